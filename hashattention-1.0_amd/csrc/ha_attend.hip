@@ -1,0 +1,470 @@
+// Decode attention kernels (gfx950, wave64): gather-only sparse attend, dense flash-decode, split merge.
+//
+// Row layout: one K or V row is 128 elements; a 16-lane quarter-wave ("row group") owns one row at
+// a time, lane `sub` holding elements [8*sub, 8*sub+8) fetched with 128-bit loads, so one wave
+// load instruction brings in four whole rows.  A workgroup of 256 threads runs 16 such row streams,
+// each keeping its own online softmax (m, l, acc[8]) in registers in the log2 domain; the streams
+// are merged through LDS at the end, and workgroups of one row's split are merged by
+// merge_splits_kernel with the usual log-sum-exp algebra.
+#include "ha_common.h"
+
+namespace {
+
+constexpr int kAttThreads = 256;
+constexpr int kStreams = kAttThreads / 16;  // 16 row streams per workgroup
+constexpr int kUnroll = 4;                  // rows in flight per stream (K and V: 8 x 128-bit loads per lane)
+constexpr float kLog2e = 1.4426950408889634f;
+
+// sum over the 16 lanes of a DPP row; every lane ends with the total
+__device__ __forceinline__ float row16_sum(float x) {
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xF, 0xF, true));  // row_mirror
+    return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+struct SparsePlan {
+    int split_rows;  // selected rows per workgroup, multiple of kStreams
+    int nsplit_max;
+};
+inline SparsePlan sparse_plan(int B, int H, int64_t idx_cap) {
+    SparsePlan p;
+    const int64_t wg256 = (int64_t)B * H * ((idx_cap + 255) / 256);
+    p.split_rows = wg256 >= 1024 ? 256 : 128;
+    p.nsplit_max = (int)((idx_cap + p.split_rows - 1) / p.split_rows);
+    if (p.nsplit_max < 1) p.nsplit_max = 1;
+    return p;
+}
+
+struct DensePlan {
+    int chunk;  // tokens per workgroup, multiple of 256
+    int nsplit_max;
+};
+inline DensePlan dense_plan(int B, int Hkv, int max_seq_len) {
+    DensePlan p;
+    int want = (2048 + B * Hkv - 1) / (B * Hkv);
+    if (want < 1) want = 1;
+    int64_t chunk = ((int64_t)max_seq_len + want - 1) / want;
+    chunk = (chunk + 255) / 256 * 256;
+    if (chunk < 256) chunk = 256;
+    p.chunk = (int)chunk;
+    p.nsplit_max = (max_seq_len + p.chunk - 1) / p.chunk;
+    if (p.nsplit_max < 1) p.nsplit_max = 1;
+    return p;
+}
+
+// Merge the 16 streams of a workgroup.  s_m/s_l [kStreams], s_acc [kStreams][128].  Thread e < 128 returns
+// the merged (m, l, acc_e).
+__device__ __forceinline__ void merge_streams(const float *s_m, const float *s_l, const float *s_acc, int e, float &M, float &L,
+                                              float &A) {
+    M = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kStreams; ++s) M = fmaxf(M, s_m[s]);
+    L = 0.f;
+    A = 0.f;
+#pragma unroll
+    for (int s = 0; s < kStreams; ++s) {
+        const float w = (s_m[s] == -INFINITY) ? 0.f : fast_exp2(s_m[s] - M);
+        L += w * s_l[s];
+        A += w * s_acc[s * HA_HEAD_DIM + e];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
+template <typename E>
+__global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+                                                                    const void *__restrict__ k, const void *__restrict__ v,
+                                                                    int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int G,
+                                                                    const int32_t *__restrict__ idx, int64_t idx_cap,
+                                                                    const int32_t *__restrict__ counts, float scale_log2e,
+                                                                    int split_rows, int nsplit_max, float *__restrict__ part_acc,
+                                                                    float *__restrict__ part_ml, void *__restrict__ out) {
+    using EL = Elem<E>;
+    __shared__ float s_m[kStreams], s_l[kStreams];
+    __shared__ float s_acc[kStreams * HA_HEAD_DIM];
+
+    const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
+    int64_t n = counts[b * H + h];
+    if (n > idx_cap) n = idx_cap;
+    const int nsplit = n > 0 ? (int)((n + split_rows - 1) / split_rows) : 1;
+    if (sp >= nsplit) return;
+    const int64_t row = (int64_t)b * H + h;
+    if (n == 0) {  // empty sequence: defined as a zero output
+        if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+        return;
+    }
+    const int r0 = sp * split_rows, r1 = (int)min((int64_t)r0 + split_rows, n);
+    const int32_t *ix = idx + row * idx_cap;
+    const char *kb = (const char *)k + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
+    const char *vb = (const char *)v + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
+    const int64_t row_bytes = kv_ss * EL::bytes;
+
+    float qf[8];
+    {
+        float t[8];
+        EL::unpack(EL::load8((const char *)q + (b * q_sb + h * q_sh) * EL::bytes, sub), t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[i] = t[i] * scale_log2e;
+    }
+
+    float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+
+    for (int base = r0 + stream; base < r1; base += kStreams * kUnroll) {
+        int32_t jj[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int r = base + u * kStreams;
+            ok[u] = r < r1;
+            jj[u] = ix[ok[u] ? r : base];
+        }
+        Raw8<E> kr[kUnroll], vr[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) kr[u] = EL::load8(kb + jj[u] * row_bytes, sub);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + jj[u] * row_bytes, sub);
+
+        float sc[kUnroll], mloc = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float kf[8], d = 0.f;
+            EL::unpack(kr[u], kf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
+            d = row16_sum(d);
+            sc[u] = ok[u] ? d : -INFINITY;
+            mloc = fmaxf(mloc, sc[u]);
+        }
+        const float m_new = fmaxf(m, mloc);
+        const float alpha = fast_exp2(m - m_new);  // m == -inf on the first pass gives 0
+        l *= alpha;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const float p = fast_exp2(sc[u] - m_new);
+            float vf[8];
+            EL::unpack(vr[u], vf);
+            l += p;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, vf[i], acc[i]);
+        }
+        m = m_new;
+    }
+
+    if (sub == 0) {
+        s_m[stream] = m;
+        s_l[stream] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_acc[stream * HA_HEAD_DIM + sub * 8 + i] = acc[i];
+    __syncthreads();
+    if (tid < HA_HEAD_DIM) {
+        float M, L, A;
+        merge_streams(s_m, s_l, s_acc, tid, M, L, A);
+        if (nsplit == 1) {
+            EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
+        } else {
+            const int64_t p = row * nsplit_max + sp;
+            part_acc[p * HA_HEAD_DIM + tid] = A;
+            if (tid == 0) {
+                part_ml[p * 2] = M;
+                part_ml[p * 2 + 1] = L;
+            }
+        }
+    }
+}
+
+// grid (H, B), 128 threads.  n_of_row: number of attended units of the row (selected tokens / keys);
+// rows with a single split were finished by the attend kernel.
+template <typename E>
+__global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
+                                                                   const int32_t *__restrict__ counts, int per_batch,
+                                                                   int64_t count_cap, int H, int unit, int nsplit_max,
+                                                                   void *__restrict__ out) {
+    using EL = Elem<E>;
+    const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
+    const int64_t row = (int64_t)b * H + h;
+    // counts is per (b, h) row, per sequence (per_batch), or absent (every row has count_cap units)
+    int64_t n = counts ? counts[per_batch ? b : row] : count_cap;
+    if (n > count_cap) n = count_cap;
+    const int nsplit = (int)((n + unit - 1) / unit);
+    if (nsplit <= 1) return;
+    const float *ml = part_ml + row * nsplit_max * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[s * 2]);
+    float L = 0.f, A = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float w = fast_exp2(ml[s * 2] - M);
+        L += w * ml[s * 2 + 1];
+        A += w * part_acc[(row * nsplit_max + s) * HA_HEAD_DIM + e];
+    }
+    EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, A / L);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Dense flash-decode.  grid (nsplit_max, Hkv, B).  A workgroup streams `chunk` consecutive keys of one
+// KV head once and scores them against the G query heads of the group.
+template <typename E, int G>
+__global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+                                                                   const void *__restrict__ k, const void *__restrict__ v,
+                                                                   int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int max_S,
+                                                                   const int32_t *__restrict__ seq_lens, float scale_log2e, int chunk,
+                                                                   int nsplit_max, float *__restrict__ part_acc,
+                                                                   float *__restrict__ part_ml, void *__restrict__ out) {
+    using EL = Elem<E>;
+    __shared__ float s_m[kStreams], s_l[kStreams];
+    __shared__ float s_acc[kStreams * HA_HEAD_DIM];
+
+    const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
+    int S = seq_lens ? seq_lens[b] : max_S;
+    if (S > max_S) S = max_S;
+    const int nsplit = S > 0 ? (S + chunk - 1) / chunk : 1;
+    if (sp >= nsplit) return;
+    if (S == 0) {
+        if (tid < HA_HEAD_DIM)
+            for (int g = 0; g < G; ++g) EL::store1((char *)out + ((int64_t)b * H + hk * G + g) * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+        return;
+    }
+    const int r0 = sp * chunk, r1 = min(r0 + chunk, S);
+    const char *kb = (const char *)k + (b * kv_sb + hk * kv_sh) * EL::bytes;
+    const char *vb = (const char *)v + (b * kv_sb + hk * kv_sh) * EL::bytes;
+    const int64_t row_bytes = kv_ss * EL::bytes;
+
+    float qf[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float t[8];
+        EL::unpack(EL::load8((const char *)q + (b * q_sb + (hk * G + g) * q_sh) * EL::bytes, sub), t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[g][i] = t[i] * scale_log2e;
+    }
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+    }
+
+    for (int base = r0 + stream; base < r1; base += kStreams * kUnroll) {
+        bool ok[kUnroll];
+        Raw8<E> kr[kUnroll], vr[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int r = base + u * kStreams;
+            ok[u] = r < r1;
+            kr[u] = EL::load8(kb + (ok[u] ? r : base) * row_bytes, sub);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + (ok[u] ? base + u * kStreams : base) * row_bytes, sub);
+
+        float sc[G][kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float kf[8];
+            EL::unpack(kr[u], kf);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float d = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
+                d = row16_sum(d);
+                sc[g][u] = ok[u] ? d : -INFINITY;
+            }
+        }
+        float p[G][kUnroll];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float mloc = sc[g][0];
+#pragma unroll
+            for (int u = 1; u < kUnroll; ++u) mloc = fmaxf(mloc, sc[g][u]);
+            const float m_new = fmaxf(m[g], mloc);
+            const float alpha = fast_exp2(m[g] - m_new);
+            l[g] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                p[g][u] = fast_exp2(sc[g][u] - m_new);
+                l[g] += p[g][u];
+            }
+            m[g] = m_new;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float vf[8];
+            EL::unpack(vr[u], vf);
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p[g][u], vf[i], acc[g][i]);
+        }
+    }
+
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        __syncthreads();  // the previous head's merge has finished reading LDS
+        if (sub == 0) {
+            s_m[stream] = m[g];
+            s_l[stream] = l[g];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s_acc[stream * HA_HEAD_DIM + sub * 8 + i] = acc[g][i];
+        __syncthreads();
+        if (tid < HA_HEAD_DIM) {
+            float M, L, A;
+            merge_streams(s_m, s_l, s_acc, tid, M, L, A);
+            const int64_t row = (int64_t)b * H + hk * G + g;
+            if (nsplit == 1) {
+                EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
+            } else {
+                const int64_t pi = row * nsplit_max + sp;
+                part_acc[pi * HA_HEAD_DIM + tid] = A;
+                if (tid == 0) {
+                    part_ml[pi * 2] = M;
+                    part_ml[pi * 2 + 1] = L;
+                }
+            }
+        }
+    }
+}
+
+int validate_qkv(const void *q, int64_t q_sb, int64_t q_sh, const void *k, const void *v, int kv_dtype, int64_t kv_sb, int64_t kv_sh,
+                 int64_t kv_ss, int B, int H, int Hkv, const void *out) {
+    HA_REQUIRE(q && k && v && out, HA_ERR_NULL_POINTER, "q/k/v/out is NULL");
+    HA_REQUIRE(kv_dtype == HA_F32 || kv_dtype == HA_BF16 || kv_dtype == HA_F16, HA_ERR_BAD_DTYPE, "kv_dtype %d", kv_dtype);
+    HA_REQUIRE(B > 0 && H > 0 && Hkv > 0 && B <= 65535 && H <= 65535, HA_ERR_BAD_SHAPE, "B, H, Hkv must be in 1..65535");
+    HA_REQUIRE(H % Hkv == 0, HA_ERR_BAD_SHAPE, "H=%d not a multiple of Hkv=%d", H, Hkv);
+    HA_REQUIRE(kv_ss >= HA_HEAD_DIM && kv_sh >= 0 && kv_sb >= 0 && q_sh >= HA_HEAD_DIM && q_sb >= 0, HA_ERR_BAD_SHAPE,
+               "strides smaller than a 128-element row");
+    const int eb = ha_dtype_bytes(kv_dtype);
+    HA_REQUIRE(ha_aligned(q, 16) && ha_aligned(k, 16) && ha_aligned(v, 16) && ha_aligned(out, 16), HA_ERR_MISALIGNED,
+               "q/k/v/out must be 16-byte aligned");
+    HA_REQUIRE((kv_ss * eb) % 16 == 0 && (kv_sh * eb) % 16 == 0 && (kv_sb * eb) % 16 == 0 && (q_sh * eb) % 16 == 0 &&
+                   (q_sb * eb) % 16 == 0,
+               HA_ERR_MISALIGNED, "strides must keep rows 16-byte aligned");
+    return HA_OK;
+}
+
+size_t part_bytes(int64_t rows, int nsplit_max) { return (size_t)rows * nsplit_max * (HA_HEAD_DIM + 2) * sizeof(float); }
+
+}  // namespace
+
+extern "C" {
+
+size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap) {
+    if (B <= 0 || H <= 0 || idx_cap <= 0) return 0;
+    return part_bytes((int64_t)B * H, sparse_plan(B, H, idx_cap).nsplit_max);
+}
+
+int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                     int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, const int32_t *idx,
+                     int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace, size_t workspace_bytes,
+                     void *stream) {
+    int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
+    if (st) return st;
+    HA_REQUIRE(idx && counts, HA_ERR_NULL_POINTER, "idx/counts is NULL");
+    HA_REQUIRE(idx_cap > 0, HA_ERR_BAD_SHAPE, "idx_cap must be positive");
+    const size_t need = ha_sparse_decode_workspace_bytes(B, H, idx_cap);
+    HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "sparse decode workspace: need %zu bytes, got %zu", need,
+               workspace ? workspace_bytes : (size_t)0);
+    HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "workspace must be 256-byte aligned");
+    if ((st = ha_require_device())) return st;
+
+    const SparsePlan plan = sparse_plan(B, H, idx_cap);
+    const int64_t rows = (int64_t)B * H;
+    float *part_acc = (float *)workspace;
+    float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(plan.nsplit_max, H, B), mgrid(H, B);
+    const float sl2 = sm_scale * kLog2e;
+    const int G = H / Hkv;
+#define HA_SPARSE_LAUNCH(E_)                                                                                                      \
+    do {                                                                                                                          \
+        hipLaunchKernelGGL(sparse_attend_kernel<E_>, grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v, kv_stride_b, \
+                           kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows, plan.nsplit_max, part_acc, \
+                           part_ml, out);                                                                                         \
+        HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
+        if (plan.nsplit_max > 1) {                                                                                                \
+            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
+                               plan.split_rows, plan.nsplit_max, out);                                                            \
+            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
+        }                                                                                                                         \
+    } while (0)
+    if (kv_dtype == HA_BF16) HA_SPARSE_LAUNCH(ElemBF16);
+    else if (kv_dtype == HA_F16) HA_SPARSE_LAUNCH(ElemF16);
+    else HA_SPARSE_LAUNCH(ElemF32);
+#undef HA_SPARSE_LAUNCH
+    return HA_OK;
+}
+
+size_t ha_dense_decode_workspace_bytes(int B, int H, int max_seq_len) {
+    if (B <= 0 || H <= 0 || max_seq_len <= 0) return 0;
+    // the plan depends on Hkv only through the workgroup count; size for the worst case Hkv = 1
+    int worst = 1;
+    for (int hkv = 1; hkv <= H; hkv *= 2) {
+        const int ns = dense_plan(B, hkv, max_seq_len).nsplit_max;
+        if (ns > worst) worst = ns;
+    }
+    return part_bytes((int64_t)B * H, worst);
+}
+
+int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                    int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, int max_seq_len,
+                    const int32_t *seq_lens, float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
+    if (st) return st;
+    HA_REQUIRE(max_seq_len > 0, HA_ERR_BAD_SHAPE, "max_seq_len must be positive");
+    const int G = H / Hkv;
+    HA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, HA_ERR_BAD_SHAPE, "H/Hkv=%d, must be 1, 2, 4 or 8", G);
+    const DensePlan plan = dense_plan(B, Hkv, max_seq_len);
+    const size_t need = part_bytes((int64_t)B * H, plan.nsplit_max);
+    HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "dense decode workspace: need %zu bytes, got %zu", need,
+               workspace ? workspace_bytes : (size_t)0);
+    HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "workspace must be 256-byte aligned");
+    if ((st = ha_require_device())) return st;
+
+    const int64_t rows = (int64_t)B * H;
+    float *part_acc = (float *)workspace;
+    float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(plan.nsplit_max, Hkv, B), mgrid(H, B);
+    const float sl2 = sm_scale * kLog2e;
+#define HA_DENSE_LAUNCH(E_, G_)                                                                                                    \
+    do {                                                                                                                           \
+        hipLaunchKernelGGL((dense_attend_kernel<E_, G_>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,          \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, plan.chunk, plan.nsplit_max,      \
+                           part_acc, part_ml, out);                                                                                \
+        HA_CHECK_LAUNCH("dense_attend_kernel");                                                                                    \
+        if (plan.nsplit_max > 1) {                                                                                                 \
+            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, seq_lens, 1,            \
+                               (int64_t)max_seq_len, H, plan.chunk, plan.nsplit_max, out);                                         \
+            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                                \
+        }                                                                                                                          \
+    } while (0)
+#define HA_DENSE_DISPATCH(E_)                \
+    do {                                     \
+        if (G == 1) HA_DENSE_LAUNCH(E_, 1);  \
+        else if (G == 2) HA_DENSE_LAUNCH(E_, 2); \
+        else if (G == 4) HA_DENSE_LAUNCH(E_, 4); \
+        else HA_DENSE_LAUNCH(E_, 8);         \
+    } while (0)
+    if (kv_dtype == HA_BF16) HA_DENSE_DISPATCH(ElemBF16);
+    else if (kv_dtype == HA_F16) HA_DENSE_DISPATCH(ElemF16);
+    else HA_DENSE_DISPATCH(ElemF32);
+#undef HA_DENSE_DISPATCH
+#undef HA_DENSE_LAUNCH
+    return HA_OK;
+}
+
+}  // extern "C"

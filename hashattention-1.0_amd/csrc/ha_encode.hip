@@ -1,0 +1,142 @@
+// Hash-MLP encode into packed sign codes (gfx950): the scalar-FMA kernel used at decode time
+// (a handful of new keys and queries per step) and as the exact-arithmetic path.
+//
+// One workgroup = one MLP head x a tile of kRows input rows.  Thread o owns output neuron o of
+// every layer; weights are read transposed ([in][out], coalesced over o) and reused for the
+// kRows rows held in LDS.  Arithmetic is fixed so results are reproducible bit for bit:
+//   acc = bias[o]; for k ascending: acc = fmaf(x[k], W[k][o], acc); SiLU(a) = a / (1 + expf(-a)).
+// HA_ARITH_BF16 additionally rounds the input, every Linear output and every SiLU output to bf16,
+// which is what a hash module kept in bf16 computes.
+#include "ha_common.h"
+
+namespace {
+
+constexpr int kEncThreads = 128;
+constexpr int kRows = 8;
+constexpr int kMaxDim = 256;
+
+__global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__restrict__ x, int x_dtype, int64_t x_sb, int64_t x_sh,
+                                                                  int64_t x_st, int B, int x_heads, int n_heads, int T,
+                                                                  const float *__restrict__ weights, int64_t per_head, int n_layers,
+                                                                  int d_in, int d_int, int d_out, int arith,
+                                                                  uint32_t *__restrict__ codes, int64_t c_sb, int64_t c_sh, int pos0,
+                                                                  const int32_t *__restrict__ pos_dev, float *__restrict__ logits) {
+    __shared__ float s_buf[2][kRows][kMaxDim];
+    const int head = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+    const int in_head = head / (n_heads / x_heads);
+    const int64_t n_rows = (int64_t)B * T;
+    const int64_t row0 = (int64_t)tile * kRows;
+
+    for (int i = tid; i < kRows * d_in; i += kEncThreads) {
+        const int r = i / d_in, e = i % d_in;
+        const int64_t row = row0 + r;
+        float val = 0.f;
+        if (row < n_rows) {
+            const int64_t b = row / T, t = row % T;
+            val = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
+            if (arith == HA_ARITH_BF16) val = ha_round_bf16(val);
+        }
+        s_buf[0][r][e] = val;
+    }
+    __syncthreads();
+
+    const float *w = weights + head * per_head;
+    int cur = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        const int in = (l == 0) ? d_in : d_int;
+        const int out = (l == n_layers - 1) ? d_out : d_int;
+        const float *Wt = w, *bias = w + (int64_t)in * out;
+        w += (int64_t)in * out + out;
+        for (int o = tid; o < out; o += kEncThreads) {
+            float acc[kRows];
+            const float bo = bias[o];
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) acc[r] = bo;
+            for (int kk = 0; kk < in; ++kk) {
+                const float wv = Wt[(int64_t)kk * out + o];
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) acc[r] = fmaf(s_buf[cur][r][kk], wv, acc[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                float a = acc[r];
+                if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
+                if (l + 1 < n_layers) {
+                    a = a / (1.0f + expf(-a));
+                    if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
+                }
+                s_buf[cur ^ 1][r][o] = a;
+            }
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // sign bits -> words.  Wave w packs output dims [64w, 64w+64): ballot low half = word 2w, high half = word 2w+1.
+    const int W = d_out / 32;
+    const int wave = tid >> 6, lane = tid & 63;
+    for (int r = 0; r < kRows; ++r) {
+        const int64_t row = row0 + r;
+        if (row >= n_rows) break;  // uniform
+        const int64_t b = row / T, t = row % T;
+        const bool bit = tid < d_out && s_buf[cur][r][tid] > 0.0f;
+        const uint64_t bal = __ballot(bit);
+        if (logits && tid < d_out) logits[((b * n_heads + head) * T + t) * d_out + tid] = s_buf[cur][r][tid];
+        const int64_t pos = (pos_dev ? pos_dev[b] : pos0) + t;
+        uint32_t *c = codes + b * c_sb + head * c_sh + pos * W;
+        if (lane == 0 && wave * 2 < W) c[wave * 2] = (uint32_t)bal;
+        if (lane == 32 && wave * 2 + 1 < W) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
+    }
+}
+
+int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const void *weights, int n_layers, int head_dim,
+                    int int_dim, int final_dim, const uint32_t *codes, int64_t c_sb, int64_t c_sh, int pos0) {
+    HA_REQUIRE(x && weights && codes, HA_ERR_NULL_POINTER, "x/weights/codes is NULL");
+    HA_REQUIRE(B > 0 && x_heads > 0 && n_heads > 0 && T > 0, HA_ERR_BAD_SHAPE, "B, x_heads, n_heads, T must be positive");
+    HA_REQUIRE(n_heads <= 65535, HA_ERR_BAD_SHAPE, "n_heads is limited to 65535");
+    HA_REQUIRE(n_heads % x_heads == 0, HA_ERR_BAD_SHAPE, "n_heads=%d not a multiple of x_heads=%d", n_heads, x_heads);
+    HA_REQUIRE(n_layers >= 1 && n_layers <= 3, HA_ERR_BAD_SHAPE, "n_layers=%d, must be 1..3", n_layers);
+    HA_REQUIRE(head_dim > 0 && head_dim <= kMaxDim && int_dim > 0 && int_dim <= kMaxDim, HA_ERR_BAD_SHAPE,
+               "head_dim and int_dim must be in 1..%d", kMaxDim);
+    HA_REQUIRE(final_dim == 32 || final_dim == 64, HA_ERR_BAD_SHAPE, "final_dim=%d, must be 32 or 64", final_dim);
+    HA_REQUIRE(pos0 >= 0, HA_ERR_BAD_SHAPE, "pos0 must be non-negative");
+    HA_REQUIRE(c_sh >= 0 && c_sb >= 0, HA_ERR_BAD_SHAPE, "negative code stride");
+    HA_REQUIRE(ha_aligned(codes, 4) && ha_aligned(weights, 4), HA_ERR_MISALIGNED, "codes/weights misaligned");
+    return HA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t ha_usa_packed_floats(int n_layers, int head_dim, int int_dim, int final_dim) {
+    if (n_layers < 1 || n_layers > 3 || head_dim <= 0 || int_dim <= 0 || final_dim <= 0) return 0;
+    int64_t n = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        const int64_t in = (l == 0) ? head_dim : int_dim, out = (l == n_layers - 1) ? final_dim : int_dim;
+        n += in * out + out;
+    }
+    return n;
+}
+
+int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t, int B, int x_heads,
+                   int n_heads, int T, const float *weights, int n_layers, int head_dim, int int_dim, int final_dim, int arith,
+                   uint32_t *codes, int64_t c_stride_b, int64_t c_stride_h, int pos0, const int32_t *pos_dev, float *logits,
+                   void *stream) {
+    int st = validate_encode(x, B, x_heads, n_heads, T, weights, n_layers, head_dim, int_dim, final_dim, codes, c_stride_b,
+                             c_stride_h, pos0);
+    if (st) return st;
+    HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
+    HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
+    const int64_t tiles = ((int64_t)B * T + kRows - 1) / kRows;
+    HA_REQUIRE(tiles <= 2147483647LL, HA_ERR_BAD_SHAPE, "too many rows for one launch");
+    if ((st = ha_require_device())) return st;
+    const int64_t per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    hipLaunchKernelGGL(encode_pack_kernel, dim3((unsigned)tiles, n_heads), dim3(kEncThreads), 0, (hipStream_t)stream, x, x_dtype,
+                       x_stride_b, x_stride_h, x_stride_t, B, x_heads, n_heads, T, weights, per_head, n_layers, head_dim, int_dim,
+                       final_dim, arith, codes, c_stride_b, c_stride_h, pos0, pos_dev, logits);
+    HA_CHECK_LAUNCH("encode_pack_kernel");
+    return HA_OK;
+}
+
+}  // extern "C"

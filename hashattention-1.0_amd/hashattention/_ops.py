@@ -1,0 +1,240 @@
+"""ctypes binding of libhashattn.so (the C ABI declared in include/hashattn.h).
+
+Every wrapper takes torch tensors that already live on the GPU, passes raw pointers, sizes and
+the current HIP stream, and raises `HashAttnError` on a non-zero status.  There is no CPU
+fallback: without the built library, or without a GPU, the calls fail loudly.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Tuple
+
+import torch
+
+_LIB_NAME = "libhashattn.so"
+_lib = None
+
+HA_F32, HA_BF16, HA_F16 = 0, 1, 2
+HA_ARITH_F32, HA_ARITH_BF16 = 0, 1
+HA_SELECT_SIMPLE, HA_SELECT_THRESHOLD = 0, 1
+
+_DTYPE = {torch.float32: HA_F32, torch.bfloat16: HA_BF16, torch.float16: HA_F16}
+
+
+class HashAttnError(RuntimeError):
+    def __init__(self, status: int, where: str, detail: str):
+        self.status = status
+        super().__init__(f"{where} failed with status {status}: {detail}")
+
+
+def lib_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+
+def load_library() -> C.CDLL:
+    """Load the built library once; raise if it has not been built (no silent fallback)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python hashattention-1.0_amd/build.py` "
+                          "(hipcc --offload-arch=gfx950); there is no CPU fallback")
+    lib = C.CDLL(path)
+    vp, i32, i64, f32, f64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_double, C.c_size_t
+    lib.ha_version.restype = i32
+    lib.ha_status_string.restype = C.c_char_p
+    lib.ha_status_string.argtypes = [i32]
+    lib.ha_last_error_string.restype = C.c_char_p
+    lib.ha_device_count.restype = i32
+    lib.ha_usa_packed_floats.restype = i64
+    lib.ha_usa_packed_floats.argtypes = [i32, i32, i32, i32]
+    lib.ha_encode_pack.restype = i32
+    lib.ha_encode_pack.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32, i32,
+                                   vp, i64, i64, i32, vp, vp, vp]
+    lib.ha_encode_pack_prefill.restype = i32
+    lib.ha_encode_pack_prefill.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32,
+                                           vp, i64, i64, i32, vp, vp]
+    lib.ha_hamming_score.restype = i32
+    lib.ha_hamming_score.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, vp, vp]
+    lib.ha_select_workspace_bytes.restype = sz
+    lib.ha_select_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
+    lib.ha_select.restype = i32
+    lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32,
+                              vp, i64, vp, vp, sz, vp]
+    lib.ha_sparse_decode_workspace_bytes.restype = sz
+    lib.ha_sparse_decode_workspace_bytes.argtypes = [i32, i32, i64]
+    lib.ha_sparse_decode.restype = i32
+    lib.ha_sparse_decode.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
+                                     vp, vp, sz, vp]
+    lib.ha_dense_decode_workspace_bytes.restype = sz
+    lib.ha_dense_decode_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.ha_dense_decode.restype = i32
+    lib.ha_dense_decode.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, f32,
+                                    vp, vp, sz, vp]
+    _lib = lib
+    return lib
+
+
+def _check(status: int, where: str):
+    if status != 0:
+        raise HashAttnError(status, where, load_library().ha_last_error_string().decode())
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("hashattention ops take GPU tensors only (there is no CPU path)")
+
+
+def workspace(nbytes: int, device) -> torch.Tensor:
+    """A byte buffer of at least nbytes (torch's allocator returns >= 256-byte aligned blocks)."""
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+# ------------------------------------------------------------------------------------------ encode
+
+def pack_usa_weights(layers_per_head, device=None) -> torch.Tensor:
+    """[[(W [out,in], b [out]), ...] per head] -> fp32 blob [n_heads, per_head]: W^T [in][out] then b, per layer."""
+    blobs = []
+    for layers in layers_per_head:
+        parts = []
+        for (W, b) in layers:
+            parts.append(W.detach().float().t().contiguous().reshape(-1))
+            parts.append(b.detach().float().reshape(-1))
+        blobs.append(torch.cat(parts))
+    out = torch.stack(blobs).contiguous()
+    return out.to(device) if device is not None else out
+
+
+def pack_usa_weights_bf16(layers_per_head, device=None) -> torch.Tensor:
+    """Blob for the MFMA encoder: per layer W [out][in] (native nn.Linear orientation) then b, in bf16."""
+    blobs = []
+    for layers in layers_per_head:
+        parts = []
+        for (W, b) in layers:
+            parts.append(W.detach().to(torch.bfloat16).contiguous().reshape(-1))
+            parts.append(b.detach().to(torch.bfloat16).reshape(-1))
+        blobs.append(torch.cat(parts))
+    out = torch.stack(blobs).contiguous()
+    return out.to(device) if device is not None else out
+
+
+def encode_pack(x: torch.Tensor, weights: torch.Tensor, n_layers: int, int_dim: int, final_dim: int,
+                codes: torch.Tensor, pos0: int = 0, pos_dev: Optional[torch.Tensor] = None,
+                arith: int = HA_ARITH_F32, want_logits: bool = False) -> Optional[torch.Tensor]:
+    """x [B, x_heads, T, d]; weights [n_heads, per_head] fp32; codes [B, n_heads, S_cap, W] int32 (written in place)."""
+    _require_cuda(x, weights, codes, pos_dev)
+    lib = load_library()
+    B, xh, T, d = x.shape
+    n_heads = weights.shape[0]
+    assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3]
+    assert codes.dtype == torch.int32 and weights.dtype == torch.float32 and weights.is_contiguous()
+    assert weights.shape[1] == lib.ha_usa_packed_floats(n_layers, d, int_dim, final_dim)
+    if pos_dev is None:
+        assert pos0 + T <= codes.shape[2]
+    logits = torch.empty(B, n_heads, T, final_dim, dtype=torch.float32, device=x.device) if want_logits else None
+    _check(lib.ha_encode_pack(_ptr(x), _DTYPE[x.dtype], x.stride(0), x.stride(1), x.stride(2), B, xh, n_heads, T,
+                              _ptr(weights), n_layers, d, int_dim, final_dim, arith,
+                              _ptr(codes), codes.stride(0), codes.stride(1), pos0, _ptr(pos_dev), _ptr(logits), _stream(x)),
+           "ha_encode_pack")
+    return logits
+
+
+def encode_pack_prefill(x: torch.Tensor, weights_bf16: torch.Tensor, n_layers: int, int_dim: int, final_dim: int,
+                        codes: torch.Tensor, pos0: int = 0, pos_dev: Optional[torch.Tensor] = None) -> None:
+    """bf16 MFMA bulk encode; same tensor conventions as `encode_pack`, weights from `pack_usa_weights_bf16`."""
+    _require_cuda(x, weights_bf16, codes, pos_dev)
+    lib = load_library()
+    B, xh, T, d = x.shape
+    n_heads = weights_bf16.shape[0]
+    assert x.dtype == torch.bfloat16 and weights_bf16.dtype == torch.bfloat16 and weights_bf16.is_contiguous()
+    assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3] and codes.dtype == torch.int32
+    if pos_dev is None:
+        assert pos0 + T <= codes.shape[2]
+    _check(lib.ha_encode_pack_prefill(_ptr(x), x.stride(0), x.stride(1), x.stride(2), B, xh, n_heads, T,
+                                      _ptr(weights_bf16), n_layers, d, int_dim, final_dim,
+                                      _ptr(codes), codes.stride(0), codes.stride(1), pos0, _ptr(pos_dev), _stream(x)),
+           "ha_encode_pack_prefill")
+
+
+# ------------------------------------------------------------------------------------------ score / select
+
+def hamming_score(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int,
+                  seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """kcodes [B, Hc, S_cap, W] int32, qcodes [B, H, W] int32 -> uint8 [B, H, max_seq_len] (rows >= seq_len are 255)."""
+    _require_cuda(kcodes, qcodes, seq_lens)
+    lib = load_library()
+    B, Hc, _, W = kcodes.shape
+    H = qcodes.shape[1]
+    assert qcodes.is_contiguous() and kcodes.stride(3) == 1 and kcodes.stride(2) == W
+    scores = torch.full((B, H, max_seq_len), 255, dtype=torch.uint8, device=kcodes.device)
+    _check(lib.ha_hamming_score(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
+                                _ptr(seq_lens), _ptr(scores), _stream(kcodes)), "ha_hamming_score")
+    return scores
+
+
+def select_workspace_bytes(B, H, Hc, W, max_seq_len) -> int:
+    return load_library().ha_select_workspace_bytes(B, H, Hc, W, max_seq_len)
+
+
+def select(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
+           init_budget: int, recent_budget: int, heavy_budget: float, out_idx: torch.Tensor, out_counts: torch.Tensor,
+           ws: torch.Tensor, mode: int = HA_SELECT_SIMPLE, depth: int = 0) -> None:
+    """Ascending index lists out_idx [B, H, idx_cap] int32 and out_counts [B, H] int32 (both written in place)."""
+    _require_cuda(kcodes, qcodes, seq_lens, out_idx, out_counts, ws)
+    lib = load_library()
+    B, Hc, _, W = kcodes.shape
+    H = qcodes.shape[1]
+    assert qcodes.is_contiguous() and kcodes.stride(3) == 1 and kcodes.stride(2) == W
+    assert out_idx.is_contiguous() and out_idx.dtype == torch.int32 and out_counts.is_contiguous() and out_counts.dtype == torch.int32
+    assert seq_lens is None or (seq_lens.dtype == torch.int32 and seq_lens.is_contiguous())
+    _check(lib.ha_select(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
+                         _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth,
+                         _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select")
+
+
+# ------------------------------------------------------------------------------------------ attention
+
+def sparse_decode_workspace_bytes(B, H, idx_cap) -> int:
+    return load_library().ha_sparse_decode_workspace_bytes(B, H, idx_cap)
+
+
+def _kv_args(q, k, v):
+    assert q.dim() == 3 and k.dim() == 4 and v.shape == k.shape and v.stride() == k.stride()
+    assert q.stride(2) == 1 and k.stride(3) == 1 and q.dtype == k.dtype == v.dtype
+    return (_ptr(q), q.stride(0), q.stride(1), _ptr(k), _ptr(v), _DTYPE[k.dtype], k.stride(0), k.stride(1), k.stride(2))
+
+
+def sparse_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor,
+                  sm_scale: float, out: torch.Tensor, ws: torch.Tensor) -> None:
+    """q [B,H,128]; k,v [B,Hkv,S_cap,128]; idx [B,H,idx_cap] int32; counts [B,H] int32; out [B,H,128] (in place)."""
+    _require_cuda(q, k, v, idx, counts, out, ws)
+    lib = load_library()
+    B, H, _ = q.shape
+    assert out.is_contiguous() and out.dtype == q.dtype and idx.is_contiguous() and counts.is_contiguous()
+    _check(lib.ha_sparse_decode(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
+                                float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_sparse_decode")
+
+
+def dense_decode_workspace_bytes(B, H, max_seq_len) -> int:
+    return load_library().ha_dense_decode_workspace_bytes(B, H, max_seq_len)
+
+
+def dense_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
+                 sm_scale: float, out: torch.Tensor, ws: torch.Tensor) -> None:
+    _require_cuda(q, k, v, seq_lens, out, ws)
+    lib = load_library()
+    B, H, _ = q.shape
+    assert out.is_contiguous() and out.dtype == q.dtype
+    _check(lib.ha_dense_decode(*_kv_args(q, k, v), B, H, k.shape[1], max_seq_len, _ptr(seq_lens), float(sm_scale),
+                               _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_dense_decode")

@@ -1,0 +1,165 @@
+/*
+ * hashattn.h - C ABI of the MI355X (gfx950) HashAttention sparse-decode library.
+ *
+ * The reference (xAlg-ai/HashAttention-1.0) has no FFI: its boundary is the Python module API
+ * `load_usa` / `convert_usa` (hashattention/hashattention_llama.py:633-667) whose patched attention
+ * layer runs the decode branch (:551-631) in eager PyTorch.  This header is what the patched layer
+ * of this build binds through ctypes instead; each entry names the reference code it replaces.
+ *
+ * Conventions
+ *   - every function returns HA_OK (0) or a negative ha_status; nothing throws or aborts;
+ *   - arguments are validated before the first HIP call, so bad arguments are reported
+ *     identically with or without a GPU; ha_last_error_string() holds the detail (thread-local);
+ *   - all pointers are device pointers unless named host_*; `stream` is a hipStream_t (NULL = the
+ *     null stream); calls are stream-ordered, never synchronise, never allocate: the caller owns
+ *     every buffer including workspaces (sized by the *_workspace_bytes functions);
+ *   - strides are in ELEMENTS of the tensor's type; the innermost dimension is contiguous;
+ *   - head_dim is 128; codes are W = 1 or 2 uint32 words per token (32- or 64-bit hashes);
+ *   - dtype codes: HA_F32, HA_BF16, HA_F16.
+ */
+#ifndef HASHATTN_H
+#define HASHATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HA_VERSION 100 /* 0.1.0 */
+
+typedef enum ha_status {
+    HA_OK = 0,
+    HA_ERR_NULL_POINTER = -1,
+    HA_ERR_BAD_SHAPE = -2,      /* a size, head count, word count or budget outside what the kernels support */
+    HA_ERR_BAD_DTYPE = -3,
+    HA_ERR_MISALIGNED = -4,     /* pointer or stride not aligned for 128-bit row loads */
+    HA_ERR_WORKSPACE = -5,      /* workspace missing or smaller than *_workspace_bytes() */
+    HA_ERR_NO_DEVICE = -6,      /* no HIP device visible to this process */
+    HA_ERR_HIP = -7             /* a HIP runtime call or kernel launch failed */
+} ha_status;
+
+#define HA_F32 0
+#define HA_BF16 1
+#define HA_F16 2
+
+#define HA_ARITH_F32 0  /* hash MLP in fp32 FMA chains (module kept in fp32) */
+#define HA_ARITH_BF16 1 /* activations rounded to bf16 after every Linear and SiLU (module kept in bf16) */
+
+#define HA_SELECT_SIMPLE 0    /* usa_eval_mode == 'simple': exactly k_eff heavy tokens */
+#define HA_SELECT_THRESHOLD 1 /* otherwise: every candidate within the distance threshold, ties included */
+
+int ha_version(void);
+const char *ha_status_string(int status);
+const char *ha_last_error_string(void);
+/* number of HIP devices visible (0 without a GPU); never fails */
+int ha_device_count(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Hash-MLP weights.  One head's MLP is 1-3 Linear layers head_dim -> int_dim (-> int_dim) ->
+ * final_dim with SiLU between them (USA.__init__, hashattention_llama.py:99-128).  The kernels read
+ * a packed fp32 blob per head: for each layer, W transposed to [in][out], then bias [out].
+ * ha_usa_packed_floats() is the blob length of ONE head; heads are concatenated.
+ * Limits: head_dim, int_dim <= 256; final_dim in {32, 64}.
+ */
+int64_t ha_usa_packed_floats(int n_layers, int head_dim, int int_dim, int final_dim);
+
+/*
+ * Encode rows through the per-head hash MLP and pack sign bits: bit i of a code = (logit_i > 0),
+ * least significant bit = output dim 0.  Replaces USA.k_embedding / q_embedding and the MLP +
+ * sign of USA.forward (hashattention_llama.py:159-173, 204-226) and the bit packing of
+ * efficiency/kernels/torchatt.py:55-56, 159, 183-184.
+ *
+ *   x        [B, x_heads, T, head_dim] of x_dtype, strides x_stride_{b,h,t}
+ *   weights  packed blob of n_heads heads; MLP head i reads x head i / (n_heads / x_heads)
+ *   codes    [B, n_heads, ., W] uint32, strides c_stride_{b,h} in words; token t of sequence b is
+ *            written at position pos0 + t, or pos_dev[b] + t when pos_dev (int32 [B]) is given:
+ *            this is the append into the per-layer bit-cache
+ *   logits   optional fp32 [B, n_heads, T, final_dim] contiguous (tests, diagnostics); may be NULL
+ */
+int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t,
+                   int B, int x_heads, int n_heads, int T,
+                   const float *weights, int n_layers, int head_dim, int int_dim, int final_dim, int arith,
+                   uint32_t *codes, int64_t c_stride_b, int64_t c_stride_h, int pos0, const int32_t *pos_dev,
+                   float *logits, void *stream);
+
+/*
+ * Bulk (prefill) encode on the matrix cores: the same mapping as ha_encode_pack in HA_ARITH_BF16
+ * arithmetic, computed as three chained bf16 MFMA GEMMs per 128-token tile.  x must be bf16,
+ * head_dim == int_dim == 128.  `weights_bf16` is the blob of ha_usa_packed_floats() elements per
+ * head converted to bf16 in the NATIVE nn.Linear orientation: per layer W [out][in], then bias [out].
+ * Replaces the un-timed prefill encode of efficiency/kernels/torchatt.py:183-184.
+ */
+int ha_encode_pack_prefill(const void *x, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t,
+                           int B, int x_heads, int n_heads, int T,
+                           const void *weights_bf16, int n_layers, int head_dim, int int_dim, int final_dim,
+                           uint32_t *codes, int64_t c_stride_b, int64_t c_stride_h, int pos0, const int32_t *pos_dev,
+                           void *stream);
+
+/*
+ * Hamming distance of every cached code to the query code: scores[b, h, j] =
+ * popcount(kcodes[b, h / (H/Hc), j] ^ qcodes[b, h]) for j < seq_len[b].  Diagnostic/test entry;
+ * ha_select fuses this.  Replaces efficiency/kernels/bit_count_uint32.py:4-33, bit_count_long.py:4-33
+ * and the xor of torchatt.py:58 (span = final_dim - 2 * distance, hashattention_llama.py:180-187).
+ *   kcodes [B, Hc, ., W] strides kc_stride_{b,h} words; qcodes [B, H, W] contiguous;
+ *   seq_lens int32 [B] or NULL (all = max_seq_len); scores uint8 [B, H, max_seq_len] contiguous.
+ */
+int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                     int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                     uint8_t *scores, void *stream);
+
+/*
+ * Token selection for one decode query per sequence.  For sequence length S: candidates are
+ * j in [init, S - recent); k_eff = min(heavy, #candidates) with heavy = (heavy_budget > 1) ?
+ * (int)heavy_budget : (int)(S * heavy_budget); the k_eff candidates of smallest Hamming distance
+ * (ties: lowest index) are kept together with the sink [0, init) and recent [S - recent, S)
+ * windows.  HA_SELECT_THRESHOLD keeps every candidate with distance <=
+ * min(d_min + depth, d_(k_eff)) instead.  Replaces compute_mask_multi / compute_mask
+ * (hashattention_llama.py:401-493; the sort at :430) and torch.topk of torchatt.py:46, 66.
+ *
+ *   out_idx    int32 [B, H, idx_cap]: ascending token indices; nothing is written past idx_cap
+ *   out_counts int32 [B, H]: number selected (the true count, even if it exceeds idx_cap)
+ *   workspace  ha_select_workspace_bytes(...) bytes, 256-byte aligned
+ */
+size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len);
+int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+              int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+              int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
+              int32_t *out_idx, int64_t idx_cap, int32_t *out_counts,
+              void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Gather-only decode attention: out[b, h] = softmax(q[b, h] . K[b, h/G, idx] * sm_scale) V[b, h/G, idx]
+ * over the first counts[b, h] entries of idx[b, h]; fp32 online softmax, split over the index list
+ * and merged by log-sum-exp.  Replaces flash_fwd_sparse / fwd_sparse
+ * (efficiency/kernels/flash_fwd_sparse.py:396-554, 775-815; sparse.py:12-187) and the masked dense
+ * softmax of hashattention_llama.py:585-615.
+ *   q   [B, H, 128] kv_dtype, strides q_stride_{b,h}
+ *   k,v [B, Hkv, ., 128] kv_dtype, strides kv_stride_{b,h,s}; rows 16-byte aligned
+ *   out [B, H, 128] kv_dtype contiguous
+ */
+size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap);
+int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                     const void *k, const void *v, int kv_dtype,
+                     int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                     int B, int H, int Hkv, const int32_t *idx, int64_t idx_cap, const int32_t *counts,
+                     float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).
+ * Replaces flash_decode_attention_fwd (efficiency/kernels/flash_fwd_sparse.py:21-321) and
+ * torch_attention_naive (efficiency/kernels/torchatt.py:17-30).  Each K/V row is read once per KV
+ * head and shared by the query heads of its group.
+ */
+size_t ha_dense_decode_workspace_bytes(int B, int H, int max_seq_len);
+int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                    const void *k, const void *v, int kv_dtype,
+                    int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                    int B, int H, int Hkv, int max_seq_len, const int32_t *seq_lens,
+                    float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HASHATTN_H */

@@ -1,0 +1,301 @@
+"""CPU restatement of HashAttention's sparse decode path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker the HIP kernels are compared with.  Nothing in the
+shipped package imports it: only the tests, the smoke run and the benchmark's
+CPU-baseline leg may.  Every function names the lines of the reference
+(`/root/reference`, xAlg-ai/HashAttention-1.0) whose behaviour it restates.
+
+Stages
+  usa_mlp / usa_logits      hash MLP of one head / all heads       hashattention/hashattention_llama.py:99-128, 159-169
+  usa_forward_hard          ternary sign, span = <sign q, sign k>  hashattention_llama.py:151-200, 51-55
+  pack_codes                bit i = logit_i > 0, LSB = dim 0       efficiency/kernels/torchatt.py:55-56, 159, 183-184
+  hamming                   popcount(q ^ k)                        efficiency/kernels/bit_count_uint32.py:4-12, torchatt.py:58-62
+  compute_mask_multi        sink | recent | top-k heavy mask       hashattention_llama.py:401-446
+  select_indices            the same selection as index lists (canonical lowest-index tie-break)
+  masked_decode_attention   dense QK^T, mask, fp32 softmax, AV     hashattention_llama.py:578-623
+  sparse_attend             gather-only attention                  efficiency/kernels/sparse.py:190-214
+  merge_splits              split-K log-sum-exp merge              efficiency/kernels/flash_fwd_sparse.py:451-508, 535-553
+  repeat_kv / rotate_half / apply_rotary_pos_emb   textbook restatements of the `transformers`
+                            helpers the reference imports (hashattention_llama.py:18); the reference
+                            holds no test at that boundary: parity unpinned there.
+  reference_decode_attention  the whole emulated layer-step (used as the timed CPU baseline)
+
+Tie-break.  The reference sorts with `span.sort(descending=True)` without
+`stable=True` (hashattention_llama.py:430), so which of the equal-score tokens
+fill the last places is implementation-defined.  This oracle fixes the
+canonical rule "lowest index first" (`stable=True`); `tie_invariant_equal`
+compares two masks up to that freedom.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+# --------------------------------------------------------------------------- hash MLP
+
+
+def usa_mlp(x: torch.Tensor, layers: Sequence[Tuple[torch.Tensor, torch.Tensor]]) -> torch.Tensor:
+    """`nn.Sequential(Linear, SiLU, Linear, SiLU, Linear)` of one head (1-3 Linear layers).
+
+    reference: hashattention_llama.py:99-128 (module construction), :168-169 (application).
+    """
+    h = x
+    for i, (W, b) in enumerate(layers):
+        h = F.linear(h, W.to(h.dtype), b.to(h.dtype))
+        if i + 1 < len(layers):
+            h = F.silu(h)
+    return h
+
+
+def usa_logits(x: torch.Tensor, heads: Sequence[Sequence[Tuple[torch.Tensor, torch.Tensor]]]) -> torch.Tensor:
+    """Per-head MLP over x [b, n_in_heads, t, d] -> logits [b, n_heads, t, D].
+
+    Head i of the MLP list reads input head i // (n_heads / n_in_heads): with one K MLP per
+    query head the reference feeds it `repeat_kv`'d keys (hashattention_llama.py:578, 605, 159-169),
+    i.e. KV head i // group.
+    """
+    b, n_in, t, _ = x.shape
+    n_heads = len(heads)
+    rep = n_heads // n_in
+    outs = [usa_mlp(x[:, i // rep], heads[i]) for i in range(n_heads)]
+    return torch.stack(outs, dim=1)
+
+
+def usa_forward_hard(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads) -> Tuple[torch.Tensor, torch.Tensor]:
+    """`USA.forward(K, Q, hard=True)`: span[b,h,t,s] = sum_i sign(q)_i sign(k)_i, non-causal -> finfo.min.
+
+    reference: hashattention_llama.py:151-200.  K, Q are [b, H, s|t, d] (K already repeat_kv'd).
+    torch.sign maps 0 to 0 (:55), so an exactly-zero logit contributes nothing to the span.
+    """
+    kl = usa_logits(K, k_heads)
+    ql = usa_logits(Q, q_heads)
+    ks, qs = torch.sign(kl), torch.sign(ql)
+    span = torch.einsum("bhtd,bhsd->bhts", qs, ks)
+    t, s = Q.shape[-2], K.shape[-2]
+    causal = torch.tril(torch.ones(t, s), diagonal=s - t).bool()
+    span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype))
+    return span, ks
+
+
+def pack_codes(logits: torch.Tensor) -> torch.Tensor:
+    """logits [..., D] (D multiple of 32) -> int64 tensor [..., D/32] holding uint32 words.
+
+    bit i of the code = (logit_i > 0) (`relu(sign(x))`), least significant bit = output dim 0
+    (`power = 2**arange(32)`): efficiency/kernels/torchatt.py:55-56, 159, 183-184.
+    """
+    D = logits.shape[-1]
+    assert D % 32 == 0
+    bits = (logits > 0).to(torch.int64).reshape(*logits.shape[:-1], D // 32, 32)
+    power = (2 ** torch.arange(32, dtype=torch.int64))
+    return (bits * power).sum(dim=-1)
+
+
+def popcount_u32(x: torch.Tensor) -> torch.Tensor:
+    """Element-wise population count of uint32 values held in an int64 tensor (SWAR).
+
+    reference: `__popc` kernel, efficiency/kernels/bit_count_uint32.py:4-12.
+    """
+    x = x & 0xFFFFFFFF
+    x = x - ((x >> 1) & 0x55555555)
+    x = (x & 0x33333333) + ((x >> 2) & 0x33333333)
+    x = (x + (x >> 4)) & 0x0F0F0F0F
+    return ((x * 0x01010101) & 0xFFFFFFFF) >> 24
+
+
+def hamming(qcodes: torch.Tensor, kcodes: torch.Tensor) -> torch.Tensor:
+    """qcodes [B, H, W], kcodes [B, Hc, S, W] (uint32 words in int64) -> Hamming distance [B, H, S].
+
+    Query head h is scored against code head h // (H / Hc).  The reference prototype ranks by
+    popcount(~(q ^ k)) (torchatt.py:58-66), which is monotone decreasing in this distance, and
+    the model path by span = D - 2 * hamming (hashattention_llama.py:180-187).
+    """
+    B, H, W = qcodes.shape
+    Hc = kcodes.shape[1]
+    kc = kcodes.repeat_interleave(H // Hc, dim=1)
+    x = qcodes[:, :, None, :] ^ kc
+    return popcount_u32(x).sum(dim=-1)
+
+
+# --------------------------------------------------------------------------- selection
+
+
+def heavy_count(seq_len: int, heavy_budget: float) -> int:
+    """reference: hashattention_llama.py:431-434 (fraction of the current length, or absolute if > 1)."""
+    return int(heavy_budget) if heavy_budget > 1.0 else int(seq_len * heavy_budget)
+
+
+def compute_mask_multi(span: torch.Tensor, init_budget: int, recent_budget: int, heavy_budget: float,
+                       mode: str = "simple", retrieve_depth: float = 0.0, stable: bool = True) -> torch.Tensor:
+    """Keep-mask [b, H, q, S] from span scores [b, H, q, S]; restates hashattention_llama.py:423-446.
+
+    `stable=True` is the canonical lowest-index tie-break; `stable=False` reproduces the
+    reference call verbatim (implementation-defined order among ties).
+    """
+    span = span.clone()
+    q, k = span.shape[-2], span.shape[-1]
+    chr_mask = torch.tril(torch.ones(q, k), diagonal=k - q - recent_budget).bool()
+    chr_mask[:, :init_budget] = False
+    span.masked_fill_(~chr_mask, torch.finfo(span.dtype).min)
+    mask = torch.zeros_like(span).bool()
+    mask[:, :, :, :] = torch.tril(torch.ones(q, k), diagonal=k - q).bool()
+    mask = mask * (~chr_mask)
+    values, indices = span.sort(dim=-1, descending=True, stable=stable)
+    hb = heavy_count(k, heavy_budget)
+    if mode == "simple":
+        mask.scatter_(3, indices[:, :, :, :hb], True)
+    else:
+        depth_thold = values[:, :, :, :1] - 2 * retrieve_depth
+        num_thold = values[:, :, :, hb - 1:hb]
+        mask.masked_fill_(span >= torch.maximum(depth_thold, num_thold), True)
+    return mask
+
+
+def select_indices(ham: torch.Tensor, seq_len: int, init_budget: int, recent_budget: int, heavy_budget: float,
+                   mode: str = "simple", retrieve_depth: int = 0) -> List[List[int]]:
+    """Index-set formulation of the q_len == 1 selection for one sequence.
+
+    ham: Hamming distances [H, >=seq_len]; returns one ascending list per head:
+    sink [0, init) | the k_eff = min(heavy, #candidates) candidates of [init, seq_len - recent)
+    with the smallest distance (ties: lowest index) | recent [seq_len - recent, seq_len).
+    Derived independently of `compute_mask_multi` (no tril/scatter) so each checks the other.
+    """
+    out = []
+    lo, hi = min(init_budget, seq_len), max(min(init_budget, seq_len), seq_len - recent_budget)
+    kk = min(heavy_count(seq_len, heavy_budget), hi - lo)
+    for h in range(ham.shape[0]):
+        cand = list(range(lo, hi))
+        row = ham[h].tolist()
+        if mode == "simple":
+            heavy = sorted(sorted(cand, key=lambda j: (row[j], j))[:kk])
+        elif cand and kk > 0:
+            order = sorted(row[j] for j in cand)
+            thold = min(order[0] + int(math.floor(retrieve_depth)), order[kk - 1])
+            heavy = [j for j in cand if row[j] <= thold]
+        else:
+            heavy = []
+        out.append(list(range(0, lo)) + heavy + list(range(hi, seq_len)))
+    return out
+
+
+def select_indices_np(ham: np.ndarray, seq_len: int, init_budget: int, recent_budget: int,
+                      heavy_budget: float) -> np.ndarray:
+    """Vectorised `select_indices` ('simple' mode) for full-size rows: [H, n_sel] int32, ascending."""
+    lo, hi = min(init_budget, seq_len), max(min(init_budget, seq_len), seq_len - recent_budget)
+    kk = min(heavy_count(seq_len, heavy_budget), hi - lo)
+    H = ham.shape[0]
+    cand = ham[:, lo:hi].astype(np.int64)
+    order = np.argsort(cand, axis=1, kind="stable")[:, :kk] + lo
+    order.sort(axis=1)
+    sink = np.broadcast_to(np.arange(0, lo), (H, lo))
+    recent = np.broadcast_to(np.arange(hi, seq_len), (H, seq_len - hi))
+    return np.concatenate([sink, order, recent], axis=1).astype(np.int32)
+
+
+def mask_from_indices(idx: Sequence[Sequence[int]], seq_len: int) -> torch.Tensor:
+    m = torch.zeros(len(idx), seq_len, dtype=torch.bool)
+    for h, row in enumerate(idx):
+        m[h, torch.as_tensor(list(row), dtype=torch.long)] = True
+    return m
+
+
+def tie_invariant_equal(mask_a: torch.Tensor, mask_b: torch.Tensor, score: torch.Tensor) -> bool:
+    """True when two keep-masks [.., S] agree up to the choice among equal scores.
+
+    For every row: same number kept, and the kept multiset of scores is identical.
+    """
+    if mask_a.shape != mask_b.shape or not torch.equal(mask_a.sum(-1), mask_b.sum(-1)):
+        return False
+    big = score.max().item() + 1
+    sa = torch.where(mask_a, score, torch.full_like(score, big)).sort(dim=-1).values
+    sb = torch.where(mask_b, score, torch.full_like(score, big)).sort(dim=-1).values
+    return torch.equal(sa, sb)
+
+
+# --------------------------------------------------------------------------- attention
+
+
+def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """[b, Hkv, s, d] -> [b, Hkv * n_rep, s, d], each KV head repeated n_rep times in place
+    (= repeat_interleave on dim 1); third-party `transformers` helper used at hashattention_llama.py:578-579."""
+    return x.repeat_interleave(n_rep, dim=1)
+
+
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    d = x.shape[-1] // 2
+    return torch.cat((-x[..., d:], x[..., :d]), dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin):
+    """Rotate-half RoPE (third-party helper used at hashattention_llama.py:571); cos/sin [b, t, d]."""
+    cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+    return q * cos + rotate_half(q) * sin, k * cos + rotate_half(k) * sin
+
+
+def masked_decode_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+    """Dense scores, mask to finfo.min, softmax in fp32 cast back to Q's dtype, times V.
+
+    reference: hashattention_llama.py:585, 606, 613, 615.  Q [b,H,q,d]; K,V [b,H,S,d]; mask [b,H,q,S].
+    """
+    w = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(Q.shape[-1])
+    w = w.masked_fill(~mask, torch.finfo(w.dtype).min)
+    w = F.softmax(w, dim=-1, dtype=torch.float32).to(Q.dtype)
+    return torch.matmul(w, V)
+
+
+def sparse_attend(q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, idx: Sequence[int], sm_scale: float) -> torch.Tensor:
+    """One (batch, head): softmax(q . K[idx] * scale) @ V[idx] in fp32.
+
+    reference: `torch_fwd_sparse`, efficiency/kernels/sparse.py:190-214 (fp32 softmax, zero mask).
+    q [d]; K, V [S, d].
+    """
+    ii = torch.as_tensor(np.asarray(idx), dtype=torch.long)
+    k, v = K[ii].float(), V[ii].float()
+    a = (k @ q.float()) * sm_scale
+    p = torch.softmax(a, dim=0)
+    return p @ v
+
+
+def merge_splits(part_o: torch.Tensor, part_lse: torch.Tensor) -> torch.Tensor:
+    """Merge per-split normalised outputs [n, d] with their log-sum-exp [n] into one output [d].
+
+    reference: stage-2 epilogue and stage-3 loop, efficiency/kernels/flash_fwd_sparse.py:496-508, 535-553.
+    """
+    m = part_lse.max()
+    w = torch.exp(part_lse - m)
+    return (w[:, None] * part_o).sum(0) / w.sum()
+
+
+def dense_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor) -> torch.Tensor:
+    """`torch_attention_naive`, efficiency/kernels/torchatt.py:17-30, without its final transpose."""
+    w = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(Q.shape[-1])
+    w = F.softmax(w, dim=-1, dtype=torch.float32).to(Q.dtype)
+    return torch.matmul(w, V)
+
+
+def reference_decode_attention(Q, K, V, k_heads, q_heads, init_budget, recent_budget, heavy_budget,
+                               mode="simple", retrieve_depth=0.0, stable=True, usa_dtype=None):
+    """The reference's emulated decode step between RoPE/cache update and o_proj.
+
+    reference: hashattention_llama.py:578-623 with compute_mask_multi :401-446: repeat K/V over the
+    group, dense QK^T, re-hash every key, full sort, masked fp32 softmax, AV.
+    Q [b,H,q,d]; K,V [b,Hkv,S,d].  Returns (attn_output [b,H,q,d], keep mask [b,H,q,S]).
+    """
+    H, Hkv = Q.shape[1], K.shape[1]
+    Kr, Vr = repeat_kv(K, H // Hkv), repeat_kv(V, H // Hkv)
+    ud = usa_dtype or Q.dtype
+    # the K MLP list has either one entry per query head or one per KV head
+    Kin = Kr if len(k_heads) == H else K
+    kl = usa_logits(Kin.to(ud), k_heads)
+    if kl.shape[1] != H:
+        kl = repeat_kv(kl, H // kl.shape[1])
+    ql = usa_logits(Q.to(ud), q_heads)
+    span = torch.einsum("bhtd,bhsd->bhts", torch.sign(ql), torch.sign(kl))
+    t, s = Q.shape[-2], K.shape[-2]
+    causal = torch.tril(torch.ones(t, s), diagonal=s - t).bool()
+    span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype))
+    mask = compute_mask_multi(span, init_budget, recent_budget, heavy_budget, mode, retrieve_depth, stable)
+    return masked_decode_attention(Q, Kr, Vr, mask), mask

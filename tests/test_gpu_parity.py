@@ -1,0 +1,112 @@
+"""GPU parity: every stage of the HIP decode path, called through the C ABI, against the oracle.
+
+Integer stages (codes from given logits' signs, Hamming distances, selected index lists, counts) must be
+bit-exact; attention outputs within 2e-2 max-abs for bf16/fp16 and 2e-5 for fp32 of the double-precision
+oracle.  Sizes are chosen so the oracle finishes in seconds.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.parity_util import run_decode_case, small_workload
+
+pytestmark = pytest.mark.gpu
+
+
+def _announce(name):
+    print(f"\n[case] {name}", flush=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_small_decode_all_stages(dtype):
+    _announce(f"small {dtype}")
+    run_decode_case(small_workload(dtype=dtype), verbose=True)
+
+
+def test_one_code_head_per_query_head():
+    # reference-exact layout: every query head has its own K hash MLP (hashattention_llama.py:642)
+    _announce("Hc == H")
+    run_decode_case(small_workload(n_code_heads=8, seed=11), verbose=True)
+
+
+@pytest.mark.parametrize("gq", [1, 2, 4, 8])
+def test_group_sizes(gq):
+    _announce(f"H/Hc = {gq}")
+    run_decode_case(small_workload(n_q_heads=8, n_kv_heads=8 // gq, n_code_heads=8 // gq, seed=20 + gq), verbose=True)
+
+
+def test_64bit_codes_ragged():
+    # 2-layer MLP, 64-bit codes (two words), ragged batch: the configs[4] shape in small
+    _announce("W=2 ragged")
+    w = small_workload(batch=3, seq_lens=[2300, 700, 1025], lth_num_layers=2, lth_final_dim=64, heavy_budget=1.0 / 16, seed=3)
+    run_decode_case(w, verbose=True)
+
+
+def test_one_layer_mlp():
+    _announce("1-layer MLP")
+    run_decode_case(small_workload(lth_num_layers=1, seed=5), verbose=True)
+
+
+@pytest.mark.parametrize("seq_lens", [[1], [5, 31], [32, 33], [40, 64], [1024, 1023, 1025], [2048, 4097]])
+def test_short_and_boundary_lengths(seq_lens):
+    # init = recent = 16: lengths below, at and just above init + recent; chunk boundaries of the select kernels
+    _announce(f"lengths {seq_lens}")
+    run_decode_case(small_workload(batch=len(seq_lens), seq_lens=seq_lens, seed=100 + seq_lens[0]), verbose=True)
+
+
+@pytest.mark.parametrize("heavy", [0.0, 0.5, 1.0, 40.0, 100000.0])
+def test_heavy_budget_forms(heavy):
+    # fraction of the length, 1.0 (fraction: everything), absolute count, absolute count above the candidates
+    _announce(f"heavy_budget {heavy}")
+    run_decode_case(small_workload(heavy_budget=heavy, seed=31), verbose=True)
+
+
+@pytest.mark.parametrize("init,recent", [(0, 0), (0, 16), (16, 0), (128, 128)])
+def test_window_forms(init, recent):
+    _announce(f"init {init} recent {recent}")
+    run_decode_case(small_workload(init_budget=init, recent_budget=recent, seed=41), verbose=True)
+
+
+@pytest.mark.parametrize("depth", [0, 2, 40])
+def test_threshold_mode(depth):
+    # usa_eval_mode != 'simple': every candidate within the distance threshold, all ties (hashattention_llama.py:439-443)
+    _announce(f"threshold depth {depth}")
+    run_decode_case(small_workload(seed=51), mode="threshold", depth=depth, verbose=True)
+
+
+def test_index_capacity_is_respected():
+    # a list shorter than the selection: nothing is written past idx_cap, the count still reports the full size
+    _announce("idx_cap clamp")
+    from hashattention import _ops
+    from oracle import c_oracle
+    from tests.parity_util import oracle_codes, to_i32
+    from hashattention.synthetic import make_problem
+    w = small_workload(seed=61)
+    p = make_problem(w)
+    _, _, kc64, qc64 = oracle_codes(p)
+    kc_np, qc_np = to_i32(kc64), to_i32(qc64)
+    dev = "cuda:0"
+    cap = 100
+    guard = 64
+    idx = torch.full((w.batch, w.n_q_heads, cap + guard), -7, dtype=torch.int32, device=dev)
+    view = idx[:, :, :cap]
+    # the ABI takes a contiguous [B, H, idx_cap] block: emulate a tight buffer followed by guard words
+    tight = torch.full((w.batch * w.n_q_heads * cap + guard,), -7, dtype=torch.int32, device=dev)
+    out_idx = tight[: w.batch * w.n_q_heads * cap].view(w.batch, w.n_q_heads, cap)
+    counts = torch.zeros(w.batch, w.n_q_heads, dtype=torch.int32, device=dev)
+    ws = _ops.workspace(_ops.select_workspace_bytes(w.batch, w.n_q_heads, w.n_code_heads, 1, w.max_seq_len), dev)
+    _ops.select(torch.from_numpy(kc_np).to(dev), torch.from_numpy(qc_np).to(dev), w.max_seq_len, p.seq_lens.to(dev),
+                w.init_budget, w.recent_budget, w.heavy_budget, out_idx, counts, ws)
+    ref_idx, ref_counts = c_oracle.select(kc_np, qc_np, p.seq_lens.numpy(), w.init_budget, w.recent_budget, w.heavy_budget, cap)
+    assert np.array_equal(counts.cpu().numpy(), ref_counts) and ref_counts.max() > cap
+    assert np.array_equal(out_idx.cpu().numpy(), ref_idx)
+    assert (tight[-guard:] == -7).all()
+    del view
+
+
+def test_config0_shape_fp32():
+    # configs[0]: B=1, S=4096, 32 q heads / 8 KV heads, one K hash MLP per query head, fp32, heavy 0.25
+    _announce("config0")
+    from hashattention.synthetic import named_workload
+    r = run_decode_case(named_workload("config0"), verbose=True)
+    assert r["n_selected"] == 1280

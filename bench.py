@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Benchmark of the HashAttention sparse decode step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config config2]
+
+A step is one pass of the hot path over one batch of synthetic input for a single attention layer:
+hash-encode of the new key and the query, Hamming select over the bit-cache, gather-only attention.
+The workload is the configuration the metric is quoted on (config2: Llama-3.1-8B attention shape,
+batch 16, 64K context, 32x sparse); K/V and the bit-cache are resident in HBM before timing starts.
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (os.path.join(ROOT, "hashattention-1.0_amd"), ROOT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published peak
+
+
+def algorithmic_bytes(w, n_sel_rows):
+    """Algorithmic HBM bytes of one layer-step, per stage.  n_sel_rows = sum over (b, h) of selected tokens."""
+    d, H, B = w.head_dim, w.n_q_heads, w.batch
+    eb = 2 if str(w.dtype) != "torch.float32" else 4
+    tokens = sum(w.seq_lens)
+    score = w.n_code_heads * tokens * 4 * w.code_words                  # every cached code read once
+    select = n_sel_rows * 4                                             # index lists written
+    gather = n_sel_rows * (2 * d * eb) + n_sel_rows * 4 + B * H * d * eb * 2   # K+V rows, index read, q read + out write
+    dense = w.n_kv_heads * tokens * 2 * d * eb
+    return dict(score=score, select=select, gather=gather, dense=dense)
+
+
+def time_gpu(fn, steps, warmup, torch):
+    """Average ms per call over `steps` back-to-back calls, HIP events on the stream the kernels run on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(w, torch):
+    """The oracle's restatement of the reference decode step (dense QK^T, every key re-hashed, full sort, masked
+    fp32 softmax) timed on the host for ONE sequence of the workload, scaled linearly to the batch."""
+    from hashattention.synthetic import Workload, make_problem
+    from oracle import hashattn_oracle as orc
+    w1 = Workload(**{**w.__dict__, "name": w.name + "-cpu", "batch": 1, "seq_lens": [w.seq_lens[0]]})
+    p = make_problem(w1)
+    q, k, v = p.q.float(), p.k.float(), p.v.float()
+    orc.reference_decode_attention(q[:, :, :, :], k[:, :, :4096], v[:, :, :4096], p.usa.k, p.usa.q, w.init_budget,
+                                   w.recent_budget, w.heavy_budget)     # warm-up on a prefix
+    t0 = time.perf_counter()
+    orc.reference_decode_attention(q, k, v, p.usa.k, p.usa.q, w.init_budget, w.recent_budget, w.heavy_budget)
+    dt = time.perf_counter() - t0
+    return {"value": dt * 1e6 * w.batch, "unit": "us/layer", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of {w.batch} sequences (S={w.seq_lens[0]}, fp32, torch CPU, {os.cpu_count()} logical cpus), "
+                      f"{dt:.2f} s measured, scaled x{w.batch}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="config2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the sparse decode path shards by (sequence, KV head) with no exchange, "
+              "and this build neither launches nor measures more than one GPU. Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from hashattention import _ops
+    from hashattention.decode import HashDecodeLayer
+    from hashattention.synthetic import make_problem_on_device, named_workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HashAttention path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    _ops.load_library()
+    dev = "cuda:0"
+    w = named_workload(args.config)
+    p = make_problem_on_device(w, dev)
+    B, H, Hkv, d, S = w.batch, w.n_q_heads, w.n_kv_heads, w.head_dim, w.max_seq_len
+    ragged = len(set(w.seq_lens)) > 1
+    seq_lens = p.seq_lens if ragged else None
+
+    layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, d, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
+                            w.init_budget, w.recent_budget, w.heavy_budget, device=dev)
+    layer.allocate(B, S)
+    # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
+    layer.encode_keys(p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
+    torch.cuda.synchronize()
+    layer.n_cached = S - 1                      # the step re-encodes the newest key, as a real decode step does
+    out = torch.empty(B, H, d, dtype=w.dtype, device=dev)
+    out_dense = torch.empty_like(out)
+    ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)
+    q3 = p.q[:, :, 0, :]
+
+    def step():
+        if ragged:
+            layer.step(p.q, p.k, p.v, S, out, seq_lens=seq_lens)
+        else:
+            layer.n_cached = S - 1
+            layer.step(p.q, p.k, p.v, S, out)
+
+    def encode_only():
+        layer.encode_keys(p.k[:, :, S - 1:S], pos0=S - 1)
+        layer.encode_query(p.q)
+
+    ms_step = time_gpu(step, args.steps, args.warmup, torch)
+    ms_encode = time_gpu(encode_only, args.steps, args.warmup, torch)
+    ms_select = time_gpu(lambda: layer.select(S, seq_lens), args.steps, args.warmup, torch)
+    ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
+    ms_dense = time_gpu(lambda: _ops.dense_decode(q3, p.k, p.v, S, seq_lens, layer.sm_scale, out_dense, ws_dense),
+                        max(10, args.steps // 4), max(2, args.warmup // 4), torch)
+
+    n_sel_rows = int(layer.counts.sum().item())
+    ab = algorithmic_bytes(w, n_sel_rows)
+    sparse_bytes = ab["score"] + ab["select"] + ab["gather"]
+    err = (out.float() - out_dense.float()).abs().max().item()   # informational: sparse vs dense output distance
+
+    res = {
+        "metric": "sparse_decode_us_per_layer",
+        "value": ms_step * 1e3,
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else str(w.dtype).replace("torch.", ""),
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: B={B} S={'ragged ' + str(min(w.seq_lens)) + '..' + str(S) if ragged else S} "
+                               f"H={H} Hkv={Hkv} d={d} code_heads={w.n_code_heads} code_bits={w.lth_final_dim} "
+                               f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} "
+                               f"n_sel={n_sel_rows // (B * H)}"},
+        "stages_us": {"encode_new_k_and_q": ms_encode * 1e3, "score_select": ms_select * 1e3,
+                      "gather_attend": ms_attend * 1e3, "dense_flash_decode": ms_dense * 1e3},
+        "hbm_gbps_step": sparse_bytes / (ms_step * 1e-3) / 1e9,
+        "hbm_frac_step": sparse_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "speedup_vs_dense": ms_dense / ms_step,
+        "dense_hbm_gbps": ab["dense"] / (ms_dense * 1e-3) / 1e9,
+        "tokens_per_s_layer": B / (ms_step * 1e-3),
+        "sparse_vs_dense_max_abs": err,
+        "roofline": {"kernel": "sparse_attend_kernel (+ split merge)", "bound": "hbm",
+                     "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(w, torch)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

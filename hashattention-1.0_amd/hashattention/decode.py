@@ -1,0 +1,120 @@
+"""Per-layer state and launch sequence of the sparse decode step.
+
+`HashDecodeLayer` owns what the reference's patched attention layer recomputes from scratch every step
+(hashattention/hashattention_llama.py:401-446, 578-615): the packed hash-MLP weights and the bit-cache of
+key codes, plus the index lists and workspaces of the kernels.  One decode step is
+
+    append   codes of the new key(s) -> bit-cache           (ha_encode_pack)
+    q codes  codes of the query                             (ha_encode_pack)
+    select   Hamming histogram + ordered compaction         (ha_select)
+    attend   gather-only split-K attention                  (ha_sparse_decode)
+
+All buffers are allocated once per (batch, capacity) and reused: the step itself allocates nothing.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _ops
+
+
+class HashDecodeLayer:
+    def __init__(self, k_layers, q_layers, n_q_heads: int, n_kv_heads: int, head_dim: int, num_layers: int, int_dim: int,
+                 final_dim: int, init_budget: int, recent_budget: int, heavy_budget: float, eval_mode: str = "simple",
+                 retrieve_depth: float = 0, arith: int = _ops.HA_ARITH_F32, device="cuda:0"):
+        """k_layers / q_layers: per head, the list of (W [out,in], b [out]) of its hash MLP.  len(k_layers) is the
+        number of code heads: n_q_heads (one K MLP per query head, as the reference builds it) or n_kv_heads."""
+        self.H, self.Hkv, self.d = n_q_heads, n_kv_heads, head_dim
+        self.Hc = len(k_layers)
+        if self.Hc not in (n_q_heads, n_kv_heads) and n_q_heads % self.Hc != 0:
+            raise ValueError("number of K hash MLPs must divide the number of query heads")
+        self.num_layers, self.int_dim, self.final_dim = num_layers, int_dim, final_dim
+        self.W = final_dim // 32
+        self.init_budget, self.recent_budget, self.heavy_budget = int(init_budget), int(recent_budget), float(heavy_budget)
+        self.mode = _ops.HA_SELECT_SIMPLE if eval_mode == "simple" else _ops.HA_SELECT_THRESHOLD
+        self.depth = int(math.floor(retrieve_depth))
+        self.arith = arith
+        self.device = torch.device(device)
+        self.wk = _ops.pack_usa_weights(k_layers, self.device)
+        self.wq = _ops.pack_usa_weights(q_layers, self.device)
+        self.wk_bf16 = None
+        if head_dim == 128 and int_dim == 128:
+            self.wk_bf16 = _ops.pack_usa_weights_bf16(k_layers, self.device)
+        self.sm_scale = 1.0 / math.sqrt(head_dim)
+        self.B = self.S_cap = 0
+        self.n_cached = 0          # tokens of every sequence already in the bit-cache (uniform batches)
+
+    # ------------------------------------------------------------------ buffers
+    def heavy_count(self, s: int) -> int:
+        hb = self.heavy_budget
+        return int(hb) if hb > 1.0 else int(s * hb)
+
+    def index_capacity(self, s_max: int) -> int:
+        if self.mode != _ops.HA_SELECT_SIMPLE:
+            return s_max                                    # threshold mode keeps all ties: no a-priori bound
+        return min(s_max, self.init_budget + self.recent_budget + self.heavy_count(s_max))
+
+    def allocate(self, B: int, S_cap: int) -> None:
+        """(Re)allocate the bit-cache and scratch for batch B and up to S_cap cached tokens."""
+        dev = self.device
+        self.B, self.S_cap = B, S_cap
+        self.codes = torch.zeros(B, self.Hc, S_cap, self.W, dtype=torch.int32, device=dev)
+        self.qcodes = torch.zeros(B, self.H, 1, self.W, dtype=torch.int32, device=dev)
+        self.idx_cap = self.index_capacity(S_cap)
+        self.idx = torch.empty(B, self.H, self.idx_cap, dtype=torch.int32, device=dev)
+        self.counts = torch.zeros(B, self.H, dtype=torch.int32, device=dev)
+        self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
+        self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
+        self.n_cached = 0
+
+    def reset(self) -> None:
+        """Forget the cached codes (a new prompt starts); buffers are kept."""
+        self.n_cached = 0
+
+    # ------------------------------------------------------------------ stages
+    def encode_keys(self, k: torch.Tensor, pos0: int = 0, pos_dev: Optional[torch.Tensor] = None, use_mfma: bool = False) -> None:
+        """k [B, Hkv, T, d]: codes of T keys per sequence into bit-cache positions pos0.. (or pos_dev[b]..)."""
+        if use_mfma:
+            if self.wk_bf16 is None or k.dtype != torch.bfloat16:
+                raise ValueError("the MFMA encoder needs bf16 keys and 128-wide MLP layers")
+            _ops.encode_pack_prefill(k, self.wk_bf16, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev)
+        else:
+            _ops.encode_pack(k, self.wk, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev, self.arith)
+
+    def encode_query(self, q: torch.Tensor) -> None:
+        """q [B, H, 1, d] -> self.qcodes."""
+        _ops.encode_pack(q, self.wq, self.num_layers, self.int_dim, self.final_dim, self.qcodes, 0, None, self.arith)
+
+    def select(self, max_seq_len: int, seq_lens: Optional[torch.Tensor]) -> None:
+        _ops.select(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
+                    self.recent_budget, self.heavy_budget, self.idx, self.counts, self.ws_select, self.mode, self.depth)
+
+    def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor) -> None:
+        _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend)
+
+    # ------------------------------------------------------------------ one decode step
+    def step(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, seq_len: int, out: torch.Tensor,
+             seq_lens: Optional[torch.Tensor] = None, n_new: int = 1) -> torch.Tensor:
+        """q [B, H, 1, d]; k_cache/v_cache [B, Hkv, >=seq_len, d] already holding the new token(s) at the end.
+
+        Uniform batches: the last `n_new` tokens (positions seq_len - n_new ..) are encoded and appended to the
+        bit-cache; everything before must already be there (`encode_keys` at prefill).  Ragged batches pass
+        `seq_lens` (int32 [B], lengths including the new token) and `seq_len` = their maximum.
+        """
+        if seq_lens is None:
+            if self.n_cached + n_new != seq_len:
+                raise RuntimeError(f"bit-cache holds {self.n_cached} tokens, step at length {seq_len} appends {n_new}")
+            self.encode_keys(k_cache[:, :, seq_len - n_new:seq_len], pos0=seq_len - n_new)
+            self.n_cached = seq_len
+        else:
+            # ragged: the new key of sequence b sits at seq_lens[b] - 1
+            pos = (seq_lens - 1).to(torch.int32)
+            newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
+            self.encode_keys(newk, pos_dev=pos)
+        self.encode_query(q)
+        self.select(seq_len, seq_lens)
+        self.attend(q[:, :, 0, :], k_cache, v_cache, out)
+        return out

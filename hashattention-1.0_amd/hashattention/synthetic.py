@@ -164,3 +164,28 @@ def sha256_of(t: torch.Tensor) -> str:
     if t.dtype == torch.bfloat16:
         t = t.view(torch.int16)
     return hashlib.sha256(t.numpy().tobytes()).hexdigest()
+
+
+def make_problem_on_device(w: Workload, device="cuda:0", with_weights: bool = True) -> Problem:
+    """Same recipe as `make_problem` drawn with the device generator: the distribution is identical, the
+    bytes are not (use `make_problem` wherever bytes must match fixtures).  Built one sequence at a time
+    so the full-size workloads never hold an fp32 copy of the whole cache."""
+    g = torch.Generator(device=device).manual_seed(w.seed)
+    B, H, Hkv, d, S = w.batch, w.n_q_heads, w.n_kv_heads, w.head_dim, w.max_seq_len
+    G = H // Hkv
+    q = torch.randn(B, H, 1, d, generator=g, device=device)
+    k = torch.zeros(B, Hkv, S, d, dtype=w.dtype, device=device)
+    v = torch.zeros(B, Hkv, S, d, dtype=w.dtype, device=device)
+    q_mean = q.view(B, Hkv, G, d).mean(dim=2)
+    for b in range(B):
+        sb = w.seq_lens[b]
+        kb = torch.randn(Hkv, sb, d, generator=g, device=device)
+        n_plant = int(w.plant_frac * sb)
+        for hk in range(Hkv):
+            pos = torch.randperm(sb, generator=g, device=device)[:n_plant]
+            kb[hk, pos] = 0.8 * q_mean[b, hk] + 0.6 * torch.randn(n_plant, d, generator=g, device=device)
+        k[b, :, :sb] = kb.to(w.dtype)
+        v[b, :, :sb] = torch.randn(Hkv, sb, d, generator=g, device=device).to(w.dtype)
+        del kb
+    return Problem(w, q.to(w.dtype), k, v, torch.tensor(w.seq_lens, dtype=torch.int32, device=device),
+                   make_usa_weights(w) if with_weights else None)

@@ -1,0 +1,97 @@
+"""GPU checks of the hash-MLP encoders.
+
+fp32 arithmetic (ha_encode_pack, HA_ARITH_F32) is covered stage by stage in test_gpu_parity.  Here:
+  - the bf16-arithmetic scalar kernel against torch running the same MLP in bf16 on the CPU;
+  - the MFMA prefill encoder against the bf16 scalar kernel (same arithmetic, different summation order);
+  - appending to the bit-cache at an offset / per-sequence offsets leaves the other positions untouched.
+bf16 rounding makes a different summation order flip a rounding now and then, so these two are judged on
+the bit-agreement rate, not exactness; the fp32 path is the bit-exact one.
+"""
+import numpy as np
+import pytest
+import torch
+
+from hashattention import _ops
+from hashattention.synthetic import make_problem
+from oracle import hashattn_oracle as orc
+from tests.parity_util import small_workload
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _bits_differing(a: torch.Tensor, b: torch.Tensor) -> int:
+    x = (a.cpu().numpy().view(np.uint32) ^ b.cpu().numpy().view(np.uint32))
+    return int(np.unpackbits(x.view(np.uint8)).sum())
+
+
+def _bf16_layers(heads):
+    return [[(W.to(torch.bfloat16), b.to(torch.bfloat16)) for W, b in layers] for layers in heads]
+
+
+@pytest.mark.parametrize("layers,final", [(3, 32), (2, 64), (1, 32), (3, 64), (2, 32), (1, 64)])
+def test_bf16_arith_and_mfma_agree(layers, final):
+    print(f"\n[case] encoders layers={layers} final={final}", flush=True)
+    w = small_workload(batch=2, seq_lens=[3000, 1700], lth_num_layers=layers, lth_final_dim=final, seed=70 + layers)
+    p = make_problem(w)
+    B, Hc, S, W = w.batch, w.n_code_heads, w.max_seq_len, w.code_words
+    k = p.k.to(DEV)
+    kb = _bf16_layers(p.usa.k)
+    # torch bf16 on the CPU: the arithmetic a hash module kept in bf16 performs
+    want = orc.pack_codes(orc.usa_logits(p.k, kb).float())
+    want_i32 = torch.from_numpy(want.numpy().astype(np.uint32).view(np.int32).copy())
+
+    wk32 = _ops.pack_usa_weights(kb, DEV)             # bf16 values, exactly representable in the fp32 blob
+    wk16 = _ops.pack_usa_weights_bf16(kb, DEV)
+    c_scalar = torch.zeros(B, Hc, S, W, dtype=torch.int32, device=DEV)
+    c_mfma = torch.full((B, Hc, S, W), -1, dtype=torch.int32, device=DEV)
+    _ops.encode_pack(k, wk32, layers, w.lth_int_dim, final, c_scalar, arith=_ops.HA_ARITH_BF16)
+    _ops.encode_pack_prefill(k, wk16, layers, w.lth_int_dim, final, c_mfma)
+    torch.cuda.synchronize()
+    total = B * Hc * S * final
+    d_ref = _bits_differing(c_scalar, want_i32) / total
+    d_mfma = _bits_differing(c_mfma, c_scalar) / total
+    print(f"  bits differing: scalar-bf16 vs torch-bf16 {d_ref:.2e}, mfma vs scalar-bf16 {d_mfma:.2e}", flush=True)
+    assert d_ref < 5e-3
+    assert d_mfma < 5e-3
+
+
+def test_mfma_tail_and_offsets():
+    # T not a multiple of the 512-token tile nor of 32; append at pos0 and at per-sequence offsets
+    print("\n[case] mfma tails/offsets", flush=True)
+    w = small_workload(batch=2, seq_lens=[777, 777], seed=81)
+    p = make_problem(w)
+    kb = _bf16_layers(p.usa.k)
+    k = p.k.to(DEV)
+    wk16 = _ops.pack_usa_weights_bf16(kb, DEV)
+    wk32 = _ops.pack_usa_weights(kb, DEV)
+    B, Hc, S, W = w.batch, w.n_code_heads, w.max_seq_len, 1
+    cap = S + 300
+    for enc in ("mfma", "scalar"):
+        full = torch.full((B, Hc, cap, W), 12345, dtype=torch.int32, device=DEV)
+        part = torch.full((B, Hc, cap, W), 12345, dtype=torch.int32, device=DEV)
+        pos = torch.tensor([100, 250], dtype=torch.int32, device=DEV)
+        if enc == "mfma":
+            _ops.encode_pack_prefill(k, wk16, 3, 128, 32, full, pos0=0)
+            _ops.encode_pack_prefill(k[:, :, 5:600], wk16, 3, 128, 32, part, pos_dev=pos)
+        else:
+            _ops.encode_pack(k, wk32, 3, 128, 32, full, pos0=0, arith=_ops.HA_ARITH_BF16)
+            _ops.encode_pack(k[:, :, 5:600], wk32, 3, 128, 32, part, pos_dev=pos, arith=_ops.HA_ARITH_BF16)
+        torch.cuda.synchronize()
+        assert (full[:, :, S:] == 12345).all(), enc
+        for b, p0 in enumerate([100, 250]):
+            assert torch.equal(part[b, :, p0:p0 + 595], full[b, :, 5:600]), enc
+            assert (part[b, :, :p0] == 12345).all() and (part[b, :, p0 + 595:] == 12345).all(), enc
+
+
+def test_exact_zero_logit_gives_bit_zero():
+    # bit = (logit > 0): an exactly-zero logit packs as 0 (efficiency/kernels/torchatt.py:55, relu(sign(0)) = 0)
+    W1 = torch.zeros(32, 128)
+    b1 = torch.zeros(32)
+    b1[::2] = 1.0
+    b1[1::4] = -1.0          # dims 3, 7, 11, ... stay exactly 0
+    x = torch.randn(1, 1, 9, 128, device=DEV)
+    codes = torch.zeros(1, 1, 9, 1, dtype=torch.int32, device=DEV)
+    _ops.encode_pack(x, _ops.pack_usa_weights([[(W1, b1)]], DEV), 1, 128, 32, codes)
+    want = sum(1 << i for i in range(0, 32, 2))
+    assert (codes.cpu().numpy().view(np.uint32) == want).all()

@@ -4,8 +4,10 @@
 // a time, lane `sub` holding elements [8*sub, 8*sub+8) fetched with 128-bit loads, so one wave
 // load instruction brings in four whole rows.  A workgroup of 256 threads runs 16 such row streams,
 // each keeping its own online softmax (m, l, acc[8]) in registers in the log2 domain; the streams
-// are merged through LDS at the end, and workgroups of one row's split are merged by
-// merge_splits_kernel with the usual log-sum-exp algebra.
+// are merged through LDS at the end.  Workgroups of one row's split publish (m, l, acc) partials and
+// take a ticket from a per-row counter; the workgroup that draws the last ticket merges the partials
+// with the usual log-sum-exp algebra and resets the counter, so a call is a single launch.  The
+// counters live at the end of the caller's workspace, which must be zero-filled before its first use.
 #include "ha_common.h"
 
 namespace {
@@ -73,6 +75,40 @@ __device__ __forceinline__ void merge_streams(const float *s_m, const float *s_l
     }
 }
 
+// Publish this workgroup's partials and draw a ticket; true in every thread of the workgroup that
+// drew the last of `n` tickets.  Fences: the partial stores are made visible device-wide before the
+// ticket is drawn, and the last workgroup re-acquires before it reads the other workgroups' partials.
+__device__ __forceinline__ bool last_ticket(int32_t *ticket, int n, int *s_last) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) *s_last = (atomicAdd(ticket, 1) == n - 1) ? 1 : 0;
+    __syncthreads();
+    const bool last = *s_last != 0;
+    if (last) __threadfence();
+    return last;
+}
+
+// Threads e < 128 merge `nsplit` partials (acc [nsplit][128], ml [nsplit][2]) into one output row.
+template <typename E>
+__device__ __forceinline__ void merge_partials(const float *acc, const float *ml, int nsplit, char *out_row, int32_t *ticket,
+                                               bool reset) {
+    const int e = threadIdx.x;
+    if (e < HA_HEAD_DIM) {
+        float M = -INFINITY;
+#pragma unroll 4
+        for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[s * 2]);
+        float L = 0.f, A = 0.f;
+#pragma unroll 4
+        for (int s = 0; s < nsplit; ++s) {
+            const float w = fast_exp2(ml[s * 2] - M);
+            L += w * ml[s * 2 + 1];
+            A += w * acc[(int64_t)s * HA_HEAD_DIM + e];
+        }
+        Elem<E>::store1(out_row, e, A / L);
+    }
+    if (reset && e == 0) *ticket = 0;  // leave the counter ready for the next call
+}
+
 // ------------------------------------------------------------------------------------------------
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
 template <typename E>
@@ -82,10 +118,12 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
                                                                     const int32_t *__restrict__ idx, int64_t idx_cap,
                                                                     const int32_t *__restrict__ counts, float scale_log2e,
                                                                     int split_rows, int nsplit_max, float *__restrict__ part_acc,
-                                                                    float *__restrict__ part_ml, void *__restrict__ out) {
+                                                                    float *__restrict__ part_ml, int32_t *__restrict__ tickets,
+                                                                    void *__restrict__ out) {
     using EL = Elem<E>;
     __shared__ float s_m[kStreams], s_l[kStreams];
     __shared__ float s_acc[kStreams * HA_HEAD_DIM];
+    __shared__ int s_last;
 
     const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
@@ -180,33 +218,10 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
             }
         }
     }
-}
-
-// grid (H, B), 128 threads.  n_of_row: number of attended units of the row (selected tokens / keys);
-// rows with a single split were finished by the attend kernel.
-template <typename E>
-__global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
-                                                                   const int32_t *__restrict__ counts, int per_batch,
-                                                                   int64_t count_cap, int H, int unit, int nsplit_max,
-                                                                   void *__restrict__ out) {
-    using EL = Elem<E>;
-    const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
-    const int64_t row = (int64_t)b * H + h;
-    // counts is per (b, h) row, per sequence (per_batch), or absent (every row has count_cap units)
-    int64_t n = counts ? counts[per_batch ? b : row] : count_cap;
-    if (n > count_cap) n = count_cap;
-    const int nsplit = (int)((n + unit - 1) / unit);
-    if (nsplit <= 1) return;
-    const float *ml = part_ml + row * nsplit_max * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[s * 2]);
-    float L = 0.f, A = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float w = fast_exp2(ml[s * 2] - M);
-        L += w * ml[s * 2 + 1];
-        A += w * part_acc[(row * nsplit_max + s) * HA_HEAD_DIM + e];
-    }
-    EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, A / L);
+    if (nsplit == 1) return;  // uniform
+    if (last_ticket(&tickets[row], nsplit, &s_last))
+        merge_partials<E>(part_acc + row * nsplit_max * HA_HEAD_DIM, part_ml + row * nsplit_max * 2, nsplit,
+                          (char *)out + row * HA_HEAD_DIM * EL::bytes, &tickets[row], true);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -218,10 +233,12 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
                                                                    int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int max_S,
                                                                    const int32_t *__restrict__ seq_lens, float scale_log2e, int chunk,
                                                                    int nsplit_max, float *__restrict__ part_acc,
-                                                                   float *__restrict__ part_ml, void *__restrict__ out) {
+                                                                   float *__restrict__ part_ml, int32_t *__restrict__ tickets,
+                                                                   void *__restrict__ out) {
     using EL = Elem<E>;
     __shared__ float s_m[kStreams], s_l[kStreams];
     __shared__ float s_acc[kStreams * HA_HEAD_DIM];
+    __shared__ int s_last;
 
     const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
@@ -337,6 +354,16 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
             }
         }
     }
+    if (nsplit == 1) return;  // uniform
+    int32_t *ticket = &tickets[b * (H / G) + hk];
+    if (last_ticket(ticket, nsplit, &s_last)) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int64_t row = (int64_t)b * H + hk * G + g;
+            merge_partials<E>(part_acc + row * nsplit_max * HA_HEAD_DIM, part_ml + row * nsplit_max * 2, nsplit,
+                              (char *)out + row * HA_HEAD_DIM * EL::bytes, ticket, g == G - 1);
+        }
+    }
 }
 
 int validate_qkv(const void *q, int64_t q_sb, int64_t q_sh, const void *k, const void *v, int kv_dtype, int64_t kv_sb, int64_t kv_sh,
@@ -356,7 +383,10 @@ int validate_qkv(const void *q, int64_t q_sb, int64_t q_sh, const void *k, const
     return HA_OK;
 }
 
-size_t part_bytes(int64_t rows, int nsplit_max) { return (size_t)rows * nsplit_max * (HA_HEAD_DIM + 2) * sizeof(float); }
+// partial accumulators, partial (m, l) pairs, then one ticket counter per row
+size_t part_bytes(int64_t rows, int nsplit_max) {
+    return (size_t)rows * nsplit_max * (HA_HEAD_DIM + 2) * sizeof(float) + (size_t)rows * sizeof(int32_t);
+}
 
 }  // namespace
 
@@ -385,21 +415,17 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, cons
     const int64_t rows = (int64_t)B * H;
     float *part_acc = (float *)workspace;
     float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
+    int32_t *tickets = (int32_t *)(part_ml + rows * plan.nsplit_max * 2);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(plan.nsplit_max, H, B), mgrid(H, B);
+    const dim3 grid(plan.nsplit_max, H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
 #define HA_SPARSE_LAUNCH(E_)                                                                                                      \
     do {                                                                                                                          \
         hipLaunchKernelGGL(sparse_attend_kernel<E_>, grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v, kv_stride_b, \
                            kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows, plan.nsplit_max, part_acc, \
-                           part_ml, out);                                                                                         \
+                           part_ml, tickets, out);                                                                                \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
-        if (plan.nsplit_max > 1) {                                                                                                \
-            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
-                               plan.split_rows, plan.nsplit_max, out);                                                            \
-            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
-        }                                                                                                                         \
     } while (0)
     if (kv_dtype == HA_BF16) HA_SPARSE_LAUNCH(ElemBF16);
     else if (kv_dtype == HA_F16) HA_SPARSE_LAUNCH(ElemF16);
@@ -437,20 +463,16 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const
     const int64_t rows = (int64_t)B * H;
     float *part_acc = (float *)workspace;
     float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
+    int32_t *tickets = (int32_t *)(part_ml + rows * plan.nsplit_max * 2);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(plan.nsplit_max, Hkv, B), mgrid(H, B);
+    const dim3 grid(plan.nsplit_max, Hkv, B);
     const float sl2 = sm_scale * kLog2e;
 #define HA_DENSE_LAUNCH(E_, G_)                                                                                                    \
     do {                                                                                                                           \
         hipLaunchKernelGGL((dense_attend_kernel<E_, G_>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,          \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, plan.chunk, plan.nsplit_max,      \
-                           part_acc, part_ml, out);                                                                                \
+                           part_acc, part_ml, tickets, out);                                                                       \
         HA_CHECK_LAUNCH("dense_attend_kernel");                                                                                    \
-        if (plan.nsplit_max > 1) {                                                                                                 \
-            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, seq_lens, 1,            \
-                               (int64_t)max_seq_len, H, plan.chunk, plan.nsplit_max, out);                                         \
-            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                                \
-        }                                                                                                                          \
     } while (0)
 #define HA_DENSE_DISPATCH(E_)                \
     do {                                     \

@@ -1,19 +1,33 @@
 // Hash-MLP encode into packed sign codes (gfx950): the scalar-FMA kernel used at decode time
 // (a handful of new keys and queries per step) and as the exact-arithmetic path.
 //
-// One workgroup = one MLP head x a tile of kRows input rows.  Thread o owns output neuron o of
-// every layer; weights are read transposed ([in][out], coalesced over o) and reused for the
-// kRows rows held in LDS.  Arithmetic is fixed so results are reproducible bit for bit:
-//   acc = bias[o]; for k ascending: acc = fmaf(x[k], W[k][o], acc); SiLU(a) = a / (1 + expf(-a)).
+// One workgroup = one MLP head x a tile of kRows input rows, 512 threads.  A decode step has little
+// work and a long dependency chain (three layers), so the kernel is built for latency: every thread
+// owns one output neuron and one quarter of the reduction (thread = (o, segment)), fetches its 32
+// weights of the NEXT layer before finishing the current one, and the quarters meet in LDS.
+// Weights are read transposed ([in][out], coalesced over o).
+//
+// The arithmetic is fixed, so results are reproducible bit for bit (the C oracle mirrors it):
+//   p_s = 0; for k ascending in segment s (a quarter of the inputs): p_s = fmaf(x[k], W[k][o], p_s)
+//   y   = (((bias[o] + p_0) + p_1) + p_2) + p_3;          SiLU(y) = y / (1 + expf(-y))
 // HA_ARITH_BF16 additionally rounds the input, every Linear output and every SiLU output to bf16,
 // which is what a hash module kept in bf16 computes.
 #include "ha_common.h"
 
 namespace {
 
-constexpr int kEncThreads = 128;
-constexpr int kRows = 8;
+constexpr int kEncThreads = 512;
+constexpr int kSeg = 4;        // reduction segments per output
+constexpr int kRows = 4;       // input rows per workgroup
 constexpr int kMaxDim = 256;
+constexpr int kMaxPerSeg = kMaxDim / kSeg;
+
+// the weights thread (o, seg) needs for one layer: W[k][o] for k in its segment
+__device__ __forceinline__ void fetch_weights(const float *Wt, int in, int out, int o, int seg, bool active, float (&w)[kMaxPerSeg]) {
+    const int per = in / kSeg;
+#pragma unroll
+    for (int i = 0; i < kMaxPerSeg; ++i) w[i] = (active && i < per) ? Wt[(int64_t)(seg * per + i) * out + o] : 0.f;
+}
 
 __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__restrict__ x, int x_dtype, int64_t x_sb, int64_t x_sh,
                                                                   int64_t x_st, int B, int x_heads, int n_heads, int T,
@@ -21,11 +35,20 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__
                                                                   int d_in, int d_int, int d_out, int arith,
                                                                   uint32_t *__restrict__ codes, int64_t c_sb, int64_t c_sh, int pos0,
                                                                   const int32_t *__restrict__ pos_dev, float *__restrict__ logits) {
-    __shared__ float s_buf[2][kRows][kMaxDim];
+    __shared__ float s_act[2][kRows][kMaxDim];
+    __shared__ float s_part[kSeg][kRows][kMaxDim];
     const int head = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
     const int in_head = head / (n_heads / x_heads);
     const int64_t n_rows = (int64_t)B * T;
     const int64_t row0 = (int64_t)tile * kRows;
+
+    const float *w = weights + head * per_head;
+    // thread -> (o, seg) of a layer with `out` outputs: the first out*kSeg threads, o fastest; wider layers loop
+    float wreg[kMaxPerSeg];
+    {
+        const int out0 = (n_layers == 1) ? d_out : d_int;
+        fetch_weights(w, d_in, out0, tid % out0, tid / out0, tid < out0 * kSeg && out0 * kSeg <= kEncThreads, wreg);
+    }
 
     for (int i = tid; i < kRows * d_in; i += kEncThreads) {
         const int r = i / d_in, e = i % d_in;
@@ -36,37 +59,67 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__
             val = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
             if (arith == HA_ARITH_BF16) val = ha_round_bf16(val);
         }
-        s_buf[0][r][e] = val;
+        s_act[0][r][e] = val;
     }
     __syncthreads();
 
-    const float *w = weights + head * per_head;
     int cur = 0;
     for (int l = 0; l < n_layers; ++l) {
         const int in = (l == 0) ? d_in : d_int;
         const int out = (l == n_layers - 1) ? d_out : d_int;
+        const int per = in / kSeg;
         const float *Wt = w, *bias = w + (int64_t)in * out;
         w += (int64_t)in * out + out;
-        for (int o = tid; o < out; o += kEncThreads) {
-            float acc[kRows];
-            const float bo = bias[o];
+        const bool fits = out * kSeg <= kEncThreads;  // one (o, seg) per thread: weights were prefetched
+
+        if (fits) {
+            if (tid < out * kSeg) {
+                const int o = tid % out, seg = tid / out;
+                float p[kRows];
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) acc[r] = bo;
-            for (int kk = 0; kk < in; ++kk) {
-                const float wv = Wt[(int64_t)kk * out + o];
+                for (int r = 0; r < kRows; ++r) p[r] = 0.f;
 #pragma unroll
-                for (int r = 0; r < kRows; ++r) acc[r] = fmaf(s_buf[cur][r][kk], wv, acc[r]);
-            }
+                for (int i = 0; i < kMaxPerSeg; ++i) {
+                    if (i < per) {
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) {
-                float a = acc[r];
-                if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
-                if (l + 1 < n_layers) {
-                    a = a / (1.0f + expf(-a));
-                    if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
+                        for (int r = 0; r < kRows; ++r) p[r] = fmaf(s_act[cur][r][seg * per + i], wreg[i], p[r]);
+                    }
                 }
-                s_buf[cur ^ 1][r][o] = a;
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) s_part[seg][r][o] = p[r];
             }
+        } else {  // layers wider than 128 outputs: plain loop, no prefetch
+            for (int t2 = tid; t2 < out * kSeg; t2 += kEncThreads) {
+                const int o = t2 % out, seg = t2 / out;
+                float p[kRows];
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) p[r] = 0.f;
+                for (int i = 0; i < per; ++i) {
+                    const float wv = Wt[(int64_t)(seg * per + i) * out + o];
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r) p[r] = fmaf(s_act[cur][r][seg * per + i], wv, p[r]);
+                }
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) s_part[seg][r][o] = p[r];
+            }
+        }
+        // next layer's weights: issue the loads before the barrier so their latency overlaps the reduction
+        if (l + 1 < n_layers) {
+            const int nout = (l + 1 == n_layers - 1) ? d_out : d_int;
+            fetch_weights(w, d_int, nout, tid % nout, tid / nout, tid < nout * kSeg && nout * kSeg <= kEncThreads, wreg);
+        }
+        __syncthreads();
+        for (int t2 = tid; t2 < out * kRows; t2 += kEncThreads) {
+            const int o = t2 % out, r = t2 / out;
+            float a = bias[o];
+#pragma unroll
+            for (int sgm = 0; sgm < kSeg; ++sgm) a += s_part[sgm][r][o];
+            if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
+            if (l + 1 < n_layers) {
+                a = a / (1.0f + expf(-a));
+                if (arith == HA_ARITH_BF16) a = ha_round_bf16(a);
+            }
+            s_act[cur ^ 1][r][o] = a;
         }
         __syncthreads();
         cur ^= 1;
@@ -79,9 +132,9 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__
         const int64_t row = row0 + r;
         if (row >= n_rows) break;  // uniform
         const int64_t b = row / T, t = row % T;
-        const bool bit = tid < d_out && s_buf[cur][r][tid] > 0.0f;
+        const bool bit = tid < d_out && s_act[cur][r][tid] > 0.0f;
         const uint64_t bal = __ballot(bit);
-        if (logits && tid < d_out) logits[((b * n_heads + head) * T + t) * d_out + tid] = s_buf[cur][r][tid];
+        if (logits && tid < d_out) logits[((b * n_heads + head) * T + t) * d_out + tid] = s_act[cur][r][tid];
         const int64_t pos = (pos_dev ? pos_dev[b] : pos0) + t;
         uint32_t *c = codes + b * c_sb + head * c_sh + pos * W;
         if (lane == 0 && wave * 2 < W) c[wave * 2] = (uint32_t)bal;
@@ -96,8 +149,8 @@ int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const
     HA_REQUIRE(n_heads <= 65535, HA_ERR_BAD_SHAPE, "n_heads is limited to 65535");
     HA_REQUIRE(n_heads % x_heads == 0, HA_ERR_BAD_SHAPE, "n_heads=%d not a multiple of x_heads=%d", n_heads, x_heads);
     HA_REQUIRE(n_layers >= 1 && n_layers <= 3, HA_ERR_BAD_SHAPE, "n_layers=%d, must be 1..3", n_layers);
-    HA_REQUIRE(head_dim > 0 && head_dim <= kMaxDim && int_dim > 0 && int_dim <= kMaxDim, HA_ERR_BAD_SHAPE,
-               "head_dim and int_dim must be in 1..%d", kMaxDim);
+    HA_REQUIRE(head_dim > 0 && head_dim <= kMaxDim && int_dim > 0 && int_dim <= kMaxDim && head_dim % kSeg == 0 && int_dim % kSeg == 0,
+               HA_ERR_BAD_SHAPE, "head_dim and int_dim must be multiples of %d in 1..%d", kSeg, kMaxDim);
     HA_REQUIRE(final_dim == 32 || final_dim == 64, HA_ERR_BAD_SHAPE, "final_dim=%d, must be 32 or 64", final_dim);
     HA_REQUIRE(pos0 >= 0, HA_ERR_BAD_SHAPE, "pos0 must be non-negative");
     HA_REQUIRE(c_sh >= 0 && c_sb >= 0, HA_ERR_BAD_SHAPE, "negative code stride");

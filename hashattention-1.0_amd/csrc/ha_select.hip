@@ -3,48 +3,82 @@
 // Selection never sorts.  Distances take only NL = 32*W + 1 values, so the k-th smallest distance
 // T of a row follows from a histogram, and "the k nearest, lowest index first" is
 //     { j : d_j < T }  union  the first r = k - #{d < T} tokens with d_j == T in index order.
-// Two streaming passes over the codes of a (sequence, code head):
-//   1. select_hist_kernel     per-chunk histograms of the distances of every query head of the group
-//   2. select_compact_kernel  T and r from the summed histograms, then an ordered wave-ballot
-//                             compaction that writes ascending index lists (sink | heavy | recent)
-// The second pass re-reads the codes (4*W bytes per token) from L2 / Infinity Cache.
+// Three launches per call:
+//   1. select_hist_kernel       grid (chunk, code head, sequence): per-chunk histograms of the distances
+//                               of every query head of the group, one streaming pass over the codes
+//   2. select_threshold_kernel  grid (head, sequence): T, r, per-chunk output offsets, window indices, counts
+//   3. select_compact_kernel    grid as 1: ordered wave-ballot compaction into ascending index lists
+// Pass 3 re-reads the codes (4*W bytes per token) from L2 / Infinity Cache.
+//
+// Both streaming kernels fetch all codes of their chunk before using any: a lane holds 4 consecutive
+// codes per 1024-code block (128-bit loads), up to 4 blocks per workgroup, so a workgroup has its whole
+// chunk in flight at once instead of paying one memory round trip per tile.
 #include "ha_common.h"
 
 namespace {
 
 constexpr int kSelThreads = 256;
 constexpr int kSelWaves = kSelThreads / HA_WAVE;
-constexpr int kMaxChunks = 32;
+constexpr int kBlock = 1024;      // codes per workgroup per block: 4 waves x 64 lanes x 4 codes
+constexpr int kMaxBlocks = 4;     // blocks per chunk held in registers
+constexpr int kMaxChunks = 1024;  // per row
 
 struct SelectPlan {
-    int chunk;   // tokens per workgroup, multiple of 1024
-    int nchunk;  // <= kMaxChunks
+    int blocks;  // 1024-code blocks per chunk, 1..kMaxBlocks
+    int nchunk;
 };
 
-inline SelectPlan select_plan(int max_seq_len) {
+inline SelectPlan select_plan(int B, int Hc, int max_seq_len) {
     SelectPlan p;
-    int64_t per = ((int64_t)max_seq_len + kMaxChunks - 1) / kMaxChunks;
-    p.chunk = (int)((per + 1023) / 1024) * 1024;
-    if (p.chunk < 1024) p.chunk = 1024;
-    p.nchunk = (max_seq_len + p.chunk - 1) / p.chunk;
-    if (p.nchunk < 1) p.nchunk = 1;
+    p.blocks = kMaxBlocks;
+    // prefer many small workgroups while the grid is short of ~8 workgroups per CU
+    while (p.blocks > 1 && (int64_t)B * Hc * ((max_seq_len + p.blocks * kBlock - 1) / (p.blocks * kBlock)) < 2048) p.blocks /= 2;
+    p.nchunk = (max_seq_len + p.blocks * kBlock - 1) / (p.blocks * kBlock);
     return p;
 }
 
 template <int W> struct Code;
 template <> struct Code<1> {
     uint32_t w0;
-    __device__ static __forceinline__ Code load(const uint32_t *p, int64_t j) { return Code{p[j]}; }
     __device__ __forceinline__ int dist(const Code &q) const { return __popc(w0 ^ q.w0); }
 };
 template <> struct Code<2> {
     uint32_t w0, w1;
-    __device__ static __forceinline__ Code load(const uint32_t *p, int64_t j) {
-        uint2 v = reinterpret_cast<const uint2 *>(p)[j];
-        return Code{v.x, v.y};
-    }
     __device__ __forceinline__ int dist(const Code &q) const { return __popc(w0 ^ q.w0) + __popc(w1 ^ q.w1); }
 };
+
+template <int W> __device__ __forceinline__ Code<W> load_code(const uint32_t *p, int64_t j) {
+    if constexpr (W == 1) return Code<1>{p[j]};
+    else {
+        const uint2 v = reinterpret_cast<const uint2 *>(p)[j];
+        return Code<2>{v.x, v.y};
+    }
+}
+
+// Four consecutive codes j0..j0+3 (j0 % 4 == 0).  `vec`: the row is 16-byte aligned and padded to whole
+// groups of four, so one (W=1) or two (W=2) 128-bit loads are safe; otherwise element loads, only for
+// indices inside [beg, end).  Codes outside [beg, end) are returned as zero and must be masked by the caller.
+template <int W>
+__device__ __forceinline__ void load_code4(const uint32_t *kc, int j0, int beg, int end, bool vec, Code<W> (&k)[4]) {
+    if (vec) {
+        if constexpr (W == 1) {
+            const uint4 v = reinterpret_cast<const uint4 *>(kc)[j0 >> 2];
+            k[0].w0 = v.x; k[1].w0 = v.y; k[2].w0 = v.z; k[3].w0 = v.w;
+        } else {
+            const uint4 a = reinterpret_cast<const uint4 *>(kc)[(j0 >> 1)], b = reinterpret_cast<const uint4 *>(kc)[(j0 >> 1) + 1];
+            k[0].w0 = a.x; k[0].w1 = a.y; k[1].w0 = a.z; k[1].w1 = a.w;
+            k[2].w0 = b.x; k[2].w1 = b.y; k[3].w0 = b.z; k[3].w1 = b.w;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int j = j0 + e;
+            if (j >= beg && j < end) k[e] = load_code<W>(kc, j);
+            else if constexpr (W == 1) k[e] = Code<1>{0u};
+            else k[e] = Code<2>{0u, 0u};
+        }
+    }
+}
 
 template <int W> __device__ __forceinline__ Code<W> load_qcode(const uint32_t *qcodes, int64_t row) {
     if constexpr (W == 1) return Code<1>{qcodes[row]};
@@ -66,9 +100,32 @@ __device__ __forceinline__ RowBudget row_budget(int S, int init, int recent, dou
     r.hi = (S - recent > r.lo) ? S - recent : r.lo;
     int heavy = heavy_budget > 1.0 ? (int)heavy_budget : (int)((double)S * heavy_budget);
     if (heavy < 0) heavy = 0;
-    int ncand = r.hi - r.lo;
+    const int ncand = r.hi - r.lo;
     r.kk = heavy < ncand ? heavy : ncand;
     return r;
+}
+
+// The chunk of a workgroup, fetched up front.  k[blk][e] is code j = j0(blk) + e.
+template <int W> struct ChunkRegs {
+    Code<W> k[kMaxBlocks][4];
+    int j0[kMaxBlocks];
+};
+template <int W>
+__device__ __forceinline__ void load_chunk(const uint32_t *kc, int chunk_start, int blocks, int beg, int end, bool vec, int wave, int lane,
+                                           ChunkRegs<W> &cr) {
+#pragma unroll
+    for (int blk = 0; blk < kMaxBlocks; ++blk) {
+        cr.j0[blk] = chunk_start + blk * kBlock + wave * (HA_WAVE * 4) + lane * 4;
+        const bool live = blk < blocks && cr.j0[blk] + 4 > beg && cr.j0[blk] < end;
+        if (live) load_code4<W>(kc, cr.j0[blk], beg, end, vec, cr.k[blk]);
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if constexpr (W == 1) cr.k[blk][e] = Code<1>{0u};
+                else cr.k[blk][e] = Code<2>{0u, 0u};
+            }
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -82,28 +139,31 @@ __global__ __launch_bounds__(256) void hamming_score_kernel(const uint32_t *__re
     if (j >= S || j >= max_S) return;
     const Code<W> q = load_qcode<W>(qcodes, (int64_t)b * H + h);
     const uint32_t *kc = kcodes + b * kc_sb + (h / (H / Hc)) * kc_sh;
-    scores[((int64_t)b * H + h) * max_S + j] = (uint8_t)Code<W>::load(kc, j).dist(q);
+    scores[((int64_t)b * H + h) * max_S + j] = (uint8_t)load_code<W>(kc, j).dist(q);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Pass 1.  grid (nchunk, Hc, B).  hist[b, h, chunk, level] = #candidates of the chunk at that distance.
-// The LDS histogram is replicated REP times (bank = lane % REP) so that the ~10 hot levels of a
-// binomial-like distance distribution do not serialise the ds_add.
+// The LDS histogram is replicated REP times (replica = lane % REP, which is also the bank) so that the
+// few hot levels of a binomial-like distance distribution do not serialise the ds_add.
 template <int W, int GQ, int REP>
 __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
                                                                   const uint32_t *__restrict__ qcodes, int H, int max_S,
                                                                   const int32_t *__restrict__ seq_lens, int init, int recent,
-                                                                  int chunk, int nchunk, uint32_t *__restrict__ hist) {
+                                                                  int blocks, int nchunk, int vec, uint32_t *__restrict__ hist) {
     constexpr int NL = 32 * W + 1;
     __shared__ uint32_t lh[GQ * NL * REP];
     const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;
     const int lo = init < S ? init : S;
     const int hi = (S - recent > lo) ? S - recent : lo;
+    const int chunk = blocks * kBlock;
     const int beg = max(lo, c * chunk), end = min(hi, (c + 1) * chunk);
 
+    ChunkRegs<W> cr;
+    if (beg < end) load_chunk<W>(kcodes + b * kc_sb + hc * kc_sh, c * chunk, blocks, beg, end, vec != 0, wave, lane, cr);
     for (int i = tid; i < GQ * NL * REP; i += kSelThreads) lh[i] = 0;
     __syncthreads();
 
@@ -111,13 +171,18 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
         Code<W> q[GQ];
 #pragma unroll
         for (int g = 0; g < GQ; ++g) q[g] = load_qcode<W>(qcodes, (int64_t)b * H + hc * GQ + g);
-        const uint32_t *kc = kcodes + b * kc_sb + hc * kc_sh;
         const int rep = tid % REP;
-        for (int j = c * chunk + tid; j < end; j += kSelThreads) {
-            if (j < beg) continue;
-            const Code<W> k = Code<W>::load(kc, j);
 #pragma unroll
-            for (int g = 0; g < GQ; ++g) atomicAdd(&lh[(g * NL + k.dist(q[g])) * REP + rep], 1u);
+        for (int blk = 0; blk < kMaxBlocks; ++blk) {
+            if (blk >= blocks) break;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = cr.j0[blk] + e;
+                if (j >= beg && j < end) {
+#pragma unroll
+                    for (int g = 0; g < GQ; ++g) atomicAdd(&lh[(g * NL + cr.k[blk][e].dist(q[g])) * REP + rep], 1u);
+                }
+            }
         }
     }
     __syncthreads();
@@ -131,47 +196,48 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
 }
 
 // ------------------------------------------------------------------------------------------------
-// Pass 2.  grid (nchunk, Hc, B).  Each wave owns a contiguous quarter of the chunk, so output order
-// is chunk-major, wave-major, tile-major, lane-major = ascending token index.
-template <int W, int GQ>
-__global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
-                                                                     const uint32_t *__restrict__ qcodes, int H, int max_S,
-                                                                     const int32_t *__restrict__ seq_lens, int init, int recent,
-                                                                     double heavy_budget, int mode, int depth, int chunk, int nchunk,
-                                                                     const uint32_t *__restrict__ hist, int32_t *__restrict__ out_idx,
-                                                                     int64_t idx_cap, int32_t *__restrict__ out_counts) {
+// Pass 2.  grid (H, B), 256 threads.  meta[row] = {T, r, n_heavy, 0}; chunk_pre[row][c] = {#selected with
+// d < T in chunks before c, #tokens with d == T in chunks before c}.  Also writes the sink and recent
+// window indices and the row's count.
+template <int W>
+__global__ __launch_bounds__(kSelThreads) void select_threshold_kernel(const uint32_t *__restrict__ hist, int H, int max_S,
+                                                                       const int32_t *__restrict__ seq_lens, int init, int recent,
+                                                                       double heavy_budget, int mode, int depth, int nchunk,
+                                                                       int32_t *__restrict__ meta, int32_t *__restrict__ chunk_pre,
+                                                                       int32_t *__restrict__ out_idx, int64_t idx_cap,
+                                                                       int32_t *__restrict__ out_counts) {
     constexpr int NL = 32 * W + 1;
-    __shared__ uint32_t s_tot[GQ][NL], s_pre[GQ][NL];
-    __shared__ int s_T[GQ], s_r[GQ], s_ltpre[GQ], s_eqpre[GQ], s_nheavy[GQ];
-    __shared__ int s_wcnt[kSelWaves][GQ][2];
+    constexpr int TC = 32;  // chunks per LDS tile
+    __shared__ uint32_t s_tile[TC * NL];
+    __shared__ uint32_t s_tot[NL];
+    __shared__ int s_T, s_nheavy, s_carry_lt, s_carry_eq;
 
-    const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int64_t row = (int64_t)b * H + h;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;
     const RowBudget rb = row_budget(S, init, recent, heavy_budget);
+    const uint32_t *hp = hist + row * nchunk * NL;
 
-    // ---- chunk-summed histograms and the part that lies in earlier chunks
-    for (int p = tid; p < GQ * NL; p += kSelThreads) {
-        const int g = p / NL, l = p % NL;
-        const uint32_t *hp = hist + ((int64_t)b * H + hc * GQ + g) * nchunk * NL + l;
-        uint32_t tot = 0, pre = 0;
-        for (int cc = 0; cc < nchunk; ++cc) {
-            const uint32_t v = hp[(int64_t)cc * NL];
-            tot += v;
-            if (cc < c) pre += v;
+    if (tid < NL) s_tot[tid] = 0;
+    for (int c0 = 0; c0 < nchunk; c0 += TC) {
+        const int n = min(TC, nchunk - c0) * NL;
+        __syncthreads();
+        for (int i = tid; i < n; i += kSelThreads) s_tile[i] = hp[(int64_t)c0 * NL + i];
+        __syncthreads();
+        if (tid < NL) {
+            uint32_t s = 0;
+            for (int cc = 0; cc * NL < n; ++cc) s += s_tile[cc * NL + tid];
+            s_tot[tid] += s;
         }
-        s_tot[g][l] = tot;
-        s_pre[g][l] = pre;
     }
     __syncthreads();
-    if (tid < GQ) {
-        const int g = tid;
+    if (tid == 0) {
         int T = 0, r = 0, nheavy = 0;
         if (rb.kk > 0) {
             int cum = 0, l = 0, dmin = -1;
             for (; l < NL; ++l) {
-                const int t = (int)s_tot[g][l];
+                const int t = (int)s_tot[l];
                 if (dmin < 0 && t > 0) dmin = l;
                 if (cum + t >= rb.kk) break;
                 cum += t;
@@ -185,104 +251,176 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
                 const int th = min(dmin + depth, l);
                 T = th + 1;  // every distance <= th, no partial tie bucket
                 r = 0;
-                for (int i = 0; i <= th; ++i) nheavy += (int)s_tot[g][i];
+                for (int i = 0; i <= th; ++i) nheavy += (int)s_tot[i];
             }
         }
-        int ltpre = 0;
-        for (int i = 0; i < T && i < NL; ++i) ltpre += (int)s_pre[g][i];
-        s_T[g] = T;
-        s_r[g] = r;
-        s_ltpre[g] = ltpre;
-        s_eqpre[g] = (T < NL) ? (int)s_pre[g][T] : 0;
-        s_nheavy[g] = nheavy;
+        s_T = T;
+        s_nheavy = nheavy;
+        s_carry_lt = 0;
+        s_carry_eq = 0;
+        meta[row * 4 + 0] = T;
+        meta[row * 4 + 1] = r;
+        meta[row * 4 + 2] = nheavy;
+        meta[row * 4 + 3] = 0;
     }
     __syncthreads();
+    const int T = s_T, nheavy = s_nheavy;
 
-    // ---- windows and counts: written once per row, by the workgroup of chunk 0
-    if (c == 0) {
-        const int n_recent = rb.S - rb.hi;
+    // exclusive prefix over chunks of (#d < T, #d == T); wave 0 scans a tile of 32 chunks at a time
+    for (int c0 = 0; c0 < nchunk; c0 += TC) {
+        const int nc = min(TC, nchunk - c0);
+        __syncthreads();
+        for (int i = tid; i < nc * NL; i += kSelThreads) s_tile[i] = hp[(int64_t)c0 * NL + i];
+        __syncthreads();
+        if (tid < HA_WAVE) {
+            int a = 0, e = 0;
+            if (tid < nc) {
+                for (int l = 0; l < T && l < NL; ++l) a += (int)s_tile[tid * NL + l];
+                if (T < NL) e = (int)s_tile[tid * NL + T];
+            }
+            int ia = a, ie = e;  // inclusive scan over lanes 0..31
 #pragma unroll
-        for (int g = 0; g < GQ; ++g) {
-            int32_t *o = out_idx + ((int64_t)b * H + hc * GQ + g) * idx_cap;
-            const int64_t rbase = (int64_t)rb.lo + s_nheavy[g];
-            for (int i = tid; i < rb.lo; i += kSelThreads)
-                if (i < idx_cap) o[i] = i;
-            for (int i = tid; i < n_recent; i += kSelThreads)
-                if (rbase + i < idx_cap) o[rbase + i] = rb.hi + i;
-            if (tid == 0) out_counts[b * H + hc * GQ + g] = (int32_t)(rbase + n_recent);
+            for (int off = 1; off < TC; off <<= 1) {
+                const int ta = __shfl_up(ia, off), te = __shfl_up(ie, off);
+                if (tid >= off) {
+                    ia += ta;
+                    ie += te;
+                }
+            }
+            const int base_lt = s_carry_lt, base_eq = s_carry_eq;
+            if (tid < nc) {
+                chunk_pre[(row * nchunk + c0 + tid) * 2 + 0] = base_lt + ia - a;
+                chunk_pre[(row * nchunk + c0 + tid) * 2 + 1] = base_eq + ie - e;
+            }
+            if (tid == nc - 1) {
+                s_carry_lt = base_lt + ia;
+                s_carry_eq = base_eq + ie;
+            }
         }
     }
 
-    const int beg = max(rb.lo, c * chunk), end = min(rb.hi, (c + 1) * chunk);
-    if (beg >= end || rb.kk == 0) return;  // uniform over the workgroup
+    // windows and count
+    int32_t *o = out_idx + row * idx_cap;
+    const int n_recent = rb.S - rb.hi;
+    const int64_t rbase = (int64_t)rb.lo + nheavy;
+    for (int i = tid; i < rb.lo; i += kSelThreads)
+        if (i < idx_cap) o[i] = i;
+    for (int i = tid; i < n_recent; i += kSelThreads)
+        if (rbase + i < idx_cap) o[rbase + i] = rb.hi + i;
+    if (tid == 0) out_counts[row] = (int32_t)(rbase + n_recent);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Pass 3.  grid (nchunk, Hc, B).  Output order = block, wave, lane, element = ascending token index.
+template <int W, int GQ>
+__global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
+                                                                     const uint32_t *__restrict__ qcodes, int H, int max_S,
+                                                                     const int32_t *__restrict__ seq_lens, int init, int recent,
+                                                                     int blocks, int nchunk, int vec, const int32_t *__restrict__ meta,
+                                                                     const int32_t *__restrict__ chunk_pre,
+                                                                     int32_t *__restrict__ out_idx, int64_t idx_cap) {
+    __shared__ int s_cnt[kMaxBlocks][kSelWaves][GQ][2];
+
+    const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int S = seq_lens ? seq_lens[b] : max_S;
+    if (S > max_S) S = max_S;
+    const int lo = init < S ? init : S;
+    const int hi = (S - recent > lo) ? S - recent : lo;
+    const int chunk = blocks * kBlock;
+    const int beg = max(lo, c * chunk), end = min(hi, (c + 1) * chunk);
+    if (beg >= end) return;  // uniform over the workgroup
+
+    ChunkRegs<W> cr;
+    load_chunk<W>(kcodes + b * kc_sb + hc * kc_sh, c * chunk, blocks, beg, end, vec != 0, wave, lane, cr);
 
     Code<W> q[GQ];
-    int T[GQ], cnt_lt[GQ], cnt_eq[GQ];
+    int T[GQ], r[GQ], lt_pre[GQ], eq_pre[GQ];
+    bool any = false;
 #pragma unroll
     for (int g = 0; g < GQ; ++g) {
-        q[g] = load_qcode<W>(qcodes, (int64_t)b * H + hc * GQ + g);
-        T[g] = s_T[g];
-        cnt_lt[g] = cnt_eq[g] = 0;
+        const int64_t row = (int64_t)b * H + hc * GQ + g;
+        q[g] = load_qcode<W>(qcodes, row);
+        T[g] = meta[row * 4 + 0];
+        r[g] = meta[row * 4 + 1];
+        any = any || meta[row * 4 + 2] > 0;
+        lt_pre[g] = chunk_pre[(row * nchunk + c) * 2 + 0];
+        eq_pre[g] = chunk_pre[(row * nchunk + c) * 2 + 1];
     }
-    const uint32_t *kc = kcodes + b * kc_sb + hc * kc_sh;
-    const int seg = chunk / kSelWaves;
-    const int wbeg = c * chunk + wave * seg, wend = min(wbeg + seg, end);
+    if (!any) return;  // uniform: nothing heavy to write for this group
 
-    // ---- pass A: per-wave counts
-    for (int j0 = wbeg; j0 < wend; j0 += HA_WAVE) {
-        const int j = j0 + lane;
-        const bool valid = j >= beg && j < wend;
-        Code<W> k = q[0];
-        if (valid) k = Code<W>::load(kc, j);
+    // ---- counts per (block, wave)
+#pragma unroll
+    for (int blk = 0; blk < kMaxBlocks; ++blk) {
+        if (blk >= blocks) break;
 #pragma unroll
         for (int g = 0; g < GQ; ++g) {
-            const int d = k.dist(q[g]);
-            cnt_lt[g] += __popcll(__ballot(valid && d < T[g]));
-            cnt_eq[g] += __popcll(__ballot(valid && d == T[g]));
-        }
-    }
-    if (lane == 0) {
+            int nlt = 0, neq = 0;
 #pragma unroll
-        for (int g = 0; g < GQ; ++g) {
-            s_wcnt[wave][g][0] = cnt_lt[g];
-            s_wcnt[wave][g][1] = cnt_eq[g];
+            for (int e = 0; e < 4; ++e) {
+                const int j = cr.j0[blk] + e;
+                const bool valid = j >= beg && j < end;
+                const int d = cr.k[blk][e].dist(q[g]);
+                nlt += __popcll(__ballot(valid && d < T[g]));
+                neq += __popcll(__ballot(valid && d == T[g]));
+            }
+            if (lane == 0) {
+                s_cnt[blk][wave][g][0] = nlt;
+                s_cnt[blk][wave][g][1] = neq;
+            }
         }
     }
     __syncthreads();
 
-    int run_sel[GQ], run_eq[GQ], r[GQ];
+    // ---- ordered compaction
+    int run_lt[GQ], run_eq[GQ];
 #pragma unroll
     for (int g = 0; g < GQ; ++g) {
-        int lt_before = s_ltpre[g], eq_before = s_eqpre[g];
-        for (int w = 0; w < wave; ++w) {
-            lt_before += s_wcnt[w][g][0];
-            eq_before += s_wcnt[w][g][1];
-        }
-        r[g] = s_r[g];
-        run_eq[g] = eq_before;
-        run_sel[g] = rb.lo + lt_before + min(eq_before, r[g]);
+        run_lt[g] = lt_pre[g];
+        run_eq[g] = eq_pre[g];
     }
-
-    // ---- pass B: ordered compaction
-    for (int j0 = wbeg; j0 < wend; j0 += HA_WAVE) {
-        const int j = j0 + lane;
-        const bool valid = j >= beg && j < wend;
-        Code<W> k = q[0];
-        if (valid) k = Code<W>::load(kc, j);
+#pragma unroll
+    for (int blk = 0; blk < kMaxBlocks; ++blk) {
+        if (blk >= blocks) break;
 #pragma unroll
         for (int g = 0; g < GQ; ++g) {
-            const int d = k.dist(q[g]);
-            const bool is_lt = valid && d < T[g];
-            const bool is_eq = valid && d == T[g];
-            const uint64_t bal_eq = __ballot(is_eq);
-            const bool sel = is_lt || (is_eq && run_eq[g] + lanes_below(bal_eq) < r[g]);
-            const uint64_t bal_sel = __ballot(sel);
-            if (sel) {
-                const int64_t pos = (int64_t)run_sel[g] + lanes_below(bal_sel);
-                if (pos < idx_cap) out_idx[((int64_t)b * H + hc * GQ + g) * idx_cap + pos] = j;
+            int lt_before = run_lt[g], eq_before = run_eq[g];
+            for (int w = 0; w < wave; ++w) {
+                lt_before += s_cnt[blk][w][g][0];
+                eq_before += s_cnt[blk][w][g][1];
             }
-            run_eq[g] += __popcll(bal_eq);
-            run_sel[g] += __popcll(bal_sel);
+            // lane-level prefix over the 4 elements of every lower lane, then over this lane's earlier elements
+            bool is_lt[4], is_eq[4];
+            uint64_t bal_lt[4], bal_eq[4];
+            int lt_lane = 0, eq_lane = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = cr.j0[blk] + e;
+                const bool valid = j >= beg && j < end;
+                const int d = cr.k[blk][e].dist(q[g]);
+                is_lt[e] = valid && d < T[g];
+                is_eq[e] = valid && d == T[g];
+                bal_lt[e] = __ballot(is_lt[e]);
+                bal_eq[e] = __ballot(is_eq[e]);
+                lt_lane += lanes_below(bal_lt[e]);
+                eq_lane += lanes_below(bal_eq[e]);
+            }
+            int n_lt = lt_before + lt_lane, n_eq = eq_before + eq_lane;  // tokens before (lane, element 0)
+            int32_t *o = out_idx + ((int64_t)b * H + hc * GQ + g) * idx_cap;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bool sel = is_lt[e] || (is_eq[e] && n_eq < r[g]);
+                if (sel) {
+                    const int64_t pos = (int64_t)lo + n_lt + min(n_eq, r[g]);
+                    if (pos < idx_cap) o[pos] = cr.j0[blk] + e;
+                }
+                n_lt += is_lt[e] ? 1 : 0;
+                n_eq += is_eq[e] ? 1 : 0;
+            }
+            for (int w = 0; w < kSelWaves; ++w) {
+                run_lt[g] += s_cnt[blk][w][g][0];
+                run_eq[g] += s_cnt[blk][w][g][1];
+            }
         }
     }
 }
@@ -297,9 +435,39 @@ int validate_codes(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, const u
     const int gq = H / Hc;
     HA_REQUIRE(gq == 1 || gq == 2 || gq == 4 || gq == 8, HA_ERR_BAD_SHAPE, "H/Hc=%d, must be 1, 2, 4 or 8", gq);
     HA_REQUIRE(kc_sh >= (int64_t)max_seq_len * W && kc_sb >= kc_sh, HA_ERR_BAD_SHAPE, "code strides smaller than the rows they span");
+    HA_REQUIRE((int64_t)max_seq_len <= (int64_t)kMaxChunks * kMaxBlocks * kBlock, HA_ERR_BAD_SHAPE, "max_seq_len above %d",
+               kMaxChunks * kMaxBlocks * kBlock);
     HA_REQUIRE(ha_aligned(kcodes, 4 * W) && ha_aligned(qcodes, 4) && (W == 1 || (kc_sb % 2 == 0 && kc_sh % 2 == 0)),
                HA_ERR_MISALIGNED, "codes must be aligned to their word count");
     return HA_OK;
+}
+
+// rows start 16-byte aligned and hold whole groups of four codes: 128-bit loads never leave a row
+bool rows_vectorisable(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, int W) {
+    return ha_aligned(kcodes, 16) && kc_sb % (4 * W) == 0 && kc_sh % (4 * W) == 0;
+}
+
+struct SelectWorkspace {
+    uint32_t *hist;
+    int32_t *meta, *chunk_pre;
+    size_t bytes;
+};
+SelectWorkspace carve_select_ws(void *base, int64_t rows, int nchunk, int W) {
+    SelectWorkspace w;
+    size_t off = 0;
+    auto take = [&](size_t n) {
+        size_t o = off;
+        off += (n + 255) / 256 * 256;
+        return o;
+    };
+    const size_t o_hist = take((size_t)rows * nchunk * (32 * W + 1) * 4);
+    const size_t o_meta = take((size_t)rows * 4 * 4);
+    const size_t o_pre = take((size_t)rows * nchunk * 2 * 4);
+    w.hist = (uint32_t *)((char *)base + o_hist);
+    w.meta = (int32_t *)((char *)base + o_meta);
+    w.chunk_pre = (int32_t *)((char *)base + o_pre);
+    w.bytes = off;
+    return w;
 }
 
 }  // namespace
@@ -324,20 +492,23 @@ int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
 }
 
 size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
-    (void)Hc;
-    if (B <= 0 || H <= 0 || max_seq_len <= 0 || (W != 1 && W != 2)) return 0;
-    const SelectPlan p = select_plan(max_seq_len);
-    return (size_t)B * H * p.nchunk * (32 * W + 1) * sizeof(uint32_t);
+    if (B <= 0 || H <= 0 || Hc <= 0 || max_seq_len <= 0 || (W != 1 && W != 2)) return 0;
+    const SelectPlan p = select_plan(B, Hc, max_seq_len);
+    return carve_select_ws(nullptr, (int64_t)B * H, p.nchunk, W).bytes;
 }
 
 #define HA_SELECT_LAUNCH(W_, GQ_, REP_)                                                                                           \
     do {                                                                                                                          \
         hipLaunchKernelGGL((select_hist_kernel<W_, GQ_, REP_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,  \
-                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.chunk, plan.nchunk, hist);          \
+                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.hist);  \
         HA_CHECK_LAUNCH("select_hist_kernel");                                                                                    \
+        hipLaunchKernelGGL(select_threshold_kernel<W_>, dim3(H, B), dim3(kSelThreads), 0, s, ws.hist, H, max_seq_len, seq_lens,   \
+                           init_budget, recent_budget, heavy_budget, mode, depth, plan.nchunk, ws.meta, ws.chunk_pre, out_idx,    \
+                           idx_cap, out_counts);                                                                                  \
+        HA_CHECK_LAUNCH("select_threshold_kernel");                                                                               \
         hipLaunchKernelGGL((select_compact_kernel<W_, GQ_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,     \
-                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, heavy_budget, mode, depth, plan.chunk,   \
-                           plan.nchunk, hist, out_idx, idx_cap, out_counts);                                                      \
+                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.meta,  \
+                           ws.chunk_pre, out_idx, idx_cap);                                                                       \
         HA_CHECK_LAUNCH("select_compact_kernel");                                                                                 \
     } while (0)
 
@@ -359,8 +530,9 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
     HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "select workspace must be 256-byte aligned");
     if ((st = ha_require_device())) return st;
 
-    const SelectPlan plan = select_plan(max_seq_len);
-    uint32_t *hist = (uint32_t *)workspace;
+    const SelectPlan plan = select_plan(B, Hc, max_seq_len);
+    const SelectWorkspace ws = carve_select_ws(workspace, (int64_t)B * H, plan.nchunk, W);
+    const int vec = rows_vectorisable(kcodes, kc_stride_b, kc_stride_h, W) ? 1 : 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(plan.nchunk, Hc, B);
     const int gq = H / Hc;

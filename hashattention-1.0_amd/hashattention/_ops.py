@@ -97,8 +97,9 @@ def _require_cuda(*tensors):
 
 
 def workspace(nbytes: int, device) -> torch.Tensor:
-    """A byte buffer of at least nbytes (torch's allocator returns >= 256-byte aligned blocks)."""
-    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+    """A zero-filled byte buffer of at least nbytes (torch's allocator returns >= 256-byte aligned blocks).
+    The decode workspaces end with ticket counters that must start at zero."""
+    return torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
 # ------------------------------------------------------------------------------------------ encode

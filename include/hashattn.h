@@ -138,6 +138,9 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
  *   q   [B, H, 128] kv_dtype, strides q_stride_{b,h}
  *   k,v [B, Hkv, ., 128] kv_dtype, strides kv_stride_{b,h,s}; rows 16-byte aligned
  *   out [B, H, 128] kv_dtype contiguous
+ *   workspace  ha_sparse_decode_workspace_bytes(...) bytes, 256-byte aligned.  It ends with one ticket
+ *              counter per row: ZERO-FILL the workspace once before its first use; every completed
+ *              call leaves the counters at zero again.  Calls sharing a workspace must not overlap.
  */
 size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap);
 int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
@@ -150,7 +153,8 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
  * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).
  * Replaces flash_decode_attention_fwd (efficiency/kernels/flash_fwd_sparse.py:21-321) and
  * torch_attention_naive (efficiency/kernels/torchatt.py:17-30).  Each K/V row is read once per KV
- * head and shared by the query heads of its group.
+ * head and shared by the query heads of its group.  Workspace rules as for ha_sparse_decode
+ * (zero-filled before first use, not shared by overlapping calls).
  */
 size_t ha_dense_decode_workspace_bytes(int B, int H, int max_seq_len);
 int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,

@@ -109,8 +109,9 @@ void orc_select(const uint32_t *kcodes, const uint32_t *qcodes, int B, int H, in
 }
 
 /*
- * Hash MLP of one head over n rows, canonical fp32 arithmetic: every Linear is
- * acc = b[o]; for k ascending acc = fmaf(x[k], W[o][k], acc); SiLU(x) = x / (1 + expf(-x)).
+ * Hash MLP of one head over n rows in the fixed fp32 arithmetic of the GPU's exact encoder: the inputs
+ * of a Linear are split in four contiguous quarters, each reduced by an ascending fmaf chain from 0,
+ * y = (((b[o] + p0) + p1) + p2) + p3; SiLU(y) = y / (1 + expf(-y)).  Input widths are multiples of 4.
  * W is nn.Linear layout [out, in].  logits [n, final] (may be NULL), codes [n, final/32].
  */
 void orc_encode(const float *x, int64_t n, int n_layers, const int32_t *dims /* n_layers+1 */,
@@ -128,7 +129,11 @@ void orc_encode(const float *x, int64_t n, int n_layers, const int32_t *dims /* 
                 int in = dims[l], out = dims[l + 1];
                 for (int o = 0; o < out; ++o) {
                     float acc = bl[l][o];
-                    for (int k = 0; k < in; ++k) acc = fmaf(a[k], Wl[l][(int64_t)o * in + k], acc);
+                    for (int s = 0; s < 4; ++s) {
+                        float p = 0.0f;
+                        for (int k = s * (in / 4); k < (s + 1) * (in / 4); ++k) p = fmaf(a[k], Wl[l][(int64_t)o * in + k], p);
+                        acc += p;
+                    }
                     if (l + 1 < n_layers) acc = acc / (1.0f + expf(-acc));
                     c[o] = acc;
                 }

@@ -4,10 +4,12 @@
 // a time, lane `sub` holding elements [8*sub, 8*sub+8) fetched with 128-bit loads, so one wave
 // load instruction brings in four whole rows.  A workgroup of 256 threads runs 16 such row streams,
 // each keeping its own online softmax (m, l, acc[8]) in registers in the log2 domain; the streams
-// are merged through LDS at the end.  Workgroups of one row's split publish (m, l, acc) partials and
-// take a ticket from a per-row counter; the workgroup that draws the last ticket merges the partials
-// with the usual log-sum-exp algebra and resets the counter, so a call is a single launch.  The
-// counters live at the end of the caller's workspace, which must be zero-filled before its first use.
+// are merged through LDS at the end, and workgroups of one row's split are merged by
+// merge_splits_kernel with the usual log-sum-exp algebra (launched only when a row is split at all).
+// The sparse kernel is software-pipelined: the K/V rows of step i+1 and the indices of step i+2 are in
+// flight while step i is reduced, so a wave always has 8 x 1 KiB of row data outstanding.
+#include <stdlib.h>
+
 #include "ha_common.h"
 
 namespace {
@@ -28,15 +30,36 @@ __device__ __forceinline__ float row16_sum(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+constexpr int kMinSplitRows = 64;
+
+// Tuning overrides (read once): HASHATTN_SPARSE_SPLIT_ROWS = rows of the index list per workgroup
+// (0 = whole list, no split merge), HASHATTN_SPARSE_THREADS = 256 or 512.
+inline int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return (e && *e) ? atoi(e) : dflt;
+}
+
 struct SparsePlan {
-    int split_rows;  // selected rows per workgroup, multiple of kStreams
+    int threads;     // workgroup size: 256 (16 row streams) or 512 (32)
+    int split_rows;  // selected rows per workgroup, multiple of 64
     int nsplit_max;
 };
 inline SparsePlan sparse_plan(int B, int H, int64_t idx_cap) {
+    static const int env_split = env_int("HASHATTN_SPARSE_SPLIT_ROWS", -1);
+    static const int env_threads = env_int("HASHATTN_SPARSE_THREADS", -1);
     SparsePlan p;
-    const int64_t wg256 = (int64_t)B * H * ((idx_cap + 255) / 256);
-    p.split_rows = wg256 >= 1024 ? 256 : 128;
-    p.nsplit_max = (int)((idx_cap + p.split_rows - 1) / p.split_rows);
+    const int64_t rows = (int64_t)B * H;
+    p.threads = env_threads == 256 || env_threads == 512 ? env_threads : 512;
+    // enough workgroups to keep 256 CUs busy (two 512-thread workgroups per CU), but no finer: when the
+    // rows alone supply them a row is not split and the merge launch disappears
+    int64_t want_splits = (512 + rows - 1) / rows;
+    int64_t split = (idx_cap + want_splits - 1) / want_splits;
+    if (env_split == 0) split = idx_cap;
+    else if (env_split > 0) split = env_split;
+    split = (split + kMinSplitRows - 1) / kMinSplitRows * kMinSplitRows;
+    if (split < kMinSplitRows) split = kMinSplitRows;
+    p.split_rows = (int)split;
+    p.nsplit_max = (int)((idx_cap + split - 1) / split);
     if (p.nsplit_max < 1) p.nsplit_max = 1;
     return p;
 }
@@ -58,72 +81,39 @@ inline DensePlan dense_plan(int B, int Hkv, int max_seq_len) {
     return p;
 }
 
-// Merge the 16 streams of a workgroup.  s_m/s_l [kStreams], s_acc [kStreams][128].  Thread e < 128 returns
+// Merge the NS streams of a workgroup.  s_m/s_l [NS], s_acc [NS][128].  Thread e < 128 returns
 // the merged (m, l, acc_e).
+template <int NS>
 __device__ __forceinline__ void merge_streams(const float *s_m, const float *s_l, const float *s_acc, int e, float &M, float &L,
                                               float &A) {
     M = -INFINITY;
 #pragma unroll
-    for (int s = 0; s < kStreams; ++s) M = fmaxf(M, s_m[s]);
+    for (int s = 0; s < NS; ++s) M = fmaxf(M, s_m[s]);
     L = 0.f;
     A = 0.f;
 #pragma unroll
-    for (int s = 0; s < kStreams; ++s) {
+    for (int s = 0; s < NS; ++s) {
         const float w = (s_m[s] == -INFINITY) ? 0.f : fast_exp2(s_m[s] - M);
         L += w * s_l[s];
         A += w * s_acc[s * HA_HEAD_DIM + e];
     }
 }
 
-// Publish this workgroup's partials and draw a ticket; true in every thread of the workgroup that
-// drew the last of `n` tickets.  Fences: the partial stores are made visible device-wide before the
-// ticket is drawn, and the last workgroup re-acquires before it reads the other workgroups' partials.
-__device__ __forceinline__ bool last_ticket(int32_t *ticket, int n, int *s_last) {
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) *s_last = (atomicAdd(ticket, 1) == n - 1) ? 1 : 0;
-    __syncthreads();
-    const bool last = *s_last != 0;
-    if (last) __threadfence();
-    return last;
-}
-
-// Threads e < 128 merge `nsplit` partials (acc [nsplit][128], ml [nsplit][2]) into one output row.
-template <typename E>
-__device__ __forceinline__ void merge_partials(const float *acc, const float *ml, int nsplit, char *out_row, int32_t *ticket,
-                                               bool reset) {
-    const int e = threadIdx.x;
-    if (e < HA_HEAD_DIM) {
-        float M = -INFINITY;
-#pragma unroll 4
-        for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[s * 2]);
-        float L = 0.f, A = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < nsplit; ++s) {
-            const float w = fast_exp2(ml[s * 2] - M);
-            L += w * ml[s * 2 + 1];
-            A += w * acc[(int64_t)s * HA_HEAD_DIM + e];
-        }
-        Elem<E>::store1(out_row, e, A / L);
-    }
-    if (reset && e == 0) *ticket = 0;  // leave the counter ready for the next call
-}
-
 // ------------------------------------------------------------------------------------------------
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
-template <typename E>
-__global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
-                                                                    const void *__restrict__ k, const void *__restrict__ v,
-                                                                    int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int G,
-                                                                    const int32_t *__restrict__ idx, int64_t idx_cap,
-                                                                    const int32_t *__restrict__ counts, float scale_log2e,
-                                                                    int split_rows, int nsplit_max, float *__restrict__ part_acc,
-                                                                    float *__restrict__ part_ml, int32_t *__restrict__ tickets,
-                                                                    void *__restrict__ out) {
+// NT threads = NT/16 row streams; U rows per stream per step.
+template <typename E, int NT, int U>
+__global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+                                                           const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
+                                                           int64_t kv_sh, int64_t kv_ss, int H, int G,
+                                                           const int32_t *__restrict__ idx, int64_t idx_cap,
+                                                           const int32_t *__restrict__ counts, float scale_log2e, int split_rows,
+                                                           int nsplit_max, float *__restrict__ part_acc,
+                                                           float *__restrict__ part_ml, void *__restrict__ out) {
     using EL = Elem<E>;
-    __shared__ float s_m[kStreams], s_l[kStreams];
-    __shared__ float s_acc[kStreams * HA_HEAD_DIM];
-    __shared__ int s_last;
+    constexpr int NS = NT / 16;  // row streams
+    __shared__ float s_m[NS], s_l[NS];
+    __shared__ float s_acc[NS * HA_HEAD_DIM];
 
     const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
@@ -141,6 +131,7 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
     const char *kb = (const char *)k + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const char *vb = (const char *)v + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;
+    constexpr int STEP = NS * U;  // rows of the list consumed per step by the workgroup
 
     float qf[8];
     {
@@ -149,52 +140,75 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
 #pragma unroll
         for (int i = 0; i < 8; ++i) qf[i] = t[i] * scale_log2e;
     }
-
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
 
-    for (int base = r0 + stream; base < r1; base += kStreams * kUnroll) {
-        int32_t jj[kUnroll];
-        bool ok[kUnroll];
+    // list position of (step base, u) for this stream; positions >= r1 are padded with the split's first row
+    auto list_index = [&](int base, int u) {
+        const int r = base + stream + u * NS;
+        return ix[r < r1 ? r : r0];
+    };
+    int32_t j_next[U];   // indices of the step after the one in flight
+    Raw8<E> kr[U], vr[U];
+    {
+        int32_t j0[U];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int r = base + u * kStreams;
-            ok[u] = r < r1;
-            jj[u] = ix[ok[u] ? r : base];
-        }
-        Raw8<E> kr[kUnroll], vr[kUnroll];
+        for (int u = 0; u < U; ++u) j0[u] = list_index(r0, u);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) kr[u] = EL::load8(kb + jj[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) j_next[u] = list_index(r0 + STEP, u);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + jj[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) kr[u] = EL::load8(kb + j0[u] * row_bytes, sub);
+#pragma unroll
+        for (int u = 0; u < U; ++u) vr[u] = EL::load8(vb + j0[u] * row_bytes, sub);
+    }
 
-        float sc[kUnroll], mloc = -INFINITY;
+    for (int base = r0; base < r1; base += STEP) {
+        // ---- issue the loads of the next step (harmless duplicates of row r0 past the end)
+        Raw8<E> kn[U], vn[U];
+        int32_t j_after[U];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
+        for (int u = 0; u < U; ++u) kn[u] = EL::load8(kb + j_next[u] * row_bytes, sub);
+#pragma unroll
+        for (int u = 0; u < U; ++u) vn[u] = EL::load8(vb + j_next[u] * row_bytes, sub);
+#pragma unroll
+        for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
+
+        // ---- reduce the current step
+        float sc[U], mloc = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
             float kf[8], d = 0.f;
             EL::unpack(kr[u], kf);
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
             d = row16_sum(d);
-            sc[u] = ok[u] ? d : -INFINITY;
+            sc[u] = (base + stream + u * NS < r1) ? d : -INFINITY;
             mloc = fmaxf(mloc, sc[u]);
         }
-        const float m_new = fmaxf(m, mloc);
-        const float alpha = fast_exp2(m - m_new);  // m == -inf on the first pass gives 0
-        l *= alpha;
+        if (mloc > -INFINITY) {  // at least one live row in this stream's step
+            const float m_new = fmaxf(m, mloc);
+            const float alpha = fast_exp2(m - m_new);  // m == -inf on the first pass gives 0
+            l *= alpha;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+            for (int i = 0; i < 8; ++i) acc[i] *= alpha;
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const float p = fast_exp2(sc[u] - m_new);
-            float vf[8];
-            EL::unpack(vr[u], vf);
-            l += p;
+            for (int u = 0; u < U; ++u) {
+                const float p = fast_exp2(sc[u] - m_new);
+                float vf[8];
+                EL::unpack(vr[u], vf);
+                l += p;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, vf[i], acc[i]);
+                for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, vf[i], acc[i]);
+            }
+            m = m_new;
         }
-        m = m_new;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            kr[u] = kn[u];
+            vr[u] = vn[u];
+            j_next[u] = j_after[u];
+        }
     }
 
     if (sub == 0) {
@@ -206,7 +220,7 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
     __syncthreads();
     if (tid < HA_HEAD_DIM) {
         float M, L, A;
-        merge_streams(s_m, s_l, s_acc, tid, M, L, A);
+        merge_streams<NS>(s_m, s_l, s_acc, tid, M, L, A);
         if (nsplit == 1) {
             EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
         } else {
@@ -218,10 +232,36 @@ __global__ __launch_bounds__(kAttThreads) void sparse_attend_kernel(const void *
             }
         }
     }
-    if (nsplit == 1) return;  // uniform
-    if (last_ticket(&tickets[row], nsplit, &s_last))
-        merge_partials<E>(part_acc + row * nsplit_max * HA_HEAD_DIM, part_ml + row * nsplit_max * 2, nsplit,
-                          (char *)out + row * HA_HEAD_DIM * EL::bytes, &tickets[row], true);
+}
+
+// grid (H, B), 128 threads: merge the split partials of a row.  `unit` = rows (sparse) or keys (dense) per
+// split; counts is per (b, h) row, per sequence (per_batch), or absent (every row has count_cap units).
+// Rows with a single split were finished by the attend kernel.
+template <typename E>
+__global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
+                                                                   const int32_t *__restrict__ counts, int per_batch,
+                                                                   int64_t count_cap, int H, int unit, int nsplit_max,
+                                                                   void *__restrict__ out) {
+    using EL = Elem<E>;
+    const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
+    const int64_t row = (int64_t)b * H + h;
+    int64_t n = counts ? counts[per_batch ? b : row] : count_cap;
+    if (n > count_cap) n = count_cap;
+    const int nsplit = (int)((n + unit - 1) / unit);
+    if (nsplit <= 1) return;
+    const float *ml = part_ml + row * nsplit_max * 2;
+    const float *pa = part_acc + row * nsplit_max * HA_HEAD_DIM + e;
+    float M = -INFINITY;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[s * 2]);
+    float L = 0.f, A = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) {
+        const float w = fast_exp2(ml[s * 2] - M);
+        L += w * ml[s * 2 + 1];
+        A += w * pa[(int64_t)s * HA_HEAD_DIM];
+    }
+    EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, A / L);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -233,12 +273,10 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
                                                                    int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int max_S,
                                                                    const int32_t *__restrict__ seq_lens, float scale_log2e, int chunk,
                                                                    int nsplit_max, float *__restrict__ part_acc,
-                                                                   float *__restrict__ part_ml, int32_t *__restrict__ tickets,
-                                                                   void *__restrict__ out) {
+                                                                   float *__restrict__ part_ml, void *__restrict__ out) {
     using EL = Elem<E>;
     __shared__ float s_m[kStreams], s_l[kStreams];
     __shared__ float s_acc[kStreams * HA_HEAD_DIM];
-    __shared__ int s_last;
 
     const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
@@ -340,7 +378,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
         __syncthreads();
         if (tid < HA_HEAD_DIM) {
             float M, L, A;
-            merge_streams(s_m, s_l, s_acc, tid, M, L, A);
+            merge_streams<kStreams>(s_m, s_l, s_acc, tid, M, L, A);
             const int64_t row = (int64_t)b * H + hk * G + g;
             if (nsplit == 1) {
                 EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
@@ -352,16 +390,6 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
                     part_ml[pi * 2 + 1] = L;
                 }
             }
-        }
-    }
-    if (nsplit == 1) return;  // uniform
-    int32_t *ticket = &tickets[b * (H / G) + hk];
-    if (last_ticket(ticket, nsplit, &s_last)) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const int64_t row = (int64_t)b * H + hk * G + g;
-            merge_partials<E>(part_acc + row * nsplit_max * HA_HEAD_DIM, part_ml + row * nsplit_max * 2, nsplit,
-                              (char *)out + row * HA_HEAD_DIM * EL::bytes, ticket, g == G - 1);
         }
     }
 }
@@ -383,10 +411,7 @@ int validate_qkv(const void *q, int64_t q_sb, int64_t q_sh, const void *k, const
     return HA_OK;
 }
 
-// partial accumulators, partial (m, l) pairs, then one ticket counter per row
-size_t part_bytes(int64_t rows, int nsplit_max) {
-    return (size_t)rows * nsplit_max * (HA_HEAD_DIM + 2) * sizeof(float) + (size_t)rows * sizeof(int32_t);
-}
+size_t part_bytes(int64_t rows, int nsplit_max) { return (size_t)rows * nsplit_max * (HA_HEAD_DIM + 2) * sizeof(float); }
 
 }  // namespace
 
@@ -394,7 +419,8 @@ extern "C" {
 
 size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap) {
     if (B <= 0 || H <= 0 || idx_cap <= 0) return 0;
-    return part_bytes((int64_t)B * H, sparse_plan(B, H, idx_cap).nsplit_max);
+    // sized for the finest split any plan uses, so tuning overrides never outgrow a caller's buffer
+    return part_bytes((int64_t)B * H, (int)((idx_cap + kMinSplitRows - 1) / kMinSplitRows));
 }
 
 int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
@@ -415,28 +441,38 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, cons
     const int64_t rows = (int64_t)B * H;
     float *part_acc = (float *)workspace;
     float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
-    int32_t *tickets = (int32_t *)(part_ml + rows * plan.nsplit_max * 2);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(plan.nsplit_max, H, B);
+    const dim3 grid(plan.nsplit_max, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-#define HA_SPARSE_LAUNCH(E_)                                                                                                      \
+#define HA_SPARSE_LAUNCH(E_, NT_, U_)                                                                                             \
     do {                                                                                                                          \
-        hipLaunchKernelGGL(sparse_attend_kernel<E_>, grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v, kv_stride_b, \
-                           kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows, plan.nsplit_max, part_acc, \
-                           part_ml, tickets, out);                                                                                \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,           \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
+                           plan.nsplit_max, part_acc, part_ml, out);                                                              \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
+        if (plan.nsplit_max > 1) {                                                                                                \
+            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
+                               plan.split_rows, plan.nsplit_max, out);                                                            \
+            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
+        }                                                                                                                         \
     } while (0)
-    if (kv_dtype == HA_BF16) HA_SPARSE_LAUNCH(ElemBF16);
-    else if (kv_dtype == HA_F16) HA_SPARSE_LAUNCH(ElemF16);
-    else HA_SPARSE_LAUNCH(ElemF32);
+#define HA_SPARSE_DISPATCH(E_, U_)                       \
+    do {                                                 \
+        if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_); \
+        else HA_SPARSE_LAUNCH(E_, 256, U_);              \
+    } while (0)
+    if (kv_dtype == HA_BF16) HA_SPARSE_DISPATCH(ElemBF16, 4);
+    else if (kv_dtype == HA_F16) HA_SPARSE_DISPATCH(ElemF16, 4);
+    else HA_SPARSE_DISPATCH(ElemF32, 2);
+#undef HA_SPARSE_DISPATCH
 #undef HA_SPARSE_LAUNCH
     return HA_OK;
 }
 
 size_t ha_dense_decode_workspace_bytes(int B, int H, int max_seq_len) {
     if (B <= 0 || H <= 0 || max_seq_len <= 0) return 0;
-    // the plan depends on Hkv only through the workgroup count; size for the worst case Hkv = 1
+    // the plan depends on Hkv only through the workgroup count; size for the worst case over Hkv
     int worst = 1;
     for (int hkv = 1; hkv <= H; hkv *= 2) {
         const int ns = dense_plan(B, hkv, max_seq_len).nsplit_max;
@@ -463,23 +499,27 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const
     const int64_t rows = (int64_t)B * H;
     float *part_acc = (float *)workspace;
     float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
-    int32_t *tickets = (int32_t *)(part_ml + rows * plan.nsplit_max * 2);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(plan.nsplit_max, Hkv, B);
+    const dim3 grid(plan.nsplit_max, Hkv, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
 #define HA_DENSE_LAUNCH(E_, G_)                                                                                                    \
     do {                                                                                                                           \
         hipLaunchKernelGGL((dense_attend_kernel<E_, G_>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,          \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, plan.chunk, plan.nsplit_max,      \
-                           part_acc, part_ml, tickets, out);                                                                       \
+                           part_acc, part_ml, out);                                                                                \
         HA_CHECK_LAUNCH("dense_attend_kernel");                                                                                    \
+        if (plan.nsplit_max > 1) {                                                                                                 \
+            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, seq_lens, 1,            \
+                               (int64_t)max_seq_len, H, plan.chunk, plan.nsplit_max, out);                                         \
+            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                                \
+        }                                                                                                                          \
     } while (0)
-#define HA_DENSE_DISPATCH(E_)                \
-    do {                                     \
-        if (G == 1) HA_DENSE_LAUNCH(E_, 1);  \
+#define HA_DENSE_DISPATCH(E_)                    \
+    do {                                         \
+        if (G == 1) HA_DENSE_LAUNCH(E_, 1);      \
         else if (G == 2) HA_DENSE_LAUNCH(E_, 2); \
         else if (G == 4) HA_DENSE_LAUNCH(E_, 4); \
-        else HA_DENSE_LAUNCH(E_, 8);         \
+        else HA_DENSE_LAUNCH(E_, 8);             \
     } while (0)
     if (kv_dtype == HA_BF16) HA_DENSE_DISPATCH(ElemBF16);
     else if (kv_dtype == HA_F16) HA_DENSE_DISPATCH(ElemF16);

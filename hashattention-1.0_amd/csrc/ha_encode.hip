@@ -29,18 +29,48 @@ __device__ __forceinline__ void fetch_weights(const float *Wt, int in, int out, 
     for (int i = 0; i < kMaxPerSeg; ++i) w[i] = (active && i < per) ? Wt[(int64_t)(seg * per + i) * out + o] : 0.f;
 }
 
-__global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__restrict__ x, int x_dtype, int64_t x_sb, int64_t x_sh,
-                                                                  int64_t x_st, int B, int x_heads, int n_heads, int T,
-                                                                  const float *__restrict__ weights, int64_t per_head, int n_layers,
-                                                                  int d_in, int d_int, int d_out, int arith,
-                                                                  uint32_t *__restrict__ codes, int64_t c_sb, int64_t c_sh, int pos0,
-                                                                  const int32_t *__restrict__ pos_dev, float *__restrict__ logits) {
+// One input tensor with its MLP heads and its destination in a code buffer.
+struct EncSide {
+    const void *x;
+    int x_dtype;
+    int64_t x_sb, x_sh, x_st;
+    int x_heads, n_heads;
+    const float *weights;
+    uint32_t *codes;
+    int64_t c_sb, c_sh;
+    int pos0;
+    const int32_t *pos_dev;
+    float *logits;
+};
+// Up to two sides share one launch (the new keys and the queries of a decode step): blockIdx.y runs over
+// the heads of side 0, then those of side 1.
+struct EncArgs {
+    EncSide side[2];
+    int B, T, n_layers, d_in, d_int, d_out, arith;
+    int64_t per_head;
+};
+
+__global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs a) {
     __shared__ float s_act[2][kRows][kMaxDim];
     __shared__ float s_part[kSeg][kRows][kMaxDim];
-    const int head = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
-    const int in_head = head / (n_heads / x_heads);
-    const int64_t n_rows = (int64_t)B * T;
-    const int64_t row0 = (int64_t)tile * kRows;
+    const bool second = (int)blockIdx.y >= a.side[0].n_heads;
+    const EncSide &sd = a.side[second ? 1 : 0];
+    const int head = second ? blockIdx.y - a.side[0].n_heads : blockIdx.y;
+    const int tile = blockIdx.x, tid = threadIdx.x;
+    const void *__restrict__ x = sd.x;
+    const int x_dtype = sd.x_dtype;
+    const int64_t x_sb = sd.x_sb, x_sh = sd.x_sh, x_st = sd.x_st;
+    const int n_heads = sd.n_heads, T = a.T, n_layers = a.n_layers, d_in = a.d_in, d_int = a.d_int, d_out = a.d_out, arith = a.arith;
+    const float *__restrict__ weights = sd.weights;
+    const int64_t per_head = a.per_head;
+    uint32_t *__restrict__ codes = sd.codes;
+    const int64_t c_sb = sd.c_sb, c_sh = sd.c_sh;
+    const int pos0 = sd.pos0;
+    const int32_t *__restrict__ pos_dev = sd.pos_dev;
+    float *__restrict__ logits = sd.logits;
+    const int in_head = head / (n_heads / sd.x_heads);
+    const int n_rows = a.B * T;  // < 2^31, validated on the host
+    const int row0 = tile * kRows;
 
     const float *w = weights + head * per_head;
     // thread -> (o, seg) of a layer with `out` outputs: the first out*kSeg threads, o fastest; wider layers loop
@@ -52,10 +82,10 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__
 
     for (int i = tid; i < kRows * d_in; i += kEncThreads) {
         const int r = i / d_in, e = i % d_in;
-        const int64_t row = row0 + r;
+        const int row = row0 + r;
         float val = 0.f;
         if (row < n_rows) {
-            const int64_t b = row / T, t = row % T;
+            const int b = row / T, t = row % T;
             val = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
             if (arith == HA_ARITH_BF16) val = ha_round_bf16(val);
         }
@@ -129,13 +159,13 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const void *__
     const int W = d_out / 32;
     const int wave = tid >> 6, lane = tid & 63;
     for (int r = 0; r < kRows; ++r) {
-        const int64_t row = row0 + r;
+        const int row = row0 + r;
         if (row >= n_rows) break;  // uniform
-        const int64_t b = row / T, t = row % T;
+        const int b = row / T, t = row % T;
         const bool bit = tid < d_out && s_act[cur][r][tid] > 0.0f;
         const uint64_t bal = __ballot(bit);
-        if (logits && tid < d_out) logits[((b * n_heads + head) * T + t) * d_out + tid] = s_act[cur][r][tid];
-        const int64_t pos = (pos_dev ? pos_dev[b] : pos0) + t;
+        if (logits && tid < d_out) logits[(((int64_t)b * n_heads + head) * T + t) * d_out + tid] = s_act[cur][r][tid];
+        const int64_t pos = (int64_t)(pos_dev ? pos_dev[b] : pos0) + t;
         uint32_t *c = codes + b * c_sb + head * c_sh + pos * W;
         if (lane == 0 && wave * 2 < W) c[wave * 2] = (uint32_t)bal;
         if (lane == 32 && wave * 2 + 1 < W) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
@@ -181,13 +211,44 @@ int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_str
     if (st) return st;
     HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
     HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
-    const int64_t tiles = ((int64_t)B * T + kRows - 1) / kRows;
-    HA_REQUIRE(tiles <= 2147483647LL, HA_ERR_BAD_SHAPE, "too many rows for one launch");
+    HA_REQUIRE((int64_t)B * T < 2147483647LL - kRows, HA_ERR_BAD_SHAPE, "too many rows for one launch");
     if ((st = ha_require_device())) return st;
-    const int64_t per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
-    hipLaunchKernelGGL(encode_pack_kernel, dim3((unsigned)tiles, n_heads), dim3(kEncThreads), 0, (hipStream_t)stream, x, x_dtype,
-                       x_stride_b, x_stride_h, x_stride_t, B, x_heads, n_heads, T, weights, per_head, n_layers, head_dim, int_dim,
-                       final_dim, arith, codes, c_stride_b, c_stride_h, pos0, pos_dev, logits);
+    EncArgs a = {};
+    a.side[0] = EncSide{x, x_dtype, x_stride_b, x_stride_h, x_stride_t, x_heads, n_heads, weights, codes, c_stride_b, c_stride_h,
+                        pos0, pos_dev, logits};
+    a.side[1] = a.side[0];
+    a.side[1].n_heads = 0;
+    a.B = B; a.T = T; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
+    a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    const unsigned tiles = (unsigned)(((int64_t)B * T + kRows - 1) / kRows);
+    hipLaunchKernelGGL(encode_pack_kernel, dim3(tiles, n_heads), dim3(kEncThreads), 0, (hipStream_t)stream, a);
+    HA_CHECK_LAUNCH("encode_pack_kernel");
+    return HA_OK;
+}
+
+int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_t, const void *q, int64_t q_stride_b,
+                   int64_t q_stride_h, int x_dtype, int B, int Hkv, int Hc, int H, int T_new, const float *weights_k,
+                   const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim, int arith, uint32_t *kcodes,
+                   int64_t kc_stride_b, int64_t kc_stride_h, int pos0, const int32_t *pos_dev, uint32_t *qcodes, void *stream) {
+    int st = validate_encode(k_new, B, Hkv, Hc, T_new, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b,
+                             kc_stride_h, pos0);
+    if (st) return st;
+    HA_REQUIRE(q && weights_q && qcodes, HA_ERR_NULL_POINTER, "q/weights_q/qcodes is NULL");
+    HA_REQUIRE(H > 0 && H + Hc <= 65535, HA_ERR_BAD_SHAPE, "H must be positive and H + Hc <= 65535");
+    HA_REQUIRE(T_new == 1, HA_ERR_BAD_SHAPE, "ha_encode_step encodes one new key per sequence (T_new=%d)", T_new);
+    HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
+    HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
+    if ((st = ha_require_device())) return st;
+    const int W = final_dim / 32;
+    EncArgs a = {};
+    a.side[0] = EncSide{k_new, x_dtype, k_stride_b, k_stride_h, k_stride_t, Hkv, Hc, weights_k, kcodes, kc_stride_b, kc_stride_h,
+                        pos0, pos_dev, nullptr};
+    a.side[1] = EncSide{q, x_dtype, q_stride_b, q_stride_h, (int64_t)head_dim, H, H, weights_q, qcodes, (int64_t)H * W, (int64_t)W,
+                        0, nullptr, nullptr};
+    a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
+    a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);
+    hipLaunchKernelGGL(encode_pack_kernel, dim3(tiles, Hc + H), dim3(kEncThreads), 0, (hipStream_t)stream, a);
     HA_CHECK_LAUNCH("encode_pack_kernel");
     return HA_OK;
 }

@@ -7,12 +7,12 @@
 //   1. select_hist_kernel       grid (chunk, code head, sequence): per-chunk histograms of the distances
 //                               of every query head of the group, one streaming pass over the codes
 //   2. select_threshold_kernel  grid (head, sequence): T, r, per-chunk output offsets, window indices, counts
-//   3. select_compact_kernel    grid as 1: ordered wave-ballot compaction into ascending index lists
+//   3. select_compact_kernel    grid as 1: ordered compaction (bit masks + one DPP scan) into ascending index lists
 // Pass 3 re-reads the codes (4*W bytes per token) from L2 / Infinity Cache.
 //
-// Both streaming kernels fetch all codes of their chunk before using any: a lane holds 4 consecutive
-// codes per 1024-code block (128-bit loads), up to 4 blocks per workgroup, so a workgroup has its whole
-// chunk in flight at once instead of paying one memory round trip per tile.
+// Both streaming kernels fetch all codes of their chunk before using any (128-bit loads, up to 16 codes
+// per lane), so a workgroup has its whole chunk in flight at once instead of paying one memory round
+// trip per tile.
 #include "ha_common.h"
 
 namespace {
@@ -311,7 +311,25 @@ __global__ __launch_bounds__(kSelThreads) void select_threshold_kernel(const uin
 }
 
 // ------------------------------------------------------------------------------------------------
-// Pass 3.  grid (nchunk, Hc, B).  Output order = block, wave, lane, element = ascending token index.
+// wave64 inclusive scan of a u32 (two packed 16-bit counters ride along for free): Hillis-Steele inside
+// each 16-lane DPP row, then the row totals are carried across rows with row_bcast15 / row_bcast31.
+#define HA_DPP_ADD(v, ctrl, row_mask) \
+    (v) += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), (row_mask), 0xF, true)
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    HA_DPP_ADD(v, 0x111, 0xF);  // row_shr:1
+    HA_DPP_ADD(v, 0x112, 0xF);  // row_shr:2
+    HA_DPP_ADD(v, 0x114, 0xF);  // row_shr:4
+    HA_DPP_ADD(v, 0x118, 0xF);  // row_shr:8
+    HA_DPP_ADD(v, 0x142, 0xA);  // row_bcast:15 into rows 1 and 3
+    HA_DPP_ADD(v, 0x143, 0xC);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+#undef HA_DPP_ADD
+
+// Pass 3.  grid (nchunk, Hc, B).  A wave owns a contiguous quarter of the chunk and a lane 4*blocks
+// consecutive codes of it, so "wave, lane, element" is ascending token order.  Per head a lane turns its
+// codes into two bit masks (d < T, d == T); one packed DPP scan gives every lane the number of such tokens
+// before it, and only the set bits are visited when the indices are written.
 template <int W, int GQ>
 __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
                                                                      const uint32_t *__restrict__ qcodes, int H, int max_S,
@@ -319,7 +337,8 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
                                                                      int blocks, int nchunk, int vec, const int32_t *__restrict__ meta,
                                                                      const int32_t *__restrict__ chunk_pre,
                                                                      int32_t *__restrict__ out_idx, int64_t idx_cap) {
-    __shared__ int s_cnt[kMaxBlocks][kSelWaves][GQ][2];
+    constexpr int CPL = 4 * kMaxBlocks;  // codes per lane at most
+    __shared__ uint32_t s_wtot[kSelWaves][GQ];
 
     const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -331,8 +350,25 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
     const int beg = max(lo, c * chunk), end = min(hi, (c + 1) * chunk);
     if (beg >= end) return;  // uniform over the workgroup
 
-    ChunkRegs<W> cr;
-    load_chunk<W>(kcodes + b * kc_sb + hc * kc_sh, c * chunk, blocks, beg, end, vec != 0, wave, lane, cr);
+    const int cpl = 4 * blocks;
+    const int j_lane = c * chunk + (wave * HA_WAVE + lane) * cpl;
+    const uint32_t *kc = kcodes + b * kc_sb + hc * kc_sh;
+    Code<W> k[CPL];
+    uint32_t vmask = 0;  // bit e: code j_lane + e is a candidate of this chunk
+#pragma unroll
+    for (int i = 0; i < kMaxBlocks; ++i) {
+        const int j0 = j_lane + 4 * i;
+        const bool live = i < blocks && j0 + 4 > beg && j0 < end;
+        Code<W> k4[4];
+        if (live) load_code4<W>(kc, j0, beg, end, vec != 0, k4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (live) k[4 * i + e] = k4[e];
+            else if constexpr (W == 1) k[4 * i + e] = Code<1>{0u};
+            else k[4 * i + e] = Code<2>{0u, 0u};
+            if (live && j0 + e >= beg && j0 + e < end) vmask |= 1u << (4 * i + e);
+        }
+    }
 
     Code<W> q[GQ];
     int T[GQ], r[GQ], lt_pre[GQ], eq_pre[GQ];
@@ -349,78 +385,46 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
     }
     if (!any) return;  // uniform: nothing heavy to write for this group
 
-    // ---- counts per (block, wave)
+    uint32_t ltm[GQ], eqm[GQ], incl[GQ];
 #pragma unroll
-    for (int blk = 0; blk < kMaxBlocks; ++blk) {
-        if (blk >= blocks) break;
+    for (int g = 0; g < GQ; ++g) {
+        uint32_t lt = 0, eq = 0;
 #pragma unroll
-        for (int g = 0; g < GQ; ++g) {
-            int nlt = 0, neq = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = cr.j0[blk] + e;
-                const bool valid = j >= beg && j < end;
-                const int d = cr.k[blk][e].dist(q[g]);
-                nlt += __popcll(__ballot(valid && d < T[g]));
-                neq += __popcll(__ballot(valid && d == T[g]));
-            }
-            if (lane == 0) {
-                s_cnt[blk][wave][g][0] = nlt;
-                s_cnt[blk][wave][g][1] = neq;
-            }
+        for (int e = 0; e < CPL; ++e) {
+            const int d = k[e].dist(q[g]);
+            lt |= (d < T[g] ? 1u : 0u) << e;
+            eq |= (d == T[g] ? 1u : 0u) << e;
         }
+        ltm[g] = lt & vmask;
+        eqm[g] = eq & vmask;
+        incl[g] = wave_inclusive_scan((uint32_t)__popc(ltm[g]) | ((uint32_t)__popc(eqm[g]) << 16));
+        if (lane == HA_WAVE - 1) s_wtot[wave][g] = incl[g];
     }
     __syncthreads();
 
-    // ---- ordered compaction
-    int run_lt[GQ], run_eq[GQ];
 #pragma unroll
     for (int g = 0; g < GQ; ++g) {
-        run_lt[g] = lt_pre[g];
-        run_eq[g] = eq_pre[g];
-    }
-#pragma unroll
-    for (int blk = 0; blk < kMaxBlocks; ++blk) {
-        if (blk >= blocks) break;
-#pragma unroll
-        for (int g = 0; g < GQ; ++g) {
-            int lt_before = run_lt[g], eq_before = run_eq[g];
-            for (int w = 0; w < wave; ++w) {
-                lt_before += s_cnt[blk][w][g][0];
-                eq_before += s_cnt[blk][w][g][1];
+        const uint32_t excl = incl[g] - ((uint32_t)__popc(ltm[g]) | ((uint32_t)__popc(eqm[g]) << 16));
+        int n_lt = lt_pre[g] + (int)(excl & 0xFFFFu), n_eq = eq_pre[g] + (int)(excl >> 16);
+        for (int w = 0; w < wave; ++w) {
+            const uint32_t t = s_wtot[w][g];
+            n_lt += (int)(t & 0xFFFFu);
+            n_eq += (int)(t >> 16);
+        }
+        const int rg = r[g];
+        int32_t *o = out_idx + ((int64_t)b * H + hc * GQ + g) * idx_cap;
+        const uint32_t em = n_eq < rg ? eqm[g] : 0u;  // past the r-th tie nothing more of the tie bucket is taken
+        uint32_t todo = ltm[g] | em;
+        while (todo) {
+            const int e = __ffs((int)todo) - 1;
+            todo &= todo - 1;
+            const bool is_eq = (em >> e) & 1u;
+            if (!is_eq || n_eq < rg) {
+                const int64_t pos = (int64_t)lo + n_lt + min(n_eq, rg);
+                if (pos < idx_cap) o[pos] = j_lane + e;
             }
-            // lane-level prefix over the 4 elements of every lower lane, then over this lane's earlier elements
-            bool is_lt[4], is_eq[4];
-            uint64_t bal_lt[4], bal_eq[4];
-            int lt_lane = 0, eq_lane = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = cr.j0[blk] + e;
-                const bool valid = j >= beg && j < end;
-                const int d = cr.k[blk][e].dist(q[g]);
-                is_lt[e] = valid && d < T[g];
-                is_eq[e] = valid && d == T[g];
-                bal_lt[e] = __ballot(is_lt[e]);
-                bal_eq[e] = __ballot(is_eq[e]);
-                lt_lane += lanes_below(bal_lt[e]);
-                eq_lane += lanes_below(bal_eq[e]);
-            }
-            int n_lt = lt_before + lt_lane, n_eq = eq_before + eq_lane;  // tokens before (lane, element 0)
-            int32_t *o = out_idx + ((int64_t)b * H + hc * GQ + g) * idx_cap;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const bool sel = is_lt[e] || (is_eq[e] && n_eq < r[g]);
-                if (sel) {
-                    const int64_t pos = (int64_t)lo + n_lt + min(n_eq, r[g]);
-                    if (pos < idx_cap) o[pos] = cr.j0[blk] + e;
-                }
-                n_lt += is_lt[e] ? 1 : 0;
-                n_eq += is_eq[e] ? 1 : 0;
-            }
-            for (int w = 0; w < kSelWaves; ++w) {
-                run_lt[g] += s_cnt[blk][w][g][0];
-                run_eq[g] += s_cnt[blk][w][g][1];
-            }
+            n_lt += is_eq ? 0 : 1;
+            n_eq += is_eq ? 1 : 0;
         }
     }
 }

@@ -53,6 +53,9 @@ def load_library() -> C.CDLL:
     lib.ha_encode_pack.restype = i32
     lib.ha_encode_pack.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32, i32,
                                    vp, i64, i64, i32, vp, vp, vp]
+    lib.ha_encode_step.restype = i32
+    lib.ha_encode_step.argtypes = [vp, i64, i64, i64, vp, i64, i64, i32, i32, i32, i32, i32, i32, vp, vp,
+                                   i32, i32, i32, i32, i32, vp, i64, i64, i32, vp, vp, vp]
     lib.ha_encode_pack_prefill.restype = i32
     lib.ha_encode_pack_prefill.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32,
                                            vp, i64, i64, i32, vp, vp]
@@ -97,9 +100,8 @@ def _require_cuda(*tensors):
 
 
 def workspace(nbytes: int, device) -> torch.Tensor:
-    """A zero-filled byte buffer of at least nbytes (torch's allocator returns >= 256-byte aligned blocks).
-    The decode workspaces end with ticket counters that must start at zero."""
-    return torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+    """A byte buffer of at least nbytes (torch's allocator returns >= 256-byte aligned blocks)."""
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
 # ------------------------------------------------------------------------------------------ encode
@@ -149,6 +151,23 @@ def encode_pack(x: torch.Tensor, weights: torch.Tensor, n_layers: int, int_dim: 
                               _ptr(codes), codes.stride(0), codes.stride(1), pos0, _ptr(pos_dev), _ptr(logits), _stream(x)),
            "ha_encode_pack")
     return logits
+
+
+def encode_step(k_new: torch.Tensor, q3: torch.Tensor, wk: torch.Tensor, wq: torch.Tensor, n_layers: int, int_dim: int,
+                final_dim: int, kcodes: torch.Tensor, qcodes: torch.Tensor, pos0: int = 0,
+                pos_dev: Optional[torch.Tensor] = None, arith: int = HA_ARITH_F32) -> None:
+    """One launch for a decode step: k_new [B, Hkv, 1, d] appended to kcodes at pos0 / pos_dev[b]; q3 [B, H, d] -> qcodes [B, H, W]."""
+    _require_cuda(k_new, q3, wk, wq, kcodes, qcodes, pos_dev)
+    lib = load_library()
+    B, Hkv, T, d = k_new.shape
+    H = q3.shape[1]
+    assert T == 1 and k_new.stride(3) == 1 and q3.stride(2) == 1 and k_new.dtype == q3.dtype
+    assert kcodes.stride(3) == 1 and kcodes.stride(2) == kcodes.shape[3] and qcodes.is_contiguous()
+    assert kcodes.dtype == torch.int32 and qcodes.dtype == torch.int32 and qcodes.numel() == B * H * (final_dim // 32)
+    _check(lib.ha_encode_step(_ptr(k_new), k_new.stride(0), k_new.stride(1), k_new.stride(2), _ptr(q3), q3.stride(0), q3.stride(1),
+                              _DTYPE[k_new.dtype], B, Hkv, wk.shape[0], H, 1, _ptr(wk), _ptr(wq), n_layers, d, int_dim, final_dim,
+                              arith, _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), pos0, _ptr(pos_dev), _ptr(qcodes),
+                              _stream(q3)), "ha_encode_step")
 
 
 def encode_pack_prefill(x: torch.Tensor, weights_bf16: torch.Tensor, n_layers: int, int_dim: int, final_dim: int,

@@ -4,8 +4,7 @@
 (hashattention/hashattention_llama.py:401-446, 578-615): the packed hash-MLP weights and the bit-cache of
 key codes, plus the index lists and workspaces of the kernels.  One decode step is
 
-    append   codes of the new key(s) -> bit-cache           (ha_encode_pack)
-    q codes  codes of the query                             (ha_encode_pack)
+    encode   code of the new key -> bit-cache, query codes  (ha_encode_step, one launch)
     select   Hamming histogram + ordered compaction         (ha_select)
     attend   gather-only split-K attention                  (ha_sparse_decode)
 
@@ -104,17 +103,21 @@ class HashDecodeLayer:
         bit-cache; everything before must already be there (`encode_keys` at prefill).  Ragged batches pass
         `seq_lens` (int32 [B], lengths including the new token) and `seq_len` = their maximum.
         """
+        q3 = q[:, :, 0, :]
         if seq_lens is None:
             if self.n_cached + n_new != seq_len:
                 raise RuntimeError(f"bit-cache holds {self.n_cached} tokens, step at length {seq_len} appends {n_new}")
-            self.encode_keys(k_cache[:, :, seq_len - n_new:seq_len], pos0=seq_len - n_new)
+            if n_new > 1:       # a short multi-token append: older tokens first, the newest rides with the query
+                self.encode_keys(k_cache[:, :, seq_len - n_new:seq_len - 1], pos0=seq_len - n_new)
+            _ops.encode_step(k_cache[:, :, seq_len - 1:seq_len], q3, self.wk, self.wq, self.num_layers, self.int_dim,
+                             self.final_dim, self.codes, self.qcodes, pos0=seq_len - 1, arith=self.arith)
             self.n_cached = seq_len
         else:
             # ragged: the new key of sequence b sits at seq_lens[b] - 1
             pos = (seq_lens - 1).to(torch.int32)
             newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
-            self.encode_keys(newk, pos_dev=pos)
-        self.encode_query(q)
+            _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
+                             self.qcodes, pos_dev=pos, arith=self.arith)
         self.select(seq_len, seq_lens)
-        self.attend(q[:, :, 0, :], k_cache, v_cache, out)
+        self.attend(q3, k_cache, v_cache, out)
         return out

@@ -85,6 +85,22 @@ int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_str
                    float *logits, void *stream);
 
 /*
+ * The encode of one decode step in a single launch: the newest key of every sequence is appended to
+ * the bit-cache (as ha_encode_pack with T = 1) and the query codes are written to qcodes [B, H, W].
+ * Replaces the q_embedding / k_embedding pair of the cached branch of compute_mask_multi
+ * (hashattention_llama.py:411-414).
+ *   k_new [B, Hkv, 1, head_dim], q [B, H, head_dim] (strides q_stride_{b,h}), both of x_dtype
+ *   weights_k: Hc heads, weights_q: H heads (packed as for ha_encode_pack)
+ */
+int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_t,
+                   const void *q, int64_t q_stride_b, int64_t q_stride_h, int x_dtype,
+                   int B, int Hkv, int Hc, int H, int T_new,
+                   const float *weights_k, const float *weights_q,
+                   int n_layers, int head_dim, int int_dim, int final_dim, int arith,
+                   uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, int pos0, const int32_t *pos_dev,
+                   uint32_t *qcodes, void *stream);
+
+/*
  * Bulk (prefill) encode on the matrix cores: the same mapping as ha_encode_pack in HA_ARITH_BF16
  * arithmetic, computed as three chained bf16 MFMA GEMMs per 128-token tile.  x must be bf16,
  * head_dim == int_dim == 128.  `weights_bf16` is the blob of ha_usa_packed_floats() elements per
@@ -138,9 +154,8 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
  *   q   [B, H, 128] kv_dtype, strides q_stride_{b,h}
  *   k,v [B, Hkv, ., 128] kv_dtype, strides kv_stride_{b,h,s}; rows 16-byte aligned
  *   out [B, H, 128] kv_dtype contiguous
- *   workspace  ha_sparse_decode_workspace_bytes(...) bytes, 256-byte aligned.  It ends with one ticket
- *              counter per row: ZERO-FILL the workspace once before its first use; every completed
- *              call leaves the counters at zero again.  Calls sharing a workspace must not overlap.
+ *   workspace  ha_sparse_decode_workspace_bytes(...) bytes, 256-byte aligned; calls that share a
+ *              workspace must not overlap
  */
 size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap);
 int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
@@ -153,8 +168,7 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
  * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).
  * Replaces flash_decode_attention_fwd (efficiency/kernels/flash_fwd_sparse.py:21-321) and
  * torch_attention_naive (efficiency/kernels/torchatt.py:17-30).  Each K/V row is read once per KV
- * head and shared by the query heads of its group.  Workspace rules as for ha_sparse_decode
- * (zero-filled before first use, not shared by overlapping calls).
+ * head and shared by the query heads of its group.  Workspace rules as for ha_sparse_decode.
  */
 size_t ha_dense_decode_workspace_bytes(int B, int H, int max_seq_len);
 int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,

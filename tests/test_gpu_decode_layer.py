@@ -1,0 +1,67 @@
+"""End-to-end decode steps through HashDecodeLayer (bit-cache append -> select -> attend) against the oracle's
+restatement of the reference layer (dense scores, every key re-hashed, stable sort, masked fp32 softmax)."""
+import numpy as np
+import pytest
+import torch
+
+from hashattention import _ops
+from hashattention.decode import HashDecodeLayer
+from hashattention.synthetic import make_problem
+from oracle import hashattn_oracle as orc
+from tests.parity_util import small_workload
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _layer(w, p, **kw):
+    return HashDecodeLayer(p.usa.k, p.usa.q, w.n_q_heads, w.n_kv_heads, w.head_dim, w.lth_num_layers, w.lth_int_dim,
+                           w.lth_final_dim, w.init_budget, w.recent_budget, w.heavy_budget, device=DEV, **kw)
+
+
+@pytest.mark.parametrize("hc", [2, 8])
+def test_three_decode_steps_match_reference_layer(hc):
+    # fp32 end to end: the step output equals the reference layer's masked dense attention on the same cache
+    print(f"\n[case] decode layer Hc={hc}", flush=True)
+    w = small_workload(batch=2, seq_lens=[900, 900], n_code_heads=hc, dtype=torch.float32, seed=17)
+    p = make_problem(w)
+    S = w.max_seq_len
+    k, v = p.k.to(DEV), p.v.to(DEV)
+    layer = _layer(w, p)
+    layer.allocate(w.batch, S)
+    s0 = S - 3
+    layer.encode_keys(k[:, :, :s0])
+    layer.n_cached = s0
+    g = torch.Generator().manual_seed(5)
+    for step in range(3):
+        s = s0 + step + 1
+        q = torch.randn(w.batch, w.n_q_heads, 1, w.head_dim, generator=g)
+        out = torch.empty(w.batch, w.n_q_heads, w.head_dim, device=DEV)
+        layer.step(q.to(DEV), k, v, s, out)
+        ref, mask = orc.reference_decode_attention(q, p.k[:, :, :s], p.v[:, :, :s], p.usa.k, p.usa.q, w.init_budget,
+                                                   w.recent_budget, w.heavy_budget)
+        # selected sets must be identical (codes may differ only at |logit| ~ 0, which would show up here)
+        idx = layer.idx.cpu().numpy()
+        cnt = layer.counts.cpu().numpy()
+        for b in range(w.batch):
+            for h in range(w.n_q_heads):
+                got = np.zeros(s, dtype=bool)
+                got[idx[b, h, :cnt[b, h]]] = True
+                assert np.array_equal(got, mask[b, h, 0].numpy()), (step, b, h)
+        err = (out.cpu() - ref[:, :, 0]).abs().max().item()
+        assert err < 2e-5, err
+
+
+def test_step_refuses_a_gap_in_the_bit_cache():
+    w = small_workload(batch=1, seq_lens=[200], seed=3)
+    p = make_problem(w)
+    layer = _layer(w, p)
+    layer.allocate(1, 200)
+    out = torch.empty(1, w.n_q_heads, 128, dtype=w.dtype, device=DEV)
+    with pytest.raises(RuntimeError):
+        layer.step(p.q.to(DEV), p.k.to(DEV), p.v.to(DEV), 200, out)   # nothing cached yet, one token appended
+
+
+def test_cpu_tensors_are_refused():
+    with pytest.raises(ValueError):
+        _ops.hamming_score(torch.zeros(1, 1, 4, 1, dtype=torch.int32), torch.zeros(1, 1, 1, dtype=torch.int32), 4)

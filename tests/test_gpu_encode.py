@@ -95,3 +95,29 @@ def test_exact_zero_logit_gives_bit_zero():
     _ops.encode_pack(x, _ops.pack_usa_weights([[(W1, b1)]], DEV), 1, 128, 32, codes)
     want = sum(1 << i for i in range(0, 32, 2))
     assert (codes.cpu().numpy().view(np.uint32) == want).all()
+
+
+def test_encode_step_equals_two_encode_packs():
+    # the single-launch step encode (new key + query) writes exactly what two separate launches write
+    print("\n[case] encode_step", flush=True)
+    for ragged in (False, True):
+        w = small_workload(batch=5, seq_lens=[300] * 5, n_q_heads=8, n_kv_heads=2, n_code_heads=2, seed=91)
+        p = make_problem(w)
+        k, q = p.k.to(DEV), p.q.to(DEV)
+        wk, wq = _ops.pack_usa_weights(p.usa.k, DEV), _ops.pack_usa_weights(p.usa.q, DEV)
+        a = torch.full((5, 2, 304, 1), 7, dtype=torch.int32, device=DEV)
+        b = a.clone()
+        qa = torch.zeros(5, 8, 1, 1, dtype=torch.int32, device=DEV)
+        qb = torch.zeros(5, 8, 1, dtype=torch.int32, device=DEV)
+        if ragged:
+            pos = torch.tensor([299, 10, 0, 150, 298], dtype=torch.int32, device=DEV)
+            newk = torch.gather(k, 2, pos.view(-1, 1, 1, 1).expand(-1, 2, 1, 128).long())
+            _ops.encode_pack(newk, wk, 3, 128, 32, a, pos_dev=pos)
+            _ops.encode_step(newk, q[:, :, 0, :], wk, wq, 3, 128, 32, b, qb, pos_dev=pos)
+        else:
+            _ops.encode_pack(k[:, :, 299:300], wk, 3, 128, 32, a, pos0=299)
+            _ops.encode_step(k[:, :, 299:300], q[:, :, 0, :], wk, wq, 3, 128, 32, b, qb, pos0=299)
+        _ops.encode_pack(q, wq, 3, 128, 32, qa)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b) and torch.equal(qa.view(5, 8, 1), qb)
+        assert int((a != 7).sum()) == 5 * 2

@@ -115,7 +115,12 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     __shared__ float s_m[NS], s_l[NS];
     __shared__ float s_acc[NS * HA_HEAD_DIM];
 
-    const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
+    // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
+    // there are 8 KV heads, i.e. on one XCD, so rows they share (the sink and recent windows, commonly
+    // selected keys) are served by that XCD's L2 instead of being fetched from HBM once per XCD.
+    const int Hkv = H / G;
+    const int sp = blockIdx.x, h = ((int)blockIdx.y % Hkv) * G + (int)blockIdx.y / Hkv, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
     int64_t n = counts[b * H + h];
     if (n > idx_cap) n = idx_cap;

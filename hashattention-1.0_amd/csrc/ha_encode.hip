@@ -22,13 +22,6 @@ constexpr int kRows = 4;       // input rows per workgroup
 constexpr int kMaxDim = 256;
 constexpr int kMaxPerSeg = kMaxDim / kSeg;
 
-// the weights thread (o, seg) needs for one layer: W[k][o] for k in its segment
-__device__ __forceinline__ void fetch_weights(const float *Wt, int in, int out, int o, int seg, bool active, float (&w)[kMaxPerSeg]) {
-    const int per = in / kSeg;
-#pragma unroll
-    for (int i = 0; i < kMaxPerSeg; ++i) w[i] = (active && i < per) ? Wt[(int64_t)(seg * per + i) * out + o] : 0.f;
-}
-
 // One input tensor with its MLP heads and its destination in a code buffer.
 struct EncSide {
     const void *x;
@@ -50,8 +43,13 @@ struct EncArgs {
     int64_t per_head;
 };
 
+// NL_/DIN_/DINT_/DOUT_ fix the MLP shape at compile time (0 = read it from the arguments).  The usual
+// shapes (128 -> 128 [-> 128] -> 32|64) are instantiated: with constant trip counts the weight fetch is
+// 72 plain loads and the kernel is a few hundred instructions, which matters because a decode step is
+// bound by this kernel's dependent-issue latency, not by its throughput.
+template <int NL_, int DIN_, int DINT_, int DOUT_>
 __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs a) {
-    __shared__ float s_act[2][kRows][kMaxDim];
+    __shared__ __align__(16) float s_act[2][kRows][kMaxDim];
     __shared__ float s_part[kSeg][kRows][kMaxDim];
     const bool second = (int)blockIdx.y >= a.side[0].n_heads;
     const EncSide &sd = a.side[second ? 1 : 0];
@@ -60,7 +58,9 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
     const void *__restrict__ x = sd.x;
     const int x_dtype = sd.x_dtype;
     const int64_t x_sb = sd.x_sb, x_sh = sd.x_sh, x_st = sd.x_st;
-    const int n_heads = sd.n_heads, T = a.T, n_layers = a.n_layers, d_in = a.d_in, d_int = a.d_int, d_out = a.d_out, arith = a.arith;
+    const int n_heads = sd.n_heads, T = a.T, arith = a.arith;
+    const int n_layers = NL_ ? NL_ : a.n_layers, d_in = DIN_ ? DIN_ : a.d_in, d_int = DINT_ ? DINT_ : a.d_int,
+              d_out = DOUT_ ? DOUT_ : a.d_out;
     const float *__restrict__ weights = sd.weights;
     const int64_t per_head = a.per_head;
     uint32_t *__restrict__ codes = sd.codes;
@@ -72,12 +72,29 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
     const int n_rows = a.B * T;  // < 2^31, validated on the host
     const int row0 = tile * kRows;
 
-    const float *w = weights + head * per_head;
-    // thread -> (o, seg) of a layer with `out` outputs: the first out*kSeg threads, o fastest; wider layers loop
-    float wreg[kMaxPerSeg];
+    // ---- every weight this thread will need, for all layers, is requested before anything else: the
+    // (o, seg) of a layer with `out` outputs is (tid % out, tid / out) for the first out*kSeg threads.
+    // Layers wider than 128 outputs do not fit one (o, seg) per thread and stream their weights instead.
+    const float *wl[3];
+    int l_in[3], l_out[3];
     {
-        const int out0 = (n_layers == 1) ? d_out : d_int;
-        fetch_weights(w, d_in, out0, tid % out0, tid / out0, tid < out0 * kSeg && out0 * kSeg <= kEncThreads, wreg);
+        const float *w = weights + head * per_head;
+        for (int l = 0; l < 3; ++l) {
+            l_in[l] = (l == 0) ? d_in : d_int;
+            l_out[l] = (l == n_layers - 1) ? d_out : d_int;
+            wl[l] = w;
+            if (l < n_layers) w += (int64_t)l_in[l] * l_out[l] + l_out[l];
+        }
+    }
+    float wreg[3][kMaxPerSeg];
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        const bool fits = l < n_layers && l_out[l] * kSeg <= kEncThreads && l_in[l] / kSeg <= kMaxPerSeg;
+        const bool active = fits && tid < l_out[l] * kSeg;
+        const int out = l < n_layers ? l_out[l] : 1, per = l < n_layers ? l_in[l] / kSeg : 0;
+        const int o = tid % out, seg = tid / out;
+#pragma unroll
+        for (int i = 0; i < kMaxPerSeg; ++i) wreg[l][i] = (active && i < per) ? wl[l][(int64_t)(seg * per + i) * out + o] : 0.f;
     }
 
     for (int i = tid; i < kRows * d_in; i += kEncThreads) {
@@ -94,13 +111,13 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
     __syncthreads();
 
     int cur = 0;
-    for (int l = 0; l < n_layers; ++l) {
-        const int in = (l == 0) ? d_in : d_int;
-        const int out = (l == n_layers - 1) ? d_out : d_int;
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        if (l >= n_layers) break;
+        const int in = l_in[l], out = l_out[l];
         const int per = in / kSeg;
-        const float *Wt = w, *bias = w + (int64_t)in * out;
-        w += (int64_t)in * out + out;
-        const bool fits = out * kSeg <= kEncThreads;  // one (o, seg) per thread: weights were prefetched
+        const float *Wt = wl[l], *bias = wl[l] + (int64_t)in * out;
+        const bool fits = out * kSeg <= kEncThreads && per <= kMaxPerSeg;
 
         if (fits) {
             if (tid < out * kSeg) {
@@ -108,17 +125,33 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
                 float p[kRows];
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) p[r] = 0.f;
+                if ((per & 3) == 0) {  // 128-bit LDS reads of four consecutive inputs
 #pragma unroll
-                for (int i = 0; i < kMaxPerSeg; ++i) {
-                    if (i < per) {
+                    for (int i = 0; i < kMaxPerSeg; i += 4) {
+                        if (i < per) {
 #pragma unroll
-                        for (int r = 0; r < kRows; ++r) p[r] = fmaf(s_act[cur][r][seg * per + i], wreg[i], p[r]);
+                            for (int r = 0; r < kRows; ++r) {
+                                const float4 xv = *reinterpret_cast<const float4 *>(&s_act[cur][r][seg * per + i]);
+                                p[r] = fmaf(xv.x, wreg[l][i], p[r]);
+                                p[r] = fmaf(xv.y, wreg[l][i + 1], p[r]);
+                                p[r] = fmaf(xv.z, wreg[l][i + 2], p[r]);
+                                p[r] = fmaf(xv.w, wreg[l][i + 3], p[r]);
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kMaxPerSeg; ++i) {
+                        if (i < per) {
+#pragma unroll
+                            for (int r = 0; r < kRows; ++r) p[r] = fmaf(s_act[cur][r][seg * per + i], wreg[l][i], p[r]);
+                        }
                     }
                 }
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) s_part[seg][r][o] = p[r];
             }
-        } else {  // layers wider than 128 outputs: plain loop, no prefetch
+        } else {
             for (int t2 = tid; t2 < out * kSeg; t2 += kEncThreads) {
                 const int o = t2 % out, seg = t2 / out;
                 float p[kRows];
@@ -132,11 +165,6 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) s_part[seg][r][o] = p[r];
             }
-        }
-        // next layer's weights: issue the loads before the barrier so their latency overlaps the reduction
-        if (l + 1 < n_layers) {
-            const int nout = (l + 1 == n_layers - 1) ? d_out : d_int;
-            fetch_weights(w, d_int, nout, tid % nout, tid / nout, tid < nout * kSeg && nout * kSeg <= kEncThreads, wreg);
         }
         __syncthreads();
         for (int t2 = tid; t2 < out * kRows; t2 += kEncThreads) {
@@ -188,6 +216,25 @@ int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const
     return HA_OK;
 }
 
+int launch_encode(const EncArgs &a, dim3 grid, hipStream_t s) {
+#define HA_ENC_CASE(NL_, DOUT_)                                                                                  \
+    if (a.n_layers == NL_ && a.d_in == 128 && (NL_ == 1 || a.d_int == 128) && a.d_out == DOUT_) {               \
+        hipLaunchKernelGGL((encode_pack_kernel<NL_, 128, 128, DOUT_>), grid, dim3(kEncThreads), 0, s, a);       \
+        HA_CHECK_LAUNCH("encode_pack_kernel");                                                                  \
+        return HA_OK;                                                                                           \
+    }
+    HA_ENC_CASE(3, 32)
+    HA_ENC_CASE(3, 64)
+    HA_ENC_CASE(2, 32)
+    HA_ENC_CASE(2, 64)
+    HA_ENC_CASE(1, 32)
+    HA_ENC_CASE(1, 64)
+#undef HA_ENC_CASE
+    hipLaunchKernelGGL((encode_pack_kernel<0, 0, 0, 0>), grid, dim3(kEncThreads), 0, s, a);
+    HA_CHECK_LAUNCH("encode_pack_kernel");
+    return HA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -221,9 +268,7 @@ int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_str
     a.B = B; a.T = T; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
     const unsigned tiles = (unsigned)(((int64_t)B * T + kRows - 1) / kRows);
-    hipLaunchKernelGGL(encode_pack_kernel, dim3(tiles, n_heads), dim3(kEncThreads), 0, (hipStream_t)stream, a);
-    HA_CHECK_LAUNCH("encode_pack_kernel");
-    return HA_OK;
+    return launch_encode(a, dim3(tiles, n_heads), (hipStream_t)stream);
 }
 
 int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_t, const void *q, int64_t q_stride_b,
@@ -248,9 +293,7 @@ int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, in
     a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
     const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);
-    hipLaunchKernelGGL(encode_pack_kernel, dim3(tiles, Hc + H), dim3(kEncThreads), 0, (hipStream_t)stream, a);
-    HA_CHECK_LAUNCH("encode_pack_kernel");
-    return HA_OK;
+    return launch_encode(a, dim3(tiles, Hc + H), (hipStream_t)stream);
 }
 
 }  // extern "C"

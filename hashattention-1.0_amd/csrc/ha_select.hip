@@ -172,13 +172,14 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
 #pragma unroll
         for (int g = 0; g < GQ; ++g) q[g] = load_qcode<W>(qcodes, (int64_t)b * H + hc * GQ + g);
         const int rep = tid % REP;
+        const bool whole = beg == c * chunk && end == (c + 1) * chunk;  // uniform: every code of the chunk is a candidate
 #pragma unroll
         for (int blk = 0; blk < kMaxBlocks; ++blk) {
             if (blk >= blocks) break;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int j = cr.j0[blk] + e;
-                if (j >= beg && j < end) {
+                if (whole || (j >= beg && j < end)) {
 #pragma unroll
                     for (int g = 0; g < GQ; ++g) atomicAdd(&lh[(g * NL + cr.k[blk][e].dist(q[g])) * REP + rep], 1u);
                 }
@@ -388,13 +389,17 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
     uint32_t ltm[GQ], eqm[GQ], incl[GQ];
 #pragma unroll
     for (int g = 0; g < GQ; ++g) {
-        uint32_t lt = 0, eq = 0;
+        // sign bit of (d - T) is "d < T", of (d - T - 1) is "d <= T"; v_alignbit shifts each into its mask.
+        // Elements are visited from the last to the first so that element e lands on bit e.
+        uint32_t lt = 0, le = 0;
+        const int neg_t = -T[g];
 #pragma unroll
-        for (int e = 0; e < CPL; ++e) {
-            const int d = k[e].dist(q[g]);
-            lt |= (d < T[g] ? 1u : 0u) << e;
-            eq |= (d == T[g] ? 1u : 0u) << e;
+        for (int e = CPL - 1; e >= 0; --e) {
+            const int key = k[e].dist(q[g]) + neg_t;
+            lt = __builtin_amdgcn_alignbit(lt, (uint32_t)key, 31);
+            le = __builtin_amdgcn_alignbit(le, (uint32_t)(key - 1), 31);
         }
+        const uint32_t eq = le & ~lt;
         ltm[g] = lt & vmask;
         eqm[g] = eq & vmask;
         incl[g] = wave_inclusive_scan((uint32_t)__popc(ltm[g]) | ((uint32_t)__popc(eqm[g]) << 16));

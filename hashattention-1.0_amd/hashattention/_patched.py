@@ -1,0 +1,309 @@
+"""Model-side half of the drop-in: the hash module `USA` and the logic shared by the patched Llama and
+Mistral attention layers.  Mirrors the reference's module API
+(hashattention/hashattention_llama.py:87-226 `USA`, :229-631 `LlamaAttention_heavy_hitter`, :633-725 helpers)
+with the decode branch running on the HIP kernels through `decode.HashDecodeLayer`.
+
+What differs from the reference on purpose
+  * the decode branch never builds dense [b, H, q, S] score/mask tensors and never re-hashes cached keys:
+    key codes live in a per-layer bit-cache that is extended as the KV cache grows (the reference keeps
+    `past_key_signatures = None`, hashattention_llama.py:407-408);
+  * ties at the top-k boundary go to the lowest token index (the reference's `sort` at :430 is unstable);
+  * softmax and the value product are fp32 throughout (the reference rounds probabilities to the query
+    dtype at :613);
+  * soft mode (`hard=False`: tanh / sigmoid, :174-176, 197-198), `CENTER` normalisation (:163-167), the LSH
+    baseline (`lth_num_layers == 0`, :130-139) and the training / statistics hooks (:304-398) are outside
+    the accelerated path and raise NotImplementedError instead of silently running something else.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Tuple
+
+import torch
+from torch import nn
+
+from . import _ops
+from .decode import HashDecodeLayer
+
+DECODE_MAX_Q_LEN = 128   # reference: `if q_len > 128 or self.train_usa` routes to the original forward (:529)
+
+
+class USA(nn.Module):
+    """Per-head learned hash: `num_heads` independent MLPs for keys and for queries.
+
+    Same constructor, parameter names and state-dict keys as the reference
+    ("learning_to_hash_transformation_{k,q}.{head}.{0,2,4}.{weight,bias}", hashattention_llama.py:99-128),
+    so reference checkpoints load unchanged.
+    """
+
+    def __init__(self, num_heads: int, head_dim: int, usa_params: dict):
+        super().__init__()
+        self.head_dim = head_dim
+        self.num_heads = num_heads
+        self.int_dim = usa_params["lth_int_dim"]
+        self.lth_final_dim = usa_params["lth_final_dim"]
+        self.lth_thold = usa_params["lth_thold"]
+        self.num_layers = usa_params.get("lth_num_layers", 3)   # the Mistral variant has no such key (mistral:566-570)
+        if self.num_layers not in (1, 2, 3):
+            raise NotImplementedError("lth_num_layers must be 1, 2 or 3 (the LSH baseline, 0, is not part of this build)")
+        if self.lth_final_dim not in (32, 64):
+            raise NotImplementedError("lth_final_dim must be 32 or 64: codes are packed in one or two 32-bit words")
+
+        def mlp():
+            if self.num_layers == 3:
+                return nn.Sequential(nn.Linear(head_dim, self.int_dim), nn.SiLU(), nn.Linear(self.int_dim, self.int_dim),
+                                     nn.SiLU(), nn.Linear(self.int_dim, self.lth_final_dim))
+            if self.num_layers == 2:
+                return nn.Sequential(nn.Linear(head_dim, self.int_dim), nn.SiLU(), nn.Linear(self.int_dim, self.lth_final_dim))
+            return nn.Sequential(nn.Linear(head_dim, self.lth_final_dim))
+
+        self.learning_to_hash_transformation_k = nn.ModuleList([mlp() for _ in range(num_heads)])
+        self.learning_to_hash_transformation_q = nn.ModuleList([mlp() for _ in range(num_heads)])
+
+    # -- weights in the form the kernels take
+    def layers(self, side: str) -> List[List[Tuple[torch.Tensor, torch.Tensor]]]:
+        mods = self.learning_to_hash_transformation_k if side == "k" else self.learning_to_hash_transformation_q
+        return [[(m.weight, m.bias) for m in seq if isinstance(m, nn.Linear)] for seq in mods]
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.learning_to_hash_transformation_k[0][-1].weight.dtype
+
+    @property
+    def arith(self) -> int:
+        """A module kept in bf16 computes with bf16 roundings after every layer; anything else in fp32."""
+        return _ops.HA_ARITH_BF16 if self.dtype == torch.bfloat16 else _ops.HA_ARITH_F32
+
+    def _embed(self, vectors: torch.Tensor, side: str, hard: bool) -> torch.Tensor:
+        if not hard:
+            raise NotImplementedError("soft (tanh) embeddings are a training feature outside this build")
+        b, a, s, d = vectors.shape
+        if a != self.num_heads:
+            raise ValueError(f"expected {self.num_heads} heads, got {a}")
+        w = _ops.pack_usa_weights(self.layers(side), vectors.device)
+        codes = torch.empty(b, a, s, self.lth_final_dim // 32, dtype=torch.int32, device=vectors.device)
+        logits = _ops.encode_pack(vectors, w, self.num_layers, self.int_dim, self.lth_final_dim, codes,
+                                  arith=self.arith, want_logits=True)
+        return torch.sign(logits), codes
+
+    def k_embedding(self, vectors: torch.Tensor, hard: bool = False) -> torch.Tensor:
+        """[b, heads, s, d] -> sign embeddings [b, heads, s, D] in fp32 (reference :204-214)."""
+        return self._embed(vectors, "k", hard)[0]
+
+    def q_embedding(self, vectors: torch.Tensor, hard: bool = False) -> torch.Tensor:
+        return self._embed(vectors, "q", hard)[0]
+
+    def forward(self, K: torch.Tensor, Q: torch.Tensor, hard: bool = False):
+        """span[b, h, t, s] = <sign q_t, sign k_s> = D - 2 * Hamming, non-causal entries at finfo.min; returns
+        (span, sign(K embeddings)) as the reference (:151-200).  Diagnostic API: the decode path does not call it."""
+        ksign, kcodes = self._embed(K, "k", hard)
+        _, qcodes = self._embed(Q, "q", hard)
+        b, a, s, _ = K.shape
+        t = Q.shape[2]
+        D = self.lth_final_dim
+        span = torch.empty(b, a, t, s, dtype=K.dtype, device=K.device)
+        for i in range(t):
+            ham = _ops.hamming_score(kcodes, qcodes[:, :, i].contiguous(), s)
+            span[:, :, i] = (D - 2 * ham.to(torch.int32)).to(K.dtype)
+        causal = torch.tril(torch.ones(t, s, device=K.device), diagonal=s - t).bool()
+        span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
+        return span, ksign.to(K.dtype)
+
+
+class HeavyHitterMixin:
+    """State and decode branch shared by `LlamaAttention_heavy_hitter` and `MistralAttention_heavy_hitter`.
+
+    The host class provides q_proj/k_proj/v_proj/o_proj, `config`, `layer_idx`, `head_dim` and the rotary
+    helper `_apply_rope(q, k, cos, sin)`.
+    """
+
+    def _init_heavy_hitter(self, config):
+        self.num_heads = config.num_attention_heads
+        self.num_key_value_heads = config.num_key_value_heads
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.hidden_size = config.hidden_size
+        self.init_budget = config.init_budget
+        self.heavy_budget = config.heavy_budget
+        self.recent_budget = config.recent_budget
+        self.usa_retrieve_depth = getattr(config, "usa_retrieve_depth", 0)
+        self.usa_eval_mode = getattr(config, "usa_eval_mode", "simple")
+        self.usa_module = None
+        self.usa_module_dtype = None
+        self.past_key_signatures = None      # kept for API parity; the bit-cache lives in self._hash_layer
+        self.use_softmax_maxtrick = False
+        self.collect_stats = False
+        self.train_usa = False
+        self.tr_loss_func = None
+        self.tr_optimizer = None
+        self.overlaps = {}
+        self.flash_forward = None
+        self._hash_layer: Optional[HashDecodeLayer] = None
+
+    def __repr__(self):
+        return (f"{super().__repr__()}\nSparsification Setting(topk:{self.heavy_budget}  edge:{self.init_budget, self.recent_budget} "
+                f"\n eval_mode:{self.usa_eval_mode} stats:{self.collect_stats}\n Istraining:{self.train_usa} )")
+
+    def _reset_state(self):
+        """A new example starts (reference :298-301): drop the cached codes."""
+        self.past_key_signatures = None
+        if self._hash_layer is not None:
+            self._hash_layer.reset()
+
+    # ---- bit-cache plumbing
+    def _ensure_hash_layer(self, batch: int, seq_len: int, device) -> HashDecodeLayer:
+        if self.usa_module is None:
+            raise RuntimeError("convert_usa() must attach a USA module before the decode branch runs")
+        hl = self._hash_layer
+        if hl is None:
+            usa = self.usa_module
+            hl = HashDecodeLayer(usa.layers("k"), usa.layers("q"), self.num_heads, self.num_key_value_heads, self.head_dim,
+                                 usa.num_layers, usa.int_dim, usa.lth_final_dim, self.init_budget, self.recent_budget,
+                                 self.heavy_budget, self.usa_eval_mode, self.usa_retrieve_depth, usa.arith, device)
+            self._hash_layer = hl
+        if hl.B != batch or hl.S_cap < seq_len:
+            keep = hl.codes[:, :, :hl.n_cached].clone() if (hl.B == batch and hl.n_cached > 0) else None
+            n = hl.n_cached if keep is not None else 0
+            hl.allocate(batch, max(2 * hl.S_cap if hl.B == batch else 0, seq_len + 1024))
+            if keep is not None:
+                hl.codes[:, :, :n] = keep
+                hl.n_cached = n
+        return hl
+
+    def _sparse_attention(self, query_states, key_states, value_states):
+        """query [b, H, q, d] (q <= 128), key/value [b, Hkv, S, d] holding the whole cache including the new tokens.
+        Returns [b, H, q, d].  Row i attends as query at absolute position S - q + i (reference :423-428)."""
+        b, H, q_len, d = query_states.shape
+        S = key_states.shape[2]
+        hl = self._ensure_hash_layer(b, S, query_states.device)
+        if hl.n_cached > S - q_len:          # the cache was rewound (new prompt without reset_usa): start over
+            hl.reset()
+        if hl.n_cached < S - q_len:          # keys cached by a prefill (or by dense steps): encode them in bulk
+            lo = hl.n_cached
+            bulk = key_states[:, :, lo:S - q_len]
+            hl.encode_keys(bulk, pos0=lo, use_mfma=(hl.arith == _ops.HA_ARITH_BF16 and bulk.dtype == torch.bfloat16
+                                                    and hl.wk_bf16 is not None))
+            hl.n_cached = S - q_len
+        out = torch.empty(b, H, q_len, d, dtype=query_states.dtype, device=query_states.device)
+        # the reference takes the heavy budget from the full key length for every query row (:431-434)
+        heavy = hl.heavy_count(S)
+        saved = hl.heavy_budget
+        hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5    # > 1: an absolute count for the kernels
+        try:
+            for i in range(q_len):
+                s_i = S - q_len + i + 1
+                o_i = torch.empty(b, H, d, dtype=query_states.dtype, device=query_states.device)
+                hl.step(query_states[:, :, i:i + 1], key_states, value_states, s_i, o_i)
+                out[:, :, i] = o_i
+        finally:
+            hl.heavy_budget = saved
+        return out
+
+    def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
+        bsz, q_len, _ = hidden_states.shape
+        if q_len > DECODE_MAX_Q_LEN or self.train_usa:
+            if self.train_usa:
+                raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
+            # prefill: the original dense forward (reference :529-550); its keys are hashed lazily at the first decode step
+            return self.flash_forward(hidden_states=hidden_states, position_embeddings=position_embeddings,
+                                      attention_mask=attention_mask, past_key_values=cache, **kwargs)
+        hidden_shape = (bsz, q_len, -1, self.head_dim)
+        query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        if position_embeddings is None:
+            raise ValueError("position_embeddings (cos, sin) are required")
+        cos, sin = position_embeddings
+        query_states, key_states = self._apply_rope(query_states, key_states, cos, sin)
+        if cache is not None:
+            key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
+        if key_states.stride(-1) != 1 or value_states.stride() != key_states.stride():
+            key_states, value_states = key_states.contiguous(), value_states.contiguous()
+        attn = self._sparse_attention(query_states.contiguous(), key_states, value_states)
+        attn = attn.transpose(1, 2).reshape(bsz, q_len, -1).contiguous()
+        return self.o_proj(attn), None
+
+    # ---- reference API kept for callers; outside the accelerated path
+    def compute_mask_multi(self, key_states, query_states):
+        """Boolean keep-mask [b, H, q, S] (reference :401-446), materialised from the kernels' index lists.
+        key_states is the repeat_kv'd key tensor as in the reference; only its first KV copy per group is read."""
+        b, H, q_len, d = query_states.shape
+        S = key_states.shape[2]
+        kv = key_states[:, ::self.num_key_value_groups].contiguous() if key_states.shape[1] == H else key_states
+        hl = self._ensure_hash_layer(b, S, query_states.device)
+        hl.reset()
+        hl.encode_keys(kv, pos0=0)
+        hl.n_cached = S
+        # one spare column collects the unused tail of every index list
+        mask = torch.zeros(b, H, q_len, S + 1, dtype=torch.bool, device=query_states.device)
+        heavy = hl.heavy_count(S)
+        saved = hl.heavy_budget
+        hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5
+        try:
+            ar = torch.arange(hl.idx_cap, device=mask.device)
+            for i in range(q_len):
+                s_i = S - q_len + i + 1
+                hl.encode_query(query_states[:, :, i:i + 1].contiguous())
+                hl.select(s_i, None)
+                valid = ar[None, None, :] < hl.counts[:, :, None]
+                where = torch.where(valid, hl.idx.long(), torch.full_like(hl.idx, S, dtype=torch.long))
+                mask[:, :, i].scatter_(2, where, True)
+        finally:
+            hl.heavy_budget = saved
+        mask = mask[..., :S]
+        return mask
+
+    def compute_mask(self, key_states, query_states):
+        assert query_states.shape[-2] == 1
+        return self.compute_mask_multi(key_states, query_states)
+
+    def train_step(self, *a, **k):
+        raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
+
+    def usa_local_compute(self, *a, **k):
+        raise NotImplementedError("recall statistics / training targets are outside this build")
+
+
+# ------------------------------------------------------------------------------------------ module-patch helpers
+
+def build_usa_modules(config, path, default_num_layers=None) -> nn.ModuleList:
+    """Body of `load_usa` (reference :633-646): one USA per decoder layer, optionally loaded from a state dict."""
+    cfg = {"lth_int_dim": config.lth_init_dim, "lth_final_dim": config.lth_final_dim, "lth_thold": config.lth_thold,
+           "lth_num_layers": getattr(config, "lth_num_layers", default_num_layers or 3)}
+    head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+    mods = nn.ModuleList([USA(config.num_attention_heads, head_dim, cfg) for _ in range(config.num_hidden_layers)])
+    if path is not None:
+        # checkpoints are plain state dicts of tensors: load them without executing anything from the file
+        mods.load_state_dict(torch.load(path, map_location="cpu", weights_only=True))
+    if not torch.cuda.is_available():
+        raise RuntimeError("load_usa() returns the modules on the GPU (reference :646) and no GPU is visible; "
+                           "this build has no CPU path")
+    _ops.load_library()
+    return mods.cuda()
+
+
+def convert_modules(model, config, usa_modules, collect_stats, train_usa, original_cls, patched_cls):
+    """Body of `convert_usa` (reference :650-667): replace every `original_cls` by `patched_cls` in place."""
+    for name, module in reversed(model._modules.items()):
+        if len(list(module.children())) > 0:
+            model._modules[name] = convert_modules(module, config, usa_modules, collect_stats, train_usa,
+                                                   original_cls, patched_cls)
+        if isinstance(module, original_cls):
+            device = next(module.parameters()).device
+            new_module = patched_cls(config, module.layer_idx).bfloat16().to(device)
+            new_module.load_state_dict(module.state_dict())
+            new_module.usa_module = usa_modules[module.layer_idx]
+            new_module.usa_module_dtype = usa_modules[module.layer_idx].dtype
+            new_module.flash_forward = module.forward
+            new_module.collect_stats = collect_stats
+            new_module.train_usa = train_usa
+            model._modules[name] = new_module
+    return model
+
+
+def walk(model, patched_cls, fn):
+    for name, module in reversed(model._modules.items()):
+        if len(list(module.children())) > 0:
+            model._modules[name] = walk(module, patched_cls, fn)
+        if isinstance(module, patched_cls):
+            fn(module)
+    return model

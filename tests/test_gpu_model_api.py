@@ -1,0 +1,133 @@
+"""The drop-in boundary on a GPU: `load_usa` / `convert_usa` / `reset_usa` on tiny random-init Llama and Mistral
+models, prefill through the original forward and decode steps through the HIP path, against the same model on
+the CPU whose attention layers run the oracle's restatement of the reference decode branch
+(hashattention/hashattention_llama.py:551-631).  fp32 everywhere so the comparison is tight."""
+import copy
+import types
+
+import pytest
+import torch
+from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM, MistralConfig, MistralForCausalLM
+
+from hashattention import hashattention_llama as hl
+from hashattention import hashattention_mistral as hm
+from oracle import hashattn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+USA_CFG = dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
+               recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple")
+
+
+def _config(cls, **kw):
+    cfg = cls(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=128, vocab_size=512, max_position_embeddings=4096, **kw)
+    for k, v in USA_CFG.items():
+        setattr(cfg, k, v)
+    return cfg
+
+
+def _oracle_forward(layer, usa, cfg, apply_rope):
+    """CPU restatement of the reference's patched forward, bound to an unpatched attention layer."""
+    orig = layer.forward
+    k_heads = [[(m.weight.detach().float().cpu(), m.bias.detach().float().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
+               for seq in usa.learning_to_hash_transformation_k]
+    q_heads = [[(m.weight.detach().float().cpu(), m.bias.detach().float().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
+               for seq in usa.learning_to_hash_transformation_q]
+
+    def forward(self, hidden_states, position_embeddings=None, attention_mask=None, past_key_values=None, **kwargs):
+        b, q_len, _ = hidden_states.shape
+        if q_len > 128:
+            return orig(hidden_states=hidden_states, position_embeddings=position_embeddings, attention_mask=attention_mask,
+                        past_key_values=past_key_values, **kwargs)
+        shape = (b, q_len, -1, self.head_dim)
+        q = self.q_proj(hidden_states).view(shape).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(shape).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
+        cos, sin = position_embeddings
+        q, k = apply_rope(q, k, cos, sin)
+        k, v = past_key_values.update(k, v, self.layer_idx)
+        out, _ = orc.reference_decode_attention(q, k, v, k_heads, q_heads, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget)
+        return self.o_proj(out.transpose(1, 2).reshape(b, q_len, -1)), None
+
+    layer.forward = types.MethodType(forward, layer)
+
+
+def _run(model, ids, steps):
+    cache = DynamicCache()
+    outs = []
+    with torch.no_grad():
+        o = model(ids[:, :-sum(steps)], past_key_values=cache, use_cache=True)
+        outs.append(o.logits[:, -1].float().cpu())
+        pos = ids.shape[1] - sum(steps)
+        for n in steps:
+            o = model(ids[:, pos:pos + n], past_key_values=cache, use_cache=True)
+            outs.append(o.logits.float().cpu())
+            pos += n
+    return outs
+
+
+@pytest.mark.parametrize("family", ["llama", "mistral"])
+def test_patched_model_matches_reference_semantics(family):
+    print(f"\n[case] model api {family}", flush=True)
+    torch.manual_seed(0)
+    if family == "llama":
+        cfg, model_cls, api = _config(LlamaConfig), LlamaForCausalLM, hl
+    else:
+        cfg, model_cls, api = _config(MistralConfig, sliding_window=None), MistralForCausalLM, hm
+    model = model_cls(cfg).bfloat16().float()           # bf16-representable weights: convert_usa's bf16 cast is then lossless
+    ref = copy.deepcopy(model)
+
+    usa = api.load_usa(cfg, None)                        # random-init hash modules, on the GPU
+    assert next(usa.parameters()).is_cuda
+    model = api.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False)
+    patched = model.model.layers[0].self_attn
+    assert type(patched).__name__.endswith("_heavy_hitter") and patched.q_proj.weight.dtype == torch.bfloat16
+    model = model.float()                                # the reference converts to bf16; compare in fp32 instead
+
+    rope = __import__(f"transformers.models.{family}.modeling_{family}", fromlist=["apply_rotary_pos_emb"]).apply_rotary_pos_emb
+    for li, layer in enumerate(ref.model.layers):
+        _oracle_forward(layer.self_attn, usa[li], cfg, rope)
+
+    ids = torch.randint(0, cfg.vocab_size, (2, 200 + 1 + 1 + 5 + 1), generator=torch.Generator().manual_seed(1))
+    steps = [1, 1, 5, 1]                                 # single-token steps and one 5-token chunk (q_len <= 128 branch)
+    got = _run(model, ids.to(DEV), steps)
+    want = _run(ref, ids, steps)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        err = (g - w).abs().max().item()
+        assert err < 2e-3, err
+
+    # a new prompt after reset_usa starts from an empty bit-cache
+    api.reset_usa(model)
+    assert model.model.layers[0].self_attn._hash_layer.n_cached == 0
+    got2 = _run(model, ids.to(DEV), steps)
+    for g, g2 in zip(got, got2):
+        assert torch.equal(g, g2)
+
+
+def test_usa_forward_and_mask_api():
+    # USA.forward / k_embedding and compute_mask_multi keep the reference's shapes and meaning
+    print("\n[case] USA.forward / compute_mask_multi", flush=True)
+    torch.manual_seed(3)
+    cfg = _config(LlamaConfig)
+    usa = hl.load_usa(cfg, None)[0]
+    K = torch.randn(1, 2, 300, 128, device=DEV).repeat_interleave(2, dim=1)   # repeat_kv'd keys, as the reference passes them
+    Q = torch.randn(1, 4, 3, 128, device=DEV)
+    span, ksign = usa(K, Q, hard=True)
+    k_heads = [[(m.weight.detach().cpu(), m.bias.detach().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
+               for seq in usa.learning_to_hash_transformation_k]
+    q_heads = [[(m.weight.detach().cpu(), m.bias.detach().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
+               for seq in usa.learning_to_hash_transformation_q]
+    span_ref, ksign_ref = orc.usa_forward_hard(K.cpu(), Q.cpu(), k_heads, q_heads)
+    assert torch.equal(span.cpu(), span_ref) and torch.equal(ksign.cpu(), ksign_ref)
+    assert torch.equal(usa.k_embedding(K, hard=True).cpu(), ksign_ref)
+    with pytest.raises(NotImplementedError):
+        usa(K, Q, hard=False)
+
+    layer = hl.LlamaAttention_heavy_hitter(cfg, 0).to(DEV)
+    layer.usa_module = usa
+    mask = layer.compute_mask_multi(K, Q)
+    mask_ref = orc.compute_mask_multi(span_ref, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget)
+    assert torch.equal(mask.cpu(), mask_ref)

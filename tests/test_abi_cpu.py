@@ -1,0 +1,146 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports every function the header declares,
+sizes its workspaces sensibly and validates arguments before it touches HIP (so a bad call is refused with the
+same status on any machine).  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from hashattention import _ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hashattn.h")
+
+HA_ERR_NULL, HA_ERR_SHAPE, HA_ERR_DTYPE, HA_ERR_ALIGN, HA_ERR_WS, HA_ERR_NODEV = -1, -2, -3, -4, -5, -6
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _ops.load_library()
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ha_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = _declared_functions()
+    assert {"ha_version", "ha_encode_pack", "ha_encode_step", "ha_encode_pack_prefill", "ha_hamming_score", "ha_select",
+            "ha_sparse_decode", "ha_dense_decode", "ha_select_workspace_bytes", "ha_sparse_decode_workspace_bytes",
+            "ha_dense_decode_workspace_bytes", "ha_usa_packed_floats", "ha_status_string", "ha_last_error_string",
+            "ha_device_count"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.ha_version() == 100
+    assert lib.ha_status_string(0) == b"ok" and lib.ha_status_string(HA_ERR_WS) == b"workspace missing or too small"
+
+
+def test_packed_weight_sizes(lib):
+    assert lib.ha_usa_packed_floats(3, 128, 128, 32) == 128 * 128 + 128 + 128 * 128 + 128 + 128 * 32 + 32 == 37152
+    assert lib.ha_usa_packed_floats(2, 128, 128, 64) == 24768
+    assert lib.ha_usa_packed_floats(1, 128, 128, 32) == 128 * 32 + 32
+    assert lib.ha_usa_packed_floats(0, 128, 128, 32) == 0
+    W = torch.arange(6.0).reshape(2, 3)
+    blob = _ops.pack_usa_weights([[(W, torch.tensor([7.0, 8.0]))]])
+    assert blob.tolist() == [[0, 3, 1, 4, 2, 5, 7, 8]]          # W^T [in][out], then the bias
+    assert _ops.pack_usa_weights_bf16([[(W, torch.tensor([7.0, 8.0]))]]).float().tolist() == [[0, 1, 2, 3, 4, 5, 7, 8]]
+
+
+def test_workspace_sizes(lib):
+    assert lib.ha_select_workspace_bytes(0, 32, 8, 1, 100) == 0 and lib.ha_select_workspace_bytes(1, 32, 8, 3, 100) == 0
+    small = lib.ha_select_workspace_bytes(1, 32, 8, 1, 4096)
+    big = lib.ha_select_workspace_bytes(16, 32, 8, 1, 65536)
+    assert 0 < small < big < 64 << 20
+    assert lib.ha_select_workspace_bytes(16, 32, 8, 2, 65536) > big
+    assert 0 < lib.ha_sparse_decode_workspace_bytes(16, 32, 2304) < 64 << 20
+    assert 0 < lib.ha_dense_decode_workspace_bytes(16, 32, 65536) < 256 << 20
+
+
+def _buf(n=4096):
+    return (C.c_char * n)()
+
+
+def _aligned(buf, a=256):
+    addr = C.addressof(buf)
+    return C.c_void_p((addr + a - 1) // a * a)
+
+
+def test_arguments_are_validated_before_any_device_work(lib):
+    """Host buffers stand in for device pointers: every call below must be refused during validation."""
+    b = _buf(1 << 16)
+    p = _aligned(b)
+    odd = C.c_void_p(p.value + 2)
+    null = None
+    # select
+    args = dict(kcodes=p, sb=1024, sh=1024, q=p, B=1, H=4, Hc=2, W=1, S=1000, sl=null, init=4, rec=4, hb=C.c_double(0.25),
+                mode=0, depth=0, idx=p, cap=300, cnt=p, ws=p, wsb=1 << 16, st=null)
+
+    def select(**kw):
+        a = {**args, **kw}
+        return lib.ha_select(a["kcodes"], a["sb"], a["sh"], a["q"], a["B"], a["H"], a["Hc"], a["W"], a["S"], a["sl"], a["init"], a["rec"],
+                             a["hb"], a["mode"], a["depth"], a["idx"], a["cap"], a["cnt"], a["ws"], a["wsb"], a["st"])
+
+    assert select(kcodes=null) == HA_ERR_NULL and b"NULL" in lib.ha_last_error_string()
+    assert select(idx=null) == HA_ERR_NULL
+    assert select(W=3) == HA_ERR_SHAPE
+    assert select(Hc=3) == HA_ERR_SHAPE                        # H not a multiple of Hc
+    assert select(H=32, Hc=2) == HA_ERR_SHAPE                  # 16 query heads per code head
+    assert select(sh=999) == HA_ERR_SHAPE                      # row stride shorter than the sequence
+    assert select(init=-1) == HA_ERR_SHAPE and select(hb=C.c_double(-0.5)) == HA_ERR_SHAPE and select(mode=7) == HA_ERR_SHAPE
+    assert select(cap=0) == HA_ERR_SHAPE
+    assert select(kcodes=odd) == HA_ERR_ALIGN
+    assert select(ws=null) == HA_ERR_WS and select(wsb=16) == HA_ERR_WS
+    assert select(ws=C.c_void_p(p.value + 64)) == HA_ERR_ALIGN
+
+    # sparse / dense decode
+    def sparse(**kw):
+        a = dict(q=p, qsb=512, qsh=128, k=p, v=p, dt=_ops.HA_BF16, sb=128000, sh=128000, ss=128, B=1, H=4, Hkv=2, idx=p, cap=300,
+                 cnt=p, sc=C.c_float(0.088), out=p, ws=p, wsb=1 << 16, st=null)
+        a.update(kw)
+        return lib.ha_sparse_decode(a["q"], a["qsb"], a["qsh"], a["k"], a["v"], a["dt"], a["sb"], a["sh"], a["ss"], a["B"], a["H"], a["Hkv"],
+                                    a["idx"], a["cap"], a["cnt"], a["sc"], a["out"], a["ws"], a["wsb"], a["st"])
+
+    assert sparse(v=null) == HA_ERR_NULL and sparse(idx=null) == HA_ERR_NULL
+    assert sparse(dt=9) == HA_ERR_DTYPE
+    assert sparse(Hkv=3) == HA_ERR_SHAPE and sparse(ss=64) == HA_ERR_SHAPE
+    assert sparse(k=odd) == HA_ERR_ALIGN and sparse(ss=132) == HA_ERR_ALIGN     # rows would not stay 16-byte aligned
+    assert sparse(wsb=8) == HA_ERR_WS
+    assert lib.ha_dense_decode(p, 512, 128, p, p, _ops.HA_F32, 128000, 128000, 128, 1, 4, 2, 0, null, C.c_float(0.1), p, p, 1 << 16,
+                               null) == HA_ERR_SHAPE           # max_seq_len must be positive
+
+    # encoders
+    def enc(**kw):
+        a = dict(x=p, dt=_ops.HA_BF16, sb=1280, sh=1280, st_=128, B=1, xh=2, nh=4, T=10, w=p, nl=3, hd=128, idim=128, fd=32, ar=0,
+                 codes=p, csb=64, csh=16, pos0=0, pd=null, lg=null, st=null)
+        a.update(kw)
+        return lib.ha_encode_pack(a["x"], a["dt"], a["sb"], a["sh"], a["st_"], a["B"], a["xh"], a["nh"], a["T"], a["w"], a["nl"], a["hd"],
+                                  a["idim"], a["fd"], a["ar"], a["codes"], a["csb"], a["csh"], a["pos0"], a["pd"], a["lg"], a["st"])
+
+    assert enc(w=null) == HA_ERR_NULL
+    assert enc(fd=48) == HA_ERR_SHAPE and enc(nl=4) == HA_ERR_SHAPE and enc(nh=3) == HA_ERR_SHAPE and enc(hd=300) == HA_ERR_SHAPE
+    assert enc(dt=5) == HA_ERR_DTYPE and enc(ar=2) == HA_ERR_DTYPE
+    assert lib.ha_encode_pack_prefill(p, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 64, 32, p, 64, 16, 0, null, null) == HA_ERR_SHAPE
+    assert lib.ha_encode_pack_prefill(odd, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 128, 32, p, 64, 16, 0, null, null) == HA_ERR_ALIGN
+    assert lib.ha_hamming_score(p, 1024, 1024, p, 1, 4, 2, 1, 1000, null, null, null) == HA_ERR_NULL
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="this check is about a machine without a GPU")
+def test_no_device_is_a_status_not_a_crash(lib):
+    b = _buf(1 << 16)
+    p = _aligned(b)
+    assert lib.ha_device_count() == 0
+    st = lib.ha_hamming_score(p, 1024, 1024, p, 1, 4, 2, 1, 1000, None, p, None)
+    assert st == HA_ERR_NODEV and b"no HIP device" in lib.ha_last_error_string()
+    with pytest.raises(ValueError):                            # the Python layer refuses CPU tensors outright
+        _ops.hamming_score(torch.zeros(1, 1, 4, 1, dtype=torch.int32), torch.zeros(1, 1, 1, dtype=torch.int32), 4)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_ops, "_lib", None)
+    monkeypatch.setattr(_ops, "lib_path", lambda: str(tmp_path / "libhashattn.so"))
+    with pytest.raises(ImportError):
+        _ops.load_library()

@@ -1,0 +1,114 @@
+"""CPU checks of the committed fixtures: the configs[0] golden (made by tests/golden/make_golden.py) and the
+vectors recorded from the reference's own code (tests/golden/make_reference_vectors.py)."""
+import os
+
+import numpy as np
+import torch
+
+from hashattention.synthetic import make_problem, named_workload, sha256_of
+from oracle import c_oracle
+from oracle import hashattn_oracle as orc
+
+HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _bits(a):
+    return np.unpackbits(a.view(np.uint8))
+
+
+def test_config0_inputs_are_reproducible_and_golden_holds():
+    g = np.load(os.path.join(HERE, "config0.npz"))
+    w = named_workload("config0")
+    p = make_problem(w)
+    assert sha256_of(p.q) == str(g["sha_q"]) and sha256_of(p.k) == str(g["sha_k"]) and sha256_of(p.v) == str(g["sha_v"])
+    kcodes, qcodes = g["kcodes"], g["qcodes"]                       # [1,32,4096,1], [1,32,1,1] uint32
+    # integer stages from the stored codes are exact on every machine
+    idx, counts = c_oracle.select(kcodes, qcodes[:, :, 0], [4096], w.init_budget, w.recent_budget, w.heavy_budget, 1280)
+    assert (counts == 1280).all() and np.array_equal(counts[0], g["n_selected"])
+    mask = np.zeros((32, 4096), dtype=bool)
+    for h in range(32):
+        mask[h, idx[0, h]] = True
+    assert np.array_equal(np.packbits(mask, axis=-1), g["mask"])
+    # python formulation of the same selection
+    ham = orc.hamming(torch.from_numpy(qcodes[:, :, 0].astype(np.int64)), torch.from_numpy(kcodes.astype(np.int64)))
+    sel = orc.select_indices_np(ham[0].numpy(), 4096, w.init_budget, w.recent_budget, w.heavy_budget)
+    assert np.array_equal(sel, idx[0])
+    # attention over the golden index lists
+    out = c_oracle.sparse_attend(p.q[:, :, 0], p.k, p.v, idx, counts, 1.0 / np.sqrt(128))
+    assert np.abs(out[0] - g["out"]).max() < 2e-5
+    # codes recomputed on this machine may differ from the stored ones only where a logit is ~0
+    kl = orc.usa_logits(orc.repeat_kv(p.k, 4), p.usa.k)
+    mine = orc.pack_codes(kl).numpy().astype(np.uint32)
+    diff = mine ^ kcodes
+    nflip = int(_bits(diff).sum())
+    assert nflip <= int(g["near_zero_logits"][0])
+    if nflip:
+        bits = ((diff[..., None] >> np.arange(32, dtype=np.uint32)) & 1).astype(bool)[:, :, :, 0, :]
+        assert (np.abs(kl.numpy())[bits] < 1e-4).all()
+
+
+def _usa_heads(g):
+    keys = [str(k) for k in g["state_keys"]]
+    sd = {k: torch.from_numpy(g[f"w{i}"]) for i, k in enumerate(keys)}
+    heads = {"k": [], "q": []}
+    for side in ("k", "q"):
+        h = 0
+        while f"learning_to_hash_transformation_{side}.{h}.0.weight" in sd:
+            layers = []
+            for l in (0, 2, 4):
+                pre = f"learning_to_hash_transformation_{side}.{h}.{l}"
+                if pre + ".weight" in sd:
+                    layers.append((sd[pre + ".weight"], sd[pre + ".bias"]))
+            heads[side].append(layers)
+            h += 1
+    return heads
+
+
+def test_oracle_matches_vectors_recorded_from_the_reference():
+    """USA.forward(hard=True) and compute_mask_multi of the reference, as recorded from its own code."""
+    g = np.load(os.path.join(HERE, "reference_vectors.npz"))
+    heads = _usa_heads(g)
+    assert len(heads["k"]) == 4 and len(heads["k"][0]) == 3
+    K = torch.from_numpy(g["K"])
+    Krep = orc.repeat_kv(K, 2)
+    for name in ("q1", "q5"):
+        Q = torch.from_numpy(g[f"{name}_Q"])
+        span, ksign = orc.usa_forward_hard(Krep, Q, heads["k"], heads["q"])
+        ref_span = torch.from_numpy(g[f"{name}_span"])
+        assert torch.equal(span, ref_span)                     # integer-valued: exact
+        assert np.array_equal(ksign.numpy().astype(np.int8), g[f"{name}_ksign"])
+        # span = D - 2 * Hamming of the packed codes, wherever the reference's causal mask keeps it
+        kc = orc.pack_codes(orc.usa_logits(Krep, heads["k"]))
+        qc = orc.pack_codes(orc.usa_logits(Q, heads["q"]))
+        for t in range(Q.shape[2]):
+            ham = orc.hamming(qc[:, :, t], kc)
+            keep = ref_span[:, :, t] > -1e30
+            assert torch.equal((32 - 2 * ham).float()[keep], ref_span[:, :, t][keep])
+        for tag in "abcd":
+            init, recent, heavy, mode, depth = g[f"{name}_{tag}_params"]
+            S = K.shape[2]
+            ref_mask = torch.from_numpy(np.unpackbits(g[f"{name}_{tag}_mask"], axis=-1)[..., :S].astype(bool))
+            mine = orc.compute_mask_multi(ref_span, int(init), int(recent), float(heavy), "simple" if mode == 0 else "thold", depth)
+            # With fewer candidates than the heavy budget the reference's `indices[:heavy_budget]` runs into the
+            # masked entries of the sort (hashattention_llama.py:437-438): window positions, already kept, and for
+            # q_len > 1 positions after the query, which the additive causal mask (:598) keeps at zero weight.
+            # Only the causal part of the mask has an effect, so only it is compared.
+            q_len = Q.shape[2]
+            causal = torch.tril(torch.ones(q_len, S), diagonal=S - q_len).bool()
+            mine, ref_mask = mine & causal, ref_mask & causal
+            score = torch.where(ref_span > -1e30, ref_span, torch.full_like(ref_span, -1e4))
+            if mode == 0:
+                # the reference's sort is unstable: equal up to the choice among equal scores ...
+                assert orc.tie_invariant_equal(mine, ref_mask, score), (name, tag)
+            else:
+                assert torch.equal(mine, ref_mask), (name, tag)        # threshold mode keeps all ties: exact
+            # ... and the index-set formulation used by the kernels agrees with the canonical mask row by row
+            hb_abs = orc.heavy_count(S, float(heavy))
+            for b in range(K.shape[0]):
+                for t in range(q_len):
+                    s_t = S - q_len + t + 1
+                    ham_bt = ((32 - ref_span[b, :, t, :s_t]) / 2).round().long()
+                    sel = orc.select_indices(ham_bt, s_t, int(init), int(recent), 0.0 if hb_abs == 0 else hb_abs + 0.5,
+                                             "simple" if mode == 0 else "thold", int(depth))
+                    assert torch.equal(orc.mask_from_indices(sel, S)[:, :s_t], mine[b, :, t, :s_t]), (name, tag, b, t)
+                    assert not mine[b, :, t, s_t:].any()

@@ -1,0 +1,74 @@
+"""The benchmark configurations at their full sizes.  Codes are made on the GPU (MFMA encoder), copied back, and
+the CPU oracle recomputes selection and attention from those same codes: index lists bit for bit, outputs within
+2e-2 (bf16).  Size-independent properties on top: ascending lists, exact counts, windows present, and the
+selected tokens' distances never exceed those of any unselected candidate."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from hashattention import _ops
+from hashattention.decode import HashDecodeLayer
+from hashattention.synthetic import make_problem_on_device, named_workload
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("name", ["config1", "config2", "config4"])
+def test_full_size_configuration(name):
+    print(f"\n[case] full size {name}", flush=True)
+    w = named_workload(name)
+    p = make_problem_on_device(w, DEV)
+    B, H, Hkv, S, W = w.batch, w.n_q_heads, w.n_kv_heads, w.max_seq_len, w.code_words
+    layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, 128, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim, w.init_budget,
+                            w.recent_budget, w.heavy_budget, device=DEV)
+    layer.allocate(B, S)
+    layer.encode_keys(p.k, use_mfma=True)
+    ragged = len(set(w.seq_lens)) > 1
+    seq = p.seq_lens if ragged else None
+    out = torch.empty(B, H, 128, dtype=w.dtype, device=DEV)
+    if ragged:
+        layer.step(p.q, p.k, p.v, S, out, seq_lens=seq)
+    else:
+        layer.n_cached = S - 1
+        layer.step(p.q, p.k, p.v, S, out)
+    torch.cuda.synchronize()
+
+    kc = layer.codes.cpu().numpy()
+    qc = layer.qcodes.view(B, H, W).cpu().numpy()
+    seq_np = np.array(w.seq_lens, dtype=np.int32)
+    idx, cnt = layer.idx.cpu().numpy(), layer.counts.cpu().numpy()
+    ref_idx, ref_cnt = c_oracle.select(kc, qc, seq_np, w.init_budget, w.recent_budget, w.heavy_budget, layer.idx_cap)
+    assert np.array_equal(cnt, ref_cnt)
+    for b in range(B):
+        assert (cnt[b] == w.n_selected(w.seq_lens[b])).all()
+        n = cnt[b, 0]
+        assert np.array_equal(idx[b, :, :n], ref_idx[b, :, :n]), b
+        assert (np.diff(idx[b, :, :n], axis=1) > 0).all()
+        assert (idx[b, :, :w.init_budget] == np.arange(w.init_budget)).all()
+        assert (idx[b, :, n - w.recent_budget:n] == np.arange(w.seq_lens[b] - w.recent_budget, w.seq_lens[b])).all()
+    # distances of the selected candidates are all <= those of the unselected ones (one row per sequence)
+    ham = c_oracle.hamming(kc, qc, seq_np)
+    for b in range(B):
+        s, n = w.seq_lens[b], cnt[b, 5]
+        sel = np.zeros(s, dtype=bool)
+        sel[idx[b, 5, :n]] = True
+        cand = np.zeros(s, dtype=bool)
+        cand[w.init_budget:s - w.recent_budget] = True
+        assert ham[b, 5, :s][sel & cand].max() <= ham[b, 5, :s][~sel & cand].min()
+
+    ref = c_oracle.sparse_attend(p.q[:, :, 0].cpu(), p.k.cpu(), p.v.cpu(), ref_idx, ref_cnt, 1 / math.sqrt(128))
+    err = np.abs(out.float().cpu().numpy() - ref).max()
+    print(f"  n_selected {cnt.min()}..{cnt.max()}, sparse max-abs error {err:.2e}", flush=True)
+    assert err <= 2e-2
+    if name != "config2":       # dense baseline against the oracle too (config2: 4 GB of K/V through a scalar loop is slow)
+        outd = torch.empty_like(out)
+        ws = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), DEV)
+        _ops.dense_decode(p.q[:, :, 0], p.k, p.v, S, seq, 1 / math.sqrt(128), outd, ws)
+        refd = c_oracle.dense_attend(p.q[:, :, 0].cpu(), p.k.cpu(), p.v.cpu(), seq_np, 1 / math.sqrt(128))
+        errd = np.abs(outd.float().cpu().numpy() - refd).max()
+        print(f"  dense max-abs error {errd:.2e}", flush=True)
+        assert errd <= 2e-2

@@ -25,6 +25,10 @@ for p in (os.path.join(ROOT, "hashattention-1.0_amd"), ROOT):
 
 HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published peak
 
+# HBM bytes per launch of the gather-attend kernel, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
+# summarised in profiles/decode_step_config2_hbm_traffic.md, each scaled on a 1 GiB copy (fetch x2.0, write x1.0).
+MEASURED_ATTEND_TRAFFIC_BYTES = {"config2": 551.8e6}
+
 
 def algorithmic_bytes(w, n_sel_rows):
     """Algorithmic HBM bytes of one layer-step, per stage.  n_sel_rows = sum over (b, h) of selected tokens."""
@@ -52,22 +56,48 @@ def time_gpu(fn, steps, warmup, torch):
     return e0.elapsed_time(e1) / steps
 
 
-def cpu_baseline(w, torch):
+def cpu_baseline(w, torch, budget_s=12.0):
     """The oracle's restatement of the reference decode step (dense QK^T, every key re-hashed, full sort, masked
-    fp32 softmax) timed on the host for ONE sequence of the workload, scaled linearly to the batch."""
+    fp32 softmax) timed on the host, one sequence of the workload at a time until `budget_s` seconds are spent,
+    then scaled linearly to the batch."""
     from hashattention.synthetic import Workload, make_problem
     from oracle import hashattn_oracle as orc
-    w1 = Workload(**{**w.__dict__, "name": w.name + "-cpu", "batch": 1, "seq_lens": [w.seq_lens[0]]})
-    p = make_problem(w1)
-    q, k, v = p.q.float(), p.k.float(), p.v.float()
-    orc.reference_decode_attention(q[:, :, :, :], k[:, :, :4096], v[:, :, :4096], p.usa.k, p.usa.q, w.init_budget,
-                                   w.recent_budget, w.heavy_budget)     # warm-up on a prefix
-    t0 = time.perf_counter()
-    orc.reference_decode_attention(q, k, v, p.usa.k, p.usa.q, w.init_budget, w.recent_budget, w.heavy_budget)
-    dt = time.perf_counter() - t0
-    return {"value": dt * 1e6 * w.batch, "unit": "us/layer", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of {w.batch} sequences (S={w.seq_lens[0]}, fp32, torch CPU, {os.cpu_count()} logical cpus), "
-                      f"{dt:.2f} s measured, scaled x{w.batch}"}
+    times = []
+    t_start = time.perf_counter()
+    for b in range(w.batch):
+        w1 = Workload(**{**w.__dict__, "name": w.name + "-cpu", "batch": 1, "seq_lens": [w.seq_lens[b]], "seed": w.seed + b})
+        p = make_problem(w1)
+        q, k, v = p.q.float(), p.k.float(), p.v.float()
+        if b == 0:     # warm-up on a prefix (thread pools, allocator)
+            orc.reference_decode_attention(q, k[:, :, :4096], v[:, :, :4096], p.usa.k, p.usa.q, w.init_budget,
+                                           w.recent_budget, w.heavy_budget)
+        t0 = time.perf_counter()
+        orc.reference_decode_attention(q, k, v, p.usa.k, p.usa.q, w.init_budget, w.recent_budget, w.heavy_budget)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > budget_s:
+            break
+    per_seq = sum(times) / len(times)
+    tokens = sum(w.seq_lens[:len(times)]) / len(times)
+    scale = sum(w.seq_lens) / tokens          # linear in cached tokens (ragged batches)
+    return {"value": per_seq * 1e6 * scale, "unit": "us/layer", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(times)} of {w.batch} sequences (fp32, torch CPU, {os.cpu_count()} logical cpus, "
+                      f"{torch.get_num_threads()} torch threads), {sum(times):.2f} s measured, scaled x{scale:.2f} by cached tokens"}
+
+
+def traffic_probe(torch, layer, q3, k, v, out):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain copy of known size, then the gather-attend
+    kernel, three launches each.  The copy gives the scale of the counter (bytes per reported KiB)."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=q3.device).random_(0, 255)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        layer.attend(q3, k, v, out)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "copy 1 GiB x3 (vectorized_elementwise copy kernel), then sparse_attend x3"}))
 
 
 def main():
@@ -78,6 +108,7 @@ def main():
     ap.add_argument("--config", default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
+    ap.add_argument("--traffic-probe", action="store_true", help="run the launches the HBM-traffic counters are read from, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the sparse decode path shards by (sequence, KV head) with no exchange, "
@@ -123,6 +154,10 @@ def main():
         _ops.encode_step(p.k[:, :, S - 1:S], q3, layer.wk, layer.wq, layer.num_layers, layer.int_dim, layer.final_dim,
                          layer.codes, layer.qcodes, pos0=S - 1)
 
+    if args.traffic_probe:
+        step()
+        traffic_probe(torch, layer, q3, p.k, p.v, out)
+        return
     ms_step_eager = time_gpu(step, args.steps, args.warmup, torch)
     # the same launch sequence captured once in a HIP graph and replayed: the step as a serving loop runs it
     side = torch.cuda.Stream()
@@ -135,8 +170,9 @@ def main():
     with torch.cuda.graph(graph):
         step()
     ref_out = out.clone()
-    ms_step = time_gpu(graph.replay, args.steps, args.warmup, torch)
+    ms_step_graph = time_gpu(graph.replay, args.steps, args.warmup, torch)
     graph_ok = bool(torch.equal(out, ref_out))
+    ms_step = min(ms_step_graph, ms_step_eager)
     ms_encode = time_gpu(encode_only, args.steps, args.warmup, torch)
     ms_select = time_gpu(lambda: layer.select(S, seq_lens), args.steps, args.warmup, torch)
     ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
@@ -156,7 +192,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_step,
-        "step_launch": "hip graph replay of the 3 calls (eager launches from Python: %.1f us)" % (ms_step_eager * 1e3),
+        "step_launch": {"value_is": "graph" if ms_step_graph <= ms_step_eager else "eager",
+                        "hip_graph_replay_us": ms_step_graph * 1e3, "eager_launches_from_python_us": ms_step_eager * 1e3},
         "graph_replay_matches_eager": graph_ok,
         "higher_is_better": False,
         "scaling": "weak",
@@ -175,9 +212,10 @@ def main():
         "dense_hbm_gbps": ab["dense"] / (ms_dense * 1e-3) / 1e9,
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
-        "roofline": {"kernel": "sparse_attend_kernel (+ split merge)", "bound": "hbm",
+        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm",
                      "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get(w.name),
                      "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
     }
     if not args.no_cpu_baseline:

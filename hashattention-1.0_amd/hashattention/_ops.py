@@ -18,6 +18,7 @@ _lib = None
 HA_F32, HA_BF16, HA_F16 = 0, 1, 2
 HA_ARITH_F32, HA_ARITH_BF16 = 0, 1
 HA_SELECT_SIMPLE, HA_SELECT_THRESHOLD = 0, 1
+HA_SELECT_ALGO_AUTO, HA_SELECT_ALGO_HISTOGRAM, HA_SELECT_ALGO_SAMPLED, HA_SELECT_ALGO_SAMPLED_EXACT_ROWS = 0, 1, 2, 3
 
 _DTYPE = {torch.float32: HA_F32, torch.bfloat16: HA_BF16, torch.float16: HA_F16}
 
@@ -64,7 +65,7 @@ def load_library() -> C.CDLL:
     lib.ha_select_workspace_bytes.restype = sz
     lib.ha_select_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.ha_select.restype = i32
-    lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32,
+    lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, i32,
                               vp, i64, vp, vp, sz, vp]
     lib.ha_sparse_decode_workspace_bytes.restype = sz
     lib.ha_sparse_decode_workspace_bytes.argtypes = [i32, i32, i64]
@@ -209,7 +210,7 @@ def select_workspace_bytes(B, H, Hc, W, max_seq_len) -> int:
 
 def select(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
            init_budget: int, recent_budget: int, heavy_budget: float, out_idx: torch.Tensor, out_counts: torch.Tensor,
-           ws: torch.Tensor, mode: int = HA_SELECT_SIMPLE, depth: int = 0) -> None:
+           ws: torch.Tensor, mode: int = HA_SELECT_SIMPLE, depth: int = 0, algo: int = HA_SELECT_ALGO_AUTO) -> None:
     """Ascending index lists out_idx [B, H, idx_cap] int32 and out_counts [B, H] int32 (both written in place)."""
     _require_cuda(kcodes, qcodes, seq_lens, out_idx, out_counts, ws)
     lib = load_library()
@@ -219,7 +220,7 @@ def select(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_len
     assert out_idx.is_contiguous() and out_idx.dtype == torch.int32 and out_counts.is_contiguous() and out_counts.dtype == torch.int32
     assert seq_lens is None or (seq_lens.dtype == torch.int32 and seq_lens.is_contiguous())
     _check(lib.ha_select(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
-                         _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth,
+                         _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth, algo,
                          _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select")
 
 

@@ -50,6 +50,12 @@ typedef enum ha_status {
 #define HA_SELECT_SIMPLE 0    /* usa_eval_mode == 'simple': exactly k_eff heavy tokens */
 #define HA_SELECT_THRESHOLD 1 /* otherwise: every candidate within the distance threshold, ties included */
 
+/* How ha_select finds the threshold; every choice returns the same lists. */
+#define HA_SELECT_ALGO_AUTO 0              /* sampled when few tokens are kept of long rows, else histogram */
+#define HA_SELECT_ALGO_HISTOGRAM 1         /* two passes over the codes: exact histogram, then compaction */
+#define HA_SELECT_ALGO_SAMPLED 2           /* sampled upper bound of the threshold, one filtering pass, exact finish */
+#define HA_SELECT_ALGO_SAMPLED_EXACT_ROWS 3 /* diagnostic: as SAMPLED with every row sent through its in-kernel exact path */
+
 int ha_version(void);
 const char *ha_status_string(int status);
 const char *ha_last_error_string(void);
@@ -141,7 +147,7 @@ int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
 size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len);
 int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
               int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
-              int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
+              int init_budget, int recent_budget, double heavy_budget, int mode, int depth, int algo,
               int32_t *out_idx, int64_t idx_cap, int32_t *out_counts,
               void *workspace, size_t workspace_bytes, void *stream);
 

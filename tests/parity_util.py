@@ -54,7 +54,8 @@ def compare_codes(name, got_u32: np.ndarray, want_u32: np.ndarray, logits: np.nd
 
 
 def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple", depth: int = 0,
-                    idx_cap: Optional[int] = None, check_dense: bool = True, verbose: bool = False, dev="cuda:0"):
+                    idx_cap: Optional[int] = None, check_dense: bool = True, verbose: bool = False, dev="cuda:0",
+                    algo: int = _ops.HA_SELECT_ALGO_AUTO):
     """encode -> hamming -> select -> sparse attend (+ dense) on the GPU, each stage against the oracle."""
     p = make_problem(w)
     B, H, Hkv, Hc, d, S, W = w.batch, w.n_q_heads, w.n_kv_heads, w.n_code_heads, w.head_dim, w.max_seq_len, w.code_words
@@ -100,7 +101,8 @@ def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple"
     counts = torch.zeros(B, H, dtype=torch.int32, device=dev)
     ws = _ops.workspace(_ops.select_workspace_bytes(B, H, Hc, W, S), dev)
     m = _ops.HA_SELECT_SIMPLE if mode == "simple" else _ops.HA_SELECT_THRESHOLD
-    _ops.select(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, idx, counts, ws, mode=m, depth=depth)
+    _ops.select(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, idx, counts, ws, mode=m, depth=depth,
+                algo=algo)
     idx_ref, counts_ref = c_oracle.select(kc_np, qc_np, seq_np, w.init_budget, w.recent_budget, w.heavy_budget, cap,
                                           mode=0 if mode == "simple" else 1, depth=depth)
     idx_np, counts_np = idx.cpu().numpy(), counts.cpu().numpy()

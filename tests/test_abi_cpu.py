@@ -54,8 +54,8 @@ def test_workspace_sizes(lib):
     assert lib.ha_select_workspace_bytes(0, 32, 8, 1, 100) == 0 and lib.ha_select_workspace_bytes(1, 32, 8, 3, 100) == 0
     small = lib.ha_select_workspace_bytes(1, 32, 8, 1, 4096)
     big = lib.ha_select_workspace_bytes(16, 32, 8, 1, 65536)
-    assert 0 < small < big < 64 << 20
-    assert lib.ha_select_workspace_bytes(16, 32, 8, 2, 65536) > big
+    assert 0 < small < big < 128 << 20
+    assert lib.ha_select_workspace_bytes(16, 32, 8, 2, 65536) >= big
     assert 0 < lib.ha_sparse_decode_workspace_bytes(16, 32, 2304) < 64 << 20
     assert 0 < lib.ha_dense_decode_workspace_bytes(16, 32, 65536) < 256 << 20
 
@@ -77,12 +77,12 @@ def test_arguments_are_validated_before_any_device_work(lib):
     null = None
     # select
     args = dict(kcodes=p, sb=1024, sh=1024, q=p, B=1, H=4, Hc=2, W=1, S=1000, sl=null, init=4, rec=4, hb=C.c_double(0.25),
-                mode=0, depth=0, idx=p, cap=300, cnt=p, ws=p, wsb=1 << 16, st=null)
+                mode=0, depth=0, algo=0, idx=p, cap=300, cnt=p, ws=p, wsb=1 << 16, st=null)
 
     def select(**kw):
         a = {**args, **kw}
         return lib.ha_select(a["kcodes"], a["sb"], a["sh"], a["q"], a["B"], a["H"], a["Hc"], a["W"], a["S"], a["sl"], a["init"], a["rec"],
-                             a["hb"], a["mode"], a["depth"], a["idx"], a["cap"], a["cnt"], a["ws"], a["wsb"], a["st"])
+                             a["hb"], a["mode"], a["depth"], a["algo"], a["idx"], a["cap"], a["cnt"], a["ws"], a["wsb"], a["st"])
 
     assert select(kcodes=null) == HA_ERR_NULL and b"NULL" in lib.ha_last_error_string()
     assert select(idx=null) == HA_ERR_NULL
@@ -91,7 +91,7 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert select(H=32, Hc=2) == HA_ERR_SHAPE                  # 16 query heads per code head
     assert select(sh=999) == HA_ERR_SHAPE                      # row stride shorter than the sequence
     assert select(init=-1) == HA_ERR_SHAPE and select(hb=C.c_double(-0.5)) == HA_ERR_SHAPE and select(mode=7) == HA_ERR_SHAPE
-    assert select(cap=0) == HA_ERR_SHAPE
+    assert select(cap=0) == HA_ERR_SHAPE and select(algo=9) == HA_ERR_SHAPE
     assert select(kcodes=odd) == HA_ERR_ALIGN
     assert select(ws=null) == HA_ERR_WS and select(wsb=16) == HA_ERR_WS
     assert select(ws=C.c_void_p(p.value + 64)) == HA_ERR_ALIGN

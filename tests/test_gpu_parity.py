@@ -110,3 +110,30 @@ def test_config0_shape_fp32():
     from hashattention.synthetic import named_workload
     r = run_decode_case(named_workload("config0"), verbose=True)
     assert r["n_selected"] == 1280
+
+
+ALGOS = {"histogram": 1, "sampled": 2, "sampled_exact_rows": 3}
+
+
+@pytest.mark.parametrize("algo", list(ALGOS))
+@pytest.mark.parametrize("case", ["plain", "ragged64", "threshold", "short", "big_budget", "gq1", "long"])
+def test_every_select_algorithm_gives_the_same_lists(algo, case):
+    # the three ways of finding the threshold (exact histogram, sampled guess, the guess's in-kernel exact path)
+    # against the same oracle; "long" makes the sample a true subsample (more than 4096 candidates per row)
+    _announce(f"select algo {algo} / {case}")
+    kw = dict(check_encode=False, check_dense=False, algo=ALGOS[algo], verbose=True)
+    if case == "plain":
+        run_decode_case(small_workload(seed=201), **kw)
+    elif case == "ragged64":
+        run_decode_case(small_workload(batch=3, seq_lens=[2300, 700, 1025], lth_num_layers=2, lth_final_dim=64, seed=202), **kw)
+    elif case == "threshold":
+        run_decode_case(small_workload(seed=203), mode="threshold", depth=1, **kw)
+    elif case == "short":
+        run_decode_case(small_workload(batch=4, seq_lens=[1, 31, 33, 40], seed=204), **kw)
+    elif case == "big_budget":      # more than half of the candidates kept: candidate segments overflow, rows go exact
+        run_decode_case(small_workload(heavy_budget=0.7, seed=205), **kw)
+    elif case == "gq1":
+        run_decode_case(small_workload(n_code_heads=8, seed=206), **kw)
+    else:
+        run_decode_case(small_workload(batch=2, seq_lens=[20000, 9000], n_q_heads=4, n_kv_heads=1, n_code_heads=1,
+                                       heavy_budget=1 / 32, seed=207), **kw)

@@ -9,7 +9,7 @@ constexpr int kSelThreads = 256;
 constexpr int kSelWaves = kSelThreads / HA_WAVE;
 constexpr int kBlock = 1024;      // codes per workgroup per block: 4 waves x 64 lanes x 4 codes
 constexpr int kMaxBlocks = 4;     // blocks per chunk held in registers
-constexpr int kMaxChunks = 1024;  // per row
+constexpr int kMaxChunks = 1024;  // per row: sequences up to 4 Mi tokens, so an index fits the low 24 bits of a candidate entry
 
 struct SelectPlan {
     int blocks;  // 1024-code blocks per chunk, 1..kMaxBlocks

@@ -14,6 +14,8 @@
 // Nothing rests on the guess being right: if a row's candidates do not contain k tokens, or a segment
 // overflows, select_finalize_kernel redoes that row exactly from the codes (slow, rare, same kernel: no
 // round trip to the host).
+#include <type_traits>
+
 #include "ha_select_common.h"
 
 using namespace ha_sel;
@@ -137,8 +139,10 @@ __global__ __launch_bounds__(kSelThreads) void select_sample_kernel(const uint32
 
 // ------------------------------------------------------------------------------------------------
 // grid (nchunk, Hc, B), 256 threads; chunk layout as select_compact_kernel (a lane owns 4*blocks consecutive codes).
-// cand[row][chunk][0..cap) = ascending indices of the chunk's candidates with d <= T_hi; cand_cnt = their number
-// (the true one, also when it exceeds cap).
+// cand[row][chunk][0..cap) = the chunk's candidates with d <= T_hi in ascending index order, each entry
+// (d << 24) | index (so the last kernel never has to gather codes again); cand_cnt = their number (the true
+// one, also when it exceeds cap).  The lane's codes are parked in LDS so that the few set bits can look
+// their code up by a run-time element number.
 template <int W, int GQ>
 __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
                                                                     const uint32_t *__restrict__ qcodes, int H, int max_S,
@@ -149,6 +153,7 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(const uint32
     constexpr int CPL = 4 * kMaxBlocks;
     constexpr int NP = (GQ + 1) / 2;  // packed scan words: two 16-bit counters each
     __shared__ uint32_t s_wtot[kSelWaves][NP];
+    __shared__ uint32_t s_codes[CPL * W * kSelThreads];  // [element][word][thread]: bank = thread % 32 for every access
 
     const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -175,28 +180,49 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(const uint32
     const int j_lane = c * chunk + (wave * HA_WAVE + lane) * cpl;
     const uint32_t *kc = kcodes + b * kc_sb + hc * kc_sh;
     Code<W> k[CPL];
-    uint32_t vmask = 0;
+    uint32_t vmask;  // bit e: code j_lane + e is a candidate of this chunk
+    if (vec && blocks == kMaxBlocks && beg == c * chunk && end == (c + 1) * chunk) {
+        // the common case, uniform over the workgroup: a full chunk strictly inside the candidate range
+        // of a 16-byte aligned row: four (eight) 128-bit loads and no per-element bounds
 #pragma unroll
-    for (int i = 0; i < kMaxBlocks; ++i) {
-        const int j0 = j_lane + 4 * i;
-        const bool live = i < blocks && j0 + 4 > beg && j0 < end;
-        Code<W> k4[4];
-        if (live) load_code4<W>(kc, j0, beg, end, vec != 0, k4);
+        for (int i = 0; i < kMaxBlocks; ++i) {
+            Code<W> k4[4];
+            load_code4<W>(kc, j_lane + 4 * i, beg, end, true, k4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (live) k[4 * i + e] = k4[e];
-            else if constexpr (W == 1) k[4 * i + e] = Code<1>{0u};
-            else k[4 * i + e] = Code<2>{0u, 0u};
-            if (live && j0 + e >= beg && j0 + e < end) vmask |= 1u << (4 * i + e);
+            for (int e = 0; e < 4; ++e) k[4 * i + e] = k4[e];
+        }
+        vmask = 0xFFFFu;
+    } else {
+        vmask = 0;
+#pragma unroll
+        for (int i = 0; i < kMaxBlocks; ++i) {
+            const int j0 = j_lane + 4 * i;
+            const bool live = i < blocks && j0 + 4 > beg && j0 < end;
+            Code<W> k4[4];
+            if (live) load_code4<W>(kc, j0, beg, end, vec != 0, k4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (live) k[4 * i + e] = k4[e];
+                else if constexpr (W == 1) k[4 * i + e] = Code<1>{0u};
+                else k[4 * i + e] = Code<2>{0u, 0u};
+                if (live && j0 + e >= beg && j0 + e < end) vmask |= 1u << (4 * i + e);
+            }
         }
     }
 
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) {
+        s_codes[(e * W) * kSelThreads + tid] = k[e].w0;
+        if constexpr (W == 2) s_codes[(e * W + 1) * kSelThreads + tid] = k[e].w1;
+    }
     uint32_t lem[GQ], packed[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) packed[p] = 0;
+    Code<W> qh[GQ];
 #pragma unroll
     for (int g = 0; g < GQ; ++g) {
-        const Code<W> q = load_qcode<W>(qcodes, (int64_t)b * H + hc * GQ + g);
+        qh[g] = load_qcode<W>(qcodes, (int64_t)b * H + hc * GQ + g);
+        const Code<W> q = qh[g];
         uint32_t le = 0;
         const int off = -t_hi[g] - 1;  // sign of d - T_hi - 1 is "d <= T_hi"; T_hi < 0 leaves it clear
 #pragma unroll
@@ -221,13 +247,17 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(const uint32
             total += t;
         }
         const int64_t row = (int64_t)b * H + hc * GQ + g;
-        int32_t *seg = cand + (row * nchunk + c) * cap;
+        int32_t *seg = cand + (row * nchunk + c) * cap;  // uniform base, 32-bit lane offsets
         uint32_t todo = lem[g];
+        uint32_t upos = (uint32_t)pos;
         while (todo) {
             const int e = __ffs((int)todo) - 1;
             todo &= todo - 1;
-            if (pos < cap) seg[pos] = j_lane + e;
-            ++pos;
+            Code<W> ce;
+            ce.w0 = s_codes[(e * W) * kSelThreads + tid];
+            if constexpr (W == 2) ce.w1 = s_codes[(e * W + 1) * kSelThreads + tid];
+            if (upos < (uint32_t)cap) seg[upos] = (ce.dist(qh[g]) << 24) | (j_lane + e);
+            ++upos;
         }
         if (tid == 0) cand_cnt[row * nchunk + c] = total;
     }
@@ -270,7 +300,10 @@ __global__ __launch_bounds__(kFinThreads) void select_finalize_kernel(const uint
                                                                       int32_t *__restrict__ out_idx, int64_t idx_cap,
                                                                       int32_t *__restrict__ out_counts) {
     constexpr int NL = 32 * W + 1;
+    constexpr int REP = 32;  // histogram replicas (replica = lane % 32 = bank): the candidates sit on a dozen levels
+    static_assert(kMaxChunks <= 2 * kFinThreads, "the chunk prefix is scanned two entries per thread");
     __shared__ int s_pre[kMaxChunks + 1];
+    __shared__ uint32_t s_rep[NL * REP];
     __shared__ uint32_t s_hist[NL];
     __shared__ uint32_t s_sa[kFinWaves], s_sb[kFinWaves];
     __shared__ int s_T, s_r, s_nheavy, s_ok;
@@ -289,29 +322,26 @@ __global__ __launch_bounds__(kFinThreads) void select_finalize_kernel(const uint
 
     int nheavy = 0;
     if (rb.kk > 0) {  // uniform
-        // ---- candidates per chunk -> exclusive prefix
+        // ---- candidates per chunk -> exclusive prefix (two chunks per thread, one block scan)
         if (tid == 0) s_ok = t_hi >= 0 ? 1 : 0;
-        if (tid < NL) s_hist[tid] = 0;
-        __syncthreads();
+        for (int i = tid; i < NL * REP; i += kFinThreads) s_rep[i] = 0;
+        int c0 = 0, c1 = 0;
         if (t_hi >= 0) {
-            for (int c = tid; c < nchunk; c += kFinThreads)
-                if (cnt[c] > cap) s_ok = 0;  // a segment overflowed (benign race: every writer stores 0)
-            if (tid == 0) {
-                int acc = 0;
-                for (int c = 0; c < nchunk; ++c) {
-                    s_pre[c] = acc;
-                    acc += min(cnt[c], cap);
-                }
-                s_pre[nchunk] = acc;
-            }
+            if (tid < nchunk) c0 = cnt[tid];
+            if (tid + kFinThreads < nchunk) c1 = cnt[tid + kFinThreads];
+        }
+        __syncthreads();
+        if (c0 > cap || c1 > cap) s_ok = 0;  // a segment overflowed (benign race: every writer stores 0)
+        {
+            int ex0, ex1, tot0, tot1;
+            block_scan2(min(c0, cap), min(c1, cap), s_sa, s_sb, ex0, ex1, tot0, tot1);
+            if (tid < nchunk) s_pre[tid] = ex0;
+            if (tid + kFinThreads < nchunk) s_pre[tid + kFinThreads] = tot0 + ex1;
+            if (tid == 0) s_pre[nchunk] = tot0 + tot1;
         }
         __syncthreads();
         const int ntot = t_hi >= 0 ? s_pre[nchunk] : 0;
-        // candidate i of the row: chunk by binary search in the prefix, then its place in the segment
-        auto cand_index = [&](int i, int &c) {
-            while (i >= s_pre[c + 1]) ++c;
-            return seg0[(int64_t)c * cap + (i - s_pre[c])];
-        };
+        // chunk that holds entry i of the row's candidate list: binary search in the prefix
         auto chunk_of = [&](int i) {
             int lo_c = 0, hi_c = nchunk - 1;
             while (lo_c < hi_c) {
@@ -321,12 +351,51 @@ __global__ __launch_bounds__(kFinThreads) void select_finalize_kernel(const uint
             }
             return lo_c;
         };
-        if (s_ok) {
+        // A thread owns a contiguous run of the candidate list, handled in batches of RB entries held in
+        // registers (index and distance come in one word): the loads of a batch are independent of each other.
+        // RB is picked per row from the run length, so short runs do not pay for a long unrolled body.
+        const int R = (ntot + kFinThreads - 1) / kFinThreads;
+        const int i0 = min(tid * R, ntot), i1 = min(i0 + R, ntot);
+        auto from_candidates = [&](auto rb_tag) {
+            constexpr int RB = decltype(rb_tag)::value;
+            const int nbatch = (R + RB - 1) / RB;  // uniform
+            int jreg[RB], dreg[RB];
+            auto load_batch = [&](int first) {  // entries [first, first + RB) of the run -> jreg / dreg (d = NL when absent)
+                int c = first < i1 ? chunk_of(first) : 0;
+                int seg_end = s_pre[c + 1];
+                const int32_t *src = seg0 + (int64_t)c * cap - s_pre[c];  // entry i of the list is src[i] while i < seg_end
+#pragma unroll
+                for (int t = 0; t < RB; ++t) {
+                    const int i = first + t;
+                    jreg[t] = -1;
+                    if (i < i1) {
+                        if (i >= seg_end) {  // the run crosses into a later chunk's segment
+                            while (i >= s_pre[c + 1]) ++c;
+                            seg_end = s_pre[c + 1];
+                            src = seg0 + (int64_t)c * cap - s_pre[c];
+                        }
+                        jreg[t] = src[i];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < RB; ++t) {
+                    dreg[t] = jreg[t] >= 0 ? (int)((uint32_t)jreg[t] >> 24) : NL;
+                    jreg[t] &= 0xFFFFFF;
+                }
+            };
             // ---- exact histogram of the candidates
-            for (int i = tid; i < ntot; i += kFinThreads) {
-                int c = chunk_of(i);
-                const int j = cand_index(i, c);
-                atomicAdd(&s_hist[load_code<W>(kc, j).dist(q)], 1u);
+            for (int bt = 0; bt < nbatch; ++bt) {
+                load_batch(i0 + bt * RB);
+#pragma unroll
+                for (int t = 0; t < RB; ++t)
+                    if (dreg[t] < NL) atomicAdd(&s_rep[dreg[t] * REP + (tid % REP)], 1u);
+            }
+            __syncthreads();
+            if (tid < NL) {
+                uint32_t sum = 0;
+#pragma unroll 8
+                for (int rr = 0; rr < REP; ++rr) sum += s_rep[tid * REP + ((rr + tid) % REP)];
+                s_hist[tid] = sum;
             }
             __syncthreads();
             if (tid == 0) {
@@ -338,36 +407,40 @@ __global__ __launch_bounds__(kFinThreads) void select_finalize_kernel(const uint
                 s_ok = ok ? 1 : 0;
             }
             __syncthreads();
-        }
-        if (s_ok) {
-            // ---- ordered compaction of the candidate list: a thread owns a contiguous run
+            if (!s_ok) return;  // uniform: the candidates do not hold k tokens
+            // ---- ordered compaction of the candidate list
             const int T = s_T, r = s_r;
-            const int R = (ntot + kFinThreads - 1) / kFinThreads;
-            const int i0 = min(tid * R, ntot), i1 = min(i0 + R, ntot);
             int nlt = 0, neq = 0;
-            if (i0 < i1) {
-                int c = chunk_of(i0);
-                for (int i = i0; i < i1; ++i) {
-                    const int d = load_code<W>(kc, cand_index(i, c)).dist(q);
-                    nlt += d < T ? 1 : 0;
-                    neq += d == T ? 1 : 0;
+            for (int bt = 0; bt < nbatch; ++bt) {
+                if (nbatch > 1) load_batch(i0 + bt * RB);  // a single batch is still in registers
+#pragma unroll
+                for (int t = 0; t < RB; ++t) {
+                    nlt += dreg[t] < T ? 1 : 0;
+                    neq += dreg[t] == T ? 1 : 0;
                 }
             }
             int ex_lt, ex_eq, tot_lt, tot_eq;
             block_scan2(nlt, neq, s_sa, s_sb, ex_lt, ex_eq, tot_lt, tot_eq);
-            if (i0 < i1) {
-                int c = chunk_of(i0);
-                for (int i = i0; i < i1; ++i) {
-                    const int j = cand_index(i, c);
-                    const int d = load_code<W>(kc, j).dist(q);
+            for (int bt = 0; bt < nbatch; ++bt) {
+                if (nbatch > 1) load_batch(i0 + bt * RB);
+#pragma unroll
+                for (int t = 0; t < RB; ++t) {
+                    const int d = dreg[t];
                     if (d < T || (d == T && ex_eq < r)) {
                         const int64_t pos = (int64_t)rb.lo + ex_lt + min(ex_eq, r);
-                        if (pos < idx_cap) o[pos] = j;
+                        if (pos < idx_cap) o[pos] = jreg[t];
                     }
                     ex_lt += d < T ? 1 : 0;
                     ex_eq += d == T ? 1 : 0;
                 }
             }
+        };
+        if (s_ok) {
+            if (R <= 8) from_candidates(std::integral_constant<int, 8>{});
+            else if (R <= 16) from_candidates(std::integral_constant<int, 16>{});
+            else from_candidates(std::integral_constant<int, 32>{});
+        }
+        if (s_ok) {
             nheavy = s_nheavy;
         } else {
             // ---- exact path from the codes: the guess was too low, a segment overflowed, or it was asked for

@@ -108,6 +108,7 @@ def main():
     ap.add_argument("--config", default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
+    ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
     ap.add_argument("--traffic-probe", action="store_true", help="run the launches the HBM-traffic counters are read from, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -134,6 +135,7 @@ def main():
     layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, d, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
                             w.init_budget, w.recent_budget, w.heavy_budget, device=dev)
     layer.allocate(B, S)
+    layer.select_algo = args.select_algo
     # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
     layer.encode_keys(p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
     torch.cuda.synchronize()

@@ -132,6 +132,38 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
 #undef HA_DPP_ADD
 
 
+#ifdef __HIPCC__
+// T (k-th smallest distance), r (how many of the tie bucket are taken) and the number of heavy tokens from a
+// histogram `tot` whose levels above `top` are unknown.  false if the known levels do not hold k tokens.
+__device__ __forceinline__ bool solve_threshold(const uint32_t *tot, int top, int NL, int kk, int mode, int depth, int &T, int &r,
+                                                int &nheavy) {
+    T = 0;
+    r = 0;
+    nheavy = 0;
+    if (kk <= 0) return true;
+    int cum = 0, l = 0, dmin = -1;
+    for (; l <= top && l < NL; ++l) {
+        const int t = (int)tot[l];
+        if (dmin < 0 && t > 0) dmin = l;
+        if (cum + t >= kk) break;
+        cum += t;
+    }
+    if (l > top || l >= NL) return false;
+    if (mode == HA_SELECT_SIMPLE) {
+        T = l;
+        r = kk - cum;
+        nheavy = kk;
+    } else {
+        const int th = min(dmin + depth, l);
+        T = th + 1;
+        r = 0;
+        for (int i = 0; i <= th; ++i) nheavy += (int)tot[i];
+    }
+    return true;
+}
+
+#endif
+
 // ---- host side -----------------------------------------------------------------------------------
 // rows start 16-byte aligned and hold whole groups of four codes: 128-bit loads never leave a row
 inline bool rows_vectorisable(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, int W) {

@@ -26,35 +26,6 @@ constexpr int kFinThreads = 512;
 constexpr int kFinWaves = kFinThreads / HA_WAVE;
 constexpr int kMaxSample = 4096;  // sampled candidates per (sequence, code head)
 
-// T (k-th smallest distance), r (how many of the tie bucket are taken) and the number of heavy tokens from a
-// histogram `tot` whose levels above `top` are unknown.  false if the known levels do not hold k tokens.
-__device__ __forceinline__ bool solve_threshold(const uint32_t *tot, int top, int NL, int kk, int mode, int depth, int &T, int &r,
-                                                int &nheavy) {
-    T = 0;
-    r = 0;
-    nheavy = 0;
-    if (kk <= 0) return true;
-    int cum = 0, l = 0, dmin = -1;
-    for (; l <= top && l < NL; ++l) {
-        const int t = (int)tot[l];
-        if (dmin < 0 && t > 0) dmin = l;
-        if (cum + t >= kk) break;
-        cum += t;
-    }
-    if (l > top || l >= NL) return false;
-    if (mode == HA_SELECT_SIMPLE) {
-        T = l;
-        r = kk - cum;
-        nheavy = kk;
-    } else {
-        const int th = min(dmin + depth, l);
-        T = th + 1;
-        r = 0;
-        for (int i = 0; i <= th; ++i) nheavy += (int)tot[i];
-    }
-    return true;
-}
-
 // ------------------------------------------------------------------------------------------------
 // grid (Hc, B), 256 threads.  thi[row] = T_hi, -1 when the row has no heavy budget, -2 = "take the exact path".
 template <int W, int GQ>

@@ -36,6 +36,7 @@ class HashDecodeLayer:
         self.mode = _ops.HA_SELECT_SIMPLE if eval_mode == "simple" else _ops.HA_SELECT_THRESHOLD
         self.depth = int(math.floor(retrieve_depth))
         self.arith = arith
+        self.select_algo = _ops.HA_SELECT_ALGO_AUTO
         self.device = torch.device(device)
         self.wk = _ops.pack_usa_weights(k_layers, self.device)
         self.wq = _ops.pack_usa_weights(q_layers, self.device)
@@ -89,7 +90,8 @@ class HashDecodeLayer:
 
     def select(self, max_seq_len: int, seq_lens: Optional[torch.Tensor]) -> None:
         _ops.select(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
-                    self.recent_budget, self.heavy_budget, self.idx, self.counts, self.ws_select, self.mode, self.depth)
+                    self.recent_budget, self.heavy_budget, self.idx, self.counts, self.ws_select, self.mode, self.depth,
+                    self.select_algo)
 
     def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor) -> None:
         _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend)

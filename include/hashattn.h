@@ -51,7 +51,7 @@ typedef enum ha_status {
 #define HA_SELECT_THRESHOLD 1 /* otherwise: every candidate within the distance threshold, ties included */
 
 /* How ha_select finds the threshold; every choice returns the same lists. */
-#define HA_SELECT_ALGO_AUTO 0              /* sampled when few tokens are kept of long rows, else histogram */
+#define HA_SELECT_ALGO_AUTO 0              /* the library's choice (currently the histogram method) */
 #define HA_SELECT_ALGO_HISTOGRAM 1         /* two passes over the codes: exact histogram, then compaction */
 #define HA_SELECT_ALGO_SAMPLED 2           /* sampled upper bound of the threshold, one filtering pass, exact finish */
 #define HA_SELECT_ALGO_SAMPLED_EXACT_ROWS 3 /* diagnostic: as SAMPLED with every row sent through its in-kernel exact path */

@@ -94,10 +94,16 @@ def traffic_probe(torch, layer, q3, k, v, out):
     for _ in range(3):
         dst.copy_(src)
     torch.cuda.synchronize()
+    from hashattention import _ops
+    w = layer
     for _ in range(3):
-        layer.attend(q3, k, v, out)
+        if layer.overlap_windows:
+            _ops.sparse_decode_heavy(q3, k, v, w.idx, w.counts, w.sm_scale, out, w.ws_attend, w.win, w.init_budget,
+                                     w.recent_budget, k.shape[2], None)
+        else:
+            layer.attend(q3, k, v, out)
     torch.cuda.synchronize()
-    print(json.dumps({"probe": "copy 1 GiB x3 (vectorized_elementwise copy kernel), then sparse_attend x3"}))
+    print(json.dumps({"probe": "copy 1 GiB x3 (runtime copy kernel), then the step's sparse_attend launch x3"}))
 
 
 def main():
@@ -109,6 +115,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
+    ap.add_argument("--overlap-windows", action="store_true", help="attend to sink|recent on a second stream (ha_window_partial)")
     ap.add_argument("--traffic-probe", action="store_true", help="run the launches the HBM-traffic counters are read from, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -136,6 +143,7 @@ def main():
                             w.init_budget, w.recent_budget, w.heavy_budget, device=dev)
     layer.allocate(B, S)
     layer.select_algo = args.select_algo
+    layer.overlap_windows = args.overlap_windows
     # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
     layer.encode_keys(p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
     torch.cuda.synchronize()
@@ -177,12 +185,27 @@ def main():
     ms_step = min(ms_step_graph, ms_step_eager)
     ms_encode = time_gpu(encode_only, args.steps, args.warmup, torch)
     ms_select = time_gpu(lambda: layer.select(S, seq_lens), args.steps, args.warmup, torch)
-    ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
+    if layer.overlap_windows:      # the dominant kernel as the step launches it: heavy tokens only, window partial merged
+        _ops.window_partial(q3, p.k, p.v, S, seq_lens, w.init_budget, w.recent_budget, layer.sm_scale, layer.win)
+        ms_attend = time_gpu(lambda: _ops.sparse_decode_heavy(q3, p.k, p.v, layer.idx, layer.counts, layer.sm_scale, out,
+                                                              layer.ws_attend, layer.win, w.init_budget, w.recent_budget, S,
+                                                              seq_lens), args.steps, args.warmup, torch)
+        ms_window = time_gpu(lambda: _ops.window_partial(q3, p.k, p.v, S, seq_lens, w.init_budget, w.recent_budget,
+                                                         layer.sm_scale, layer.win), args.steps, args.warmup, torch)
+    else:
+        ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
+        ms_window = 0.0
     ms_dense = time_gpu(lambda: _ops.dense_decode(q3, p.k, p.v, S, seq_lens, layer.sm_scale, out_dense, ws_dense),
                         max(10, args.steps // 4), max(2, args.warmup // 4), torch)
 
     n_sel_rows = int(layer.counts.sum().item())
     ab = algorithmic_bytes(w, n_sel_rows)
+    eb = 2 if w.dtype != torch.float32 else 4
+    if layer.overlap_windows:      # bytes of the heavy-only launch: its rows, their indices, q, out and the window partial
+        n_win_rows = sum(H * (min(w.init_budget, s) + s - max(s - w.recent_budget, min(w.init_budget, s))) for s in w.seq_lens)
+        attend_bytes = (n_sel_rows - n_win_rows) * (2 * d * eb + 4) + B * H * (2 * d * eb + 130 * 4)
+    else:
+        attend_bytes = ab["gather"]
     sparse_bytes = ab["score"] + ab["select"] + ab["gather"]
     err = (out.float() - out_dense.float()).abs().max().item()   # informational: sparse vs dense output distance
 
@@ -207,7 +230,8 @@ def main():
                                f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} "
                                f"n_sel={n_sel_rows // (B * H)}"},
         "stages_us": {"encode_new_k_and_q": ms_encode * 1e3, "score_select": ms_select * 1e3,
-                      "gather_attend": ms_attend * 1e3, "dense_flash_decode": ms_dense * 1e3},
+                      "gather_attend": ms_attend * 1e3, "window_partial_second_stream": ms_window * 1e3,
+                      "dense_flash_decode": ms_dense * 1e3},
         "hbm_gbps_step": sparse_bytes / (ms_step * 1e-3) / 1e9,
         "hbm_frac_step": sparse_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "speedup_vs_dense": ms_dense / ms_step,
@@ -215,10 +239,10 @@ def main():
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
         "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm",
-                     "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "achieved": attend_bytes / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": attend_bytes / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get(w.name),
-                     "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
+                     "algorithmic_bytes": attend_bytes, "us": ms_attend * 1e3},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)

@@ -109,7 +109,9 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
                                                            const int32_t *__restrict__ idx, int64_t idx_cap,
                                                            const int32_t *__restrict__ counts, float scale_log2e, int split_rows,
                                                            int nsplit_max, float *__restrict__ part_acc,
-                                                           float *__restrict__ part_ml, void *__restrict__ out) {
+                                                           float *__restrict__ part_ml, void *__restrict__ out,
+                                                           const float *__restrict__ win_part, int win_init, int win_recent,
+                                                           const int32_t *__restrict__ seq_lens, int max_S) {
     using EL = Elem<E>;
     constexpr int NS = NT / 16;  // row streams
     __shared__ float s_m[NS], s_l[NS];
@@ -124,14 +126,25 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
     int64_t n = counts[b * H + h];
     if (n > idx_cap) n = idx_cap;
+    // win_part: the sink and recent windows were attended by another launch; their entries (the first
+    // min(init, S) and the last S - max(S - recent, min(init, S)) of the list) are skipped here and the
+    // partial is merged at the end
+    int skip_front = 0;
+    if (win_part) {
+        int S = seq_lens ? seq_lens[b] : max_S;
+        if (S > max_S) S = max_S;
+        const int lo = min(win_init, S), hi = max(S - win_recent, lo);
+        skip_front = lo;
+        n = max((int64_t)0, n - lo - (S - hi));
+    }
     const int nsplit = n > 0 ? (int)((n + split_rows - 1) / split_rows) : 1;
     if (sp >= nsplit) return;
     const int64_t row = (int64_t)b * H + h;
-    if (n == 0) {  // empty sequence: defined as a zero output
+    if (n == 0 && !win_part) {  // empty sequence: defined as a zero output
         if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
         return;
     }
-    const int r0 = sp * split_rows, r1 = (int)min((int64_t)r0 + split_rows, n);
+    const int r0 = skip_front + sp * split_rows, r1 = (int)min((int64_t)r0 + split_rows, skip_front + n);
     const int32_t *ix = idx + row * idx_cap;
     const char *kb = (const char *)k + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const char *vb = (const char *)v + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
@@ -227,7 +240,15 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
         float M, L, A;
         merge_streams<NS>(s_m, s_l, s_acc, tid, M, L, A);
         if (nsplit == 1) {
-            EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
+            if (win_part) {  // partial of the windows: acc[128], m, l
+                const float *wp = win_part + row * (HA_HEAD_DIM + 2);
+                const float wm = wp[HA_HEAD_DIM], wl = wp[HA_HEAD_DIM + 1];
+                const float M2 = fmaxf(M, wm);
+                const float sh = (M == -INFINITY) ? 0.f : fast_exp2(M - M2), sw = (wm == -INFINITY) ? 0.f : fast_exp2(wm - M2);
+                A = A * sh + wp[tid] * sw;
+                L = L * sh + wl * sw;
+            }
+            EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, L > 0.f ? A / L : 0.f);
         } else {
             const int64_t p = row * nsplit_max + sp;
             part_acc[p * HA_HEAD_DIM + tid] = A;
@@ -246,12 +267,20 @@ template <typename E>
 __global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *__restrict__ part_acc, const float *__restrict__ part_ml,
                                                                    const int32_t *__restrict__ counts, int per_batch,
                                                                    int64_t count_cap, int H, int unit, int nsplit_max,
-                                                                   void *__restrict__ out) {
+                                                                   void *__restrict__ out, const float *__restrict__ win_part,
+                                                                   int win_init, int win_recent,
+                                                                   const int32_t *__restrict__ win_seq_lens, int win_max_S) {
     using EL = Elem<E>;
     const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
     const int64_t row = (int64_t)b * H + h;
     int64_t n = counts ? counts[per_batch ? b : row] : count_cap;
     if (n > count_cap) n = count_cap;
+    if (win_part) {  // the attend kernel skipped the window entries of the list (see sparse_attend_kernel)
+        int win_S = win_seq_lens ? win_seq_lens[b] : win_max_S;
+        if (win_S > win_max_S) win_S = win_max_S;
+        const int lo = min(win_init, win_S), hi = max(win_S - win_recent, lo);
+        n = max((int64_t)0, n - lo - (win_S - hi));
+    }
     const int nsplit = (int)((n + unit - 1) / unit);
     if (nsplit <= 1) return;
     const float *ml = part_ml + row * nsplit_max * 2;
@@ -266,19 +295,30 @@ __global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *
         L += w * ml[s * 2 + 1];
         A += w * pa[(int64_t)s * HA_HEAD_DIM];
     }
+    if (win_part) {
+        const float *wp = win_part + row * (HA_HEAD_DIM + 2);
+        const float wm = wp[HA_HEAD_DIM], M2 = fmaxf(M, wm);
+        const float sh = fast_exp2(M - M2), sw = (wm == -INFINITY) ? 0.f : fast_exp2(wm - M2);
+        A = A * sh + wp[e] * sw;
+        L = L * sh + wp[HA_HEAD_DIM + 1] * sw;
+    }
     EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, A / L);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Dense flash-decode.  grid (nsplit_max, Hkv, B).  A workgroup streams `chunk` consecutive keys of one
 // KV head once and scores them against the G query heads of the group.
-template <typename E, int G>
+// WIN: the same over the sink and recent windows only (win_init, win_recent; grid (1, Hkv, B)): the result is
+// left as an unnormalised partial (acc, m, l) per row for the sparse kernel to merge, so this small launch can
+// run on another stream while the selection is still being computed.
+template <typename E, int G, bool WIN>
 __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                                    const void *__restrict__ k, const void *__restrict__ v,
                                                                    int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int max_S,
                                                                    const int32_t *__restrict__ seq_lens, float scale_log2e, int chunk,
                                                                    int nsplit_max, float *__restrict__ part_acc,
-                                                                   float *__restrict__ part_ml, void *__restrict__ out) {
+                                                                   float *__restrict__ part_ml, void *__restrict__ out, int win_init,
+                                                                   int win_recent) {
     using EL = Elem<E>;
     __shared__ float s_m[kStreams], s_l[kStreams];
     __shared__ float s_acc[kStreams * HA_HEAD_DIM];
@@ -287,14 +327,19 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;
-    const int nsplit = S > 0 ? (S + chunk - 1) / chunk : 1;
+    // WIN: list position t < n_sink is token t, the others are tokens win_hi + (t - n_sink)
+    const int n_sink = WIN ? min(win_init, S) : 0;
+    const int win_hi = WIN ? max(S - win_recent, n_sink) : 0;
+    const int n_rows = WIN ? n_sink + (S - win_hi) : S;
+    const int nsplit = WIN ? 1 : (S > 0 ? (S + chunk - 1) / chunk : 1);
     if (sp >= nsplit) return;
-    if (S == 0) {
+    if (!WIN && S == 0) {
         if (tid < HA_HEAD_DIM)
             for (int g = 0; g < G; ++g) EL::store1((char *)out + ((int64_t)b * H + hk * G + g) * HA_HEAD_DIM * EL::bytes, tid, 0.f);
         return;
     }
-    const int r0 = sp * chunk, r1 = min(r0 + chunk, S);
+    const int r0 = WIN ? 0 : sp * chunk, r1 = WIN ? n_rows : min(r0 + chunk, S);
+    auto token = [&](int r) { return WIN ? (r < n_sink ? r : win_hi + (r - n_sink)) : r; };
     const char *kb = (const char *)k + (b * kv_sb + hk * kv_sh) * EL::bytes;
     const char *vb = (const char *)v + (b * kv_sb + hk * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;
@@ -323,10 +368,10 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
         for (int u = 0; u < kUnroll; ++u) {
             const int r = base + u * kStreams;
             ok[u] = r < r1;
-            kr[u] = EL::load8(kb + (ok[u] ? r : base) * row_bytes, sub);
+            kr[u] = EL::load8(kb + token(ok[u] ? r : base) * row_bytes, sub);
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + (ok[u] ? base + u * kStreams : base) * row_bytes, sub);
+        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + token(ok[u] ? base + u * kStreams : base) * row_bytes, sub);
 
         float sc[G][kUnroll];
 #pragma unroll
@@ -385,7 +430,13 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
             float M, L, A;
             merge_streams<kStreams>(s_m, s_l, s_acc, tid, M, L, A);
             const int64_t row = (int64_t)b * H + hk * G + g;
-            if (nsplit == 1) {
+            if (WIN) {  // one record per row: acc[128], m, l
+                part_acc[row * (HA_HEAD_DIM + 2) + tid] = A;
+                if (tid == 0) {
+                    part_acc[row * (HA_HEAD_DIM + 2) + HA_HEAD_DIM] = M;
+                    part_acc[row * (HA_HEAD_DIM + 2) + HA_HEAD_DIM + 1] = L;
+                }
+            } else if (nsplit == 1) {
                 EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, A / L);
             } else {
                 const int64_t pi = row * nsplit_max + sp;
@@ -428,10 +479,11 @@ size_t ha_sparse_decode_workspace_bytes(int B, int H, int64_t idx_cap) {
     return part_bytes((int64_t)B * H, (int)((idx_cap + kMinSplitRows - 1) / kMinSplitRows));
 }
 
-int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
-                     int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, const int32_t *idx,
-                     int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace, size_t workspace_bytes,
-                     void *stream) {
+static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                              int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv,
+                              const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace,
+                              size_t workspace_bytes, const float *win_part, int win_init, int win_recent, const int32_t *seq_lens,
+                              int max_seq_len, void *stream) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(idx && counts, HA_ERR_NULL_POINTER, "idx/counts is NULL");
@@ -454,11 +506,11 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, cons
     do {                                                                                                                          \
         hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,           \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
-                           plan.nsplit_max, part_acc, part_ml, out);                                                              \
+                           plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len);       \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
         if (plan.nsplit_max > 1) {                                                                                                \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
-                               plan.split_rows, plan.nsplit_max, out);                                                            \
+                               plan.split_rows, plan.nsplit_max, out, win_part, win_init, win_recent, seq_lens, max_seq_len);     \
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
         }                                                                                                                         \
     } while (0)
@@ -472,6 +524,67 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, cons
     else HA_SPARSE_DISPATCH(ElemF32, 2);
 #undef HA_SPARSE_DISPATCH
 #undef HA_SPARSE_LAUNCH
+    return HA_OK;
+}
+
+int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                     int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, const int32_t *idx,
+                     int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace, size_t workspace_bytes,
+                     void *stream) {
+    return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
+                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0, stream);
+}
+
+int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, const int32_t *idx,
+                           int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace,
+                           size_t workspace_bytes, const float *window_partial, int init_budget, int recent_budget,
+                           int max_seq_len, const int32_t *seq_lens, void *stream) {
+    HA_REQUIRE(window_partial, HA_ERR_NULL_POINTER, "window_partial is NULL");
+    HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && max_seq_len > 0, HA_ERR_BAD_SHAPE, "bad window budgets or max_seq_len");
+    return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
+                              counts, sm_scale, out, workspace, workspace_bytes, window_partial, init_budget, recent_budget, seq_lens,
+                              max_seq_len, stream);
+}
+
+size_t ha_window_partial_bytes(int B, int H) {
+    if (B <= 0 || H <= 0) return 0;
+    return (size_t)B * H * (HA_HEAD_DIM + 2) * sizeof(float);
+}
+
+int ha_window_partial(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                      int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, int max_seq_len,
+                      const int32_t *seq_lens, int init_budget, int recent_budget, float sm_scale, float *window_partial,
+                      void *stream) {
+    HA_REQUIRE(window_partial, HA_ERR_NULL_POINTER, "window_partial is NULL");
+    int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, window_partial);
+    if (st) return st;
+    HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && max_seq_len > 0, HA_ERR_BAD_SHAPE, "bad window budgets or max_seq_len");
+    const int G = H / Hkv;
+    HA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, HA_ERR_BAD_SHAPE, "H/Hkv=%d, must be 1, 2, 4 or 8", G);
+    if ((st = ha_require_device())) return st;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(1, Hkv, B);
+    const float sl2 = sm_scale * kLog2e;
+#define HA_WIN_LAUNCH(E_, G_)                                                                                                      \
+    do {                                                                                                                           \
+        hipLaunchKernelGGL((dense_attend_kernel<E_, G_, true>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,    \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, 0, 1, window_partial,             \
+                           (float *)nullptr, (void *)nullptr, init_budget, recent_budget);                                         \
+        HA_CHECK_LAUNCH("dense_attend_kernel<window>");                                                                            \
+    } while (0)
+#define HA_WIN_DISPATCH(E_)                    \
+    do {                                       \
+        if (G == 1) HA_WIN_LAUNCH(E_, 1);      \
+        else if (G == 2) HA_WIN_LAUNCH(E_, 2); \
+        else if (G == 4) HA_WIN_LAUNCH(E_, 4); \
+        else HA_WIN_LAUNCH(E_, 8);             \
+    } while (0)
+    if (kv_dtype == HA_BF16) HA_WIN_DISPATCH(ElemBF16);
+    else if (kv_dtype == HA_F16) HA_WIN_DISPATCH(ElemF16);
+    else HA_WIN_DISPATCH(ElemF32);
+#undef HA_WIN_DISPATCH
+#undef HA_WIN_LAUNCH
     return HA_OK;
 }
 
@@ -509,13 +622,14 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const
     const float sl2 = sm_scale * kLog2e;
 #define HA_DENSE_LAUNCH(E_, G_)                                                                                                    \
     do {                                                                                                                           \
-        hipLaunchKernelGGL((dense_attend_kernel<E_, G_>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,          \
+        hipLaunchKernelGGL((dense_attend_kernel<E_, G_, false>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,   \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, plan.chunk, plan.nsplit_max,      \
-                           part_acc, part_ml, out);                                                                                \
+                           part_acc, part_ml, out, 0, 0);                                                                          \
         HA_CHECK_LAUNCH("dense_attend_kernel");                                                                                    \
         if (plan.nsplit_max > 1) {                                                                                                 \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, seq_lens, 1,            \
-                               (int64_t)max_seq_len, H, plan.chunk, plan.nsplit_max, out);                                         \
+                               (int64_t)max_seq_len, H, plan.chunk, plan.nsplit_max, out, (const float *)nullptr, 0, 0,            \
+                               (const int32_t *)nullptr, 0);                                                                       \
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                                \
         }                                                                                                                          \
     } while (0)

@@ -72,6 +72,13 @@ def load_library() -> C.CDLL:
     lib.ha_sparse_decode.restype = i32
     lib.ha_sparse_decode.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
                                      vp, vp, sz, vp]
+    lib.ha_window_partial_bytes.restype = sz
+    lib.ha_window_partial_bytes.argtypes = [i32, i32]
+    lib.ha_window_partial.restype = i32
+    lib.ha_window_partial.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, f32, vp, vp]
+    lib.ha_sparse_decode_heavy.restype = i32
+    lib.ha_sparse_decode_heavy.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
+                                           vp, vp, sz, vp, i32, i32, i32, vp, vp]
     lib.ha_dense_decode_workspace_bytes.restype = sz
     lib.ha_dense_decode_workspace_bytes.argtypes = [i32, i32, i32]
     lib.ha_dense_decode.restype = i32
@@ -245,6 +252,30 @@ def sparse_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.
     assert out.is_contiguous() and out.dtype == q.dtype and idx.is_contiguous() and counts.is_contiguous()
     _check(lib.ha_sparse_decode(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
                                 float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_sparse_decode")
+
+
+def window_partial(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
+                   init_budget: int, recent_budget: int, sm_scale: float, win: torch.Tensor) -> None:
+    """Attention over the sink and recent windows only -> win [B, H, 130] fp32 (acc[128], m, l), unnormalised."""
+    _require_cuda(q, k, v, seq_lens, win)
+    lib = load_library()
+    B, H, _ = q.shape
+    assert win.dtype == torch.float32 and win.is_contiguous() and win.numel() == B * H * 130
+    _check(lib.ha_window_partial(*_kv_args(q, k, v), B, H, k.shape[1], max_seq_len, _ptr(seq_lens), init_budget, recent_budget,
+                                 float(sm_scale), _ptr(win), _stream(q)), "ha_window_partial")
+
+
+def sparse_decode_heavy(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor,
+                        sm_scale: float, out: torch.Tensor, ws: torch.Tensor, win: torch.Tensor, init_budget: int,
+                        recent_budget: int, max_seq_len: int, seq_lens: Optional[torch.Tensor]) -> None:
+    """`sparse_decode` that skips the window entries of the lists and merges the partial made by `window_partial`."""
+    _require_cuda(q, k, v, idx, counts, out, ws, win, seq_lens)
+    lib = load_library()
+    B, H, _ = q.shape
+    assert out.is_contiguous() and out.dtype == q.dtype and idx.is_contiguous() and counts.is_contiguous()
+    _check(lib.ha_sparse_decode_heavy(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
+                                      float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _ptr(win), init_budget, recent_budget,
+                                      max_seq_len, _ptr(seq_lens), _stream(q)), "ha_sparse_decode_heavy")
 
 
 def dense_decode_workspace_bytes(B, H, max_seq_len) -> int:

@@ -4,9 +4,11 @@
 (hashattention/hashattention_llama.py:401-446, 578-615): the packed hash-MLP weights and the bit-cache of
 key codes, plus the index lists and workspaces of the kernels.  One decode step is
 
+    windows  attention over sink | recent, second stream    (ha_window_partial, overlaps the next two)
     encode   code of the new key -> bit-cache, query codes  (ha_encode_step, one launch)
     select   Hamming histogram + ordered compaction         (ha_select)
-    attend   gather-only split-K attention                  (ha_sparse_decode)
+    attend   gather-only attention over the heavy tokens,   (ha_sparse_decode_heavy; ha_sparse_decode when
+             merged with the window partial                   overlap_windows is off)
 
 All buffers are allocated once per (batch, capacity) and reused: the step itself allocates nothing.
 """
@@ -37,6 +39,9 @@ class HashDecodeLayer:
         self.depth = int(math.floor(retrieve_depth))
         self.arith = arith
         self.select_algo = _ops.HA_SELECT_ALGO_AUTO
+        # attend to sink | recent on a second stream while the selection runs.  Off by default: at 64K-token rows the
+        # windows are already served from L2 to the heads of a group and the fork/join costs more than it hides.
+        self.overlap_windows = False
         self.device = torch.device(device)
         self.wk = _ops.pack_usa_weights(k_layers, self.device)
         self.wq = _ops.pack_usa_weights(q_layers, self.device)
@@ -68,6 +73,8 @@ class HashDecodeLayer:
         self.counts = torch.zeros(B, self.H, dtype=torch.int32, device=dev)
         self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
         self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
+        self.win = torch.empty(B, self.H, 130, dtype=torch.float32, device=dev)
+        self.side_stream = torch.cuda.Stream(device=dev)
         self.n_cached = 0
 
     def reset(self) -> None:
@@ -106,6 +113,14 @@ class HashDecodeLayer:
         `seq_lens` (int32 [B], lengths including the new token) and `seq_len` = their maximum.
         """
         q3 = q[:, :, 0, :]
+        main = torch.cuda.current_stream(self.device)
+        if self.overlap_windows:
+            # fork: the sink and recent windows need no selection, so their share of the attention runs on a second
+            # stream under the (latency-bound) encode and select launches; joined before the heavy tokens are attended
+            self.side_stream.wait_stream(main)
+            with torch.cuda.stream(self.side_stream):
+                _ops.window_partial(q3, k_cache, v_cache, seq_len, seq_lens, self.init_budget, self.recent_budget,
+                                    self.sm_scale, self.win)
         if seq_lens is None:
             if self.n_cached + n_new != seq_len:
                 raise RuntimeError(f"bit-cache holds {self.n_cached} tokens, step at length {seq_len} appends {n_new}")
@@ -121,5 +136,10 @@ class HashDecodeLayer:
             _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
                              self.qcodes, pos_dev=pos, arith=self.arith)
         self.select(seq_len, seq_lens)
-        self.attend(q3, k_cache, v_cache, out)
+        if self.overlap_windows:
+            main.wait_stream(self.side_stream)
+            _ops.sparse_decode_heavy(q3, k_cache, v_cache, self.idx, self.counts, self.sm_scale, out, self.ws_attend, self.win,
+                                     self.init_budget, self.recent_budget, seq_len, seq_lens)
+        else:
+            self.attend(q3, k_cache, v_cache, out)
         return out

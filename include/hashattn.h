@@ -171,6 +171,30 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
                      float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same attention in two launches that may overlap in time.  The sink [0, init) and recent [S - recent, S)
+ * windows are known before any selection is made and are shared by the query heads of a KV group:
+ * ha_window_partial attends to them alone (each row read once per KV head) and leaves an unnormalised partial
+ * (acc[128], m, l: ha_window_partial_bytes) per (sequence, query head).  It depends only on q, K and V, so a
+ * caller can issue it on a second stream while ha_encode_step and ha_select run.  ha_sparse_decode_heavy then
+ * takes the index lists of ha_select (same budgets, same seq_lens), skips their window entries and merges the
+ * partial: the output equals ha_sparse_decode's up to fp32 summation order.  No counterpart in the reference,
+ * whose prototype has no windows at all (efficiency/kernels/torchatt.py:52-71).
+ */
+size_t ha_window_partial_bytes(int B, int H);
+int ha_window_partial(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                      const void *k, const void *v, int kv_dtype,
+                      int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                      int B, int H, int Hkv, int max_seq_len, const int32_t *seq_lens,
+                      int init_budget, int recent_budget, float sm_scale, float *window_partial, void *stream);
+int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                           const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                           int B, int H, int Hkv, const int32_t *idx, int64_t idx_cap, const int32_t *counts,
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes,
+                           const float *window_partial, int init_budget, int recent_budget,
+                           int max_seq_len, const int32_t *seq_lens, void *stream);
+
+/*
  * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).
  * Replaces flash_decode_attention_fwd (efficiency/kernels/flash_fwd_sparse.py:21-321) and
  * torch_attention_naive (efficiency/kernels/torchatt.py:17-30).  Each K/V row is read once per KV

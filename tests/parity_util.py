@@ -120,6 +120,15 @@ def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple"
     assert err <= ATOL[w.dtype], f"sparse attend max-abs error {err} > {ATOL[w.dtype]}"
     report.update(sparse_err=err)
 
+    # ---- the same attention as window partial + heavy-only launch
+    win = torch.empty(B, H, 130, dtype=torch.float32, device=dev)
+    out2 = torch.empty_like(out)
+    _ops.window_partial(q3, k, v, S, seq, w.init_budget, w.recent_budget, sm_scale, win)
+    _ops.sparse_decode_heavy(q3, k, v, idx, counts, sm_scale, out2, ws2, win, w.init_budget, w.recent_budget, S, seq)
+    err2 = float(np.abs(out2.float().cpu().numpy() - ref).max())
+    assert err2 <= ATOL[w.dtype], f"window + heavy attend max-abs error {err2} > {ATOL[w.dtype]}"
+    report.update(split_window_err=err2)
+
     if check_dense:
         outd = torch.empty(B, H, d, dtype=w.dtype, device=dev)
         ws3 = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)

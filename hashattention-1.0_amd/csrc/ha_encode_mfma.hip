@@ -30,10 +30,14 @@ constexpr int kKSteps = kDim / 16;
 // LDS bytes of one layer's permuted weights: [out/32][8 k-steps][64 lanes][8 bf16]
 constexpr int wp_bytes(int out) { return (out / 32) * kKSteps * 64 * 16; }
 
+// SiLU of a Linear output in bf16 arithmetic: the accumulator is rounded to bf16, y * sigmoid(y) is evaluated
+// in fp32 with the hardware exp2 and reciprocal (1 ulp each, far below the bf16 rounding that follows in the
+// caller).  Two of the five operations are quarter-rate transcendentals: with 256 activations per (token,
+// head) against 72 MFMA cycles, this, not the matrix pipe, bounds the kernel.
 __device__ __forceinline__ float silu_bf16(float acc) {
     const float y = (float)(__bf16)acc;
-    const float s = y / (1.0f + __expf(-y));
-    return s;
+    const float t = __builtin_amdgcn_exp2f(y * -1.4426950408889634f);
+    return y * __builtin_amdgcn_rcpf(1.0f + t);
 }
 
 // Copy W [out][128] (bf16, global) into the MFMA A-operand order.  c_perm selects the k permutation:

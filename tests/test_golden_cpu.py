@@ -112,3 +112,23 @@ def test_oracle_matches_vectors_recorded_from_the_reference():
                                              "simple" if mode == 0 else "thold", int(depth))
                     assert torch.equal(orc.mask_from_indices(sel, S)[:, :s_t], mine[b, :, t, :s_t]), (name, tag, b, t)
                     assert not mine[b, :, t, s_t:].any()
+
+
+def test_usa_state_dict_layout_matches_the_reference_checkpoints():
+    """`load_usa` reads reference checkpoints by key: the hash module of this build must expose exactly the keys
+    and shapes of the reference's `USA.state_dict()` (recorded in reference_vectors.npz), values interchangeable."""
+    from hashattention._patched import USA
+    g = np.load(os.path.join(HERE, "reference_vectors.npz"))
+    keys = [str(k) for k in g["state_keys"]]
+    usa = USA(4, 128, {"lth_int_dim": 32, "lth_final_dim": 32, "lth_thold": 0, "lth_num_layers": 3})
+    sd = usa.state_dict()
+    assert list(sd.keys()) == keys
+    ref_sd = {k: torch.from_numpy(g[f"w{i}"]) for i, k in enumerate(keys)}
+    for k in keys:
+        assert sd[k].shape == ref_sd[k].shape, k
+    usa.load_state_dict(ref_sd)                      # a reference state dict loads as is
+    heads = usa.layers("k")
+    assert torch.equal(heads[2][1][0], ref_sd["learning_to_hash_transformation_k.2.2.weight"])
+    # and the ModuleList wrapping of load_usa gives the "{layer}." prefix of the shipped checkpoints
+    ml = torch.nn.ModuleList([usa])
+    assert list(ml.state_dict().keys())[0] == "0." + keys[0]

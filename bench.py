@@ -106,6 +106,87 @@ def traffic_probe(torch, layer, q3, k, v, out):
     print(json.dumps({"probe": "copy 1 GiB x3 (runtime copy kernel), then the step's sparse_attend launch x3"}))
 
 
+def decoder_bench(args, torch):
+    """--config config3: the whole 32-layer Llama-3.1-8B-shaped decoder step (random-init weights, synthetic cache of
+    131072 tokens per sequence, batch 4) with the sparse attention step in every layer; decode tokens/s."""
+    from hashattention import _ops
+    from hashattention.decoder import LlamaShapedDecoder
+    from hashattention.synthetic import named_workload
+    w = named_workload("config3")
+    B, S = w.batch, w.max_seq_len
+    dev = "cuda:0"
+    dec = LlamaShapedDecoder(n_layers=args.layers, n_code_heads=w.n_code_heads, init_budget=w.init_budget,
+                             recent_budget=w.recent_budget, heavy_budget=w.heavy_budget, dtype=torch.bfloat16, device=dev)
+    dec.allocate(B, S)
+    t0 = time.perf_counter()
+    ms_prefill_encode = dec.fill_cache_synthetic(S - 1)
+    fill_s = time.perf_counter() - t0
+    tokens = torch.randint(0, dec.vocab, (B,), device=dev)
+    logits = [None]
+
+    def step(dense=False):
+        with torch.no_grad():
+            logits[0] = dec.decode_step(tokens, advance=False, dense=dense)
+
+    def graphed(fn):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
+
+    ms_eager = time_gpu(step, args.steps, args.warmup, torch)
+    eager_logits = logits[0].clone()
+    g = graphed(step)
+    ms_graph = time_gpu(g.replay, args.steps, args.warmup, torch)
+    graph_ok = bool(torch.equal(logits[0], eager_logits))
+    ms_step = min(ms_eager, ms_graph)
+    gd = graphed(lambda: step(dense=True))
+    ms_dense = time_gpu(gd.replay, max(5, args.steps // 8), 2, torch)
+    # the attention step of one layer alone, at this shape
+    hl0 = dec.hash[0]
+    q = torch.randn(B, dec.H, 1, dec.d, device=dev).to(torch.bfloat16)
+    out = torch.empty(B, dec.H, dec.d, dtype=torch.bfloat16, device=dev)
+
+    def layer_step():
+        hl0.n_cached = S - 1
+        hl0.step(q, dec.k_cache[0], dec.v_cache[0], S, out)
+
+    ms_layer = time_gpu(layer_step, args.steps, args.warmup, torch)
+    ms_attend = time_gpu(lambda: hl0.attend(q[:, :, 0, :], dec.k_cache[0], dec.v_cache[0], out), args.steps, args.warmup, torch)
+    n_sel_rows = int(hl0.counts.sum().item())
+    ab = algorithmic_bytes(w, n_sel_rows)
+    n_params = sum(t.numel() for p in dec.layers for t in p.values()) + dec.lm_head.numel()
+    step_bytes = 2 * n_params + dec.L * (ab["score"] + ab["select"] + ab["gather"])
+    res = {
+        "metric": "decode_tokens_per_s", "value": B / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "step_launch": {"value_is": "graph" if ms_graph <= ms_eager else "eager", "hip_graph_replay_ms": ms_graph,
+                        "eager_launches_from_python_ms": ms_eager},
+        "graph_replay_matches_eager": graph_ok,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config3: {dec.L}-layer Llama-3.1-8B-shaped decoder step, B={B} context={S} H={dec.H} Hkv={dec.Hkv} "
+                               f"d={dec.d} hidden={dec.hidden} ffn={dec.ffn} vocab={dec.vocab} code_heads={dec.Hc} "
+                               f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} n_sel={n_sel_rows // (B * dec.H)}"},
+        "dense_attention_step_ms": ms_dense, "speedup_vs_dense_attention": ms_dense / ms_step,
+        "dense_tokens_per_s": B / (ms_dense * 1e-3),
+        "attention_step_us_per_layer": ms_layer * 1e3, "attention_share_of_step": dec.L * ms_layer / ms_step,
+        "prefill_encode_ms_per_layer": ms_prefill_encode,
+        "prefill_encode_tflops": 2 * B * dec.Hc * (S - 1) * (128 * 128 * 2 + 128 * 32) / (ms_prefill_encode * 1e-3) / 1e12,
+        "cache_fill_seconds": fill_s,
+        "hbm_gbps_step": step_bytes / (ms_step * 1e-3) / 1e9, "hbm_frac_step": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None, "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +197,8 @@ def main():
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
     ap.add_argument("--overlap-windows", action="store_true", help="attend to sink|recent on a second stream (ha_window_partial)")
+    ap.add_argument("--layers", type=int, default=32, help="decoder layers of the config3 whole-step workload")
+    ap.add_argument("--layer-only", action="store_true", help="config3: time one attention layer-step instead of the whole decoder")
     ap.add_argument("--traffic-probe", action="store_true", help="run the launches the HBM-traffic counters are read from, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -132,6 +215,9 @@ def main():
         print("bench.py needs a GPU: the HashAttention path has no CPU fallback", file=sys.stderr)
         sys.exit(2)
     _ops.load_library()
+    if args.config == "config3" and not args.layer_only:
+        decoder_bench(args, torch)
+        return
     dev = "cuda:0"
     w = named_workload(args.config)
     p = make_problem_on_device(w, dev)

@@ -1,0 +1,178 @@
+"""A Llama-shaped decoder step around the sparse attention op: the tokens/s harness of the 32-layer workload.
+
+The reference measures end-to-end decode throughput with a gpt-fast fork (efficiency/generate.py:386-434,
+efficiency/model.py:98-345: RMSNorm, rotary embedding, SwiGLU feed-forward, static KV cache).  That fork is not
+runnable as shipped and drives Double-Sparsity labels, not hashes; this module is the same decoder shape with
+the HashAttention step in every layer.  Everything outside attention is plain library work (rocBLAS GEMMs,
+`F.rms_norm`, elementwise ops): the point is to time the whole step, and to check the plumbing around the op
+(rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
+
+Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no
+per-step concatenation.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import _ops
+from .decode import HashDecodeLayer
+from .synthetic import UsaWeights, layer_dims
+
+
+class LlamaShapedDecoder:
+    def __init__(self, n_layers=32, hidden=4096, ffn=14336, n_heads=32, n_kv_heads=8, head_dim=128, vocab=128256,
+                 rope_theta=500000.0, rms_eps=1e-5, n_code_heads=8, lth_num_layers=3, lth_int_dim=128, lth_final_dim=32,
+                 init_budget=128, recent_budget=128, heavy_budget=1.0 / 32, dtype=torch.bfloat16, device="cuda:0", seed=0):
+        self.L, self.hidden, self.ffn, self.H, self.Hkv, self.d, self.vocab = n_layers, hidden, ffn, n_heads, n_kv_heads, head_dim, vocab
+        self.theta, self.eps, self.dtype, self.device = rope_theta, rms_eps, dtype, torch.device(device)
+        self.Hc = n_code_heads
+        self.usa_shape = (lth_num_layers, lth_int_dim, lth_final_dim)
+        self.budgets = (init_budget, recent_budget, heavy_budget)
+        g = torch.Generator(device=device).manual_seed(seed)
+
+        def w(*shape, fan_in):
+            return (torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * fan_in ** -0.5).to(dtype)
+
+        q_out, kv_out = n_heads * head_dim, n_kv_heads * head_dim
+        self.embed = w(vocab, hidden, fan_in=1.0)
+        self.lm_head = w(vocab, hidden, fan_in=hidden)                     # [out, in] as nn.Linear
+        self.final_norm = torch.ones(hidden, dtype=dtype, device=device)
+        self.layers = []
+        for _ in range(n_layers):
+            self.layers.append(dict(
+                attn_norm=torch.ones(hidden, dtype=dtype, device=device), ffn_norm=torch.ones(hidden, dtype=dtype, device=device),
+                wqkv=w(q_out + 2 * kv_out, hidden, fan_in=hidden), wo=w(hidden, q_out, fan_in=q_out),
+                w13=w(2 * ffn, hidden, fan_in=hidden), w2=w(hidden, ffn, fan_in=ffn)))
+        self.hash: List[HashDecodeLayer] = []
+        self.k_cache: List[torch.Tensor] = []
+        self.v_cache: List[torch.Tensor] = []
+        self.B = self.S_cap = self.seq_len = 0
+        inv = 1.0 / (rope_theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+        self.inv_freq = inv
+
+    # ------------------------------------------------------------------ setup
+    def random_usa(self, seed: int) -> UsaWeights:
+        g = torch.Generator().manual_seed(seed)
+        nl, idim, fdim = self.usa_shape
+        out = UsaWeights()
+        for side, n in (("k", self.Hc), ("q", self.H)):
+            heads = []
+            for _ in range(n):
+                heads.append([(torch.randn(fo, fi, generator=g) * fi ** -0.5, torch.randn(fo, generator=g) * 0.01)
+                              for fi, fo in layer_dims(self.d, idim, fdim, nl)])
+            setattr(out, side, heads)
+        return out
+
+    def allocate(self, B: int, S_cap: int, usa_per_layer: Optional[List[UsaWeights]] = None) -> None:
+        self.B, self.S_cap, self.seq_len = B, S_cap, 0
+        nl, idim, fdim = self.usa_shape
+        init, recent, heavy = self.budgets
+        arith = _ops.HA_ARITH_BF16 if self.dtype == torch.bfloat16 else _ops.HA_ARITH_F32
+        self.k_cache, self.v_cache, self.hash = [], [], []
+        for l in range(self.L):
+            self.k_cache.append(torch.zeros(B, self.Hkv, S_cap, self.d, dtype=self.dtype, device=self.device))
+            self.v_cache.append(torch.zeros(B, self.Hkv, S_cap, self.d, dtype=self.dtype, device=self.device))
+            usa = usa_per_layer[l] if usa_per_layer is not None else self.random_usa(1000 + l)
+            hl = HashDecodeLayer(usa.k, usa.q, self.H, self.Hkv, self.d, nl, idim, fdim, init, recent, heavy, arith=arith,
+                                 device=self.device)
+            hl.allocate(B, S_cap)
+            self.hash.append(hl)
+        self.attn_out = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
+        self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
+
+    def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
+        """Put `seq_len` synthetic tokens (N(0,1) keys/values) in every layer's cache and hash all keys with the MFMA
+        encoder.  Returns the milliseconds the hashing of one layer took (HIP events)."""
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        ms = []
+        for l in range(self.L):
+            for b in range(self.B):
+                self.k_cache[l][b, :, :seq_len] = torch.randn(self.Hkv, seq_len, self.d, generator=g, device=self.device).to(self.dtype)
+                self.v_cache[l][b, :, :seq_len] = torch.randn(self.Hkv, seq_len, self.d, generator=g, device=self.device).to(self.dtype)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            self.hash[l].encode_keys(self.k_cache[l][:, :, :seq_len], pos0=0,
+                                     use_mfma=self.dtype == torch.bfloat16 and self.hash[l].wk_bf16 is not None)
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+            self.hash[l].n_cached = seq_len
+        self.seq_len = seq_len
+        return sum(ms) / len(ms)
+
+    def load_cache(self, keys: List[torch.Tensor], values: List[torch.Tensor]) -> None:
+        """Take over a prefilled cache: per layer keys/values [B, Hkv, S, d] (rotary already applied to the keys)."""
+        S = keys[0].shape[2]
+        for l in range(self.L):
+            self.k_cache[l][:, :, :S] = keys[l]
+            self.v_cache[l][:, :, :S] = values[l]
+            self.hash[l].encode_keys(self.k_cache[l][:, :, :S], pos0=0)
+            self.hash[l].n_cached = S
+        self.seq_len = S
+
+    # ------------------------------------------------------------------ one decode step
+    def _rope_table(self, pos: int):
+        """cos/sin [d] of absolute position `pos` (fp32 angles, cast to the model dtype as transformers' Llama does)."""
+        ang = pos * self.inv_freq
+        return torch.cat([ang.cos(), ang.cos()]).to(self.dtype), torch.cat([ang.sin(), ang.sin()]).to(self.dtype)
+
+    def _rope(self, x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+        """Rotate-half RoPE of x [B, heads, d]."""
+        half = self.d // 2
+        rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+        return x * cos + rot * sin
+
+    def decode_step(self, tokens: torch.Tensor, advance: bool = True, dense: bool = False) -> torch.Tensor:
+        """tokens [B] int64 -> logits [B, vocab].  The new token sits at position `seq_len`; with advance=False the
+        step can be replayed (HIP graph) at a fixed context length.  dense=True attends to the whole cache with the
+        dense flash-decode kernel instead (the baseline the sparse step is compared with)."""
+        B, H, Hkv, d = self.B, self.H, self.Hkv, self.d
+        pos = self.seq_len
+        S = pos + 1
+        x = self.embed[tokens]                                            # [B, hidden]
+        cos, sin = self._rope_table(pos)
+        for l, p in enumerate(self.layers):
+            h = F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps)
+            qkv = F.linear(h, p["wqkv"])
+            q = self._rope(qkv[:, :H * d].view(B, H, d), cos, sin)
+            k = self._rope(qkv[:, H * d:(H + Hkv) * d].view(B, Hkv, d), cos, sin)
+            v = qkv[:, (H + Hkv) * d:].view(B, Hkv, d)
+            self.k_cache[l][:, :, pos] = k
+            self.v_cache[l][:, :, pos] = v
+            hl = self.hash[l]
+            if dense:
+                _ops.dense_decode(q, self.k_cache[l], self.v_cache[l], S, None, hl.sm_scale, self.attn_out, self.ws_dense)
+            else:
+                hl.n_cached = pos
+                hl.step(q.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
+            x = x + F.linear(self.attn_out.view(B, H * d), p["wo"])
+            h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
+            gu = F.linear(h, p["w13"])
+            x = x + F.linear(F.silu(gu[:, :self.ffn]) * gu[:, self.ffn:], p["w2"])
+        if advance:
+            self.seq_len = S
+        x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)
+        return F.linear(x, self.lm_head)
+
+    # ------------------------------------------------------------------ weights from a transformers Llama
+    def load_hf_llama(self, model) -> None:
+        """Copy the weights of a `transformers` LlamaForCausalLM of the same shape (used by the plumbing test)."""
+        sd = model.state_dict()
+        cast = lambda t: t.detach().to(self.device, self.dtype)
+        self.embed = cast(sd["model.embed_tokens.weight"])
+        self.lm_head = cast(sd["lm_head.weight"])
+        self.final_norm = cast(sd["model.norm.weight"])
+        # the model's own rotary frequencies: a buffer, so a dtype round trip of the model (`.bfloat16().float()`) has
+        # rounded them, and the cache it filled was rotated with the rounded values
+        self.inv_freq = model.model.rotary_emb.inv_freq.detach().to(self.device, torch.float32)
+        for l, p in enumerate(self.layers):
+            pre = f"model.layers.{l}."
+            p["attn_norm"] = cast(sd[pre + "input_layernorm.weight"])
+            p["ffn_norm"] = cast(sd[pre + "post_attention_layernorm.weight"])
+            p["wqkv"] = torch.cat([cast(sd[pre + f"self_attn.{n}_proj.weight"]) for n in "qkv"], dim=0)
+            p["wo"] = cast(sd[pre + "self_attn.o_proj.weight"])
+            p["w13"] = torch.cat([cast(sd[pre + "mlp.gate_proj.weight"]), cast(sd[pre + "mlp.up_proj.weight"])], dim=0)
+            p["w2"] = cast(sd[pre + "mlp.down_proj.weight"])

@@ -67,6 +67,10 @@ def load_library() -> C.CDLL:
     lib.ha_select.restype = i32
     lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, i32,
                               vp, i64, vp, vp, sz, vp]
+    lib.ha_rope_append.restype = i32
+    lib.ha_rope_append.argtypes = [vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]
+    lib.ha_swiglu.restype = i32
+    lib.ha_swiglu.argtypes = [vp, i64, i32, i32, i32, vp, vp]
     lib.ha_sparse_decode_workspace_bytes.restype = sz
     lib.ha_sparse_decode_workspace_bytes.argtypes = [i32, i32, i64]
     lib.ha_sparse_decode.restype = i32
@@ -290,3 +294,26 @@ def dense_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, max_seq_len:
     assert out.is_contiguous() and out.dtype == q.dtype
     _check(lib.ha_dense_decode(*_kv_args(q, k, v), B, H, k.shape[1], max_seq_len, _ptr(seq_lens), float(sm_scale),
                                _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_dense_decode")
+
+
+# ------------------------------------------------------------------------------------------ decoder plumbing
+def rope_append(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, pos: int, inv_freq: torch.Tensor, q_out: torch.Tensor,
+                k_cache: torch.Tensor, v_cache: torch.Tensor, pos_dev: Optional[torch.Tensor] = None) -> None:
+    """qkv [B, (H + 2 Hkv) * 128] of one new token per sequence -> rotated q into q_out [B, H, 128], rotated k and v into
+    the caches [B, Hkv, S_cap, 128] at position pos (or pos_dev[b])."""
+    _require_cuda(qkv, inv_freq, q_out, k_cache, v_cache, pos_dev)
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and q_out.is_contiguous() and q_out.dtype == qkv.dtype == k_cache.dtype == v_cache.dtype
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == 64 and inv_freq.is_contiguous()
+    assert k_cache.stride() == v_cache.stride() and k_cache.stride(3) == 1
+    B = qkv.shape[0]
+    _check(load_library().ha_rope_append(_ptr(qkv), qkv.stride(0), _DTYPE[qkv.dtype], B, n_q_heads, n_kv_heads, int(pos), _ptr(pos_dev),
+                                         _ptr(inv_freq), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
+                                         k_cache.stride(1), k_cache.stride(2), k_cache.shape[2], _stream(qkv)), "ha_rope_append")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """gate_up [B, 2F] (gate | up) -> out [B, F] = silu(gate) * up."""
+    _require_cuda(gate_up, out)
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and out.is_contiguous() and out.dtype == gate_up.dtype
+    B, F = out.shape
+    _check(load_library().ha_swiglu(_ptr(gate_up), gate_up.stride(0), _DTYPE[gate_up.dtype], B, F, _ptr(out), _stream(gate_up)), "ha_swiglu")

@@ -3,8 +3,9 @@
 The reference measures end-to-end decode throughput with a gpt-fast fork (efficiency/generate.py:386-434,
 efficiency/model.py:98-345: RMSNorm, rotary embedding, SwiGLU feed-forward, static KV cache).  That fork is not
 runnable as shipped and drives Double-Sparsity labels, not hashes; this module is the same decoder shape with
-the HashAttention step in every layer.  Everything outside attention is plain library work (rocBLAS GEMMs,
-`F.rms_norm`, elementwise ops): the point is to time the whole step, and to check the plumbing around the op
+the HashAttention step in every layer.  Outside attention the GEMMs and RMSNorm are library calls (hipBLASLt,
+`F.rms_norm`); RoPE + cache append and SwiGLU are one launch each (`ha_rope_append`, `ha_swiglu`) and the residual adds
+ride in the GEMMs: the point is to time the whole step, and to check the plumbing around the op
 (rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
 
 Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no
@@ -81,6 +82,8 @@ class LlamaShapedDecoder:
             hl.allocate(B, S_cap)
             self.hash.append(hl)
         self.attn_out = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
+        self.q_rot = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
+        self.ffn_act = torch.empty(B, self.ffn, dtype=self.dtype, device=self.device)
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
@@ -114,44 +117,31 @@ class LlamaShapedDecoder:
         self.seq_len = S
 
     # ------------------------------------------------------------------ one decode step
-    def _rope_table(self, pos: int):
-        """cos/sin [d] of absolute position `pos` (fp32 angles, cast to the model dtype as transformers' Llama does)."""
-        ang = pos * self.inv_freq
-        return torch.cat([ang.cos(), ang.cos()]).to(self.dtype), torch.cat([ang.sin(), ang.sin()]).to(self.dtype)
-
-    def _rope(self, x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-        """Rotate-half RoPE of x [B, heads, d]."""
-        half = self.d // 2
-        rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
-        return x * cos + rot * sin
-
     def decode_step(self, tokens: torch.Tensor, advance: bool = True, dense: bool = False) -> torch.Tensor:
         """tokens [B] int64 -> logits [B, vocab].  The new token sits at position `seq_len`; with advance=False the
         step can be replayed (HIP graph) at a fixed context length.  dense=True attends to the whole cache with the
-        dense flash-decode kernel instead (the baseline the sparse step is compared with)."""
+        dense flash-decode kernel instead (the baseline the sparse step is compared with).
+
+        Per layer: RMSNorm, QKV GEMM, ha_rope_append, the attention step, output GEMM with the residual folded in
+        (addmm), RMSNorm, gate/up GEMM, ha_swiglu, down GEMM with the residual folded in."""
         B, H, Hkv, d = self.B, self.H, self.Hkv, self.d
         pos = self.seq_len
         S = pos + 1
         x = self.embed[tokens]                                            # [B, hidden]
-        cos, sin = self._rope_table(pos)
         for l, p in enumerate(self.layers):
             h = F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps)
             qkv = F.linear(h, p["wqkv"])
-            q = self._rope(qkv[:, :H * d].view(B, H, d), cos, sin)
-            k = self._rope(qkv[:, H * d:(H + Hkv) * d].view(B, Hkv, d), cos, sin)
-            v = qkv[:, (H + Hkv) * d:].view(B, Hkv, d)
-            self.k_cache[l][:, :, pos] = k
-            self.v_cache[l][:, :, pos] = v
+            _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
             hl = self.hash[l]
             if dense:
-                _ops.dense_decode(q, self.k_cache[l], self.v_cache[l], S, None, hl.sm_scale, self.attn_out, self.ws_dense)
+                _ops.dense_decode(self.q_rot, self.k_cache[l], self.v_cache[l], S, None, hl.sm_scale, self.attn_out, self.ws_dense)
             else:
                 hl.n_cached = pos
-                hl.step(q.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
-            x = x + F.linear(self.attn_out.view(B, H * d), p["wo"])
+                hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
+            x = torch.addmm(x, self.attn_out.view(B, H * d), p["wo"].t())
             h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
-            gu = F.linear(h, p["w13"])
-            x = x + F.linear(F.silu(gu[:, :self.ffn]) * gu[:, self.ffn:], p["w2"])
+            _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
+            x = torch.addmm(x, self.ffn_act, p["w2"].t())
         if advance:
             self.seq_len = S
         x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)

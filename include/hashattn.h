@@ -207,6 +207,23 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
                     int B, int H, int Hkv, int max_seq_len, const int32_t *seq_lens,
                     float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * The two elementwise steps of a decoder layer next to the attention step, for a decode loop that wants them as
+ * one launch each (the reference's end-to-end harness leaves them to torch.compile: efficiency/model.py:236-250
+ * QKV split, rotary embedding and cache update, :88-96 KVCache.update, :304-305 FeedForward).
+ *
+ * ha_rope_append: qkv [B, >= (H + 2 Hkv) * 128] holds one new token per sequence, heads in the order q | k | v.
+ * q and k are rotated in the rotate-half convention (pairs (i, i + 64), transformers' apply_rotary_pos_emb; not
+ * the interleaved pairs of efficiency/model.py:333-345) by the angle pos * inv_freq[i], the cos/sin table rounded
+ * to `dtype` as transformers does; q goes to q_out [B, H, 128], k and v into the caches at token position `pos`
+ * (or pos_dev[b] when pos_dev is not NULL; the caller guarantees pos_dev[b] < cache_len).  Cache strides in elements.
+ * ha_swiglu: out[b, i] = silu(gate_up[b, i]) * gate_up[b, F + i], silu rounded to `dtype` before the product.
+ */
+int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int H, int Hkv, int pos, const int32_t *pos_dev,
+                   const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
+                   int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, void *stream);
+int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, int F, void *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -127,6 +127,19 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert lib.ha_encode_pack_prefill(odd, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 128, 32, p, 64, 16, 0, null, null) == HA_ERR_ALIGN
     assert lib.ha_hamming_score(p, 1024, 1024, p, 1, 4, 2, 1, 1000, null, null, null) == HA_ERR_NULL
 
+    # decoder plumbing
+    def rope(**kw):
+        a = dict(qkv=p, sb=768, dt=_ops.HA_BF16, B=1, H=4, Hkv=1, pos=5, pd=null, f=p, q=p, k=p, v=p, ksb=12800, ksh=12800, kss=128,
+                 cl=100, st=null)
+        a.update(kw)
+        return lib.ha_rope_append(a["qkv"], a["sb"], a["dt"], a["B"], a["H"], a["Hkv"], a["pos"], a["pd"], a["f"], a["q"], a["k"], a["v"],
+                                  a["ksb"], a["ksh"], a["kss"], a["cl"], a["st"])
+
+    assert rope(f=null) == HA_ERR_NULL and rope(dt=7) == HA_ERR_DTYPE
+    assert rope(sb=512) == HA_ERR_SHAPE and rope(pos=100) == HA_ERR_SHAPE and rope(pos=-1) == HA_ERR_SHAPE and rope(kss=64) == HA_ERR_SHAPE
+    assert lib.ha_swiglu(null, 64, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_NULL
+    assert lib.ha_swiglu(p, 63, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_SHAPE and lib.ha_swiglu(p, 64, 9, 1, 32, p, null) == HA_ERR_DTYPE
+
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="this check is about a machine without a GPU")
 def test_no_device_is_a_status_not_a_crash(lib):

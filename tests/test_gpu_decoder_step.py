@@ -57,3 +57,42 @@ def test_decoder_step_matches_converted_llama():
             print(f"step {t}: max-abs logit difference {err:.2e}", flush=True)
             assert err < 2e-3, err
     assert dec.seq_len == S0 + steps
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_rope_append_and_swiglu_against_torch(dtype):
+    # the two plumbing kernels alone, against transformers' rotate-half formula and F.silu, host position and per-sequence positions
+    print(f"\n[case] rope_append / swiglu {dtype}", flush=True)
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    from hashattention import _ops
+    g = torch.Generator(device=DEV).manual_seed(5)
+    B, H, Hkv, d, cap = 3, 8, 2, 128, 40
+    qkv_full = torch.randn(B, (H + 2 * Hkv) * d + 64, generator=g, device=DEV).to(dtype)     # a row stride wider than the payload
+    qkv = qkv_full[:, :(H + 2 * Hkv) * d]
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    for pos_dev in (None, torch.tensor([7, 0, 39], dtype=torch.int32, device=DEV)):
+        k_cache = torch.zeros(B, Hkv, cap, d, dtype=dtype, device=DEV)
+        v_cache = torch.zeros_like(k_cache)
+        q_out = torch.empty(B, H, d, dtype=dtype, device=DEV)
+        _ops.rope_append(qkv, H, Hkv, 11, inv_freq, q_out, k_cache, v_cache, pos_dev)
+        pos = pos_dev.long() if pos_dev is not None else torch.full((B,), 11, device=DEV)
+        ang = pos[:, None].float() * inv_freq[None, :]
+        cos, sin = torch.cat([ang.cos(), ang.cos()], -1).to(dtype), torch.cat([ang.sin(), ang.sin()], -1).to(dtype)
+        q = qkv[:, :H * d].view(B, H, 1, d).float()
+        k = qkv[:, H * d:(H + Hkv) * d].view(B, Hkv, 1, d).float()
+        qr, kr = apply_rotary_pos_emb(q, k, cos.float()[:, None, :], sin.float()[:, None, :])       # [B, 1, d] tables, fp32 math
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        assert (q_out.float() - qr[:, :, 0]).abs().max().item() <= tol
+        want_k = torch.zeros_like(k_cache, dtype=torch.float32)
+        want_v = torch.zeros_like(want_k)
+        for b in range(B):
+            want_k[b, :, pos[b]] = kr[b, :, 0]
+            want_v[b, :, pos[b]] = qkv[b, (H + Hkv) * d:].view(Hkv, d).float()
+        assert (k_cache.float() - want_k).abs().max().item() <= tol           # also: nothing written at any other position
+        assert torch.equal(v_cache.float(), want_v)
+    F_ = 1000
+    gu = torch.randn(B, 2 * F_, generator=g, device=DEV).to(dtype)
+    out = torch.empty(B, F_, dtype=dtype, device=DEV)
+    _ops.swiglu(gu, out)
+    want = torch.nn.functional.silu(gu[:, :F_]) * gu[:, F_:]
+    assert (out.float() - want.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 2e-2)

@@ -51,10 +51,23 @@ template <int NL_, int DIN_, int DINT_, int DOUT_>
 __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs a) {
     __shared__ __align__(16) float s_act[2][kRows][kMaxDim];
     __shared__ float s_part[kSeg][kRows][kMaxDim];
-    const bool second = (int)blockIdx.y >= a.side[0].n_heads;
+    // Workgroups go to the 8 XCDs round-robin in linear launch order.  When the grid divides evenly, renumber them so
+    // that each XCD owns whole heads: the tiles of a head then share one L2 and its weights leave HBM once, not once
+    // per tile.
+    int bx = blockIdx.x, by = blockIdx.y;
+    {
+        const int n = gridDim.x * gridDim.y;
+        if (n % 8 == 0 && gridDim.x > 1) {
+            const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+            const int v = (lin % 8) * (n / 8) + lin / 8;
+            bx = v % gridDim.x;
+            by = v / gridDim.x;
+        }
+    }
+    const bool second = by >= a.side[0].n_heads;
     const EncSide &sd = a.side[second ? 1 : 0];
-    const int head = second ? blockIdx.y - a.side[0].n_heads : blockIdx.y;
-    const int tile = blockIdx.x, tid = threadIdx.x;
+    const int head = second ? by - a.side[0].n_heads : by;
+    const int tile = bx, tid = threadIdx.x;
     const void *__restrict__ x = sd.x;
     const int x_dtype = sd.x_dtype;
     const int64_t x_sb = sd.x_sb, x_sh = sd.x_sh, x_st = sd.x_st;

@@ -84,7 +84,7 @@ def cpu_baseline(w, torch, budget_s=12.0):
                       f"{torch.get_num_threads()} torch threads), {sum(times):.2f} s measured, scaled x{scale:.2f} by cached tokens"}
 
 
-def traffic_probe(torch, layer, q3, k, v, out):
+def traffic_probe(torch, layer, q3, k, v, out, fused_attend=None):
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain copy of known size, then the gather-attend
     kernel, three launches each.  The copy gives the scale of the counter (bytes per reported KiB)."""
     n = 1 << 30
@@ -97,7 +97,9 @@ def traffic_probe(torch, layer, q3, k, v, out):
     from hashattention import _ops
     w = layer
     for _ in range(3):
-        if layer.overlap_windows:
+        if fused_attend is not None:
+            fused_attend()
+        elif layer.overlap_windows:
             _ops.sparse_decode_heavy(q3, k, v, w.idx, w.counts, w.sm_scale, out, w.ws_attend, w.win, w.init_budget,
                                      w.recent_budget, k.shape[2], None)
         else:
@@ -180,7 +182,7 @@ def decoder_bench(args, torch):
         "prefill_encode_tflops": 2 * B * dec.Hc * (S - 1) * (128 * 128 * 2 + 128 * 32) / (ms_prefill_encode * 1e-3) / 1e12,
         "cache_fill_seconds": fill_s,
         "hbm_gbps_step": step_bytes / (ms_step * 1e-3) / 1e9, "hbm_frac_step": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
+        "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
     }
@@ -196,6 +198,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
+    ap.add_argument("--two-launch", action="store_true", help="ha_select + ha_sparse_decode instead of the fused select-attend path")
     ap.add_argument("--overlap-windows", action="store_true", help="attend to sink|recent on a second stream (ha_window_partial)")
     ap.add_argument("--layers", type=int, default=32, help="decoder layers of the config3 whole-step workload")
     ap.add_argument("--layer-only", action="store_true", help="config3: time one attention layer-step instead of the whole decoder")
@@ -230,6 +233,8 @@ def main():
     layer.allocate(B, S)
     layer.select_algo = args.select_algo
     layer.overlap_windows = args.overlap_windows
+    layer.use_fused = not args.two_launch
+    fused = layer.use_fused and layer.fused_ok and not layer.overlap_windows
     # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
     layer.encode_keys(p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
     torch.cuda.synchronize()
@@ -252,7 +257,8 @@ def main():
 
     if args.traffic_probe:
         step()
-        traffic_probe(torch, layer, q3, p.k, p.v, out)
+        traffic_probe(torch, layer, q3, p.k, p.v, out,
+                      (lambda: layer.attend_fused(q3, p.k, p.v, out, S, seq_lens)) if fused else None)
         return
     ms_step_eager = time_gpu(step, args.steps, args.warmup, torch)
     # the same launch sequence captured once in a HIP graph and replayed: the step as a serving loop runs it
@@ -278,12 +284,20 @@ def main():
                                                               seq_lens), args.steps, args.warmup, torch)
         ms_window = time_gpu(lambda: _ops.window_partial(q3, p.k, p.v, S, seq_lens, w.init_budget, w.recent_budget,
                                                          layer.sm_scale, layer.win), args.steps, args.warmup, torch)
+    elif fused:    # the step's dominant launch: list rebuilt from the codes in LDS + gather-attend (thresholds already in the workspace)
+        layer.select(S, seq_lens)              # leaves the same thresholds as select_prepare, plus the lists for the comparison below
+        ms_attend_lists = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
+        ms_prepare = time_gpu(lambda: layer.select_prepare(S, seq_lens), args.steps, args.warmup, torch)
+        ms_attend = time_gpu(lambda: layer.attend_fused(q3, p.k, p.v, out, S, seq_lens), args.steps, args.warmup, torch)
+        ms_window = 0.0
     else:
         ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
         ms_window = 0.0
     ms_dense = time_gpu(lambda: _ops.dense_decode(q3, p.k, p.v, S, seq_lens, layer.sm_scale, out_dense, ws_dense),
                         max(10, args.steps // 4), max(2, args.warmup // 4), torch)
 
+    if fused:
+        layer.select(S, seq_lens)
     n_sel_rows = int(layer.counts.sum().item())
     ab = algorithmic_bytes(w, n_sel_rows)
     eb = 2 if w.dtype != torch.float32 else 4
@@ -315,16 +329,20 @@ def main():
                                f"H={H} Hkv={Hkv} d={d} code_heads={w.n_code_heads} code_bits={w.lth_final_dim} "
                                f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} "
                                f"n_sel={n_sel_rows // (B * H)}"},
-        "stages_us": {"encode_new_k_and_q": ms_encode * 1e3, "score_select": ms_select * 1e3,
-                      "gather_attend": ms_attend * 1e3, "window_partial_second_stream": ms_window * 1e3,
-                      "dense_flash_decode": ms_dense * 1e3},
+        "path": "ha_encode_step + ha_select_prepare + ha_sparse_decode_fused" if fused else
+                "ha_encode_step + ha_select + " + ("ha_window_partial + ha_sparse_decode_heavy" if layer.overlap_windows else "ha_sparse_decode"),
+        "stages_us": {"encode_new_k_and_q": ms_encode * 1e3,
+                      **({"select_prepare": ms_prepare * 1e3, "select_attend_fused": ms_attend * 1e3,
+                          "two_launch_select": ms_select * 1e3, "two_launch_attend": ms_attend_lists * 1e3} if fused else
+                         {"score_select": ms_select * 1e3, "gather_attend": ms_attend * 1e3}),
+                      "window_partial_second_stream": ms_window * 1e3, "dense_flash_decode": ms_dense * 1e3},
         "hbm_gbps_step": sparse_bytes / (ms_step * 1e-3) / 1e9,
         "hbm_frac_step": sparse_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "speedup_vs_dense": ms_dense / ms_step,
         "dense_hbm_gbps": ab["dense"] / (ms_dense * 1e-3) / 1e9,
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
-        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm",
+        "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm",
                      "achieved": attend_bytes / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": attend_bytes / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get(w.name),

@@ -10,7 +10,7 @@
 // flight while step i is reduced, so a wave always has 8 x 1 KiB of row data outstanding.
 #include <stdlib.h>
 
-#include "ha_common.h"
+#include "ha_select_common.h"
 
 namespace {
 
@@ -100,9 +100,164 @@ __device__ __forceinline__ void merge_streams(const float *s_m, const float *s_l
 }
 
 // ------------------------------------------------------------------------------------------------
+// Selection fused into the attend kernel (FW = code words, 0 = the list comes from memory).  After
+// ha_select_prepare the workspace holds, per row, the threshold T, the number r of ties taken and n_heavy, and per
+// (row, chunk) how many tokens with d < T / d == T precede the chunk.  That is all a workgroup needs to rebuild its
+// part of the ordered index list in LDS straight from the codes - the list never goes through memory, and the
+// compaction launch disappears.  A workgroup owns `cps` consecutive chunks (all of them when rows are not split);
+// the first also takes the sink window, the last the recent window.
+constexpr int kFusedListCap = 8192;  // entries of the LDS list (32 KiB)
+struct FusedSel {
+    const uint32_t *kcodes;
+    int64_t kc_sb, kc_sh;
+    const uint32_t *qcodes;
+    const int32_t *meta, *chunk_pre;
+    int nchunk, chunk, cps, gq, init, recent, vec;
+};
+
+// NSLAB slabs of 256 codes of one chunk, all requested before the first is used: the selected ones go to their list
+// positions.  n_lt / n_eq: tokens with d < T / d == T before the first slab (row-wide), updated.
+template <int W, int NSLAB>
+__device__ __forceinline__ void scan_slabs(const uint32_t *kc, const ha_sel::Code<W> &q, int j_first, int beg, int end, bool whole, int T,
+                                           int r, int lo, int p0, int n, int lane, int &n_lt, int &n_eq, int32_t *s_list) {
+    using namespace ha_sel;
+    Code<W> k[NSLAB][4];
+#pragma unroll
+    for (int s = 0; s < NSLAB; ++s) load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
+#pragma unroll
+    for (int s = 0; s < NSLAB; ++s) {
+        const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
+        uint32_t lt4 = 0, eq4 = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int d = k[s][e].dist(q);
+            const bool in = whole || (j0 + e >= beg && j0 + e < end);
+            lt4 |= (in && d < T) ? (1u << e) : 0u;
+            eq4 |= (in && d == T) ? (1u << e) : 0u;
+        }
+        const uint32_t cnt = (uint32_t)__popc(lt4) | ((uint32_t)__popc(eq4) << 16);
+        const uint32_t incl = wave_inclusive_scan(cnt);
+        const uint32_t excl = incl - cnt;
+        int a = n_lt + (int)(excl & 0xFFFFu), t = n_eq + (int)(excl >> 16);
+        const uint32_t em = t < r ? eq4 : 0u;  // past the r-th tie nothing more of the tie bucket is taken
+        uint32_t todo = lt4 | em;
+        while (todo) {
+            const int e = __ffs((int)todo) - 1;
+            todo &= todo - 1;
+            const bool is_eq = (em >> e) & 1u;
+            if (!is_eq || t < r) {
+                const int pos = lo + a + min(t, r) - p0;
+                if (pos >= 0 && pos < n) s_list[pos] = j0 + e;
+            }
+            a += is_eq ? 0 : 1;
+            t += is_eq ? 1 : 0;
+        }
+        const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
+        n_lt += (int)(tot & 0xFFFFu);
+        n_eq += (int)(tot >> 16);
+    }
+}
+
+// The same for a chunk whose ties are taken all or not at all (every chunk but the one holding the r-th tie): the
+// NSLAB * 4 codes of a lane become one bit mask and one wave scan places them, in (lane, slab, element) order inside
+// the group - the list holds the same tokens as the ordered one, in a different but fixed order.
+template <int W, int NSLAB>
+__device__ __forceinline__ void scan_slabs_unordered(const uint32_t *kc, const ha_sel::Code<W> &q, int j_first, int beg, int end, bool whole,
+                                                     int T, bool take_ties, int base, int n, int lane, int &n_sel, int32_t *s_list) {
+    using namespace ha_sel;
+    Code<W> k[NSLAB][4];
+#pragma unroll
+    for (int s = 0; s < NSLAB; ++s) load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
+    // sign bit of (d - T') is "d < T'"; T' = T + 1 when ties count.  Last code first so that code (s, e) lands on bit 4 s + e.
+    const int neg_t = -(T + (take_ties ? 1 : 0));
+    uint32_t m = 0;
+#pragma unroll
+    for (int s = NSLAB - 1; s >= 0; --s)
+#pragma unroll
+        for (int e = 3; e >= 0; --e) m = __builtin_amdgcn_alignbit(m, (uint32_t)(k[s][e].dist(q) + neg_t), 31);
+    if (!whole) {
+        uint32_t valid = 0;
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) {
+            const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) valid |= (j0 + e >= beg && j0 + e < end) ? (1u << (4 * s + e)) : 0u;
+        }
+        m &= valid;
+    }
+    const uint32_t cnt = (uint32_t)__popc(m);
+    const uint32_t incl = wave_inclusive_scan(cnt);
+    int pos = base + n_sel + (int)(incl - cnt);
+    const int j_lane = j_first + lane * 4;
+    while (m) {
+        const int bit = __ffs((int)m) - 1;
+        m &= m - 1;
+        if (pos >= 0 && pos < n) s_list[pos] = j_lane + (bit >> 2) * (HA_WAVE * 4) + (bit & 3);
+        ++pos;
+    }
+    n_sel += __builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
+}
+
+// Fills s_list[0, n) with the list positions [p0, p0 + n) of row `row`; returns n.  All threads of the workgroup call it.
+template <int W, int NT>
+__device__ __forceinline__ int build_list(const FusedSel &f, int b, int h, int H, int64_t row, int S, int sp, int32_t *s_list) {
+    using namespace ha_sel;
+    constexpr int NW = NT / HA_WAVE;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lo = min(f.init, S), hi = max(S - f.recent, lo);
+    const int T = f.meta[row * 4 + 0], r = f.meta[row * 4 + 1], nheavy = f.meta[row * 4 + 2];
+    const int c0 = sp * f.cps, c1 = min(c0 + f.cps, f.nchunk);
+    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
+    const int p0 = sp == 0 ? 0 : lo + pre[c0 * 2] + min(pre[c0 * 2 + 1], r);
+    const int p1 = c1 >= f.nchunk ? lo + nheavy + (S - hi) : lo + pre[c1 * 2] + min(pre[c1 * 2 + 1], r);
+    const int n = min(max(p1 - p0, 0), kFusedListCap);
+    if (sp == 0)
+        for (int i = tid; i < lo && i < n; i += NT) s_list[i] = i;
+    if (c1 >= f.nchunk) {
+        const int base = lo + nheavy - p0;
+        for (int i = tid; i < S - hi; i += NT)
+            if (base + i < n) s_list[base + i] = hi + i;
+    }
+    if (nheavy > 0) {
+        const Code<W> q = load_qcode<W>(f.qcodes, row);
+        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+        constexpr int GS = W == 1 ? 8 : 4;  // slabs per request group: 32 VGPRs of codes in flight per lane
+        for (int c = c0 + wave; c < c1; c += NW) {  // uniform per wave
+            const int cb = c * f.chunk;
+            const int beg = max(lo, cb), end = min(hi, cb + f.chunk);
+            if (beg >= end) continue;
+            int n_lt = pre[c * 2], n_eq = pre[c * 2 + 1];
+            const bool whole = f.vec && beg == cb && end == cb + f.chunk;
+            // ties of this chunk: none taken, all taken, or (the chunk of the r-th tie, and the last chunk, whose tie
+            // count is not recorded) the first few in token order
+            const bool none = n_eq >= r;
+            const bool all = !none && c + 1 < f.nchunk && pre[(c + 1) * 2 + 1] <= r;
+            if (none || all) {
+                int n_sel = n_lt + min(n_eq, r);
+                if (f.chunk % (GS * HA_WAVE * 4) == 0) {
+                    for (int j = cb; j < cb + f.chunk; j += GS * HA_WAVE * 4)
+                        scan_slabs_unordered<W, GS>(kc, q, j, beg, end, whole, T, all, lo - p0, n, lane, n_sel, s_list);
+                } else {
+                    for (int j = cb; j < cb + f.chunk; j += 4 * HA_WAVE * 4)
+                        scan_slabs_unordered<W, 4>(kc, q, j, beg, end, whole, T, all, lo - p0, n, lane, n_sel, s_list);
+                }
+            } else if (f.chunk % (GS * HA_WAVE * 4) == 0) {
+                for (int j = cb; j < cb + f.chunk; j += GS * HA_WAVE * 4)
+                    scan_slabs<W, GS>(kc, q, j, beg, end, whole, T, r, lo, p0, n, lane, n_lt, n_eq, s_list);
+            } else {  // 1024-code chunks (short rows): four slabs at a time
+                for (int j = cb; j < cb + f.chunk; j += 4 * HA_WAVE * 4)
+                    scan_slabs<W, 4>(kc, q, j, beg, end, whole, T, r, lo, p0, n, lane, n_lt, n_eq, s_list);
+            }
+        }
+    }
+    __syncthreads();
+    return n;
+}
+
+// ------------------------------------------------------------------------------------------------
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
 // NT threads = NT/16 row streams; U rows per stream per step.
-template <typename E, int NT, int U>
+template <typename E, int NT, int U, int FW>
 __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
@@ -111,11 +266,12 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
                                                            int nsplit_max, float *__restrict__ part_acc,
                                                            float *__restrict__ part_ml, void *__restrict__ out,
                                                            const float *__restrict__ win_part, int win_init, int win_recent,
-                                                           const int32_t *__restrict__ seq_lens, int max_S) {
+                                                           const int32_t *__restrict__ seq_lens, int max_S, const FusedSel fsel) {
     using EL = Elem<E>;
     constexpr int NS = NT / 16;  // row streams
     __shared__ float s_m[NS], s_l[NS];
     __shared__ float s_acc[NS * HA_HEAD_DIM];
+    __shared__ int32_t s_list[FW > 0 ? kFusedListCap : 1];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
     // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
@@ -124,28 +280,43 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     const int Hkv = H / G;
     const int sp = blockIdx.x, h = ((int)blockIdx.y % Hkv) * G + (int)blockIdx.y / Hkv, b = blockIdx.z;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
-    int64_t n = counts[b * H + h];
-    if (n > idx_cap) n = idx_cap;
-    // win_part: the sink and recent windows were attended by another launch; their entries (the first
-    // min(init, S) and the last S - max(S - recent, min(init, S)) of the list) are skipped here and the
-    // partial is merged at the end
-    int skip_front = 0;
-    if (win_part) {
+    const int64_t row = (int64_t)b * H + h;
+    int r0, r1, nsplit;
+    const int32_t *ix = nullptr;
+    if constexpr (FW > 0) {
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
-        const int lo = min(win_init, S), hi = max(S - win_recent, lo);
-        skip_front = lo;
-        n = max((int64_t)0, n - lo - (S - hi));
+        nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
+        r0 = 0;
+        r1 = build_list<FW, NT>(fsel, b, h, H, row, S, sp, s_list);
+        if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output
+            if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+            return;
+        }
+    } else {
+        int64_t n = counts[b * H + h];
+        if (n > idx_cap) n = idx_cap;
+        // win_part: the sink and recent windows were attended by another launch; their entries (the first
+        // min(init, S) and the last S - max(S - recent, min(init, S)) of the list) are skipped here and the
+        // partial is merged at the end
+        int skip_front = 0;
+        if (win_part) {
+            int S = seq_lens ? seq_lens[b] : max_S;
+            if (S > max_S) S = max_S;
+            const int lo = min(win_init, S), hi = max(S - win_recent, lo);
+            skip_front = lo;
+            n = max((int64_t)0, n - lo - (S - hi));
+        }
+        nsplit = n > 0 ? (int)((n + split_rows - 1) / split_rows) : 1;
+        if (sp >= nsplit) return;
+        if (n == 0 && !win_part) {  // empty sequence: defined as a zero output
+            if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+            return;
+        }
+        r0 = skip_front + sp * split_rows;
+        r1 = (int)min((int64_t)r0 + split_rows, skip_front + n);
+        ix = idx + row * idx_cap;
     }
-    const int nsplit = n > 0 ? (int)((n + split_rows - 1) / split_rows) : 1;
-    if (sp >= nsplit) return;
-    const int64_t row = (int64_t)b * H + h;
-    if (n == 0 && !win_part) {  // empty sequence: defined as a zero output
-        if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
-        return;
-    }
-    const int r0 = skip_front + sp * split_rows, r1 = (int)min((int64_t)r0 + split_rows, skip_front + n);
-    const int32_t *ix = idx + row * idx_cap;
     const char *kb = (const char *)k + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const char *vb = (const char *)v + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;
@@ -165,7 +336,8 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     // list position of (step base, u) for this stream; positions >= r1 are padded with the split's first row
     auto list_index = [&](int base, int u) {
         const int r = base + stream + u * NS;
-        return ix[r < r1 ? r : r0];
+        if constexpr (FW > 0) return r < r1 ? s_list[r] : (r1 > 0 ? s_list[0] : 0);
+        else return ix[r < r1 ? r : r0];
     };
     int32_t j_next[U];   // indices of the step after the one in flight
     Raw8<E> kr[U], vr[U];
@@ -291,18 +463,18 @@ __global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *
     float L = 0.f, A = 0.f;
 #pragma unroll 8
     for (int s = 0; s < nsplit; ++s) {
-        const float w = fast_exp2(ml[s * 2] - M);
+        const float w = (ml[s * 2] == -INFINITY) ? 0.f : fast_exp2(ml[s * 2] - M);  // an empty split leaves (m, l) = (-inf, 0)
         L += w * ml[s * 2 + 1];
         A += w * pa[(int64_t)s * HA_HEAD_DIM];
     }
     if (win_part) {
         const float *wp = win_part + row * (HA_HEAD_DIM + 2);
         const float wm = wp[HA_HEAD_DIM], M2 = fmaxf(M, wm);
-        const float sh = fast_exp2(M - M2), sw = (wm == -INFINITY) ? 0.f : fast_exp2(wm - M2);
+        const float sh = (M == -INFINITY) ? 0.f : fast_exp2(M - M2), sw = (wm == -INFINITY) ? 0.f : fast_exp2(wm - M2);
         A = A * sh + wp[e] * sw;
         L = L * sh + wp[HA_HEAD_DIM + 1] * sw;
     }
-    EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, A / L);
+    EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, e, L > 0.f ? A / L : 0.f);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -504,9 +676,10 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
     const int G = H / Hkv;
 #define HA_SPARSE_LAUNCH(E_, NT_, U_)                                                                                             \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,           \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,        \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
-                           plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len);       \
+                           plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len,        \
+                           FusedSel{});                                                                                           \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
         if (plan.nsplit_max > 1) {                                                                                                \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
@@ -545,6 +718,102 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
     return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
                               counts, sm_scale, out, workspace, workspace_bytes, window_partial, init_budget, recent_budget, seq_lens,
                               max_seq_len, stream);
+}
+
+// chunks per workgroup of the fused path: whole rows when the rows alone fill the GPU, else enough splits for ~512 workgroups
+static int fused_chunks_per_split(int B, int H, int nchunk) {
+    const int64_t rows = (int64_t)B * H;
+    int64_t want = (512 + rows - 1) / rows;
+    if (want > nchunk) want = nchunk;
+    if (want < 1) want = 1;
+    return (int)((nchunk + want - 1) / want);
+}
+
+int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len, int init_budget, int recent_budget, double heavy_budget,
+                                   int mode) {
+    if (B <= 0 || H <= 0 || Hc <= 0 || max_seq_len <= 0 || (W != 1 && W != 2) || H % Hc != 0) return 0;
+    if (mode != HA_SELECT_SIMPLE || init_budget < 0 || recent_budget < 0 || heavy_budget < 0.0) return 0;
+    const double heavy = heavy_budget > 1.0 ? heavy_budget : (double)max_seq_len * heavy_budget;
+    return (double)init_budget + (double)recent_budget + heavy <= (double)kFusedListCap ? 1 : 0;
+}
+
+size_t ha_sparse_decode_fused_workspace_bytes(int B, int H, int Hc, int max_seq_len) {
+    if (B <= 0 || H <= 0 || Hc <= 0 || max_seq_len <= 0) return 0;
+    const ha_sel::SelectPlan plan = ha_sel::select_plan(B, Hc, max_seq_len);
+    return part_bytes((int64_t)B * H, plan.nchunk);
+}
+
+int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes, int64_t kc_stride_b,
+                           int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W, int max_seq_len,
+                           const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                           const void *select_workspace, size_t select_workspace_bytes, float sm_scale, void *out, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+    int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
+    if (st) return st;
+    HA_REQUIRE(kcodes && qcodes && select_workspace, HA_ERR_NULL_POINTER, "kcodes/qcodes/select_workspace is NULL");
+    HA_REQUIRE(Hc > 0 && H % Hc == 0 && (W == 1 || W == 2) && max_seq_len > 0, HA_ERR_BAD_SHAPE, "bad Hc, W or max_seq_len");
+    HA_REQUIRE(kc_stride_h >= (int64_t)max_seq_len * W && kc_stride_b >= kc_stride_h, HA_ERR_BAD_SHAPE,
+               "code strides smaller than the rows they span");
+    HA_REQUIRE(ha_sparse_decode_fused_applies(B, H, Hc, W, max_seq_len, init_budget, recent_budget, heavy_budget, HA_SELECT_SIMPLE),
+               HA_ERR_BAD_SHAPE, "selection larger than the %d-entry list of the fused path: use ha_select + ha_sparse_decode",
+               kFusedListCap);
+    HA_REQUIRE(select_workspace_bytes >= ha_select_workspace_bytes(B, H, Hc, W, max_seq_len), HA_ERR_WORKSPACE,
+               "select workspace smaller than ha_select_workspace_bytes");
+    const size_t need = ha_sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len);
+    HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "fused decode workspace: need %zu bytes, got %zu", need,
+               workspace ? workspace_bytes : (size_t)0);
+    HA_REQUIRE(ha_aligned(workspace, 256) && ha_aligned(select_workspace, 256) && ha_aligned(kcodes, 4 * W) && ha_aligned(qcodes, 4),
+               HA_ERR_MISALIGNED, "workspaces must be 256-byte aligned, codes aligned to their word count");
+    if ((st = ha_require_device())) return st;
+
+    const ha_sel::SelectPlan plan = ha_sel::select_plan(B, Hc, max_seq_len);
+    const ha_sel::SelectWorkspace sw = ha_sel::carve_select_ws(const_cast<void *>(select_workspace), (int64_t)B * H, plan.nchunk, W);
+    FusedSel f;
+    f.kcodes = kcodes;
+    f.kc_sb = kc_stride_b;
+    f.kc_sh = kc_stride_h;
+    f.qcodes = qcodes;
+    f.meta = sw.meta;
+    f.chunk_pre = sw.chunk_pre;
+    f.nchunk = plan.nchunk;
+    f.chunk = plan.blocks * ha_sel::kBlock;
+    f.cps = fused_chunks_per_split(B, H, plan.nchunk);
+    f.gq = H / Hc;
+    f.init = init_budget;
+    f.recent = recent_budget;
+    f.vec = ha_sel::rows_vectorisable(kcodes, kc_stride_b, kc_stride_h, W) ? 1 : 0;
+    const int nsplit = (plan.nchunk + f.cps - 1) / f.cps;
+    const int64_t rows = (int64_t)B * H;
+    float *part_acc = (float *)workspace;
+    float *part_ml = part_acc + rows * nsplit * HA_HEAD_DIM;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(nsplit, H, B), mgrid(H, B);
+    const float sl2 = sm_scale * kLog2e;
+    const int G = H / Hkv;
+#define HA_FUSED_LAUNCH(E_, U_, FW_)                                                                                              \
+    do {                                                                                                                          \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,      \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f);                                      \
+        HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
+        if (nsplit > 1) {                                                                                                         \
+            hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \
+                               (int64_t)nsplit, H, 1, nsplit, out, nullptr, 0, 0, nullptr, 0);                                    \
+            HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
+        }                                                                                                                         \
+    } while (0)
+    if (W == 1) {
+        if (kv_dtype == HA_BF16) HA_FUSED_LAUNCH(ElemBF16, 4, 1);
+        else if (kv_dtype == HA_F16) HA_FUSED_LAUNCH(ElemF16, 4, 1);
+        else HA_FUSED_LAUNCH(ElemF32, 2, 1);
+    } else {
+        if (kv_dtype == HA_BF16) HA_FUSED_LAUNCH(ElemBF16, 4, 2);
+        else if (kv_dtype == HA_F16) HA_FUSED_LAUNCH(ElemF16, 4, 2);
+        else HA_FUSED_LAUNCH(ElemF32, 2, 2);
+    }
+#undef HA_FUSED_LAUNCH
+    return HA_OK;
 }
 
 size_t ha_window_partial_bytes(int B, int H) {

@@ -176,10 +176,12 @@ __global__ __launch_bounds__(kSelThreads) void select_threshold_kernel(const uin
     int32_t *o = out_idx + row * idx_cap;
     const int n_recent = rb.S - rb.hi;
     const int64_t rbase = (int64_t)rb.lo + nheavy;
-    for (int i = tid; i < rb.lo; i += kSelThreads)
-        if (i < idx_cap) o[i] = i;
-    for (int i = tid; i < n_recent; i += kSelThreads)
-        if (rbase + i < idx_cap) o[rbase + i] = rb.hi + i;
+    if (out_idx) {
+        for (int i = tid; i < rb.lo; i += kSelThreads)
+            if (i < idx_cap) o[i] = i;
+        for (int i = tid; i < n_recent; i += kSelThreads)
+            if (rbase + i < idx_cap) o[rbase + i] = rb.hi + i;
+    }
     if (tid == 0) out_counts[row] = (int32_t)(rbase + n_recent);
 }
 
@@ -322,29 +324,6 @@ int validate_codes(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, const u
     return HA_OK;
 }
 
-struct SelectWorkspace {
-    uint32_t *hist;
-    int32_t *meta, *chunk_pre;
-    size_t bytes;
-};
-SelectWorkspace carve_select_ws(void *base, int64_t rows, int nchunk, int W) {
-    SelectWorkspace w;
-    size_t off = 0;
-    auto take = [&](size_t n) {
-        size_t o = off;
-        off += (n + 255) / 256 * 256;
-        return o;
-    };
-    const size_t o_hist = take((size_t)rows * nchunk * (32 * W + 1) * 4);
-    const size_t o_meta = take((size_t)rows * 4 * 4);
-    const size_t o_pre = take((size_t)rows * nchunk * 2 * 4);
-    w.hist = (uint32_t *)((char *)base + o_hist);
-    w.meta = (int32_t *)((char *)base + o_meta);
-    w.chunk_pre = (int32_t *)((char *)base + o_pre);
-    w.bytes = off;
-    return w;
-}
-
 }  // namespace
 
 extern "C" {
@@ -384,19 +363,20 @@ size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
                            init_budget, recent_budget, heavy_budget, mode, depth, plan.nchunk, ws.meta, ws.chunk_pre, out_idx,    \
                            idx_cap, out_counts);                                                                                  \
         HA_CHECK_LAUNCH("select_threshold_kernel");                                                                               \
+        if (!out_idx) break; /* ha_select_prepare: thresholds and offsets only */                                                 \
         hipLaunchKernelGGL((select_compact_kernel<W_, GQ_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,     \
                            qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.meta,  \
                            ws.chunk_pre, out_idx, idx_cap);                                                                       \
         HA_CHECK_LAUNCH("select_compact_kernel");                                                                                 \
     } while (0)
 
-int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc, int W,
-              int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget, int mode,
-              int depth, int algo, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
-              size_t workspace_bytes, void *stream) {
+static int select_impl(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
+                       int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                       int mode, int depth, int algo, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
+                       size_t workspace_bytes, void *stream, bool prepare_only) {
     int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len);
     if (st) return st;
-    HA_REQUIRE(out_idx && out_counts, HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
+    HA_REQUIRE((prepare_only || out_idx) && out_counts, HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
     HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && heavy_budget >= 0.0 && depth >= 0, HA_ERR_BAD_SHAPE,
                "budgets and depth must be non-negative");
     HA_REQUIRE(heavy_budget < 2147483647.0, HA_ERR_BAD_SHAPE, "heavy_budget too large");
@@ -409,6 +389,7 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
     HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "select workspace must be 256-byte aligned");
     if ((st = ha_require_device())) return st;
 
+    if (prepare_only) algo = HA_SELECT_ALGO_HISTOGRAM;
     if (algo == HA_SELECT_ALGO_AUTO) {
         // Measured on MI355X (16 x 64K-token rows, 1/32 kept): histogram 33.7 us, sampled 36.9 us.  Both are
         // bound by per-launch latency chains at these sizes, so the simpler method is the default.
@@ -436,6 +417,22 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
         else HA_SELECT_LAUNCH(2, 8, 16);
     }
     return HA_OK;
+}
+
+int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc, int W,
+              int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget, int mode,
+              int depth, int algo, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
+              size_t workspace_bytes, void *stream) {
+    return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
+                       heavy_budget, mode, depth, algo, out_idx, idx_cap, out_counts, workspace, workspace_bytes, stream, false);
+}
+
+int ha_select_prepare(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
+                      int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                      int mode, int depth, int32_t *out_counts, void *workspace, size_t workspace_bytes, void *stream) {
+    return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
+                       heavy_budget, mode, depth, HA_SELECT_ALGO_HISTOGRAM, nullptr, 1, out_counts, workspace, workspace_bytes, stream,
+                       true);
 }
 
 }  // extern "C"

@@ -171,6 +171,32 @@ inline bool rows_vectorisable(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_
 }
 
 
+// workspace of the histogram selection: per-chunk histograms, row meta {T, r, n_heavy, 0}, per-chunk prefixes
+// {#d < T before the chunk, #d == T before the chunk}
+struct SelectWorkspace {
+    uint32_t *hist;
+    int32_t *meta, *chunk_pre;
+    size_t bytes;
+};
+inline SelectWorkspace carve_select_ws(void *base, int64_t rows, int nchunk, int W) {
+    SelectWorkspace w;
+    size_t off = 0;
+    auto take = [&](size_t n) {
+        size_t o = off;
+        off += (n + 255) / 256 * 256;
+        return o;
+    };
+    const size_t o_hist = take((size_t)rows * nchunk * (32 * W + 1) * 4);
+    const size_t o_meta = take((size_t)rows * 4 * 4);
+    const size_t o_pre = take((size_t)rows * nchunk * 2 * 4);
+    w.hist = (uint32_t *)((char *)base + o_hist);
+    w.meta = (int32_t *)((char *)base + o_meta);
+    w.chunk_pre = (int32_t *)((char *)base + o_pre);
+    w.bytes = off;
+    return w;
+}
+
+
 // workspace of the sampled-threshold selection: T_hi per row, candidate count per (row, chunk), candidate segments
 struct SampledWorkspace {
     int32_t *thi, *cand_cnt, *cand;

@@ -6,9 +6,11 @@ key codes, plus the index lists and workspaces of the kernels.  One decode step 
 
     windows  attention over sink | recent, second stream    (ha_window_partial, overlaps the next two)
     encode   code of the new key -> bit-cache, query codes  (ha_encode_step, one launch)
-    select   Hamming histogram + ordered compaction         (ha_select)
-    attend   gather-only attention over the heavy tokens,   (ha_sparse_decode_heavy; ha_sparse_decode when
-             merged with the window partial                   overlap_windows is off)
+    select   Hamming histogram + threshold per row          (ha_select_prepare)
+    attend   index list rebuilt in LDS from the codes,      (ha_sparse_decode_fused)
+             gather-only attention over it
+or, for threshold mode and lists above 8192 entries, ha_select (histogram, threshold, ordered compaction into
+memory) + ha_sparse_decode (ha_sparse_decode_heavy merged with the window partial when overlap_windows is on).
 
 All buffers are allocated once per (batch, capacity) and reused: the step itself allocates nothing.
 """
@@ -42,6 +44,9 @@ class HashDecodeLayer:
         # attend to sink | recent on a second stream while the selection runs.  Off by default: at 64K-token rows the
         # windows are already served from L2 to the heads of a group and the fork/join costs more than it hides.
         self.overlap_windows = False
+        # rebuild the index list in LDS inside the attend launch instead of writing it to memory (simple mode, lists of
+        # up to 8192 entries; decided per allocation)
+        self.use_fused = True
         self.device = torch.device(device)
         self.wk = _ops.pack_usa_weights(k_layers, self.device)
         self.wq = _ops.pack_usa_weights(q_layers, self.device)
@@ -73,6 +78,9 @@ class HashDecodeLayer:
         self.counts = torch.zeros(B, self.H, dtype=torch.int32, device=dev)
         self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
         self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
+        self.fused_ok = _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget, self.recent_budget,
+                                           self.heavy_budget, self.mode)
+        self.ws_fused = _ops.workspace(_ops.sparse_decode_fused_workspace_bytes(B, self.H, self.Hc, S_cap), dev)
         self.win = torch.empty(B, self.H, 130, dtype=torch.float32, device=dev)
         self.side_stream = torch.cuda.Stream(device=dev)
         self.n_cached = 0
@@ -99,6 +107,16 @@ class HashDecodeLayer:
         _ops.select(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
                     self.recent_budget, self.heavy_budget, self.idx, self.counts, self.ws_select, self.mode, self.depth,
                     self.select_algo)
+
+    def select_prepare(self, max_seq_len: int, seq_lens: Optional[torch.Tensor]) -> None:
+        _ops.select_prepare(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
+                            self.recent_budget, self.heavy_budget, self.counts, self.ws_select, self.mode, self.depth)
+
+    def attend_fused(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, max_seq_len: int,
+                     seq_lens: Optional[torch.Tensor]) -> None:
+        _ops.sparse_decode_fused(q3, k, v, self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens,
+                                 self.init_budget, self.recent_budget, self.heavy_budget, self.ws_select, self.sm_scale, out,
+                                 self.ws_fused)
 
     def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor) -> None:
         _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend)
@@ -135,6 +153,10 @@ class HashDecodeLayer:
             newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
             _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
                              self.qcodes, pos_dev=pos, arith=self.arith)
+        if self.use_fused and self.fused_ok and not self.overlap_windows:
+            self.select_prepare(seq_len, seq_lens)
+            self.attend_fused(q3, k_cache, v_cache, out, seq_len, seq_lens)
+            return out
         self.select(seq_len, seq_lens)
         if self.overlap_windows:
             main.wait_stream(self.side_stream)

@@ -195,6 +195,34 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
                            int max_seq_len, const int32_t *seq_lens, void *stream);
 
 /*
+ * Selection fused into the attention launch.  ha_select_prepare runs the first two launches of the histogram
+ * method only: it leaves in the workspace, per (sequence, query head), the threshold distance T, the number of ties
+ * taken and the heavy count, and per 1024..4096-token chunk how many selected tokens precede it, and writes
+ * out_counts.  ha_sparse_decode_fused then rebuilds each row's ordered index list in LDS straight from the codes
+ * (same order as ha_select's list, so the output equals ha_select + ha_sparse_decode bit for bit when rows are not
+ * split) and attends to it: the list never travels through memory and the compaction launch disappears.
+ * Budgets, seq_lens and code arguments must be those given to ha_select_prepare; `select_workspace` is the
+ * workspace it filled.  Only HA_SELECT_SIMPLE, and only while init + recent + heavy <= 8192 entries
+ * (ha_sparse_decode_fused_applies returns 1); otherwise use ha_select + ha_sparse_decode.  Replaces the same
+ * reference lines as those two (hashattention_llama.py:401-446, 585-615; efficiency/kernels/torchatt.py:52-71).
+ */
+int ha_select_prepare(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                      int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                      int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
+                      int32_t *out_counts, void *workspace, size_t workspace_bytes, void *stream);
+int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
+                                   int init_budget, int recent_budget, double heavy_budget, int mode);
+size_t ha_sparse_decode_fused_workspace_bytes(int B, int H, int Hc, int max_seq_len);
+int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                           const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                           const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                           int B, int H, int Hkv, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                           int init_budget, int recent_budget, double heavy_budget,
+                           const void *select_workspace, size_t select_workspace_bytes,
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).
  * Replaces flash_decode_attention_fwd (efficiency/kernels/flash_fwd_sparse.py:21-321) and
  * torch_attention_naive (efficiency/kernels/torchatt.py:17-30).  Each K/V row is read once per KV

@@ -129,6 +129,21 @@ def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple"
     assert err2 <= ATOL[w.dtype], f"window + heavy attend max-abs error {err2} > {ATOL[w.dtype]}"
     report.update(split_window_err=err2)
 
+    # ---- selection fused into the attend launch: thresholds from ha_select_prepare, list rebuilt in LDS from the codes
+    if mode == "simple" and _ops.fused_applies(B, H, Hc, W, S, w.init_budget, w.recent_budget, w.heavy_budget):
+        counts3 = torch.full((B, H), -5, dtype=torch.int32, device=dev)
+        out3 = torch.empty_like(out)
+        ws4 = _ops.workspace(_ops.sparse_decode_fused_workspace_bytes(B, H, Hc, S), dev)
+        _ops.select_prepare(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, counts3, ws)
+        _ops.sparse_decode_fused(q3, k, v, kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws, sm_scale,
+                                 out3, ws4)
+        assert np.array_equal(counts3.cpu().numpy(), counts_ref), "fused path: counts differ"
+        err3 = float(np.abs(out3.float().cpu().numpy() - ref).max())
+        assert err3 <= ATOL[w.dtype], f"fused select+attend max-abs error {err3} > {ATOL[w.dtype]}"
+        same = float((out3.float() - out.float()).abs().max().item())
+        assert same <= (2e-6 if w.dtype == torch.float32 else 1e-2), f"fused vs two-launch output differ by {same}"
+        report.update(fused_err=err3, fused_vs_unfused=same)
+
     if check_dense:
         outd = torch.empty(B, H, d, dtype=w.dtype, device=dev)
         ws3 = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)

@@ -115,59 +115,22 @@ struct FusedSel {
     int nchunk, chunk, cps, gq, init, recent, vec;
 };
 
-// NSLAB slabs of 256 codes of one chunk, all requested before the first is used: the selected ones go to their list
-// positions.  n_lt / n_eq: tokens with d < T / d == T before the first slab (row-wide), updated.
+// NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.
 template <int W, int NSLAB>
-__device__ __forceinline__ void scan_slabs(const uint32_t *kc, const ha_sel::Code<W> &q, int j_first, int beg, int end, bool whole, int T,
-                                           int r, int lo, int p0, int n, int lane, int &n_lt, int &n_eq, int32_t *s_list) {
-    using namespace ha_sel;
-    Code<W> k[NSLAB][4];
+__device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int beg, int end, bool whole, int lane,
+                                           ha_sel::Code<W> (&k)[NSLAB][4]) {
 #pragma unroll
-    for (int s = 0; s < NSLAB; ++s) load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
-#pragma unroll
-    for (int s = 0; s < NSLAB; ++s) {
-        const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
-        uint32_t lt4 = 0, eq4 = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int d = k[s][e].dist(q);
-            const bool in = whole || (j0 + e >= beg && j0 + e < end);
-            lt4 |= (in && d < T) ? (1u << e) : 0u;
-            eq4 |= (in && d == T) ? (1u << e) : 0u;
-        }
-        const uint32_t cnt = (uint32_t)__popc(lt4) | ((uint32_t)__popc(eq4) << 16);
-        const uint32_t incl = wave_inclusive_scan(cnt);
-        const uint32_t excl = incl - cnt;
-        int a = n_lt + (int)(excl & 0xFFFFu), t = n_eq + (int)(excl >> 16);
-        const uint32_t em = t < r ? eq4 : 0u;  // past the r-th tie nothing more of the tie bucket is taken
-        uint32_t todo = lt4 | em;
-        while (todo) {
-            const int e = __ffs((int)todo) - 1;
-            todo &= todo - 1;
-            const bool is_eq = (em >> e) & 1u;
-            if (!is_eq || t < r) {
-                const int pos = lo + a + min(t, r) - p0;
-                if (pos >= 0 && pos < n) s_list[pos] = j0 + e;
-            }
-            a += is_eq ? 0 : 1;
-            t += is_eq ? 1 : 0;
-        }
-        const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
-        n_lt += (int)(tot & 0xFFFFu);
-        n_eq += (int)(tot >> 16);
-    }
+    for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
 }
 
-// The same for a chunk whose ties are taken all or not at all (every chunk but the one holding the r-th tie): the
+// Placement for a chunk whose ties are taken all or not at all (every chunk but the one holding the r-th tie): the
 // NSLAB * 4 codes of a lane become one bit mask and one wave scan places them, in (lane, slab, element) order inside
 // the group - the list holds the same tokens as the ordered one, in a different but fixed order.
 template <int W, int NSLAB>
-__device__ __forceinline__ void scan_slabs_unordered(const uint32_t *kc, const ha_sel::Code<W> &q, int j_first, int beg, int end, bool whole,
-                                                     int T, bool take_ties, int base, int n, int lane, int &n_sel, int32_t *s_list) {
+__device__ __forceinline__ void scan_slabs_unordered(const ha_sel::Code<W> (&k)[NSLAB][4], const ha_sel::Code<W> &q, int j_first, int beg,
+                                                     int end, bool whole, int T, bool take_ties, int base, int n, int lane, int &n_sel,
+                                                     int32_t *s_list) {
     using namespace ha_sel;
-    Code<W> k[NSLAB][4];
-#pragma unroll
-    for (int s = 0; s < NSLAB; ++s) load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
     // sign bit of (d - T') is "d < T'"; T' = T + 1 when ties count.  Last code first so that code (s, e) lands on bit 4 s + e.
     const int neg_t = -(T + (take_ties ? 1 : 0));
     uint32_t m = 0;
@@ -198,60 +161,191 @@ __device__ __forceinline__ void scan_slabs_unordered(const uint32_t *kc, const h
     n_sel += __builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
 }
 
-// Fills s_list[0, n) with the list positions [p0, p0 + n) of row `row`; returns n.  All threads of the workgroup call it.
-template <int W, int NT>
-__device__ __forceinline__ int build_list(const FusedSel &f, int b, int h, int H, int64_t row, int S, int sp, int32_t *s_list) {
-    using namespace ha_sel;
-    constexpr int NW = NT / HA_WAVE;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int lo = min(f.init, S), hi = max(S - f.recent, lo);
-    const int T = f.meta[row * 4 + 0], r = f.meta[row * 4 + 1], nheavy = f.meta[row * 4 + 2];
-    const int c0 = sp * f.cps, c1 = min(c0 + f.cps, f.nchunk);
+// A fused workgroup first places the selected tokens of its chunks in the LDS list (all waves; wave w owns chunks
+// c0 + w, c0 + w + NW, ...; list positions come from the chunk prefixes, so waves never talk to each other), then
+// runs the attention loop over the list.  (Dedicated producer waves feeding the loop through LDS counters were
+// tried: the loop's bandwidth follows the number of gathering waves, and giving two of eight to the scan cost
+// more than the scan itself.)
+struct FusedRow {
+    int lo, hi, T, r, nheavy, neq, c0, nc, p0, n;
+    int cstar;  // the chunk of this workgroup that holds the r-th tie (ties before it are taken, after it not), or -1
+};
+
+// All threads of the workgroup: row constants and the windows.
+template <int NTT>
+__device__ __forceinline__ FusedRow fused_setup(const FusedSel &f, int64_t row, int S, int sp, int32_t *s_list, int *s_cstar) {
+    FusedRow fr;
+    const int tid = threadIdx.x;
+    fr.lo = min(f.init, S);
+    fr.hi = max(S - f.recent, fr.lo);
+    fr.T = f.meta[row * 4 + 0];
+    fr.r = f.meta[row * 4 + 1];
+    fr.nheavy = f.meta[row * 4 + 2];
+    fr.neq = f.meta[row * 4 + 3];
+    fr.c0 = sp * f.cps;
+    const int c1 = min(fr.c0 + f.cps, f.nchunk);
+    fr.nc = c1 - fr.c0;
     const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
-    const int p0 = sp == 0 ? 0 : lo + pre[c0 * 2] + min(pre[c0 * 2 + 1], r);
-    const int p1 = c1 >= f.nchunk ? lo + nheavy + (S - hi) : lo + pre[c1 * 2] + min(pre[c1 * 2 + 1], r);
-    const int n = min(max(p1 - p0, 0), kFusedListCap);
+    auto gpos = [&](int c) { return c >= f.nchunk ? fr.lo + fr.nheavy : fr.lo + pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
+    fr.p0 = sp == 0 ? 0 : gpos(fr.c0);
+    const int p1 = c1 >= f.nchunk ? fr.lo + fr.nheavy + (S - fr.hi) : gpos(c1);
+    fr.n = min(max(p1 - fr.p0, 0), kFusedListCap);
     if (sp == 0)
-        for (int i = tid; i < lo && i < n; i += NT) s_list[i] = i;
+        for (int i = tid; i < fr.lo && i < fr.n; i += NTT) s_list[i] = i;
     if (c1 >= f.nchunk) {
-        const int base = lo + nheavy - p0;
-        for (int i = tid; i < S - hi; i += NT)
-            if (base + i < n) s_list[base + i] = hi + i;
+        const int base = fr.lo + fr.nheavy - fr.p0;
+        for (int i = tid; i < S - fr.hi; i += NTT)
+            if (base + i < fr.n) s_list[base + i] = fr.hi + i;
     }
-    if (nheavy > 0) {
-        const Code<W> q = load_qcode<W>(f.qcodes, row);
-        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
-        constexpr int GS = W == 1 ? 8 : 4;  // slabs per request group: 32 VGPRs of codes in flight per lane
-        for (int c = c0 + wave; c < c1; c += NW) {  // uniform per wave
-            const int cb = c * f.chunk;
-            const int beg = max(lo, cb), end = min(hi, cb + f.chunk);
-            if (beg >= end) continue;
-            int n_lt = pre[c * 2], n_eq = pre[c * 2 + 1];
-            const bool whole = f.vec && beg == cb && end == cb + f.chunk;
-            // ties of this chunk: none taken, all taken, or (the chunk of the r-th tie, and the last chunk, whose tie
-            // count is not recorded) the first few in token order
-            const bool none = n_eq >= r;
-            const bool all = !none && c + 1 < f.nchunk && pre[(c + 1) * 2 + 1] <= r;
-            if (none || all) {
-                int n_sel = n_lt + min(n_eq, r);
-                if (f.chunk % (GS * HA_WAVE * 4) == 0) {
-                    for (int j = cb; j < cb + f.chunk; j += GS * HA_WAVE * 4)
-                        scan_slabs_unordered<W, GS>(kc, q, j, beg, end, whole, T, all, lo - p0, n, lane, n_sel, s_list);
-                } else {
-                    for (int j = cb; j < cb + f.chunk; j += 4 * HA_WAVE * 4)
-                        scan_slabs_unordered<W, 4>(kc, q, j, beg, end, whole, T, all, lo - p0, n, lane, n_sel, s_list);
+    if (tid == 0) *s_cstar = -1;
+    __syncthreads();
+    for (int i = tid; i < fr.nc; i += NTT) {
+        const int c = fr.c0 + i;
+        const int eq0 = pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? pre[(c + 1) * 2 + 1] : fr.neq;
+        if (eq0 < fr.r && fr.r < eq1) *s_cstar = c;  // at most one chunk of the row
+    }
+    __syncthreads();
+    fr.cstar = *s_cstar;
+    return fr;
+}
+
+// One wave (p = 0 .. NP-1) of the NP that share the chunks.  Its chunks are cut into groups of NSLAB slabs; the codes
+// of group g + 1 are requested before group g is placed, so only the first memory round trip is waited out idle.
+template <int W, int NSLAB, int NP>
+__device__ __forceinline__ void fused_produce(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, int p, int32_t *s_list) {
+    using namespace ha_sel;
+    const int lane = threadIdx.x & 63;
+    const Code<W> q = load_qcode<W>(f.qcodes, row);
+    const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
+    const int lo = fr.lo, hi = fr.hi, T = fr.T, r = fr.r, p0 = fr.p0, n = fr.n;
+    constexpr int GC = NSLAB * HA_WAVE * 4;           // codes per group
+    const int gpc = f.chunk / GC;                     // groups per chunk (>= 1: the host picks NSLAB to divide the chunk)
+    const int my_chunks = fr.nc > p ? (fr.nc - p + NP - 1) / NP : 0;
+    const int G = fr.nheavy > 0 ? my_chunks * gpc : 0;
+    struct Grp {
+        int c, j_first, beg, end;
+        bool whole;
+    };
+    auto grp = [&](int g) {
+        Grp x;
+        x.c = fr.c0 + p + (g / gpc) * NP;
+        const int cb = x.c * f.chunk;
+        x.j_first = cb + (g % gpc) * GC;
+        x.beg = max(lo, cb);
+        x.end = min(hi, cb + f.chunk);
+        x.whole = f.vec && x.beg == cb && x.end == cb + f.chunk;
+        return x;
+    };
+    Code<W> cur[NSLAB][4], nxt[NSLAB][4];
+    if (G > 0) {
+        const Grp x = grp(0);
+        load_slabs<W, NSLAB>(kc, x.j_first, x.beg, x.end, x.whole, lane, cur);
+    }
+    int n_lt = 0, n_eq = 0, n_sel = 0;
+    bool ordered = false, ties = false;
+    (void)r;
+    for (int g = 0; g < G; ++g) {
+        if (g + 1 < G) {
+            const Grp y = grp(g + 1);
+            load_slabs<W, NSLAB>(kc, y.j_first, y.beg, y.end, y.whole, lane, nxt);
+        }
+        const Grp x = grp(g);
+        if (g % gpc == 0) {  // a new chunk: where its tokens go, and how its ties are treated
+            n_lt = pre[x.c * 2];
+            n_eq = pre[x.c * 2 + 1];
+            // ties of this chunk: none taken or all taken; the one chunk where the r-th tie falls is left to
+            // fused_place_tie_chunk
+            ties = n_eq < r;          // all of them (the chunk of the r-th tie is not placed here)
+            ordered = x.c == fr.cstar;
+            n_sel = n_lt + min(n_eq, r);
+        }
+        if (x.beg < x.end && !ordered)
+            scan_slabs_unordered<W, NSLAB>(cur, q, x.j_first, x.beg, x.end, x.whole, T, ties, lo - p0, n, lane, n_sel, s_list);
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cur[s][e] = nxt[s][e];
+    }
+}
+
+// The chunk where the r-th tie falls: its ties are taken in token order, so its slabs need each other's counts.
+// All NW waves share it, one to two slabs each.  tie_chunk_count (before the other chunks are scanned, so its memory
+// round trip is not waited for on its own) leaves each slab's counts in LDS and the lane's masks in `tc`;
+// tie_chunk_place (after a workgroup barrier) places the tokens.  Both are called by every thread when
+// fr.cstar >= 0 (uniform).
+struct TieChunk {
+    uint32_t lt4[2], eq4[2], incl[2];
+};
+template <int W, int NW>
+__device__ __forceinline__ void tie_chunk_count(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, uint32_t *s_cnt /* [64] */,
+                                                TieChunk &tc) {
+    using namespace ha_sel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Code<W> q = load_qcode<W>(f.qcodes, row);
+    const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+    const int cb = fr.cstar * f.chunk;
+    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
+    const bool whole = f.vec && beg == cb && end == cb + f.chunk;
+    const int nslab = f.chunk / (HA_WAVE * 4);             // 4, 8 or 16
+    const int spw = (nslab + NW - 1) / NW;                 // slabs per wave: 1 or 2 for NW = 8
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        tc.lt4[i] = tc.eq4[i] = tc.incl[i] = 0;
+        const int sl = wave * spw + i;
+        if (i < spw && sl < nslab) {
+            const int j0 = cb + sl * (HA_WAVE * 4) + lane * 4;
+            Code<W> k4[4];
+            load_code4<W>(kc, j0, beg, end, whole, k4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int d = k4[e].dist(q);
+                const bool in = whole || (j0 + e >= beg && j0 + e < end);
+                tc.lt4[i] |= (in && d < fr.T) ? (1u << e) : 0u;
+                tc.eq4[i] |= (in && d == fr.T) ? (1u << e) : 0u;
+            }
+            tc.incl[i] = wave_inclusive_scan((uint32_t)__popc(tc.lt4[i]) | ((uint32_t)__popc(tc.eq4[i]) << 16));
+            if (lane == HA_WAVE - 1) s_cnt[sl] = tc.incl[i];
+        }
+    }
+}
+template <int NW>
+__device__ __forceinline__ void tie_chunk_place(const FusedSel &f, const FusedRow &fr, int64_t row, const uint32_t *s_cnt, const TieChunk &tc,
+                                                int32_t *s_list) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
+    const int c = fr.cstar, cb = c * f.chunk;
+    const int nslab = f.chunk / (HA_WAVE * 4);
+    const int spw = (nslab + NW - 1) / NW;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int sl = wave * spw + i;
+        if (i < spw && sl < nslab) {
+            int a = pre[c * 2], t = pre[c * 2 + 1];
+            for (int s2 = 0; s2 < sl; ++s2) {
+                const uint32_t v = s_cnt[s2];
+                a += (int)(v & 0xFFFFu);
+                t += (int)(v >> 16);
+            }
+            const uint32_t excl = tc.incl[i] - ((uint32_t)__popc(tc.lt4[i]) | ((uint32_t)__popc(tc.eq4[i]) << 16));
+            a += (int)(excl & 0xFFFFu);
+            t += (int)(excl >> 16);
+            const int j0 = cb + sl * (HA_WAVE * 4) + lane * 4;
+            const uint32_t em = t < fr.r ? tc.eq4[i] : 0u;  // past the r-th tie nothing more of the tie bucket is taken
+            uint32_t todo = tc.lt4[i] | em;
+            while (todo) {
+                const int e = __ffs((int)todo) - 1;
+                todo &= todo - 1;
+                const bool is_eq = (em >> e) & 1u;
+                if (!is_eq || t < fr.r) {
+                    const int pos = fr.lo + a + min(t, fr.r) - fr.p0;
+                    if (pos >= 0 && pos < fr.n) s_list[pos] = j0 + e;
                 }
-            } else if (f.chunk % (GS * HA_WAVE * 4) == 0) {
-                for (int j = cb; j < cb + f.chunk; j += GS * HA_WAVE * 4)
-                    scan_slabs<W, GS>(kc, q, j, beg, end, whole, T, r, lo, p0, n, lane, n_lt, n_eq, s_list);
-            } else {  // 1024-code chunks (short rows): four slabs at a time
-                for (int j = cb; j < cb + f.chunk; j += 4 * HA_WAVE * 4)
-                    scan_slabs<W, 4>(kc, q, j, beg, end, whole, T, r, lo, p0, n, lane, n_lt, n_eq, s_list);
+                a += is_eq ? 0 : 1;
+                t += is_eq ? 1 : 0;
             }
         }
     }
-    __syncthreads();
-    return n;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -272,6 +366,8 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     __shared__ float s_m[NS], s_l[NS];
     __shared__ float s_acc[NS * HA_HEAD_DIM];
     __shared__ int32_t s_list[FW > 0 ? kFusedListCap : 1];
+    __shared__ uint32_t s_cnt[FW > 0 ? 64 : 1];
+    __shared__ int s_cstar;
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
     // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
@@ -287,12 +383,25 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
+        const FusedRow fr = fused_setup<NT>(fsel, row, S, sp, s_list, &s_cstar);
         r0 = 0;
-        r1 = build_list<FW, NT>(fsel, b, h, H, row, S, sp, s_list);
-        if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output
+        r1 = fr.n;
+        if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
             if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
             return;
         }
+        TieChunk tc;
+        if (fr.cstar >= 0) tie_chunk_count<FW, NT / HA_WAVE>(fsel, fr, b, h, row, s_cnt, tc);
+        {
+            constexpr int GS = FW == 1 ? 8 : 4;  // slabs per request group: 32 VGPRs of codes per lane, twice (two groups in flight)
+            if (fsel.chunk % (GS * HA_WAVE * 4) == 0) fused_produce<FW, GS, NT / HA_WAVE>(fsel, fr, b, h, row, tid >> 6, s_list);
+            else fused_produce<FW, FW == 1 ? 4 : 2, NT / HA_WAVE>(fsel, fr, b, h, row, tid >> 6, s_list);  // 1024-code chunks
+        }
+        if (fr.cstar >= 0) {
+            __syncthreads();  // every slab's counts are in LDS
+            tie_chunk_place<NT / HA_WAVE>(fsel, fr, row, s_cnt, tc, s_list);
+        }
+        __syncthreads();  // the list is complete
     } else {
         int64_t n = counts[b * H + h];
         if (n > idx_cap) n = idx_cap;
@@ -336,7 +445,7 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     // list position of (step base, u) for this stream; positions >= r1 are padded with the split's first row
     auto list_index = [&](int base, int u) {
         const int r = base + stream + u * NS;
-        if constexpr (FW > 0) return r < r1 ? s_list[r] : (r1 > 0 ? s_list[0] : 0);
+        if constexpr (FW > 0) return r < r1 ? s_list[r] : 0;  // padding: token 0, always present
         else return ix[r < r1 ? r : r0];
     };
     int32_t j_next[U];   // indices of the step after the one in flight
@@ -793,7 +902,8 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     const int G = H / Hkv;
 #define HA_FUSED_LAUNCH(E_, U_, FW_)                                                                                              \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,      \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b,                       \
+                           q_stride_h, k, v,                                                                                      \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
                            part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f);                                      \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \

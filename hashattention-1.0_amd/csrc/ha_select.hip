@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
 }
 
 // ------------------------------------------------------------------------------------------------
-// Pass 2.  grid (H, B), 256 threads.  meta[row] = {T, r, n_heavy, 0}; chunk_pre[row][c] = {#selected with
+// Pass 2.  grid (H, B), 256 threads.  meta[row] = {T, r, n_heavy, #tokens with d == T}; chunk_pre[row][c] = {#selected with
 // d < T in chunks before c, #tokens with d == T in chunks before c}.  Also writes the sink and recent
 // window indices and the row's count.
 template <int W>
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kSelThreads) void select_threshold_kernel(const uin
         meta[row * 4 + 0] = T;
         meta[row * 4 + 1] = r;
         meta[row * 4 + 2] = nheavy;
-        meta[row * 4 + 3] = 0;
+        meta[row * 4 + 3] = (T >= 0 && T < NL) ? (int)s_tot[T] : 0;  // size of the tie bucket
     }
     __syncthreads();
     const int T = s_T, nheavy = s_nheavy;

@@ -171,7 +171,7 @@ inline bool rows_vectorisable(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_
 }
 
 
-// workspace of the histogram selection: per-chunk histograms, row meta {T, r, n_heavy, 0}, per-chunk prefixes
+// workspace of the histogram selection: per-chunk histograms, row meta {T, r, n_heavy, size of the tie bucket}, per-chunk prefixes
 // {#d < T before the chunk, #d == T before the chunk}
 struct SelectWorkspace {
     uint32_t *hist;

@@ -19,16 +19,20 @@ def _layer(w, p, **kw):
                            w.lth_final_dim, w.init_budget, w.recent_budget, w.heavy_budget, device=DEV, **kw)
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("hc", [2, 8])
-def test_three_decode_steps_match_reference_layer(hc):
-    # fp32 end to end: the step output equals the reference layer's masked dense attention on the same cache
-    print(f"\n[case] decode layer Hc={hc}", flush=True)
+def test_three_decode_steps_match_reference_layer(hc, fused):
+    # fp32 end to end: the step output equals the reference layer's masked dense attention on the same cache, through the
+    # fused select-attend launch and through ha_select + ha_sparse_decode
+    print(f"\n[case] decode layer Hc={hc} fused={fused}", flush=True)
     w = small_workload(batch=2, seq_lens=[900, 900], n_code_heads=hc, dtype=torch.float32, seed=17)
     p = make_problem(w)
     S = w.max_seq_len
     k, v = p.k.to(DEV), p.v.to(DEV)
     layer = _layer(w, p)
     layer.allocate(w.batch, S)
+    layer.use_fused = fused
+    assert layer.fused_ok
     s0 = S - 3
     layer.encode_keys(k[:, :, :s0])
     layer.n_cached = s0
@@ -38,6 +42,8 @@ def test_three_decode_steps_match_reference_layer(hc):
         q = torch.randn(w.batch, w.n_q_heads, 1, w.head_dim, generator=g)
         out = torch.empty(w.batch, w.n_q_heads, w.head_dim, device=DEV)
         layer.step(q.to(DEV), k, v, s, out)
+        if fused:           # the fused step keeps its lists in LDS: write them out for the comparison below
+            layer.select(s, None)
         ref, mask = orc.reference_decode_attention(q, p.k[:, :, :s], p.v[:, :, :s], p.usa.k, p.usa.q, w.init_budget,
                                                    w.recent_budget, w.heavy_budget)
         # selected sets must be identical (codes may differ only at |logit| ~ 0, which would show up here)

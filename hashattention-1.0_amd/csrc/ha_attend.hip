@@ -348,6 +348,119 @@ __device__ __forceinline__ void tie_chunk_place(const FusedSel &f, const FusedRo
     }
 }
 
+// One scan round of a fused workgroup: its NW waves take NW consecutive groups of GS slabs (a group is part of one
+// chunk; a chunk's groups never straddle rounds), place the selected tokens of those groups in the list, and return
+// how many leading list entries are in LDS afterwards.  Two workgroup barriers per round; called by all threads.
+// The gather loop runs between rounds, so the scan's integer work sits in the shadow of the loop's memory waits
+// instead of in front of it.
+template <int W, int GS, int NW>
+__device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, int round, int n_groups,
+                                           uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list) {
+    using namespace ha_sel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int GC = GS * HA_WAVE * 4;  // codes per group
+    const int gpc = f.chunk / GC;         // groups per chunk: 1, 2 or 4 (divides NW)
+    const int g = round * NW + wave;
+    const bool active = g < n_groups;
+    const int c = fr.c0 + (active ? g / gpc : 0), gi = active ? g % gpc : 0;
+    const int cb = c * f.chunk, j_first = cb + gi * GC;
+    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
+    const bool whole = f.vec && beg == cb && end == cb + f.chunk;
+    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
+
+    uint32_t lt = 0, le = 0;  // bit 4 s + e: code (slab s, element e) of this lane has d < T / d <= T
+    if (active && beg < end && fr.nheavy > 0) {
+        const Code<W> q = load_qcode<W>(f.qcodes, row);
+        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+        Code<W> k[GS][4];
+        load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
+        const int neg_t = -fr.T;
+#pragma unroll
+        for (int s = GS - 1; s >= 0; --s)
+#pragma unroll
+            for (int e = 3; e >= 0; --e) {
+                const int key = k[s][e].dist(q) + neg_t;  // sign bit: d < T; of key - 1: d <= T
+                lt = __builtin_amdgcn_alignbit(lt, (uint32_t)key, 31);
+                le = __builtin_amdgcn_alignbit(le, (uint32_t)(key - 1), 31);
+            }
+        if (!whole) {
+            uint32_t valid = 0;
+#pragma unroll
+            for (int s = 0; s < GS; ++s) {
+                const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) valid |= (j0 + e >= beg && j0 + e < end) ? (1u << (4 * s + e)) : 0u;
+            }
+            lt &= valid;
+            le &= valid;
+        }
+    }
+    const uint32_t eq = le & ~lt;
+    const uint32_t cnt = (uint32_t)__popc(lt) | ((uint32_t)__popc(eq) << 16);
+    const uint32_t incl = wave_inclusive_scan(cnt);
+    const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
+    if (lane == 0) s_cnt[wave] = tot;
+    __syncthreads();
+
+    // tokens of the row with d < T / d == T before this group: the chunk's prefix plus the chunk's earlier groups,
+    // which are the gi waves just below this one
+    int a = pre[c * 2], t = pre[c * 2 + 1];
+    for (int w2 = wave - gi; w2 < wave; ++w2) {
+        const uint32_t v = s_cnt[w2];
+        a += (int)(v & 0xFFFFu);
+        t += (int)(v >> 16);
+    }
+    const int r = fr.r;
+    if (active && tot != 0) {
+        const int j_lane = j_first + lane * 4;
+        if (c != fr.cstar) {
+            // ties of the chunk all taken (t < r here and through the chunk) or none (t >= r): one mask, one scan
+            const bool ties = t < r;
+            uint32_t m = ties ? le : lt;
+            const uint32_t excl = incl - cnt;
+            int pos = fr.lo + a + min(t, r) - fr.p0 + (int)(excl & 0xFFFFu) + (ties ? (int)(excl >> 16) : 0);
+            while (m) {
+                const int bit = __ffs((int)m) - 1;
+                m &= m - 1;
+                if (pos >= 0 && pos < fr.n) s_list[pos] = j_lane + (bit >> 2) * (HA_WAVE * 4) + (bit & 3);
+                ++pos;
+            }
+        } else {
+            // the chunk of the r-th tie: ties in token order, slab by slab
+            int n_lt = a, n_eq = t;
+#pragma unroll
+            for (int s = 0; s < GS; ++s) {
+                const uint32_t lt4 = (lt >> (4 * s)) & 0xFu, eq4 = (eq >> (4 * s)) & 0xFu;
+                const uint32_t c4 = (uint32_t)__popc(lt4) | ((uint32_t)__popc(eq4) << 16);
+                const uint32_t in4 = wave_inclusive_scan(c4);
+                const uint32_t ex4 = in4 - c4;
+                int a2 = n_lt + (int)(ex4 & 0xFFFFu), t2 = n_eq + (int)(ex4 >> 16);
+                const uint32_t em = t2 < r ? eq4 : 0u;  // past the r-th tie nothing more of the tie bucket is taken
+                uint32_t todo = lt4 | em;
+                while (todo) {
+                    const int e = __ffs((int)todo) - 1;
+                    todo &= todo - 1;
+                    const bool is_eq = (em >> e) & 1u;
+                    if (!is_eq || t2 < r) {
+                        const int pos = fr.lo + a2 + min(t2, r) - fr.p0;
+                        if (pos >= 0 && pos < fr.n) s_list[pos] = j_lane + s * (HA_WAVE * 4) + e;
+                    }
+                    a2 += is_eq ? 0 : 1;
+                    t2 += is_eq ? 1 : 0;
+                }
+                const uint32_t t4 = (uint32_t)__builtin_amdgcn_readlane((int)in4, HA_WAVE - 1);
+                n_lt += (int)(t4 & 0xFFFFu);
+                n_eq += (int)(t4 >> 16);
+            }
+        }
+    }
+    // the last group of the round knows where the placed prefix ends
+    const int last = min(n_groups - 1 - round * NW, NW - 1);
+    if (wave == last && lane == 0) *s_ready = fr.lo + a + (int)(tot & 0xFFFFu) + min(t + (int)(tot >> 16), r) - fr.p0;
+    __syncthreads();
+    return *s_ready;
+}
+
 // ------------------------------------------------------------------------------------------------
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
 // NT threads = NT/16 row streams; U rows per stream per step.
@@ -379,29 +492,18 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     const int64_t row = (int64_t)b * H + h;
     int r0, r1, nsplit;
     const int32_t *ix = nullptr;
+    FusedRow fr = {};
     if constexpr (FW > 0) {
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
-        const FusedRow fr = fused_setup<NT>(fsel, row, S, sp, s_list, &s_cstar);
+        fr = fused_setup<NT>(fsel, row, S, sp, s_list, &s_cstar);
         r0 = 0;
         r1 = fr.n;
         if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
             if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
             return;
         }
-        TieChunk tc;
-        if (fr.cstar >= 0) tie_chunk_count<FW, NT / HA_WAVE>(fsel, fr, b, h, row, s_cnt, tc);
-        {
-            constexpr int GS = FW == 1 ? 8 : 4;  // slabs per request group: 32 VGPRs of codes per lane, twice (two groups in flight)
-            if (fsel.chunk % (GS * HA_WAVE * 4) == 0) fused_produce<FW, GS, NT / HA_WAVE>(fsel, fr, b, h, row, tid >> 6, s_list);
-            else fused_produce<FW, FW == 1 ? 4 : 2, NT / HA_WAVE>(fsel, fr, b, h, row, tid >> 6, s_list);  // 1024-code chunks
-        }
-        if (fr.cstar >= 0) {
-            __syncthreads();  // every slab's counts are in LDS
-            tie_chunk_place<NT / HA_WAVE>(fsel, fr, row, s_cnt, tc, s_list);
-        }
-        __syncthreads();  // the list is complete
     } else {
         int64_t n = counts[b * H + h];
         if (n > idx_cap) n = idx_cap;
@@ -450,20 +552,22 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     };
     int32_t j_next[U];   // indices of the step after the one in flight
     Raw8<E> kr[U], vr[U];
-    {
+    int base = r0;
+    // needs list entries [base, base + 2 STEP)
+    auto prime = [&]() {
         int32_t j0[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) j0[u] = list_index(r0, u);
+        for (int u = 0; u < U; ++u) j0[u] = list_index(base, u);
 #pragma unroll
-        for (int u = 0; u < U; ++u) j_next[u] = list_index(r0 + STEP, u);
+        for (int u = 0; u < U; ++u) j_next[u] = list_index(base + STEP, u);
 #pragma unroll
         for (int u = 0; u < U; ++u) kr[u] = EL::load8(kb + j0[u] * row_bytes, sub);
 #pragma unroll
         for (int u = 0; u < U; ++u) vr[u] = EL::load8(vb + j0[u] * row_bytes, sub);
-    }
-
-    for (int base = r0; base < r1; base += STEP) {
-        // ---- issue the loads of the next step (harmless duplicates of row r0 past the end)
+    };
+    // consumes list entries [base, base + STEP); needs entries up to base + 3 STEP
+    auto step = [&]() {
+        // ---- issue the loads of the next step (harmless duplicates of a padding row past the end)
         Raw8<E> kn[U], vn[U];
         int32_t j_after[U];
 #pragma unroll
@@ -508,6 +612,36 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
             vr[u] = vn[u];
             j_next[u] = j_after[u];
         }
+        base += STEP;
+    };
+
+    if constexpr (FW > 0) {
+        // scan rounds and gather steps alternate: after a round the list is complete up to `ready`, and the loop runs
+        // as far as its look-ahead (3 steps) allows.  Everything here is uniform over the workgroup.
+        constexpr int NW = NT / HA_WAVE;
+        constexpr int GS = FW == 1 ? 4 : 2;  // slabs per wave and round: 16 VGPRs of codes on top of the loop's registers
+        const bool wide = true;
+        const int gc = GS * HA_WAVE * 4;
+        const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
+        const int rounds = (n_groups + NW - 1) / NW;
+        bool primed = false;
+        for (int k = 0; k < rounds; ++k) {
+            int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
+            (void)wide;
+            if (k == rounds - 1) break;
+            ready = min(ready, r1);
+            if (!primed && ready >= min(2 * STEP, r1)) {
+                prime();
+                primed = true;
+            }
+            while (primed && base + 3 * STEP <= ready) step();
+        }
+        if (rounds == 0) __syncthreads();  // the windows written by fused_setup
+        if (!primed) prime();
+        while (base < r1) step();
+    } else {
+        prime();
+        while (base < r1) step();
     }
 
     if (sub == 0) {

@@ -123,51 +123,15 @@ __device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int 
     for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
 }
 
-// Placement for a chunk whose ties are taken all or not at all (every chunk but the one holding the r-th tie): the
-// NSLAB * 4 codes of a lane become one bit mask and one wave scan places them, in (lane, slab, element) order inside
-// the group - the list holds the same tokens as the ordered one, in a different but fixed order.
-template <int W, int NSLAB>
-__device__ __forceinline__ void scan_slabs_unordered(const ha_sel::Code<W> (&k)[NSLAB][4], const ha_sel::Code<W> &q, int j_first, int beg,
-                                                     int end, bool whole, int T, bool take_ties, int base, int n, int lane, int &n_sel,
-                                                     int32_t *s_list) {
-    using namespace ha_sel;
-    // sign bit of (d - T') is "d < T'"; T' = T + 1 when ties count.  Last code first so that code (s, e) lands on bit 4 s + e.
-    const int neg_t = -(T + (take_ties ? 1 : 0));
-    uint32_t m = 0;
-#pragma unroll
-    for (int s = NSLAB - 1; s >= 0; --s)
-#pragma unroll
-        for (int e = 3; e >= 0; --e) m = __builtin_amdgcn_alignbit(m, (uint32_t)(k[s][e].dist(q) + neg_t), 31);
-    if (!whole) {
-        uint32_t valid = 0;
-#pragma unroll
-        for (int s = 0; s < NSLAB; ++s) {
-            const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) valid |= (j0 + e >= beg && j0 + e < end) ? (1u << (4 * s + e)) : 0u;
-        }
-        m &= valid;
-    }
-    const uint32_t cnt = (uint32_t)__popc(m);
-    const uint32_t incl = wave_inclusive_scan(cnt);
-    int pos = base + n_sel + (int)(incl - cnt);
-    const int j_lane = j_first + lane * 4;
-    while (m) {
-        const int bit = __ffs((int)m) - 1;
-        m &= m - 1;
-        if (pos >= 0 && pos < n) s_list[pos] = j_lane + (bit >> 2) * (HA_WAVE * 4) + (bit & 3);
-        ++pos;
-    }
-    n_sel += __builtin_amdgcn_readlane((int)incl, HA_WAVE - 1);
-}
-
-// A fused workgroup first places the selected tokens of its chunks in the LDS list (all waves; wave w owns chunks
-// c0 + w, c0 + w + NW, ...; list positions come from the chunk prefixes, so waves never talk to each other), then
-// runs the attention loop over the list.  (Dedicated producer waves feeding the loop through LDS counters were
-// tried: the loop's bandwidth follows the number of gathering waves, and giving two of eight to the scan cost
-// more than the scan itself.)
+// A fused workgroup alternates scan rounds (fused_round: its waves place the selected tokens of the next few chunks in
+// the LDS list) with as many steps of the attention loop as the list filled so far allows.  (Dedicated producer
+// waves feeding the loop through LDS counters were tried: the loop's bandwidth follows the number of gathering
+// waves, and giving two of eight to the scan cost more than the scan itself.  Building the whole list first costs
+// the scan's ~15 us up front.)
 struct FusedRow {
-    int lo, hi, T, r, nheavy, neq, c0, nc, p0, n;
+    int lo, hi, T, r, nheavy, neq, c0, nc, n;
+    int nwin;   // window entries at the head of this workgroup's list (sink if it has the first chunk, recent if the last)
+    int hbase;  // list position of a heavy token = hbase + (#d < T before it) + min(#d == T before it, r)
     int cstar;  // the chunk of this workgroup that holds the r-th tie (ties before it are taken, after it not), or -1
 };
 
@@ -186,17 +150,17 @@ __device__ __forceinline__ FusedRow fused_setup(const FusedSel &f, int64_t row, 
     const int c1 = min(fr.c0 + f.cps, f.nchunk);
     fr.nc = c1 - fr.c0;
     const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
-    auto gpos = [&](int c) { return c >= f.nchunk ? fr.lo + fr.nheavy : fr.lo + pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
-    fr.p0 = sp == 0 ? 0 : gpos(fr.c0);
-    const int p1 = c1 >= f.nchunk ? fr.lo + fr.nheavy + (S - fr.hi) : gpos(c1);
-    fr.n = min(max(p1 - fr.p0, 0), kFusedListCap);
-    if (sp == 0)
-        for (int i = tid; i < fr.lo && i < fr.n; i += NTT) s_list[i] = i;
-    if (c1 >= f.nchunk) {
-        const int base = fr.lo + fr.nheavy - fr.p0;
-        for (int i = tid; i < S - fr.hi; i += NTT)
-            if (base + i < fr.n) s_list[base + i] = fr.hi + i;
-    }
+    // heavy tokens of the row before chunk c
+    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
+    // the windows come first in the list: they are known at once, so the loop can start on them while the first
+    // chunks are being scanned
+    const int n_sink = sp == 0 ? fr.lo : 0, n_recent = c1 >= f.nchunk ? S - fr.hi : 0;
+    fr.nwin = min(n_sink + n_recent, kFusedListCap);
+    fr.hbase = fr.nwin - rank(fr.c0);
+    fr.n = min(fr.nwin + max(rank(c1) - rank(fr.c0), 0), kFusedListCap);
+    for (int i = tid; i < n_sink && i < fr.n; i += NTT) s_list[i] = i;
+    for (int i = tid; i < n_recent; i += NTT)
+        if (n_sink + i < fr.n) s_list[n_sink + i] = fr.hi + i;
     if (tid == 0) *s_cstar = -1;
     __syncthreads();
     for (int i = tid; i < fr.nc; i += NTT) {
@@ -207,145 +171,6 @@ __device__ __forceinline__ FusedRow fused_setup(const FusedSel &f, int64_t row, 
     __syncthreads();
     fr.cstar = *s_cstar;
     return fr;
-}
-
-// One wave (p = 0 .. NP-1) of the NP that share the chunks.  Its chunks are cut into groups of NSLAB slabs; the codes
-// of group g + 1 are requested before group g is placed, so only the first memory round trip is waited out idle.
-template <int W, int NSLAB, int NP>
-__device__ __forceinline__ void fused_produce(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, int p, int32_t *s_list) {
-    using namespace ha_sel;
-    const int lane = threadIdx.x & 63;
-    const Code<W> q = load_qcode<W>(f.qcodes, row);
-    const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
-    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
-    const int lo = fr.lo, hi = fr.hi, T = fr.T, r = fr.r, p0 = fr.p0, n = fr.n;
-    constexpr int GC = NSLAB * HA_WAVE * 4;           // codes per group
-    const int gpc = f.chunk / GC;                     // groups per chunk (>= 1: the host picks NSLAB to divide the chunk)
-    const int my_chunks = fr.nc > p ? (fr.nc - p + NP - 1) / NP : 0;
-    const int G = fr.nheavy > 0 ? my_chunks * gpc : 0;
-    struct Grp {
-        int c, j_first, beg, end;
-        bool whole;
-    };
-    auto grp = [&](int g) {
-        Grp x;
-        x.c = fr.c0 + p + (g / gpc) * NP;
-        const int cb = x.c * f.chunk;
-        x.j_first = cb + (g % gpc) * GC;
-        x.beg = max(lo, cb);
-        x.end = min(hi, cb + f.chunk);
-        x.whole = f.vec && x.beg == cb && x.end == cb + f.chunk;
-        return x;
-    };
-    Code<W> cur[NSLAB][4], nxt[NSLAB][4];
-    if (G > 0) {
-        const Grp x = grp(0);
-        load_slabs<W, NSLAB>(kc, x.j_first, x.beg, x.end, x.whole, lane, cur);
-    }
-    int n_lt = 0, n_eq = 0, n_sel = 0;
-    bool ordered = false, ties = false;
-    (void)r;
-    for (int g = 0; g < G; ++g) {
-        if (g + 1 < G) {
-            const Grp y = grp(g + 1);
-            load_slabs<W, NSLAB>(kc, y.j_first, y.beg, y.end, y.whole, lane, nxt);
-        }
-        const Grp x = grp(g);
-        if (g % gpc == 0) {  // a new chunk: where its tokens go, and how its ties are treated
-            n_lt = pre[x.c * 2];
-            n_eq = pre[x.c * 2 + 1];
-            // ties of this chunk: none taken or all taken; the one chunk where the r-th tie falls is left to
-            // fused_place_tie_chunk
-            ties = n_eq < r;          // all of them (the chunk of the r-th tie is not placed here)
-            ordered = x.c == fr.cstar;
-            n_sel = n_lt + min(n_eq, r);
-        }
-        if (x.beg < x.end && !ordered)
-            scan_slabs_unordered<W, NSLAB>(cur, q, x.j_first, x.beg, x.end, x.whole, T, ties, lo - p0, n, lane, n_sel, s_list);
-#pragma unroll
-        for (int s = 0; s < NSLAB; ++s)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) cur[s][e] = nxt[s][e];
-    }
-}
-
-// The chunk where the r-th tie falls: its ties are taken in token order, so its slabs need each other's counts.
-// All NW waves share it, one to two slabs each.  tie_chunk_count (before the other chunks are scanned, so its memory
-// round trip is not waited for on its own) leaves each slab's counts in LDS and the lane's masks in `tc`;
-// tie_chunk_place (after a workgroup barrier) places the tokens.  Both are called by every thread when
-// fr.cstar >= 0 (uniform).
-struct TieChunk {
-    uint32_t lt4[2], eq4[2], incl[2];
-};
-template <int W, int NW>
-__device__ __forceinline__ void tie_chunk_count(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, uint32_t *s_cnt /* [64] */,
-                                                TieChunk &tc) {
-    using namespace ha_sel;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const Code<W> q = load_qcode<W>(f.qcodes, row);
-    const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
-    const int cb = fr.cstar * f.chunk;
-    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
-    const bool whole = f.vec && beg == cb && end == cb + f.chunk;
-    const int nslab = f.chunk / (HA_WAVE * 4);             // 4, 8 or 16
-    const int spw = (nslab + NW - 1) / NW;                 // slabs per wave: 1 or 2 for NW = 8
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        tc.lt4[i] = tc.eq4[i] = tc.incl[i] = 0;
-        const int sl = wave * spw + i;
-        if (i < spw && sl < nslab) {
-            const int j0 = cb + sl * (HA_WAVE * 4) + lane * 4;
-            Code<W> k4[4];
-            load_code4<W>(kc, j0, beg, end, whole, k4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int d = k4[e].dist(q);
-                const bool in = whole || (j0 + e >= beg && j0 + e < end);
-                tc.lt4[i] |= (in && d < fr.T) ? (1u << e) : 0u;
-                tc.eq4[i] |= (in && d == fr.T) ? (1u << e) : 0u;
-            }
-            tc.incl[i] = wave_inclusive_scan((uint32_t)__popc(tc.lt4[i]) | ((uint32_t)__popc(tc.eq4[i]) << 16));
-            if (lane == HA_WAVE - 1) s_cnt[sl] = tc.incl[i];
-        }
-    }
-}
-template <int NW>
-__device__ __forceinline__ void tie_chunk_place(const FusedSel &f, const FusedRow &fr, int64_t row, const uint32_t *s_cnt, const TieChunk &tc,
-                                                int32_t *s_list) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
-    const int c = fr.cstar, cb = c * f.chunk;
-    const int nslab = f.chunk / (HA_WAVE * 4);
-    const int spw = (nslab + NW - 1) / NW;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int sl = wave * spw + i;
-        if (i < spw && sl < nslab) {
-            int a = pre[c * 2], t = pre[c * 2 + 1];
-            for (int s2 = 0; s2 < sl; ++s2) {
-                const uint32_t v = s_cnt[s2];
-                a += (int)(v & 0xFFFFu);
-                t += (int)(v >> 16);
-            }
-            const uint32_t excl = tc.incl[i] - ((uint32_t)__popc(tc.lt4[i]) | ((uint32_t)__popc(tc.eq4[i]) << 16));
-            a += (int)(excl & 0xFFFFu);
-            t += (int)(excl >> 16);
-            const int j0 = cb + sl * (HA_WAVE * 4) + lane * 4;
-            const uint32_t em = t < fr.r ? tc.eq4[i] : 0u;  // past the r-th tie nothing more of the tie bucket is taken
-            uint32_t todo = tc.lt4[i] | em;
-            while (todo) {
-                const int e = __ffs((int)todo) - 1;
-                todo &= todo - 1;
-                const bool is_eq = (em >> e) & 1u;
-                if (!is_eq || t < fr.r) {
-                    const int pos = fr.lo + a + min(t, fr.r) - fr.p0;
-                    if (pos >= 0 && pos < fr.n) s_list[pos] = j0 + e;
-                }
-                a += is_eq ? 0 : 1;
-                t += is_eq ? 1 : 0;
-            }
-        }
-    }
 }
 
 // One scan round of a fused workgroup: its NW waves take NW consecutive groups of GS slabs (a group is part of one
@@ -418,7 +243,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
             const bool ties = t < r;
             uint32_t m = ties ? le : lt;
             const uint32_t excl = incl - cnt;
-            int pos = fr.lo + a + min(t, r) - fr.p0 + (int)(excl & 0xFFFFu) + (ties ? (int)(excl >> 16) : 0);
+            int pos = fr.hbase + a + min(t, r) + (int)(excl & 0xFFFFu) + (ties ? (int)(excl >> 16) : 0);
             while (m) {
                 const int bit = __ffs((int)m) - 1;
                 m &= m - 1;
@@ -442,7 +267,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
                     todo &= todo - 1;
                     const bool is_eq = (em >> e) & 1u;
                     if (!is_eq || t2 < r) {
-                        const int pos = fr.lo + a2 + min(t2, r) - fr.p0;
+                        const int pos = fr.hbase + a2 + min(t2, r);
                         if (pos >= 0 && pos < fr.n) s_list[pos] = j_lane + s * (HA_WAVE * 4) + e;
                     }
                     a2 += is_eq ? 0 : 1;
@@ -456,7 +281,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
     }
     // the last group of the round knows where the placed prefix ends
     const int last = min(n_groups - 1 - round * NW, NW - 1);
-    if (wave == last && lane == 0) *s_ready = fr.lo + a + (int)(tot & 0xFFFFu) + min(t + (int)(tot >> 16), r) - fr.p0;
+    if (wave == last && lane == 0) *s_ready = fr.hbase + a + (int)(tot & 0xFFFFu) + min(t + (int)(tot >> 16), r);
     __syncthreads();
     return *s_ready;
 }
@@ -465,7 +290,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
 // NT threads = NT/16 row streams; U rows per stream per step.
 template <typename E, int NT, int U, int FW>
-__global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
                                                            const int32_t *__restrict__ idx, int64_t idx_cap,
@@ -493,11 +318,13 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     int r0, r1, nsplit;
     const int32_t *ix = nullptr;
     FusedRow fr = {};
+    int j_max = 0;  // fused: last token of the sequence (list entries are clamped to it: a wrong entry must not become a wild address)
     if constexpr (FW > 0) {
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
         fr = fused_setup<NT>(fsel, row, S, sp, s_list, &s_cstar);
+        j_max = max(S - 1, 0);
         r0 = 0;
         r1 = fr.n;
         if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
@@ -547,7 +374,7 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
     // list position of (step base, u) for this stream; positions >= r1 are padded with the split's first row
     auto list_index = [&](int base, int u) {
         const int r = base + stream + u * NS;
-        if constexpr (FW > 0) return r < r1 ? s_list[r] : 0;  // padding: token 0, always present
+        if constexpr (FW > 0) return r < r1 ? min(max(s_list[r], 0), j_max) : 0;  // padding: token 0, always present
         else return ix[r < r1 ? r : r0];
     };
     int32_t j_next[U];   // indices of the step after the one in flight
@@ -619,15 +446,19 @@ __global__ __launch_bounds__(NT) void sparse_attend_kernel(const void *__restric
         // scan rounds and gather steps alternate: after a round the list is complete up to `ready`, and the loop runs
         // as far as its look-ahead (3 steps) allows.  Everything here is uniform over the workgroup.
         constexpr int NW = NT / HA_WAVE;
-        constexpr int GS = FW == 1 ? 4 : 2;  // slabs per wave and round: 16 VGPRs of codes on top of the loop's registers
-        const bool wide = true;
-        const int gc = GS * HA_WAVE * 4;
+        constexpr int GS = FW == 1 ? 8 : 4;  // slabs per wave and round
+        const bool wide = fsel.chunk % (GS * HA_WAVE * 4) == 0;  // else 1024-code chunks (short rows): 4 slabs
+        const int gc = (wide ? GS : 4) * HA_WAVE * 4;
         const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
         const int rounds = (n_groups + NW - 1) / NW;
         bool primed = false;
+        if (rounds > 0 && fr.nwin >= min(2 * STEP, r1)) {  // the windows alone fill the first two steps
+            prime();
+            primed = true;
+        }
         for (int k = 0; k < rounds; ++k) {
-            int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
-            (void)wide;
+            int ready = wide ? fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list)
+                             : fused_round<FW, 4, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
             if (k == rounds - 1) break;
             ready = min(ready, r1);
             if (!primed && ready >= min(2 * STEP, r1)) {

@@ -78,8 +78,10 @@ class HashDecodeLayer:
         self.counts = torch.zeros(B, self.H, dtype=torch.int32, device=dev)
         self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
         self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
-        self.fused_ok = _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget, self.recent_budget,
-                                           self.heavy_budget, self.mode)
+        # measured: the fused launch wins when a row is cut into at most two pieces (B * H >= 256 rows keep 256 CUs busy);
+        # with more, finer pieces the two-launch path is a few microseconds ahead
+        self.fused_ok = B * self.H >= 256 and _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget,
+                                                                 self.recent_budget, self.heavy_budget, self.mode)
         self.ws_fused = _ops.workspace(_ops.sparse_decode_fused_workspace_bytes(B, self.H, self.Hc, S_cap), dev)
         self.win = torch.empty(B, self.H, 130, dtype=torch.float32, device=dev)
         self.side_stream = torch.cuda.Stream(device=dev)

@@ -32,7 +32,8 @@ def test_three_decode_steps_match_reference_layer(hc, fused):
     layer = _layer(w, p)
     layer.allocate(w.batch, S)
     layer.use_fused = fused
-    assert layer.fused_ok
+    layer.fused_ok = _ops.fused_applies(w.batch, w.n_q_heads, hc, w.code_words, S, w.init_budget, w.recent_budget, w.heavy_budget)
+    assert layer.fused_ok             # small batches default to the two-launch path: force the fused one here
     s0 = S - 3
     layer.encode_keys(k[:, :, :s0])
     layer.n_cached = s0

@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the gather-attend kernel, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
 # summarised in profiles/decode_step_config2_hbm_traffic.md, each scaled on a 1 GiB copy (fetch x2.0, write x1.0).
-MEASURED_ATTEND_TRAFFIC_BYTES = {"config2": 551.4e6}
+MEASURED_ATTEND_TRAFFIC_BYTES = {("config2", True): 577.6e6, ("config2", False): 551.4e6}   # key: (workload, selection fused)
 
 
 def algorithmic_bytes(w, n_sel_rows):
@@ -182,7 +182,7 @@ def decoder_bench(args, torch):
         "prefill_encode_tflops": 2 * B * dec.Hc * (S - 1) * (128 * 128 * 2 + 128 * 32) / (ms_prefill_encode * 1e-3) / 1e12,
         "cache_fill_seconds": fill_s,
         "hbm_gbps_step": step_bytes / (ms_step * 1e-3) / 1e9, "hbm_frac_step": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
+        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
     }
@@ -345,7 +345,7 @@ def main():
         "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm",
                      "achieved": attend_bytes / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": attend_bytes / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get(w.name),
+                     "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get((w.name, bool(fused))),
                      "algorithmic_bytes": attend_bytes, "us": ms_attend * 1e3},
     }
     if not args.no_cpu_baseline:

@@ -99,6 +99,23 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
             if (l < n_layers) w += (int64_t)l_in[l] * l_out[l] + l_out[l];
         }
     }
+    // the inputs are requested first and parked in registers: memory returns loads in order, and the first layer then
+    // needs only them and its own weights, not the whole weight prefetch
+    constexpr int kXIter = (kRows * kMaxDim + kEncThreads - 1) / kEncThreads;
+    float xs[kXIter];
+#pragma unroll
+    for (int it = 0; it < kXIter; ++it) {
+        const int i = tid + it * kEncThreads;
+        xs[it] = 0.f;
+        if (i < kRows * d_in) {
+            const int r = i / d_in, e = i % d_in;
+            const int row = row0 + r;
+            if (row < n_rows) {
+                const int b = row / T, t = row % T;
+                xs[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
+            }
+        }
+    }
     float wreg[3][kMaxPerSeg];
 #pragma unroll
     for (int l = 0; l < 3; ++l) {
@@ -109,17 +126,10 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
 #pragma unroll
         for (int i = 0; i < kMaxPerSeg; ++i) wreg[l][i] = (active && i < per) ? wl[l][(int64_t)(seg * per + i) * out + o] : 0.f;
     }
-
-    for (int i = tid; i < kRows * d_in; i += kEncThreads) {
-        const int r = i / d_in, e = i % d_in;
-        const int row = row0 + r;
-        float val = 0.f;
-        if (row < n_rows) {
-            const int b = row / T, t = row % T;
-            val = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
-            if (arith == HA_ARITH_BF16) val = ha_round_bf16(val);
-        }
-        s_act[0][r][e] = val;
+#pragma unroll
+    for (int it = 0; it < kXIter; ++it) {
+        const int i = tid + it * kEncThreads;
+        if (i < kRows * d_in) s_act[0][i / d_in][i % d_in] = arith == HA_ARITH_BF16 ? ha_round_bf16(xs[it]) : xs[it];
     }
     __syncthreads();
 

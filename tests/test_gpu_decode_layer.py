@@ -72,3 +72,45 @@ def test_step_refuses_a_gap_in_the_bit_cache():
 def test_cpu_tensors_are_refused():
     with pytest.raises(ValueError):
         _ops.hamming_score(torch.zeros(1, 1, 4, 1, dtype=torch.int32), torch.zeros(1, 1, 1, dtype=torch.int32), 4)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_step_replayed_from_a_hip_graph_matches_eager(fused):
+    # the step allocates nothing and reads its lengths from arguments, so it can be captured; every replay, with eager
+    # work and synchronisations in between, must reproduce the eager output bit for bit
+    print(f"\n[case] graph replay fused={fused}", flush=True)
+    w = small_workload(batch=8, seq_lens=[3000] * 8, n_q_heads=32, n_kv_heads=8, n_code_heads=8, seed=23)
+    p = make_problem(w)
+    S = w.max_seq_len
+    k, v, q = p.k.to(DEV), p.v.to(DEV), p.q.to(DEV)
+    layer = _layer(w, p)
+    layer.allocate(w.batch, S)
+    layer.use_fused = fused
+    assert layer.fused_ok
+    layer.encode_keys(k[:, :, :S - 1])
+    out = torch.empty(w.batch, w.n_q_heads, w.head_dim, dtype=w.dtype, device=DEV)
+
+    def step():
+        layer.n_cached = S - 1
+        layer.step(q, k, v, S, out)
+
+    step()
+    want = out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(4):
+        out.zero_()
+        layer.counts.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), i
+        scratch = torch.randn(1 << 20, device=DEV).sum().item()     # unrelated eager work between replays
+        assert scratch == scratch

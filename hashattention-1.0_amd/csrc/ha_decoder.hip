@@ -1,10 +1,188 @@
 // The two elementwise steps of a decoder layer that sit right against the attention step, each as one launch:
 //   ha_rope_append  rotate-half RoPE of the new token's q and k, k and v written into the caches in place
 //   ha_swiglu       silu(gate) * up of the feed-forward block
-// Both are a few hundred KB of traffic: latency-bound, one element pair / element per thread.
+//   ha_linear_skinny  y = x W^T (+ residual) for a handful of rows (one token per sequence): streams W once
+// The first two are a few hundred KB of traffic: latency-bound, one element pair / element per thread.
 #include "ha_common.h"
 
 namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// y[m, n] = sum_k x[m, k] W[n, k] (+ res[m, n]), bf16 in, fp32 accumulate, bf16 out, M <= 16.  HBM-bound on W
+// (2 N K bytes, read once).  One workgroup owns 16 consecutive output columns n; its NWAVE waves split K.  A wave
+// feeds v_mfma_f32_16x16x32_bf16 with A = the 16 rows of W (lane: row l % 16, 8 consecutive k at 8 (l / 16)) and
+// B = x^T padded to 16 columns, so a wave load brings 64 contiguous bytes of each of the 16 rows and two consecutive
+// loads complete every 128-byte line.  Loads of the next four k-steps are in flight while the current four are
+// multiplied (4 KiB of W per wave, 64 KiB per CU with two workgroups resident).  The matrix unit is idle most of
+// the time at these shapes: it is there to keep the VALU out of the way of the loads.
+// ------------------------------------------------------------------------------------------------
+// Row-streaming form of the same product for M <= 8 and K <= 16384 (every projection of a decode step).
+// A workgroup owns RB consecutive rows of W; its NWAVE waves cut K into slices of XCH chunks of 512 elements, and a
+// wave keeps its slice of x (M x XCH x 16 bytes per lane) in registers for the whole workgroup.  A wave load is then
+// one contiguous KiB of one row of W, the waves of a workgroup together read whole rows front to back, and the next
+// R rows are in flight while R rows are multiplied (a third stage in flight cost occupancy and was slower) (v_dot2c_f32_bf16: two MACs per lane and instruction, no
+// unpacking).  The R x MM per-lane sums are folded with a reduce-scatter inside each quad (two DPP stages, the
+// value count halving at each) and two row rotations, so a 16-lane row ends with each sum once; rows of lanes and
+// waves meet in LDS.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float dot8(const uint4 &a, const uint4 &b, float c) {
+    c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.x), __builtin_bit_cast(bf16x2, b.x), c, false);
+    c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.y), __builtin_bit_cast(bf16x2, b.y), c, false);
+    c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), __builtin_bit_cast(bf16x2, b.z), c, false);
+    c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), c, false);
+    return c;
+}
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+template <int NWAVE, int XCH, int R, int MM>
+__global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *__restrict__ x, int64_t x_sm,
+                                                               const uint16_t *__restrict__ w, int64_t w_sn,
+                                                               const uint16_t *__restrict__ res, int64_t res_sm,
+                                                               uint16_t *__restrict__ out, int64_t out_sm, int M, int N, int K, int RB) {
+    constexpr int NV = R * MM;       // sums per lane and row group: 8 or 16
+    constexpr int NP = NWAVE * 4;    // partials per sum: one per 16-lane row of every wave
+    extern __shared__ float s_part[];  // [RB * MM][NP]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int n0 = blockIdx.x * RB;
+    const int nrows = min(RB, N - n0);
+    const int kbase = wave * XCH * 512 + lane * 8;  // first element of this lane's 16 bytes in chunk 0 of its slice
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+
+    uint4 xr[XCH][MM];
+#pragma unroll
+    for (int c = 0; c < XCH; ++c)
+#pragma unroll
+        for (int m = 0; m < MM; ++m) {
+            const int k = kbase + c * 512;
+            xr[c][m] = (m < M && k < K) ? *reinterpret_cast<const uint4 *>(x + (int64_t)m * x_sm + k) : zero;
+        }
+
+    uint4 wc[R][XCH], wn[R][XCH];
+    auto fetch = [&](int r0, uint4 (&wv)[R][XCH]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < XCH; ++c) {
+                const int k = kbase + c * 512;
+                wv[r][c] = (r0 + r < nrows && k < K) ? *reinterpret_cast<const uint4 *>(w + (int64_t)(n0 + r0 + r) * w_sn + k) : zero;
+            }
+    };
+    fetch(0, wc);
+    for (int r0 = 0; r0 < nrows; r0 += R) {
+        if (r0 + R < nrows) fetch(r0 + R, wn);
+        float v[NV];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < MM; ++m) {
+                float a = 0.f;
+#pragma unroll
+                for (int c = 0; c < XCH; ++c) a = dot8(wc[r][c], xr[c][m], a);
+                v[r * MM + m] = a;
+            }
+        // reduce-scatter inside the quad: after stage 0 a lane holds the pair sums of the values with index bit 0 equal
+        // to its lane bit 0, after stage 1 the quad sums of the values i with i % 4 == lane % 4
+        float u[NV / 2], t[NV / 4];
+        const bool b0 = lane & 1, b1 = lane & 2;
+#pragma unroll
+        for (int j = 0; j < NV / 2; ++j) {
+            const float keep = b0 ? v[2 * j + 1] : v[2 * j], send = b0 ? v[2 * j] : v[2 * j + 1];
+            u[j] = keep + dpp_f<0xB1>(send);  // quad_perm [1,0,3,2]
+        }
+#pragma unroll
+        for (int j = 0; j < NV / 4; ++j) {
+            const float keep = b1 ? u[2 * j + 1] : u[2 * j], send = b1 ? u[2 * j] : u[2 * j + 1];
+            t[j] = keep + dpp_f<0x4E>(send);  // quad_perm [2,3,0,1]
+        }
+        // the four quads of a 16-lane row: rotations by 4 and 8 keep lane % 4
+#pragma unroll
+        for (int j = 0; j < NV / 4; ++j) {
+            t[j] += dpp_f<0x124>(t[j]);  // row_ror:4
+            t[j] += dpp_f<0x128>(t[j]);  // row_ror:8
+        }
+        if ((lane & 12) == 0) {  // lanes 0..3 of each row: value i = 4 j + lane % 4 of this row group
+            const int p = wave * 4 + (lane >> 4), q = lane & 3;
+#pragma unroll
+            for (int j = 0; j < NV / 4; ++j) {
+                const int i = 4 * j + q, r = i / MM, m = i % MM;
+                s_part[((r0 + r) * MM + m) * NP + p] = t[j];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < XCH; ++c) wc[r][c] = wn[r][c];
+    }
+    __syncthreads();
+    for (int o = tid; o < nrows * M; o += NWAVE * 64) {
+        const int m = o / nrows, r = o % nrows;  // consecutive threads write consecutive columns of y
+        const float *pp = s_part + (r * MM + m) * NP;
+        float y = 0.f;
+#pragma unroll 8
+        for (int p = 0; p < NP; ++p) y += pp[p];
+        if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + r] << 16);
+        out[(int64_t)m * out_sm + n0 + r] = (uint16_t)ha_f32_to_bf16_bits(y);
+    }
+}
+
+template <int NWAVE>
+__global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_t *__restrict__ x, int64_t x_sm,
+                                                                   const uint16_t *__restrict__ w, int64_t w_sn,
+                                                                   const uint16_t *__restrict__ res, int64_t res_sm,
+                                                                   uint16_t *__restrict__ out, int64_t out_sm, int M, int N, int K) {
+    constexpr int PF = 4;
+    __shared__ float s_c[NWAVE][16][17];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int n = min(n0 + r, N - 1);
+    const int steps = K / 32;                                   // k-steps of 32
+    const int per = ((steps + NWAVE - 1) / NWAVE + PF - 1) / PF * PF;  // per wave, whole groups of PF
+    const int s_beg = wave * per, s_end = min(s_beg + per, steps);
+    const uint4 *wp = reinterpret_cast<const uint4 *>(w + (int64_t)n * w_sn) + g;
+    const uint4 *xp = reinterpret_cast<const uint4 *>(x + (int64_t)min(r, M - 1) * x_sm) + g;
+    const bool x_ok = r < M;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    uint4 wc[PF], xc[PF], wn[PF], xn[PF];
+    auto fetch = [&](int s0, uint4 (&wv)[PF], uint4 (&xv)[PF]) {
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            const bool ok = s0 + i < s_end;
+            wv[i] = ok ? wp[(int64_t)(s0 + i) * 4] : zero;
+            xv[i] = (ok && x_ok) ? xp[(int64_t)(s0 + i) * 4] : zero;
+        }
+    };
+    if (s_beg < s_end) fetch(s_beg, wc, xc);
+    for (int s0 = s_beg; s0 < s_end; s0 += PF) {
+        if (s0 + PF < s_end) fetch(s0 + PF, wn, xn);
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wc[i]), __builtin_bit_cast(bf16x8, xc[i]), acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            wc[i] = wn[i];
+            xc[i] = xn[i];
+        }
+    }
+    // acc[i] = C[row 4 g + i (the column n0 + 4 g + i of y)][col r (the row m of y)]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_c[wave][4 * g + i][r] = acc[i];
+    __syncthreads();
+    for (int t = tid; t < 16 * M; t += NWAVE * 64) {
+        const int m = t >> 4, nl = t & 15;
+        if (n0 + nl >= N) continue;
+        float y = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < NWAVE; ++wv) y += s_c[wv][nl][m];
+        if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + nl] << 16);
+        out[(int64_t)m * out_sm + n0 + nl] = (uint16_t)ha_f32_to_bf16_bits(y);
+    }
+}
 
 __device__ __forceinline__ void store_elem(void *p, int64_t i, float x, int dtype) {
     if (dtype == HA_F32) reinterpret_cast<float *>(p)[i] = x;
@@ -85,6 +263,56 @@ int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, i
     if (st) return st;
     hipLaunchKernelGGL(swiglu_kernel, dim3((F + 255) / 256, B), dim3(256), 0, (hipStream_t)stream, gate_up, gate_up_stride_b, dtype, F, out);
     HA_CHECK_LAUNCH("swiglu_kernel");
+    return HA_OK;
+}
+
+int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
+                     int64_t residual_stride_m, void *out, int64_t out_stride_m, int M, int N, int K, void *stream) {
+    HA_REQUIRE(x && w && out, HA_ERR_NULL_POINTER, "x/w/out is NULL");
+    HA_REQUIRE(M >= 1 && M <= 16 && N >= 1 && K >= 32 && K % 32 == 0, HA_ERR_BAD_SHAPE, "need 1 <= M <= 16, N >= 1, K a multiple of 32");
+    HA_REQUIRE(x_stride_m >= K && w_stride_n >= K && out_stride_m >= N && (!residual || residual_stride_m >= N), HA_ERR_BAD_SHAPE,
+               "strides smaller than the rows they span");
+    HA_REQUIRE(ha_aligned(x, 16) && ha_aligned(w, 16) && x_stride_m % 8 == 0 && w_stride_n % 8 == 0, HA_ERR_MISALIGNED,
+               "x and W rows must be 16-byte aligned");
+    int st = ha_require_device();
+    if (st) return st;
+    const uint16_t *xp = (const uint16_t *)x, *wp = (const uint16_t *)w, *rp = (const uint16_t *)residual;
+    uint16_t *op = (uint16_t *)out;
+    hipStream_t s = (hipStream_t)stream;
+    if (M <= 8 && K <= 16384) {
+        // rows per workgroup: enough workgroups for two per CU, but at least 16 rows so that the slice of x a wave keeps
+        // is paid for
+        const int RB = (int64_t)N >= 64 * 1024 ? 64 : (int64_t)N >= 32 * 512 ? 32 : 16;
+        const dim3 g2((N + RB - 1) / RB);
+        const int chunks = (K + 511) / 512;
+#define HA_GEMV(NW_, XCH_, R_, MM_)                                                                                          \
+    hipLaunchKernelGGL((gemv_rows_kernel<NW_, XCH_, R_, MM_>), g2, dim3(NW_ * 64), (size_t)RB * MM_ * NW_ * 4 * sizeof(float), s, \
+                       xp, x_stride_m, wp, w_stride_n, rp, residual_stride_m, op, out_stride_m, M, N, K, RB)
+        if (chunks <= 8) {
+            if (M <= 4) HA_GEMV(8, 1, 4, 4);
+            else HA_GEMV(8, 1, 2, 8);
+        } else if (chunks <= 16) {
+            if (M <= 4) HA_GEMV(16, 1, 4, 4);
+            else HA_GEMV(16, 1, 2, 8);
+        } else {
+            if (M <= 4) HA_GEMV(16, 2, 2, 4);
+            else HA_GEMV(16, 2, 1, 8);
+        }
+#undef HA_GEMV
+        HA_CHECK_LAUNCH("gemv_rows_kernel");
+        return HA_OK;
+    }
+    const dim3 grid((N + 15) / 16);
+    // few output columns: split K eight ways so that the grid still covers the CUs with enough loads in flight
+    if ((int64_t)N * 4 < 16 * 4096)
+        hipLaunchKernelGGL(skinny_linear_kernel<8>, grid, dim3(512), 0, (hipStream_t)stream, (const uint16_t *)x, x_stride_m,
+                           (const uint16_t *)w, w_stride_n, (const uint16_t *)residual, residual_stride_m, (uint16_t *)out, out_stride_m,
+                           M, N, K);
+    else
+        hipLaunchKernelGGL(skinny_linear_kernel<4>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x, x_stride_m,
+                           (const uint16_t *)w, w_stride_n, (const uint16_t *)residual, residual_stride_m, (uint16_t *)out, out_stride_m,
+                           M, N, K);
+    HA_CHECK_LAUNCH("skinny_linear_kernel");
     return HA_OK;
 }
 

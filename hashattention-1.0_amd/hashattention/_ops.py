@@ -69,6 +69,8 @@ def load_library() -> C.CDLL:
                               vp, i64, vp, vp, sz, vp]
     lib.ha_rope_append.restype = i32
     lib.ha_rope_append.argtypes = [vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]
+    lib.ha_linear_skinny.restype = i32
+    lib.ha_linear_skinny.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
     lib.ha_swiglu.restype = i32
     lib.ha_swiglu.argtypes = [vp, i64, i32, i32, i32, vp, vp]
     lib.ha_select_prepare.restype = i32
@@ -364,3 +366,17 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and out.is_contiguous() and out.dtype == gate_up.dtype
     B, F = out.shape
     _check(load_library().ha_swiglu(_ptr(gate_up), gate_up.stride(0), _DTYPE[gate_up.dtype], B, F, _ptr(out), _stream(gate_up)), "ha_swiglu")
+
+
+def linear_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out [M, N] = x [M, K] @ w[N, K]^T (+ residual [M, N]); bf16, M <= 16.  Streams w once."""
+    _require_cuda(x, w, out, residual)
+    assert x.dtype == w.dtype == out.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2 and out.dim() == 2
+    assert x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1 and (residual is None or (residual.stride(1) == 1 and residual.dtype == x.dtype))
+    M, K = x.shape
+    N = w.shape[0]
+    assert w.shape[1] == K and out.shape == (M, N) and (residual is None or residual.shape == (M, N))
+    _check(load_library().ha_linear_skinny(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual),
+                                           residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0), M, N, K,
+                                           _stream(x)), "ha_linear_skinny")
+    return out

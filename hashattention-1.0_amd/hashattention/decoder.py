@@ -3,9 +3,10 @@
 The reference measures end-to-end decode throughput with a gpt-fast fork (efficiency/generate.py:386-434,
 efficiency/model.py:98-345: RMSNorm, rotary embedding, SwiGLU feed-forward, static KV cache).  That fork is not
 runnable as shipped and drives Double-Sparsity labels, not hashes; this module is the same decoder shape with
-the HashAttention step in every layer.  Outside attention the GEMMs and RMSNorm are library calls (hipBLASLt,
-`F.rms_norm`); RoPE + cache append and SwiGLU are one launch each (`ha_rope_append`, `ha_swiglu`) and the residual adds
-ride in the GEMMs: the point is to time the whole step, and to check the plumbing around the op
+the HashAttention step in every layer.  Outside attention: RMSNorm, the down projection and the lm_head are library
+calls (`F.rms_norm`, hipBLASLt); the QKV, output and gate/up projections go through `ha_linear_skinny` when the batch
+is at most 8 rows of bf16; RoPE + cache append and SwiGLU are one launch each (`ha_rope_append`, `ha_swiglu`); the
+residual adds ride in the projections: the point is to time the whole step, and to check the plumbing around the op
 (rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
 
 Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no
@@ -30,6 +31,7 @@ class LlamaShapedDecoder:
         self.L, self.hidden, self.ffn, self.H, self.Hkv, self.d, self.vocab = n_layers, hidden, ffn, n_heads, n_kv_heads, head_dim, vocab
         self.theta, self.eps, self.dtype, self.device = rope_theta, rms_eps, dtype, torch.device(device)
         self.Hc = n_code_heads
+        self.use_skinny = True   # ha_linear_skinny for the projections it is faster for (bf16, batch <= 8)
         self.usa_shape = (lth_num_layers, lth_int_dim, lth_final_dim)
         self.budgets = (init_budget, recent_budget, heavy_budget)
         g = torch.Generator(device=device).manual_seed(seed)
@@ -84,6 +86,9 @@ class LlamaShapedDecoder:
         self.attn_out = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
         self.q_rot = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
         self.ffn_act = torch.empty(B, self.ffn, dtype=self.dtype, device=self.device)
+        self.qkv = torch.empty(B, (self.H + 2 * self.Hkv) * self.d, dtype=self.dtype, device=self.device)
+        self.x_attn = torch.empty(B, self.hidden, dtype=self.dtype, device=self.device)
+        self.gate_up = torch.empty(B, 2 * self.ffn, dtype=self.dtype, device=self.device)
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
@@ -128,9 +133,12 @@ class LlamaShapedDecoder:
         pos = self.seq_len
         S = pos + 1
         x = self.embed[tokens]                                            # [B, hidden]
+        # the row-streaming kernel measured faster than the library GEMM for the QKV, output and gate/up projections
+        # (2.6 -> 3.3, 1.8 -> 3.0, 4.0 -> 4.4 TB/s at B = 4) and slower for the down projection and the lm_head
+        skinny = self.use_skinny and self.dtype == torch.bfloat16 and B <= 8
         for l, p in enumerate(self.layers):
             h = F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps)
-            qkv = F.linear(h, p["wqkv"])
+            qkv = _ops.linear_skinny(h, p["wqkv"], self.qkv) if skinny else F.linear(h, p["wqkv"])
             _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
             hl = self.hash[l]
             if dense:
@@ -138,9 +146,12 @@ class LlamaShapedDecoder:
             else:
                 hl.n_cached = pos
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
-            x = torch.addmm(x, self.attn_out.view(B, H * d), p["wo"].t())
+            if skinny:
+                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn, residual=x)
+            else:
+                x = torch.addmm(x, self.attn_out.view(B, H * d), p["wo"].t())
             h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
-            _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
+            _ops.swiglu(_ops.linear_skinny(h, p["w13"], self.gate_up) if skinny else F.linear(h, p["w13"]), self.ffn_act)
             x = torch.addmm(x, self.ffn_act, p["w2"].t())
         if advance:
             self.seq_len = S

@@ -251,6 +251,15 @@ int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int 
                    const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
                    int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, void *stream);
 int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, int F, void *out, void *stream);
+/*
+ * out[m, n] = sum_k x[m, k] * w[n, k] (+ residual[m, n]): a Linear layer (weight [N, K] as nn.Linear keeps it) applied to
+ * M <= 16 rows, bf16 in and out, fp32 accumulation.  The decode step's projections (efficiency/model.py:236, 261,
+ * 304-305: wqkv, wo, w1/w3, w2, and the lm_head of :158) are this shape: they stream every weight once per token, so
+ * the kernel is bound by HBM.  K must be a multiple of 32, rows 16-byte aligned; strides in elements.
+ */
+int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n,
+                     const void *residual, int64_t residual_stride_m, void *out, int64_t out_stride_m,
+                     int M, int N, int K, void *stream);
 
 #ifdef __cplusplus
 }

@@ -162,6 +162,10 @@ def test_arguments_are_validated_before_any_device_work(lib):
 
     assert rope(f=null) == HA_ERR_NULL and rope(dt=7) == HA_ERR_DTYPE
     assert rope(sb=512) == HA_ERR_SHAPE and rope(pos=100) == HA_ERR_SHAPE and rope(pos=-1) == HA_ERR_SHAPE and rope(kss=64) == HA_ERR_SHAPE
+    lin = lambda **kw: lib.ha_linear_skinny(*[{**dict(x=p, xs=4096, w=p, ws=4096, r=null, rs=0, o=p, os=4096, M=4, N=4096, K=4096, st=null), **kw}[k]
+                                              for k in ("x", "xs", "w", "ws", "r", "rs", "o", "os", "M", "N", "K", "st")])
+    assert lin(w=null) == HA_ERR_NULL and lin(M=17) == HA_ERR_SHAPE and lin(K=100) == HA_ERR_SHAPE and lin(ws=100) == HA_ERR_SHAPE
+    assert lin(x=odd) == HA_ERR_ALIGN and lin(xs=4100) == HA_ERR_ALIGN and lin(r=p, rs=10) == HA_ERR_SHAPE
     assert lib.ha_swiglu(null, 64, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_NULL
     assert lib.ha_swiglu(p, 63, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_SHAPE and lib.ha_swiglu(p, 64, 9, 1, 32, p, null) == HA_ERR_DTYPE
 

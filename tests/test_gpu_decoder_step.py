@@ -96,3 +96,45 @@ def test_rope_append_and_swiglu_against_torch(dtype):
     _ops.swiglu(gu, out)
     want = torch.nn.functional.silu(gu[:, :F_]) * gu[:, F_:]
     assert (out.float() - want.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(4, 4096, 4096), (1, 1000, 512), (16, 6144, 4096), (4, 4096, 14336), (3, 20, 64), (4, 128256, 1024),
+                                   (8, 4100, 4096), (5, 333, 8192), (7, 50, 14336), (2, 4096, 16416), (12, 77, 96)])
+def test_linear_skinny_against_fp32_matmul(M, N, K):
+    # bf16 inputs, fp32 accumulation: against the fp32 product of the same bf16 values, one bf16 rounding of the result apart
+    print(f"\n[case] linear_skinny {M}x{N}x{K}", flush=True)
+    from hashattention import _ops
+    g = torch.Generator(device=DEV).manual_seed(M * 7 + N)
+    x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device=DEV) * K ** -0.5).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g, device=DEV).to(torch.bfloat16)
+    want = x.float() @ w.float().t()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    _ops.linear_skinny(x, w, out)
+    assert (out.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+    assert torch.equal(out, want.to(torch.bfloat16)) or (out.float() - want.to(torch.bfloat16).float()).abs().max().item() <= 2 ** -6
+    _ops.linear_skinny(x, w, out, residual=res)
+    want2 = want + res.float()
+    assert (out.float() - want2).abs().max().item() <= 2e-2 * max(1.0, want2.abs().max().item())
+    # strided views (a slice of a wider buffer) for x and out
+    xw = torch.zeros(M, K + 64, dtype=torch.bfloat16, device=DEV)
+    xw[:, :K] = x
+    ow = torch.zeros(M, N + 8, dtype=torch.bfloat16, device=DEV)
+    _ops.linear_skinny(xw[:, :K], w, ow[:, :N])
+    assert (ow[:, :N].float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item()) and (ow[:, N:] == 0).all()
+
+
+def test_bf16_decoder_step_with_and_without_the_skinny_projections():
+    # the bf16 step routes three projections through ha_linear_skinny; with the library GEMMs instead the logits agree to bf16 noise
+    print("\n[case] bf16 decoder step, skinny projections on/off", flush=True)
+    dec = LlamaShapedDecoder(n_layers=2, hidden=512, ffn=1024, n_heads=4, n_kv_heads=2, head_dim=128, vocab=512, n_code_heads=2,
+                             init_budget=8, recent_budget=8, heavy_budget=0.125, dtype=torch.bfloat16, device=DEV, seed=3)
+    dec.allocate(2, 400)
+    dec.fill_cache_synthetic(300)
+    tokens = torch.tensor([5, 17], device=DEV)
+    with torch.no_grad():
+        a = dec.decode_step(tokens, advance=False).float()
+        dec.use_skinny = False
+        b = dec.decode_step(tokens, advance=False).float()
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())

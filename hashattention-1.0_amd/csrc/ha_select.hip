@@ -316,7 +316,8 @@ int validate_codes(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, const u
     HA_REQUIRE(H % Hc == 0, HA_ERR_BAD_SHAPE, "H=%d not a multiple of Hc=%d", H, Hc);
     const int gq = H / Hc;
     HA_REQUIRE(gq == 1 || gq == 2 || gq == 4 || gq == 8, HA_ERR_BAD_SHAPE, "H/Hc=%d, must be 1, 2, 4 or 8", gq);
-    HA_REQUIRE(kc_sh >= (int64_t)max_seq_len * W && kc_sb >= kc_sh, HA_ERR_BAD_SHAPE, "code strides smaller than the rows they span");
+    HA_REQUIRE(kc_sh >= (int64_t)max_seq_len * W && (kc_sb >= kc_sh || kc_sb == 0), HA_ERR_BAD_SHAPE,
+               "code strides smaller than the rows they span");
     HA_REQUIRE((int64_t)max_seq_len <= (int64_t)kMaxChunks * kMaxBlocks * kBlock, HA_ERR_BAD_SHAPE, "max_seq_len above %d",
                kMaxChunks * kMaxBlocks * kBlock);
     HA_REQUIRE(ha_aligned(kcodes, 4 * W) && ha_aligned(qcodes, 4) && (W == 1 || (kc_sb % 2 == 0 && kc_sh % 2 == 0)),

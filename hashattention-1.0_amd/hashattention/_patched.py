@@ -11,8 +11,9 @@ What differs from the reference on purpose
   * softmax and the value product are fp32 throughout (the reference rounds probabilities to the query
     dtype at :613);
   * soft mode (`hard=False`: tanh / sigmoid, :174-176, 197-198), `CENTER` normalisation (:163-167), the LSH
-    baseline (`lth_num_layers == 0`, :130-139) and the training / statistics hooks (:304-398) are outside
-    the accelerated path and raise NotImplementedError instead of silently running something else.
+    baseline (`lth_num_layers == 0`, :130-139) and the training hooks (:304-316 and the train branch of :370-371)
+    are outside the accelerated path and raise NotImplementedError instead of silently running something else;
+    the recall statistic (:319-398, eval branch) is built on the selection kernel (`usa_local_compute`).
 """
 from __future__ import annotations
 
@@ -204,8 +205,11 @@ class HeavyHitterMixin:
             if self.train_usa:
                 raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
             # prefill: the original dense forward (reference :529-550); its keys are hashed lazily at the first decode step
-            return self.flash_forward(hidden_states=hidden_states, position_embeddings=position_embeddings,
-                                      attention_mask=attention_mask, past_key_values=cache, **kwargs)
+            ret = self.flash_forward(hidden_states=hidden_states, position_embeddings=position_embeddings,
+                                     attention_mask=attention_mask, past_key_values=cache, **kwargs)
+            if self.collect_stats:
+                self.usa_local_compute(hidden_states, attention_mask, None, cache, position_embeddings)
+            return ret
         hidden_shape = (bsz, q_len, -1, self.head_dim)
         query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
         key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
@@ -259,8 +263,80 @@ class HeavyHitterMixin:
     def train_step(self, *a, **k):
         raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
 
-    def usa_local_compute(self, *a, **k):
-        raise NotImplementedError("recall statistics / training targets are outside this build")
+    def usa_local_compute(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None,
+                          position_embeddings=None):
+        """Recall statistic of the hash ranking (reference :319-398, eval branch): whenever the cache length is a multiple
+        of 1024, for every query row of this chunk, which fraction of its 32 highest true attention logits among the
+        candidates [init, pos - recent] is inside the S // 16 candidates of smallest Hamming distance.  Accumulated per
+        cache length in `self.overlaps[S] = [sum, sum of squares, count, mean, std]` as the reference does.
+
+        The hash side runs on the selection kernel: all rows of the chunk in one ha_select call against the same codes
+        (batch stride 0), each row with its own length.  Ties of the hash score go to the lowest index (the reference's
+        torch.topk leaves them open); rows with fewer than 32 candidates count only real candidates as targets."""
+        if self.train_usa:
+            raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
+        cache = past_key_value
+        if cache is None or len(cache.layers) <= self.layer_idx:
+            return
+        keys = cache.layers[self.layer_idx].keys                        # [b, Hkv, S, d], the chunk's keys already appended
+        if keys is None or keys.shape[-2] % 1024 != 0:
+            return
+        bsz, q_len, _ = hidden_states.shape
+        S = keys.shape[-2]
+        H, d = self.num_heads, self.head_dim
+        shape = (bsz, q_len, -1, d)
+        q = self.q_proj(hidden_states).view(shape).transpose(1, 2)
+        k_new = self.k_proj(hidden_states).view(shape).transpose(1, 2)
+        cos, sin = position_embeddings
+        q, _ = self._apply_rope(q, k_new, cos, sin)
+        q = q.contiguous()
+        keys = keys if keys.stride(-1) == 1 else keys.contiguous()
+        dev = q.device
+
+        # ---- hash side: codes of all keys and of every query row, one selection per row
+        hl = self._ensure_hash_layer(bsz, S, dev)
+        kc = torch.zeros(bsz, hl.Hc, S, hl.W, dtype=torch.int32, device=dev)
+        _ops.encode_pack(keys, hl.wk, hl.num_layers, hl.int_dim, hl.final_dim, kc, 0, None, hl.arith)
+        qc = torch.zeros(bsz, H, q_len, hl.W, dtype=torch.int32, device=dev)
+        _ops.encode_pack(q, hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
+        n_pred = S // 16
+        if n_pred < 2:                                  # a heavy budget <= 1 would be read as a fraction
+            return
+        cap = min(S, self.init_budget + self.recent_budget + n_pred)
+        lens = torch.arange(S - q_len + 1, S + 1, dtype=torch.int32, device=dev)      # row i sees keys [0, S - q_len + i]
+        ws = _ops.workspace(_ops.select_workspace_bytes(q_len, H, hl.Hc, hl.W, S), dev)
+        idx = torch.empty(q_len, H, cap, dtype=torch.int32, device=dev)
+        cnt = torch.empty(q_len, H, dtype=torch.int32, device=dev)
+        scale = 1.0 / math.sqrt(d)
+        top_true = 32
+        ratios = []
+        for b in range(bsz):
+            _ops.select(kc[b:b + 1].expand(q_len, -1, -1, -1), qc[b].transpose(0, 1).contiguous(), S, lens, self.init_budget,
+                        self.recent_budget, float(n_pred) + 0.5, idx, cnt, ws)
+            # lists are ascending; everything past the count becomes a sentinel so that a binary search can test membership
+            pos = torch.arange(cap, device=dev)
+            lists = torch.where(pos[None, None, :] < cnt[:, :, None], idx, torch.full_like(idx, 2 ** 31 - 1))
+            # ---- true side (reference :357-366): logits of the candidates, top 32
+            kk = keys[b].repeat_interleave(self.num_key_value_groups, dim=0).float()             # [H, S, d]
+            logits = torch.matmul(q[b].float(), kk.transpose(1, 2)) * scale                       # [H, q_len, S]
+            j = torch.arange(S, device=dev)
+            cand = (j[None, :] >= self.init_budget) & (j[None, :] <= (lens[:, None] - 1 - self.recent_budget))   # [q_len, S]
+            logits = logits.masked_fill(~cand[None], float("-inf"))
+            kt = min(top_true, S)
+            top = torch.topk(logits, kt, dim=-1)
+            tgt = top.indices.transpose(0, 1).contiguous().to(torch.int32)                       # [q_len, H, kt]
+            real = torch.isfinite(top.values).transpose(0, 1)
+            where = torch.searchsorted(lists, tgt).clamp_(max=cap - 1)
+            hit = (torch.gather(lists, 2, where) == tgt) & real
+            ratios.append(hit.sum(-1).float() / top_true)                                         # [q_len, H]
+        r = torch.stack(ratios)                                                                  # [b, q_len, H]
+        st = self.overlaps.setdefault(S, [0, 0, 0, 0, 0])                                        # sum, sqsum, ct, mean, std
+        st[0] += r.sum().item()
+        st[1] += torch.square(r).sum().item()
+        st[2] += r.numel()
+        st[3] = st[0] / st[2]
+        st[4] = math.sqrt(max(st[1] / st[2] - st[3] ** 2, 0.0))
+        self.last_overlap_ratio = r.permute(0, 2, 1)                                             # [b, H, q_len], for tests
 
 
 # ------------------------------------------------------------------------------------------ module-patch helpers

@@ -143,6 +143,9 @@ int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
  *   out_idx    int32 [B, H, idx_cap]: ascending token indices; nothing is written past idx_cap
  *   out_counts int32 [B, H]: number selected (the true count, even if it exceeds idx_cap)
  *   workspace  ha_select_workspace_bytes(...) bytes, 256-byte aligned
+ * kc_stride_b may be 0: every batch entry then reads the same codes, i.e. B queries (each with its own row of
+ * qcodes and its own seq_lens[b]) against one sequence - the rows of a multi-token chunk
+ * (hashattention_llama.py:423-428) or of the recall statistic (:319-398) in one call.
  */
 size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len);
 int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,

@@ -299,3 +299,39 @@ def reference_decode_attention(Q, K, V, k_heads, q_heads, init_budget, recent_bu
     span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype))
     mask = compute_mask_multi(span, init_budget, recent_budget, heavy_budget, mode, retrieve_depth, stable)
     return masked_decode_attention(Q, Kr, Vr, mask), mask
+
+
+def recall_overlap(q: torch.Tensor, k: torch.Tensor, k_heads, q_heads, init_budget: int, recent_budget: int,
+                   top_true: int = 32) -> torch.Tensor:
+    """The recall statistic of the reference's `usa_local_compute` (hashattention_llama.py:357-386): for every query row,
+    the fraction of its `top_true` highest-scoring candidate keys (true attention logits) that are among the S // 16
+    candidates of highest hash score.  q [b, H, q_len, d] are the last q_len positions of the S cached keys k
+    [b, Hkv, S, d]; candidates of row i are j in [init, i + S - q_len - recent].  Returns [b, H, q_len] float.
+
+    Two points where the reference is not fully specified are fixed here: ties of the hash score are broken by lowest
+    index (its torch.topk leaves them open), and rows with fewer than `top_true` candidates count only real
+    candidates as targets (its top-k would pad the target with masked positions) while still dividing by `top_true`.
+    """
+    b, H, q_len, d = q.shape
+    S = k.shape[2]
+    kk = repeat_kv(k.float(), H // k.shape[1])
+    logits = torch.matmul(q.float(), kk.transpose(2, 3)) / math.sqrt(d)                     # :358
+    cand = torch.tril(torch.ones(q_len, S), diagonal=S - q_len - recent_budget).bool()      # :360
+    cand[:, :init_budget] = False                                                            # :361
+    span, _ = usa_forward_hard(kk, q.float(), k_heads if len(k_heads) == H else [k_heads[h // (H // len(k_heads))] for h in range(H)],
+                               q_heads)
+    out = torch.zeros(b, H, q_len)
+    n_pred = S // 16                                                                         # :375
+    for i in range(q_len):
+        js = torch.nonzero(cand[i]).flatten()
+        if js.numel() == 0:
+            continue
+        for bb in range(b):
+            for h in range(H):
+                lg = logits[bb, h, i, js]
+                true_top = js[torch.topk(lg, min(top_true, js.numel())).indices]
+                sp = span[bb, h, i, js]
+                order = sorted(range(js.numel()), key=lambda t: (-float(sp[t]), int(js[t])))[:n_pred]
+                pred = set(int(js[t]) for t in order)
+                out[bb, h, i] = sum(1 for j in true_top.tolist() if j in pred) / float(top_true)
+    return out

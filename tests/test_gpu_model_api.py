@@ -131,3 +131,43 @@ def test_usa_forward_and_mask_api():
     mask = layer.compute_mask_multi(K, Q)
     mask_ref = orc.compute_mask_multi(span_ref, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget)
     assert torch.equal(mask.cpu(), mask_ref)
+
+
+def test_recall_statistic_matches_the_oracle():
+    # collect_stats=True: after a 1024-token prefill every layer holds the recall of its hash ranking (reference :319-398);
+    # layer 0 is compared row by row with the oracle on the same queries and keys
+    print("\n[case] recall statistic (collect_stats)", flush=True)
+    torch.manual_seed(4)
+    cfg = _config(LlamaConfig)
+    model = LlamaForCausalLM(cfg).bfloat16().float()
+    usa = hl.load_usa(cfg, None)
+    model = hl.convert_usa(model.to(DEV), cfg, usa, collect_stats=True, train_usa=False).float()
+    attn = model.model.layers[0].self_attn
+    seen = {}
+
+    def grab(mod, args, kwargs):
+        seen["h"] = kwargs["hidden_states"] if "hidden_states" in kwargs else args[0]
+        seen["pe"] = kwargs["position_embeddings"]
+    hook = attn.register_forward_pre_hook(grab, with_kwargs=True)
+    ids = torch.randint(0, cfg.vocab_size, (1, 1024), generator=torch.Generator().manual_seed(2)).to(DEV)
+    cache = DynamicCache()
+    with torch.no_grad():
+        model(ids, past_key_values=cache, use_cache=True)
+    hook.remove()
+    assert list(attn.overlaps) == [1024] and attn.overlaps[1024][2] == 4 * 1024
+    got = attn.last_overlap_ratio.cpu()                                                      # [1, H, q_len]
+    rope = __import__("transformers.models.llama.modeling_llama", fromlist=["apply_rotary_pos_emb"]).apply_rotary_pos_emb
+    with torch.no_grad():
+        q = attn.q_proj(seen["h"]).view(1, 1024, 4, 128).transpose(1, 2)
+        q, _ = rope(q, q, *seen["pe"])
+    keys = cache.layers[0].keys
+    lin = lambda seqs: [[(m.weight.detach().float().cpu(), m.bias.detach().float().cpu()) for m in s if isinstance(m, torch.nn.Linear)]
+                        for s in seqs]
+    rows = slice(1024 - 96, 1024)                                                            # the oracle is a Python loop: the last 96 rows
+    want = orc.recall_overlap(q[:, :, rows].float().cpu(), keys.float().cpu(), lin(usa[0].learning_to_hash_transformation_k),
+                              lin(usa[0].learning_to_hash_transformation_q), cfg.init_budget, cfg.recent_budget)
+    diff = (got[:, :, rows] - want).abs()
+    # a near tie between the 32nd and 33rd true logit may flip with the summation order of the GPU matmul: 1/32 on few rows
+    assert diff.max().item() <= 1 / 32 + 1e-6 and (diff > 0).float().mean().item() < 0.05, (diff.max().item(), (diff > 0).float().mean().item())
+    assert 0.0 < attn.overlaps[1024][3] <= 1.0
+    hl.print_stats(model)

@@ -211,3 +211,47 @@ def test_reference_decode_attention_is_consistent_with_its_stages():
     for h in range(w.n_q_heads):
         o = orc.sparse_attend(p.q[0, h, 0], p.k[0, h // 4], p.v[0, h // 4], sel[h], 1 / math.sqrt(128))
         assert torch.allclose(o, out[0, h, 0], atol=1e-5)
+
+
+def test_recall_overlap_is_pinned_by_its_special_cases_and_a_verbatim_restatement():
+    # (1) when S // 16 covers every candidate the statistic is min(32, #candidates) / 32 whatever the hashes say;
+    # (2) the dense formulation written as the reference writes it (masked logits, two torch.topk, scatter, product:
+    #     hashattention_llama.py:357-386) must lie between the canonical value with the boundary ties of the hash score
+    #     all left out and all taken in - torch.topk is free to pick any of them
+    import math
+    from hashattention.synthetic import make_usa_weights, Workload
+    g = torch.Generator().manual_seed(11)
+    w = Workload("t", 1, [96], n_q_heads=4, n_kv_heads=2, n_code_heads=4, lth_int_dim=32, seed=2)
+    usa = make_usa_weights(w)
+    S, q_len, init, recent = 96, 40, 4, 6
+    k = torch.randn(1, 2, S, 128, generator=g)
+    q = torch.randn(1, 4, q_len, 128, generator=g)
+    got = orc.recall_overlap(q, k, usa.k, usa.q, init, recent, top_true=3)                  # S // 16 = 6 predictions
+    # verbatim restatement
+    kk = orc.repeat_kv(k, 2)
+    logits = torch.matmul(q, kk.transpose(2, 3)) / math.sqrt(128)
+    keep = torch.tril(torch.ones(q_len, S), diagonal=S - q_len - recent).bool()
+    keep[:, :init] = False
+    logits = logits.masked_fill(~keep, torch.finfo(logits.dtype).min)
+    target = torch.zeros_like(logits)
+    target.scatter_(-1, torch.topk(logits, 3, dim=-1).indices, 1.0)
+    span, _ = orc.usa_forward_hard(kk, q, usa.k, usa.q)
+    span = span.masked_fill(~keep, torch.finfo(span.dtype).min)
+    pred = torch.zeros_like(span)
+    pred.scatter_(-1, torch.topk(span, S // 16, dim=-1).indices, 1.0)
+    verbatim = (pred * target).sum(-1) / target.sum(-1)
+    # bounds from the threshold value of the hash score
+    thr = torch.topk(span, S // 16, dim=-1).values[..., -1:]
+    lower = ((span > thr).float() * target).sum(-1) / 3
+    upper = ((span >= thr).float() * target).sum(-1) / 3
+    rows = keep.sum(-1) >= S // 16                                                          # rows whose candidates fill the prediction
+    assert rows.any()
+    assert ((verbatim >= lower - 1e-6) & (verbatim <= upper + 1e-6))[..., rows].all()
+    assert ((got >= lower - 1e-6) & (got <= upper + 1e-6))[..., rows].all()
+    assert (upper - lower)[..., rows].abs().max() <= 1.0 and (got[..., rows] > 0).any()
+    # special case: predictions cover all candidates
+    few = orc.recall_overlap(q, k, usa.k, usa.q, init, S - q_len - 5, top_true=3)            # at most ~ q_len candidates... per row i: i + 2
+    ncand = torch.clamp(torch.arange(q_len) + S - q_len - (S - q_len - 5) - init + 1, min=0)
+    full = ncand <= S // 16
+    want = torch.clamp(ncand, max=3).float() / 3
+    assert torch.allclose(few[0, :, full], want[full].expand(4, -1))

@@ -187,16 +187,35 @@ class HeavyHitterMixin:
         out = torch.empty(b, H, q_len, d, dtype=query_states.dtype, device=query_states.device)
         # the reference takes the heavy budget from the full key length for every query row (:431-434)
         heavy = hl.heavy_count(S)
-        saved = hl.heavy_budget
-        hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5    # > 1: an absolute count for the kernels
-        try:
-            for i in range(q_len):
-                s_i = S - q_len + i + 1
-                o_i = torch.empty(b, H, d, dtype=query_states.dtype, device=query_states.device)
-                hl.step(query_states[:, :, i:i + 1], key_states, value_states, s_i, o_i)
-                out[:, :, i] = o_i
-        finally:
-            hl.heavy_budget = saved
+        heavy_abs = 0.0 if heavy == 0 else heavy + 0.5       # > 1: an absolute count for the kernels
+        if q_len == 1:
+            saved = hl.heavy_budget
+            hl.heavy_budget = heavy_abs
+            try:
+                hl.step(query_states, key_states, value_states, S, out[:, :, 0])
+            finally:
+                hl.heavy_budget = saved
+            return out
+        # a chunk of q_len rows: the new keys join the bit-cache, then every row is one "sequence" of the kernels - same
+        # codes and K/V (batch stride 0), its own query code and its own length S - q_len + i + 1 (reference :423-428)
+        dev = query_states.device
+        hl.encode_keys(key_states[:, :, S - q_len:S], pos0=S - q_len)
+        hl.n_cached = S
+        lens = torch.arange(S - q_len + 1, S + 1, dtype=torch.int32, device=dev)
+        cap = S if hl.mode != _ops.HA_SELECT_SIMPLE else min(S, hl.init_budget + hl.recent_budget + heavy)
+        qc = torch.zeros(1, H, q_len, hl.W, dtype=torch.int32, device=dev)
+        idx = torch.empty(q_len, H, cap, dtype=torch.int32, device=dev)
+        cnt = torch.empty(q_len, H, dtype=torch.int32, device=dev)
+        ws_s = _ops.workspace(_ops.select_workspace_bytes(q_len, H, hl.Hc, hl.W, S), dev)
+        ws_a = _ops.workspace(_ops.sparse_decode_workspace_bytes(q_len, H, cap), dev)
+        o_b = torch.empty(q_len, H, d, dtype=query_states.dtype, device=dev)
+        for bi in range(b):
+            _ops.encode_pack(query_states[bi:bi + 1], hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
+            _ops.select(hl.codes[bi:bi + 1].expand(q_len, -1, -1, -1), qc[0].transpose(0, 1).contiguous(), S, lens, hl.init_budget,
+                        hl.recent_budget, heavy_abs, idx, cnt, ws_s, hl.mode, hl.depth)
+            _ops.sparse_decode(query_states[bi].transpose(0, 1).contiguous(), key_states[bi:bi + 1].expand(q_len, -1, -1, -1),
+                               value_states[bi:bi + 1].expand(q_len, -1, -1, -1), idx, cnt, hl.sm_scale, o_b, ws_a)
+            out[bi] = o_b.transpose(0, 1)
         return out
 
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):

@@ -329,7 +329,8 @@ def main():
                                f"H={H} Hkv={Hkv} d={d} code_heads={w.n_code_heads} code_bits={w.lth_final_dim} "
                                f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} "
                                f"n_sel={n_sel_rows // (B * H)}"},
-        "path": "ha_encode_step + ha_select_prepare + ha_sparse_decode_fused" if fused else
+        "path": ("ha_encode_step + ha_select_histogram + ha_sparse_decode_fused (thresholds in the attention launch)"
+                 if layer.local_thresholds else "ha_encode_step + ha_select_prepare + ha_sparse_decode_fused") if fused else
                 "ha_encode_step + ha_select + " + ("ha_window_partial + ha_sparse_decode_heavy" if layer.overlap_windows else "ha_sparse_decode"),
         "stages_us": {"encode_new_k_and_q": ms_encode * 1e3,
                       **({"select_prepare": ms_prepare * 1e3, "select_attend_fused": ms_attend * 1e3,

@@ -113,7 +113,13 @@ struct FusedSel {
     const uint32_t *qcodes;
     const int32_t *meta, *chunk_pre;
     int nchunk, chunk, cps, gq, init, recent, vec;
+    // when `hist` is set the workspace holds only the per-chunk histograms (ha_select_histogram): the workgroup derives
+    // its row's threshold and chunk prefixes itself (at most kFusedLocalChunks chunks) and writes the row's count
+    const uint32_t *hist;
+    double heavy_budget;
+    int32_t *out_counts;
 };
+constexpr int kFusedLocalChunks = 64;
 
 // NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.
 template <int W, int NSLAB>
@@ -129,6 +135,7 @@ __device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int 
 // waves, and giving two of eight to the scan cost more than the scan itself.  Building the whole list first costs
 // the scan's ~15 us up front.)
 struct FusedRow {
+    const int32_t *pre;  // {#d < T, #d == T} before each chunk of the row: the workspace's, or the workgroup's own in LDS
     int lo, hi, T, r, nheavy, neq, c0, nc, n;
     int nwin;   // window entries at the head of this workgroup's list (sink if it has the first chunk, recent if the last)
     int hbase;  // list position of a heavy token = hbase + (#d < T before it) + min(#d == T before it, r)
@@ -136,31 +143,92 @@ struct FusedRow {
 };
 
 // All threads of the workgroup: row constants and the windows.
+// Threshold and chunk prefixes of one row from its chunk histograms, by the workgroup itself (the work of
+// select_threshold_kernel for this row).  s_h: nchunk * NL words, s_pre: 2 * nchunk, s_meta: 4.
+template <int W, int NTT>
+__device__ __forceinline__ void local_thresholds(const FusedSel &f, int64_t row, int S, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
+    constexpr int NL = 32 * W + 1;
+    const int tid = threadIdx.x;
+    const uint32_t *hp = f.hist + row * f.nchunk * NL;
+    for (int i = tid; i < f.nchunk * NL; i += NTT) s_h[i] = hp[i];
+    __syncthreads();
+    uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile
+    if (tid < NL) {
+        uint32_t t = 0;
+        for (int c = 0; c < f.nchunk; ++c) t += s_h[c * NL + tid];
+        s_tot[tid] = t;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const ha_sel::RowBudget rb = ha_sel::row_budget(S, f.init, f.recent, f.heavy_budget);
+        int T, r, nheavy;
+        ha_sel::solve_threshold(s_tot, NL - 1, NL, rb.kk, HA_SELECT_SIMPLE, 0, T, r, nheavy);
+        s_meta[0] = T;
+        s_meta[1] = r;
+        s_meta[2] = nheavy;
+        s_meta[3] = T < NL ? (int)s_tot[T] : 0;
+    }
+    __syncthreads();
+    if (tid < HA_WAVE) {  // nchunk <= 64: one wave, one chunk per lane, two scans
+        const int T = s_meta[0];
+        uint32_t lt = 0, eq = 0;
+        if (tid < f.nchunk) {
+            for (int l = 0; l < T && l < NL; ++l) lt += s_h[tid * NL + l];
+            if (T < NL) eq = s_h[tid * NL + T];
+        }
+        const uint32_t ilt = ha_sel::wave_inclusive_scan(lt), ieq = ha_sel::wave_inclusive_scan(eq);
+        if (tid < f.nchunk) {
+            s_pre[tid * 2] = (int32_t)(ilt - lt);
+            s_pre[tid * 2 + 1] = (int32_t)(ieq - eq);
+        }
+    }
+    __syncthreads();
+}
+
+// Setup, first half: what is known without any threshold - the row's window geometry, this workgroup's chunks, and the
+// window entries at the head of its list (the loop can be primed on them while the second half runs).
 template <int NTT>
-__device__ __forceinline__ FusedRow fused_setup(const FusedSel &f, int64_t row, int S, int sp, int32_t *s_list, int *s_cstar) {
-    FusedRow fr;
+__device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, int32_t *s_list, FusedRow &fr) {
     const int tid = threadIdx.x;
     fr.lo = min(f.init, S);
     fr.hi = max(S - f.recent, fr.lo);
-    fr.T = f.meta[row * 4 + 0];
-    fr.r = f.meta[row * 4 + 1];
-    fr.nheavy = f.meta[row * 4 + 2];
-    fr.neq = f.meta[row * 4 + 3];
     fr.c0 = sp * f.cps;
     const int c1 = min(fr.c0 + f.cps, f.nchunk);
     fr.nc = c1 - fr.c0;
-    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
-    // heavy tokens of the row before chunk c
-    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
-    // the windows come first in the list: they are known at once, so the loop can start on them while the first
-    // chunks are being scanned
     const int n_sink = sp == 0 ? fr.lo : 0, n_recent = c1 >= f.nchunk ? S - fr.hi : 0;
     fr.nwin = min(n_sink + n_recent, kFusedListCap);
+    for (int i = tid; i < n_sink && i < fr.nwin; i += NTT) s_list[i] = i;
+    for (int i = tid; i < n_recent; i += NTT)
+        if (n_sink + i < fr.nwin) s_list[n_sink + i] = fr.hi + i;
+    __syncthreads();
+}
+
+// Setup, second half: threshold, prefixes, list length, the chunk of the r-th tie.
+template <int W, int NTT>
+__device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row, int S, int sp, int *s_cstar, uint32_t *s_h,
+                                                 int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
+    const int tid = threadIdx.x;
+    if (f.hist) {
+        local_thresholds<W, NTT>(f, row, S, s_h, s_pre, s_meta);
+        fr.T = s_meta[0];
+        fr.r = s_meta[1];
+        fr.nheavy = s_meta[2];
+        fr.neq = s_meta[3];
+        fr.pre = s_pre;
+        if (sp == 0 && tid == 0 && f.out_counts) f.out_counts[row] = fr.lo + fr.nheavy + (S - fr.hi);
+    } else {
+        fr.T = f.meta[row * 4 + 0];
+        fr.r = f.meta[row * 4 + 1];
+        fr.nheavy = f.meta[row * 4 + 2];
+        fr.neq = f.meta[row * 4 + 3];
+        fr.pre = f.chunk_pre + row * f.nchunk * 2;
+    }
+    const int c1 = fr.c0 + fr.nc;
+    const int32_t *pre = fr.pre;
+    // heavy tokens of the row before chunk c
+    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
     fr.hbase = fr.nwin - rank(fr.c0);
     fr.n = min(fr.nwin + max(rank(c1) - rank(fr.c0), 0), kFusedListCap);
-    for (int i = tid; i < n_sink && i < fr.n; i += NTT) s_list[i] = i;
-    for (int i = tid; i < n_recent; i += NTT)
-        if (n_sink + i < fr.n) s_list[n_sink + i] = fr.hi + i;
     if (tid == 0) *s_cstar = -1;
     __syncthreads();
     for (int i = tid; i < fr.nc; i += NTT) {
@@ -170,7 +238,6 @@ __device__ __forceinline__ FusedRow fused_setup(const FusedSel &f, int64_t row, 
     }
     __syncthreads();
     fr.cstar = *s_cstar;
-    return fr;
 }
 
 // One scan round of a fused workgroup: its NW waves take NW consecutive groups of GS slabs (a group is part of one
@@ -191,7 +258,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
     const int cb = c * f.chunk, j_first = cb + gi * GC;
     const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
     const bool whole = f.vec && beg == cb && end == cb + f.chunk;
-    const int32_t *pre = f.chunk_pre + row * f.nchunk * 2;
+    const int32_t *pre = fr.pre;
 
     uint32_t lt = 0, le = 0;  // bit 4 s + e: code (slab s, element e) of this lane has d < T / d <= T
     if (active && beg < end && fr.nheavy > 0) {
@@ -306,6 +373,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __shared__ int32_t s_list[FW > 0 ? kFusedListCap : 1];
     __shared__ uint32_t s_cnt[FW > 0 ? 64 : 1];
     __shared__ int s_cstar;
+    // in-kernel thresholds: the row's chunk histograms (+ their totals), chunk prefixes, {T, r, n_heavy, tie bucket}
+    __shared__ uint32_t s_h[FW > 0 ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
+    __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedLocalChunks : 1];
+    __shared__ int32_t s_meta[4];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
     // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
@@ -323,14 +394,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
-        fr = fused_setup<NT>(fsel, row, S, sp, s_list, &s_cstar);
+        fused_windows<NT>(fsel, S, sp, s_list, fr);
         j_max = max(S - 1, 0);
         r0 = 0;
-        r1 = fr.n;
-        if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
-            if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
-            return;
-        }
+        r1 = fr.nwin;  // until the thresholds are known the list is its windows
     } else {
         int64_t n = counts[b * H + h];
         if (n > idx_cap) n = idx_cap;
@@ -449,13 +516,24 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         constexpr int GS = FW == 1 ? 8 : 4;  // slabs per wave and round
         const bool wide = fsel.chunk % (GS * HA_WAVE * 4) == 0;  // else 1024-code chunks (short rows): 4 slabs
         const int gc = (wide ? GS : 4) * HA_WAVE * 4;
-        const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
-        const int rounds = (n_groups + NW - 1) / NW;
+        // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out
         bool primed = false;
-        if (rounds > 0 && fr.nwin >= min(2 * STEP, r1)) {  // the windows alone fill the first two steps
+        if (fr.nwin >= 2 * STEP) {
             prime();
             primed = true;
         }
+        {
+            int S = seq_lens ? seq_lens[b] : max_S;
+            if (S > max_S) S = max_S;
+            fused_thresholds<FW, NT>(fsel, row, S, sp, &s_cstar, s_h, s_pre, s_meta, fr);
+        }
+        r1 = fr.n;
+        if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
+            if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+            return;
+        }
+        const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
+        const int rounds = (n_groups + NW - 1) / NW;
         for (int k = 0; k < rounds; ++k) {
             int ready = wide ? fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list)
                              : fused_round<FW, 4, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
@@ -467,7 +545,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             }
             while (primed && base + 3 * STEP <= ready) step();
         }
-        if (rounds == 0) __syncthreads();  // the windows written by fused_setup
         if (!primed) prime();
         while (base < r1) step();
     } else {
@@ -811,6 +888,11 @@ int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
     return (double)init_budget + (double)recent_budget + heavy <= (double)kFusedListCap ? 1 : 0;
 }
 
+int ha_sparse_decode_fused_local_thresholds(int B, int Hc, int max_seq_len) {
+    if (B <= 0 || Hc <= 0 || max_seq_len <= 0) return 0;
+    return ha_sel::select_plan(B, Hc, max_seq_len).nchunk <= kFusedLocalChunks ? 1 : 0;
+}
+
 size_t ha_sparse_decode_fused_workspace_bytes(int B, int H, int Hc, int max_seq_len) {
     if (B <= 0 || H <= 0 || Hc <= 0 || max_seq_len <= 0) return 0;
     const ha_sel::SelectPlan plan = ha_sel::select_plan(B, Hc, max_seq_len);
@@ -821,8 +903,8 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
                            int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes, int64_t kc_stride_b,
                            int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W, int max_seq_len,
                            const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
-                           const void *select_workspace, size_t select_workspace_bytes, float sm_scale, void *out, void *workspace,
-                           size_t workspace_bytes, void *stream) {
+                           const void *select_workspace, size_t select_workspace_bytes, int thresholds_ready, int32_t *out_counts,
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(kcodes && qcodes && select_workspace, HA_ERR_NULL_POINTER, "kcodes/qcodes/select_workspace is NULL");
@@ -857,6 +939,14 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     f.init = init_budget;
     f.recent = recent_budget;
     f.vec = ha_sel::rows_vectorisable(kcodes, kc_stride_b, kc_stride_h, W) ? 1 : 0;
+    f.hist = nullptr;
+    f.heavy_budget = heavy_budget;
+    f.out_counts = out_counts;
+    if (!thresholds_ready) {
+        HA_REQUIRE(plan.nchunk <= kFusedLocalChunks, HA_ERR_BAD_SHAPE,
+                   "rows of more than %d chunks need their thresholds from ha_select_prepare", kFusedLocalChunks);
+        f.hist = sw.hist;
+    }
     const int nsplit = (plan.nchunk + f.cps - 1) / f.cps;
     const int64_t rows = (int64_t)B * H;
     float *part_acc = (float *)workspace;

@@ -360,6 +360,7 @@ size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
         hipLaunchKernelGGL((select_hist_kernel<W_, GQ_, REP_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,  \
                            qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.hist);  \
         HA_CHECK_LAUNCH("select_hist_kernel");                                                                                    \
+        if (!out_counts) break; /* ha_select_histogram: chunk histograms only */                                                  \
         hipLaunchKernelGGL(select_threshold_kernel<W_>, dim3(H, B), dim3(kSelThreads), 0, s, ws.hist, H, max_seq_len, seq_lens,   \
                            init_budget, recent_budget, heavy_budget, mode, depth, plan.nchunk, ws.meta, ws.chunk_pre, out_idx,    \
                            idx_cap, out_counts);                                                                                  \
@@ -377,7 +378,7 @@ static int select_impl(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_s
                        size_t workspace_bytes, void *stream, bool prepare_only) {
     int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len);
     if (st) return st;
-    HA_REQUIRE((prepare_only || out_idx) && out_counts, HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
+    HA_REQUIRE(prepare_only || (out_idx && out_counts), HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
     HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && heavy_budget >= 0.0 && depth >= 0, HA_ERR_BAD_SHAPE,
                "budgets and depth must be non-negative");
     HA_REQUIRE(heavy_budget < 2147483647.0, HA_ERR_BAD_SHAPE, "heavy_budget too large");
@@ -428,9 +429,17 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
                        heavy_budget, mode, depth, algo, out_idx, idx_cap, out_counts, workspace, workspace_bytes, stream, false);
 }
 
+int ha_select_histogram(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
+                        int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+    return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget, 0.0,
+                       HA_SELECT_SIMPLE, 0, HA_SELECT_ALGO_HISTOGRAM, nullptr, 1, nullptr, workspace, workspace_bytes, stream, true);
+}
+
 int ha_select_prepare(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
                       int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
                       int mode, int depth, int32_t *out_counts, void *workspace, size_t workspace_bytes, void *stream) {
+    HA_REQUIRE(out_counts, HA_ERR_NULL_POINTER, "out_counts is NULL");
     return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
                        heavy_budget, mode, depth, HA_SELECT_ALGO_HISTOGRAM, nullptr, 1, out_counts, workspace, workspace_bytes, stream,
                        true);

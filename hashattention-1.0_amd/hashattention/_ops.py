@@ -75,13 +75,17 @@ def load_library() -> C.CDLL:
     lib.ha_swiglu.argtypes = [vp, i64, i32, i32, i32, vp, vp]
     lib.ha_select_prepare.restype = i32
     lib.ha_select_prepare.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, vp, vp, sz, vp]
+    lib.ha_select_histogram.restype = i32
+    lib.ha_select_histogram.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, vp, sz, vp]
+    lib.ha_sparse_decode_fused_local_thresholds.restype = i32
+    lib.ha_sparse_decode_fused_local_thresholds.argtypes = [i32, i32, i32]
     lib.ha_sparse_decode_fused_applies.restype = i32
     lib.ha_sparse_decode_fused_applies.argtypes = [i32, i32, i32, i32, i32, i32, i32, f64, i32]
     lib.ha_sparse_decode_fused_workspace_bytes.restype = sz
     lib.ha_sparse_decode_fused_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.ha_sparse_decode_fused.restype = i32
     lib.ha_sparse_decode_fused.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp,
-                                           i32, i32, f64, vp, sz, f32, vp, vp, sz, vp]
+                                           i32, i32, f64, vp, sz, i32, vp, f32, vp, vp, sz, vp]
     lib.ha_sparse_decode_workspace_bytes.restype = sz
     lib.ha_sparse_decode_workspace_bytes.argtypes = [i32, i32, i64]
     lib.ha_sparse_decode.restype = i32
@@ -260,6 +264,24 @@ def select_prepare(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int,
                                  _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select_prepare")
 
 
+def select_histogram(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
+                     init_budget: int, recent_budget: int, ws: torch.Tensor) -> None:
+    """Per-chunk distance histograms into the workspace: all the fused attention launch needs when it derives the
+    thresholds itself (sparse_decode_fused(..., thresholds_ready=False))."""
+    _require_cuda(kcodes, qcodes, seq_lens, ws)
+    lib = load_library()
+    B, Hc, _, W = kcodes.shape
+    H = qcodes.shape[1]
+    assert kcodes.stride(3) == 1 and kcodes.stride(2) == W and qcodes.is_contiguous()
+    _check(lib.ha_select_histogram(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
+                                   _ptr(seq_lens), init_budget, recent_budget, _ptr(ws), ws.numel(), _stream(kcodes)),
+           "ha_select_histogram")
+
+
+def fused_local_thresholds(B, Hc, max_seq_len) -> bool:
+    return bool(load_library().ha_sparse_decode_fused_local_thresholds(B, Hc, max_seq_len))
+
+
 def fused_applies(B, H, Hc, W, max_seq_len, init_budget, recent_budget, heavy_budget, mode=HA_SELECT_SIMPLE) -> bool:
     return bool(load_library().ha_sparse_decode_fused_applies(B, H, Hc, W, max_seq_len, init_budget, recent_budget,
                                                               float(heavy_budget), mode))
@@ -271,17 +293,19 @@ def sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len) -> int:
 
 def sparse_decode_fused(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kcodes: torch.Tensor, qcodes: torch.Tensor,
                         max_seq_len: int, seq_lens: Optional[torch.Tensor], init_budget: int, recent_budget: int,
-                        heavy_budget: float, ws_select: torch.Tensor, sm_scale: float, out: torch.Tensor, ws: torch.Tensor) -> None:
-    """Attention over the selection prepared by select_prepare (same codes, budgets and seq_lens); out [B,H,128] in place."""
-    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws)
+                        heavy_budget: float, ws_select: torch.Tensor, sm_scale: float, out: torch.Tensor, ws: torch.Tensor,
+                        thresholds_ready: bool = True, out_counts: Optional[torch.Tensor] = None) -> None:
+    """Attention over the selection prepared by select_prepare (same codes, budgets and seq_lens); out [B,H,128] in place.
+    thresholds_ready=False: the workspace was filled by select_histogram only; counts (optional, [B,H] int32) are written here."""
+    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws, out_counts)
     lib = load_library()
     B, H, _ = q.shape
     Hc, W = kcodes.shape[1], kcodes.shape[3]
     assert out.is_contiguous() and out.dtype == q.dtype and kcodes.stride(3) == 1 and kcodes.stride(2) == W and qcodes.is_contiguous()
     _check(lib.ha_sparse_decode_fused(*_kv_args(q, k, v), _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H,
                                       k.shape[1], Hc, W, max_seq_len, _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget),
-                                      _ptr(ws_select), ws_select.numel(), float(sm_scale), _ptr(out), _ptr(ws), ws.numel(),
-                                      _stream(q)), "ha_sparse_decode_fused")
+                                      _ptr(ws_select), ws_select.numel(), 1 if thresholds_ready else 0, _ptr(out_counts),
+                                      float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_sparse_decode_fused")
 
 
 # ------------------------------------------------------------------------------------------ attention

@@ -6,9 +6,10 @@ key codes, plus the index lists and workspaces of the kernels.  One decode step 
 
     windows  attention over sink | recent, second stream    (ha_window_partial, overlaps the next two)
     encode   code of the new key -> bit-cache, query codes  (ha_encode_step, one launch)
-    select   Hamming histogram + threshold per row          (ha_select_prepare)
-    attend   index list rebuilt in LDS from the codes,      (ha_sparse_decode_fused)
-             gather-only attention over it
+    select   Hamming histograms per 4096-token chunk        (ha_select_histogram; ha_select_prepare adds the
+                                                               per-row thresholds for rows of more than 64 chunks)
+    attend   threshold per row, index list rebuilt in LDS   (ha_sparse_decode_fused)
+             from the codes, gather-only attention over it
 or, for threshold mode and lists above 8192 entries, ha_select (histogram, threshold, ordered compaction into
 memory) + ha_sparse_decode (ha_sparse_decode_heavy merged with the window partial when overlap_windows is on).
 
@@ -82,6 +83,8 @@ class HashDecodeLayer:
         # with more, finer pieces the two-launch path is a few microseconds ahead
         self.fused_ok = B * self.H >= 256 and _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget,
                                                                  self.recent_budget, self.heavy_budget, self.mode)
+        # rows of up to 64 chunks: the attention launch derives the thresholds itself, the step is three launches
+        self.local_thresholds = _ops.fused_local_thresholds(B, self.Hc, S_cap)
         self.ws_fused = _ops.workspace(_ops.sparse_decode_fused_workspace_bytes(B, self.H, self.Hc, S_cap), dev)
         self.win = torch.empty(B, self.H, 130, dtype=torch.float32, device=dev)
         self.side_stream = torch.cuda.Stream(device=dev)
@@ -111,6 +114,10 @@ class HashDecodeLayer:
                     self.select_algo)
 
     def select_prepare(self, max_seq_len: int, seq_lens: Optional[torch.Tensor]) -> None:
+        if self.local_thresholds:
+            _ops.select_histogram(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
+                                  self.recent_budget, self.ws_select)
+            return
         _ops.select_prepare(self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens, self.init_budget,
                             self.recent_budget, self.heavy_budget, self.counts, self.ws_select, self.mode, self.depth)
 
@@ -118,7 +125,7 @@ class HashDecodeLayer:
                      seq_lens: Optional[torch.Tensor]) -> None:
         _ops.sparse_decode_fused(q3, k, v, self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens,
                                  self.init_budget, self.recent_budget, self.heavy_budget, self.ws_select, self.sm_scale, out,
-                                 self.ws_fused)
+                                 self.ws_fused, thresholds_ready=not self.local_thresholds, out_counts=self.counts)
 
     def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor) -> None:
         _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend)

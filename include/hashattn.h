@@ -205,16 +205,23 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
  * (same order as ha_select's list, so the output equals ha_select + ha_sparse_decode bit for bit when rows are not
  * split) and attends to it: the list never travels through memory and the compaction launch disappears.
  * Budgets, seq_lens and code arguments must be those given to ha_select_prepare; `select_workspace` is the
- * workspace it filled.  Only HA_SELECT_SIMPLE, and only while init + recent + heavy <= 8192 entries
+ * workspace it filled.  With thresholds_ready = 0 the workspace needs only the chunk histograms (ha_select_histogram,
+ * the first launch alone): every workgroup of the attention launch derives its row's threshold and prefixes
+ * itself and out_counts (may be NULL) is written by that launch - one launch less per step; rows of at most 64
+ * chunks (max_seq_len <= 262144, ha_sparse_decode_fused_local_thresholds returns 1).  Only HA_SELECT_SIMPLE, and only while init + recent + heavy <= 8192 entries
  * (ha_sparse_decode_fused_applies returns 1); otherwise use ha_select + ha_sparse_decode.  Replaces the same
  * reference lines as those two (hashattention_llama.py:401-446, 585-615; efficiency/kernels/torchatt.py:52-71).
  */
+int ha_select_histogram(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                        int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                        int init_budget, int recent_budget, void *workspace, size_t workspace_bytes, void *stream);
 int ha_select_prepare(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
                       int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
                       int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
                       int32_t *out_counts, void *workspace, size_t workspace_bytes, void *stream);
 int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
                                    int init_budget, int recent_budget, double heavy_budget, int mode);
+int ha_sparse_decode_fused_local_thresholds(int B, int Hc, int max_seq_len);
 size_t ha_sparse_decode_fused_workspace_bytes(int B, int H, int Hc, int max_seq_len);
 int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h,
                            const void *k, const void *v, int kv_dtype,
@@ -223,6 +230,7 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
                            int B, int H, int Hkv, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
                            int init_budget, int recent_budget, double heavy_budget,
                            const void *select_workspace, size_t select_workspace_bytes,
+                           int thresholds_ready, int32_t *out_counts,
                            float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*

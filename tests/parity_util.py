@@ -143,6 +143,15 @@ def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple"
         same = float((out3.float() - out.float()).abs().max().item())
         assert same <= (2e-6 if w.dtype == torch.float32 else 1e-2), f"fused vs two-launch output differ by {same}"
         report.update(fused_err=err3, fused_vs_unfused=same)
+        if _ops.fused_local_thresholds(B, Hc, S):       # thresholds derived inside the attention launch: same output bit for bit
+            counts4 = torch.full((B, H), -5, dtype=torch.int32, device=dev)
+            out4 = torch.empty_like(out)
+            ws5 = _ops.workspace(_ops.select_workspace_bytes(B, H, Hc, W, S), dev)
+            _ops.select_histogram(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, ws5)
+            _ops.sparse_decode_fused(q3, k, v, kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws5, sm_scale,
+                                     out4, ws4, thresholds_ready=False, out_counts=counts4)
+            assert np.array_equal(counts4.cpu().numpy(), counts_ref), "fused path, local thresholds: counts differ"
+            assert torch.equal(out4, out3), "fused path: local thresholds change the output"
 
     if check_dense:
         outd = torch.empty(B, H, d, dtype=w.dtype, device=dev)

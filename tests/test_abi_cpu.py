@@ -138,15 +138,17 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert lib.ha_sparse_decode_fused_applies(1, 4, 2, 1, 1000, 4, 4, C.c_double(0.25), 1) == 0          # threshold mode
     assert lib.ha_sparse_decode_fused_applies(1, 4, 2, 1, 100000, 4, 4, C.c_double(0.25), 0) == 0        # 25 008 entries > 8192
     assert lib.ha_sparse_decode_fused_workspace_bytes(1, 4, 2, 1000) > 0
+    assert lib.ha_sparse_decode_fused_local_thresholds(1, 2, 1000) == 1 and lib.ha_sparse_decode_fused_local_thresholds(1, 2, 1 << 20) == 0
+    assert lib.ha_select_histogram(p, 1024, 1024, null, 1, 4, 2, 1, 1000, null, 4, 4, p, 1 << 20, null) == HA_ERR_NULL
 
     def fused(**kw):
         a = dict(q=p, qsb=512, qsh=128, k=p, v=p, dt=_ops.HA_BF16, sb=128000, sh=128000, ss=128, kc=p, csb=1024, csh=1024, qc=p, B=1, H=4,
-                 Hkv=2, Hc=2, W=1, S=1000, sl=null, init=4, rec=4, hb=C.c_double(0.25), sws=p, swsb=1 << 20, sc=C.c_float(0.088), out=p,
-                 ws=p, wsb=1 << 20, st=null)
+                 Hkv=2, Hc=2, W=1, S=1000, sl=null, init=4, rec=4, hb=C.c_double(0.25), sws=p, swsb=1 << 20, tr=1, oc=null,
+                 sc=C.c_float(0.088), out=p, ws=p, wsb=1 << 20, st=null)
         a.update(kw)
         return lib.ha_sparse_decode_fused(a["q"], a["qsb"], a["qsh"], a["k"], a["v"], a["dt"], a["sb"], a["sh"], a["ss"], a["kc"], a["csb"],
                                           a["csh"], a["qc"], a["B"], a["H"], a["Hkv"], a["Hc"], a["W"], a["S"], a["sl"], a["init"], a["rec"],
-                                          a["hb"], a["sws"], a["swsb"], a["sc"], a["out"], a["ws"], a["wsb"], a["st"])
+                                          a["hb"], a["sws"], a["swsb"], a["tr"], a["oc"], a["sc"], a["out"], a["ws"], a["wsb"], a["st"])
 
     assert fused(kc=null) == HA_ERR_NULL and fused(sws=null) == HA_ERR_NULL and fused(dt=9) == HA_ERR_DTYPE
     assert fused(Hc=3) == HA_ERR_SHAPE and fused(csh=999) == HA_ERR_SHAPE and fused(hb=C.c_double(0.9), S=60000, csb=60000, csh=60000) == HA_ERR_SHAPE

@@ -160,7 +160,14 @@ def decoder_bench(args, torch):
         hl0.step(q, dec.k_cache[0], dec.v_cache[0], S, out)
 
     ms_layer = time_gpu(layer_step, args.steps, args.warmup, torch)
-    ms_attend = time_gpu(lambda: hl0.attend(q[:, :, 0, :], dec.k_cache[0], dec.v_cache[0], out), args.steps, args.warmup, torch)
+    # the layer's attention launch alone: the fused launch replays on the histograms and query codes the step left
+    # behind; the two-launch path's gather reads the index lists its selection wrote
+    fused0 = hl0.use_fused and hl0.fused_ok and not hl0.overlap_windows
+    if fused0:
+        attend_alone = lambda: hl0.attend_fused(q[:, :, 0, :], dec.k_cache[0], dec.v_cache[0], out, S, None)
+    else:
+        attend_alone = lambda: hl0.attend(q[:, :, 0, :], dec.k_cache[0], dec.v_cache[0], out)
+    ms_attend = time_gpu(attend_alone, args.steps, args.warmup, torch)
     n_sel_rows = int(hl0.counts.sum().item())
     ab = algorithmic_bytes(w, n_sel_rows)
     n_params = sum(t.numel() for p in dec.layers for t in p.values()) + dec.lm_head.numel()
@@ -182,7 +189,7 @@ def decoder_bench(args, torch):
         "prefill_encode_tflops": 2 * B * dec.Hc * (S - 1) * (128 * 128 * 2 + 128 * 32) / (ms_prefill_encode * 1e-3) / 1e12,
         "cache_fill_seconds": fill_s,
         "hbm_gbps_step": step_bytes / (ms_step * 1e-3) / 1e9, "hbm_frac_step": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
+        "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused0 else "sparse_attend_kernel", "bound": "hbm", "achieved": ab["gather"] / (ms_attend * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
     }
@@ -198,6 +205,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
+    ap.add_argument("--fused-min-rows", type=int, default=None, help="take the fused select-attend path from this many (sequence, head) rows on")
     ap.add_argument("--two-launch", action="store_true", help="ha_select + ha_sparse_decode instead of the fused select-attend path")
     ap.add_argument("--overlap-windows", action="store_true", help="attend to sink|recent on a second stream (ha_window_partial)")
     ap.add_argument("--layers", type=int, default=32, help="decoder layers of the config3 whole-step workload")
@@ -230,6 +238,8 @@ def main():
 
     layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, d, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
                             w.init_budget, w.recent_budget, w.heavy_budget, device=dev)
+    if args.fused_min_rows is not None:
+        layer.fused_min_rows = args.fused_min_rows
     layer.allocate(B, S)
     layer.select_algo = args.select_algo
     layer.overlap_windows = args.overlap_windows

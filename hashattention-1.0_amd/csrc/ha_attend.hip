@@ -120,6 +120,8 @@ struct FusedSel {
     int32_t *out_counts;
 };
 constexpr int kFusedLocalChunks = 64;
+constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
+constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
 
 // NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.
 template <int W, int NSLAB>
@@ -188,14 +190,16 @@ __device__ __forceinline__ void local_thresholds(const FusedSel &f, int64_t row,
 // Setup, first half: what is known without any threshold - the row's window geometry, this workgroup's chunks, and the
 // window entries at the head of its list (the loop can be primed on them while the second half runs).
 template <int NTT>
-__device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, int32_t *s_list, FusedRow &fr) {
+__device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, int cps, int row_pieces, int32_t *s_list, FusedRow &fr) {
     const int tid = threadIdx.x;
     fr.lo = min(f.init, S);
     fr.hi = max(S - f.recent, fr.lo);
-    fr.c0 = sp * f.cps;
-    const int c1 = min(fr.c0 + f.cps, f.nchunk);
+    // workgroup sp of the row owns chunks [sp * cps, (sp + 1) * cps); the row has row_pieces such workgroups
+    fr.c0 = min(sp * cps, f.nchunk);
+    const int c1 = min(fr.c0 + cps, f.nchunk);
     fr.nc = c1 - fr.c0;
-    const int n_sink = sp == 0 ? fr.lo : 0, n_recent = c1 >= f.nchunk ? S - fr.hi : 0;
+    // sink: first workgroup; recent: last workgroup of the row
+    const int n_sink = sp == 0 ? fr.lo : 0, n_recent = sp == row_pieces - 1 ? S - fr.hi : 0;
     fr.nwin = min(n_sink + n_recent, kFusedListCap);
     for (int i = tid; i < n_sink && i < fr.nwin; i += NTT) s_list[i] = i;
     for (int i = tid; i < n_recent; i += NTT)
@@ -373,6 +377,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __shared__ int32_t s_list[FW > 0 ? kFusedListCap : 1];
     __shared__ uint32_t s_cnt[FW > 0 ? 64 : 1];
     __shared__ int s_cstar;
+    __shared__ int s_plan[2];
     // in-kernel thresholds: the row's chunk histograms (+ their totals), chunk prefixes, {T, r, n_heavy, tie bucket}
     __shared__ uint32_t s_h[FW > 0 ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
     __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedLocalChunks : 1];
@@ -383,8 +388,59 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     // there are 8 KV heads, i.e. on one XCD, so rows they share (the sink and recent windows, commonly
     // selected keys) are served by that XCD's L2 instead of being fetched from HBM once per XCD.
     const int Hkv = H / G;
-    const int sp = blockIdx.x, h = ((int)blockIdx.y % Hkv) * G + (int)blockIdx.y / Hkv, b = blockIdx.z;
+    int sp = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
+    if constexpr (FW > 0) {
+        // in-kernel plan (below): walk the grid piece index slowest, so that the first pieces of all rows are dispatched
+        // first and spread over all XCDs, and the workgroups that turn out to own nothing come last
+        if (seq_lens && (int)gridDim.z <= kFusedSortBatch && gridDim.x > 1) {
+            const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), per = gridDim.y * gridDim.z;
+            sp = lin / per;
+            by = (lin % per) % (int)gridDim.y;
+            b = (lin % per) / (int)gridDim.y;
+        }
+    }
+    const int h = (by % Hkv) * G + by / Hkv;
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
+    const int slice = b;  // position of this workgroup's sequence in the walk over the batch
+    int cps = fsel.cps, row_pieces = nsplit_max;  // chunks per workgroup, workgroups of this row that own chunks
+    if constexpr (FW > 0) {
+        // Ragged batch (lengths on the device, up to kFusedSortBatch sequences): every workgroup works out the same plan
+        // from the lengths.  (1) Workgroups are dispatched in launch order, so the z-th slice of the grid takes the z-th
+        // longest sequence (ties by index) and the long rows do not start last.  (2) One piece size for the batch: the
+        // fewest chunks per workgroup for which all pieces of all rows are resident at once (kFusedResident workgroups),
+        // so a long row is cut into more pieces than a short one and no second round of workgroups is needed.
+        if (seq_lens && (int)gridDim.z <= kFusedSortBatch) {
+            const int nb = gridDim.z;
+            if (tid < nb) {
+                const int mine = seq_lens[tid];
+                int rank = 0;
+                for (int u = 0; u < nb; ++u) {
+                    const int o = seq_lens[u];
+                    rank += (o > mine || (o == mine && u < tid)) ? 1 : 0;
+                }
+                if (rank == slice) s_plan[0] = tid;
+            }
+            if (tid >= 192 && tid < 256) {  // one candidate piece size per lane of the fourth wave
+                const int cstep = (fsel.nchunk + 63) / 64;
+                const int cand = (tid - 192 + 1) * cstep;
+                int total = 0, longest = 1;
+                for (int u = 0; u < nb; ++u) {
+                    const int nc = min(max((min(seq_lens[u], max_S) + fsel.chunk - 1) / fsel.chunk, 1), fsel.nchunk);
+                    total += (nc + cand - 1) / cand;
+                    longest = max(longest, nc);
+                }
+                const unsigned long long ok = __ballot((int64_t)total * H <= kFusedResident);
+                int pick = ok ? (__ffsll((long long)ok)) * cstep : 64 * cstep;
+                pick = max(pick, (longest + (int)gridDim.x - 1) / (int)gridDim.x);  // the grid has gridDim.x workgroups per row
+                if (tid == 192) s_plan[1] = pick;
+            }
+            __syncthreads();
+            b = s_plan[0];
+            const int nc = min(max((min(seq_lens[b], max_S) + fsel.chunk - 1) / fsel.chunk, 1), fsel.nchunk);
+            row_pieces = (nc + s_plan[1] - 1) / s_plan[1];
+            cps = (nc + row_pieces - 1) / row_pieces;  // the row's chunks dealt evenly to its pieces
+        }
+    }
     const int64_t row = (int64_t)b * H + h;
     int r0, r1, nsplit;
     const int32_t *ix = nullptr;
@@ -394,7 +450,18 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
-        fused_windows<NT>(fsel, S, sp, s_list, fr);
+        if (sp >= row_pieces) {  // nothing of this row here (uniform over the workgroup): an empty partial
+            if (tid < HA_HEAD_DIM) {
+                const int64_t p = row * nsplit_max + sp;
+                part_acc[p * HA_HEAD_DIM + tid] = 0.f;
+                if (tid == 0) {
+                    part_ml[p * 2] = -INFINITY;
+                    part_ml[p * 2 + 1] = 0.f;
+                }
+            }
+            return;
+        }
+        fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr);
         j_max = max(S - 1, 0);
         r0 = 0;
         r1 = fr.nwin;  // until the thresholds are known the list is its windows
@@ -872,9 +939,13 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
 }
 
 // chunks per workgroup of the fused path: whole rows when the rows alone fill the GPU, else enough splits for ~512 workgroups
-static int fused_chunks_per_split(int B, int H, int nchunk) {
+// Workgroups per row: enough for two 512-thread workgroups on each of the 256 CUs.  With lengths on the device the
+// kernel decides per row how many of them own chunks, so the grid offers up to four times as many (at most one per
+// kFusedResident / H rows, the count a single sequence would get).
+static int fused_chunks_per_split(int B, int H, int nchunk, bool ragged) {
     const int64_t rows = (int64_t)B * H;
-    int64_t want = (512 + rows - 1) / rows;
+    int64_t want = (kFusedResident + rows - 1) / rows;
+    if (ragged && B > 1 && B <= kFusedSortBatch && rows < kFusedResident) want = std::min<int64_t>(4 * want, (kFusedResident + H - 1) / H);
     if (want > nchunk) want = nchunk;
     if (want < 1) want = 1;
     return (int)((nchunk + want - 1) / want);
@@ -934,7 +1005,7 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     f.chunk_pre = sw.chunk_pre;
     f.nchunk = plan.nchunk;
     f.chunk = plan.blocks * ha_sel::kBlock;
-    f.cps = fused_chunks_per_split(B, H, plan.nchunk);
+    f.cps = fused_chunks_per_split(B, H, plan.nchunk, seq_lens != nullptr);
     f.gq = H / Hc;
     f.init = init_budget;
     f.recent = recent_budget;

@@ -48,6 +48,7 @@ class HashDecodeLayer:
         # rebuild the index list in LDS inside the attend launch instead of writing it to memory (simple mode, lists of
         # up to 8192 entries; decided per allocation)
         self.use_fused = True
+        self.fused_min_rows = 32
         self.device = torch.device(device)
         self.wk = _ops.pack_usa_weights(k_layers, self.device)
         self.wq = _ops.pack_usa_weights(q_layers, self.device)
@@ -75,13 +76,15 @@ class HashDecodeLayer:
         self.codes = torch.zeros(B, self.Hc, S_cap, self.W, dtype=torch.int32, device=dev)
         self.qcodes = torch.zeros(B, self.H, 1, self.W, dtype=torch.int32, device=dev)
         self.idx_cap = self.index_capacity(S_cap)
-        self.idx = torch.empty(B, self.H, self.idx_cap, dtype=torch.int32, device=dev)
+        # zero-filled: the fused path never writes the lists, and a gather over lists that were never selected must
+        # stay inside the cache
+        self.idx = torch.zeros(B, self.H, self.idx_cap, dtype=torch.int32, device=dev)
         self.counts = torch.zeros(B, self.H, dtype=torch.int32, device=dev)
         self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
         self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
-        # measured: the fused launch wins when a row is cut into at most two pieces (B * H >= 256 rows keep 256 CUs busy);
-        # with more, finer pieces the two-launch path is a few microseconds ahead
-        self.fused_ok = B * self.H >= 256 and _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget,
+        # measured: with the thresholds derived in the attention launch the fused path is ahead from 32 rows on (a row
+        # is then cut into up to 16 pieces: 40.3 against 45.2 us at B = 1, 32K tokens; 84.1 against 86.5 us at B = 4, 128K)
+        self.fused_ok = B * self.H >= self.fused_min_rows and _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget,
                                                                  self.recent_budget, self.heavy_budget, self.mode)
         # rows of up to 64 chunks: the attention launch derives the thresholds itself, the step is three launches
         self.local_thresholds = _ops.fused_local_thresholds(B, self.Hc, S_cap)

@@ -138,3 +138,26 @@ def test_bf16_decoder_step_with_and_without_the_skinny_projections():
         b = dec.decode_step(tokens, advance=False).float()
     assert torch.isfinite(a).all()
     assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
+
+
+def test_decoder_step_on_the_fused_attention_path_matches_the_two_launch_path():
+    # 32 (sequence, head) rows: every layer takes ha_select_histogram + ha_sparse_decode_fused; the same step through
+    # ha_select + ha_sparse_decode must agree to bf16 noise, and the index lists the fused path never writes stay usable
+    print("\n[case] bf16 decoder step, fused attention path on/off", flush=True)
+    dec = LlamaShapedDecoder(n_layers=2, hidden=512, ffn=1024, n_heads=8, n_kv_heads=2, head_dim=128, vocab=512, n_code_heads=2,
+                             init_budget=8, recent_budget=8, heavy_budget=0.125, dtype=torch.bfloat16, device=DEV, seed=4)
+    dec.allocate(4, 3000)
+    dec.fill_cache_synthetic(2500)
+    assert all(hl.fused_ok for hl in dec.hash)
+    tokens = torch.tensor([5, 17, 40, 3], device=DEV)
+    with torch.no_grad():
+        a = dec.decode_step(tokens, advance=False).float()
+        hl0 = dec.hash[0]
+        out = torch.empty(4, 8, 128, dtype=torch.bfloat16, device=DEV)
+        hl0.attend(dec.q_rot, dec.k_cache[0], dec.v_cache[0], out)          # lists never selected: zero-filled, in bounds
+        for hl in dec.hash:
+            hl.use_fused = False
+        b = dec.decode_step(tokens, advance=False).float()
+    torch.cuda.synchronize()
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())

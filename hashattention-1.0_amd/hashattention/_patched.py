@@ -10,14 +10,17 @@ What differs from the reference on purpose
   * ties at the top-k boundary go to the lowest token index (the reference's `sort` at :430 is unstable);
   * softmax and the value product are fp32 throughout (the reference rounds probabilities to the query
     dtype at :613);
-  * soft mode (`hard=False`: tanh / sigmoid, :174-176, 197-198), `CENTER` normalisation (:163-167), the LSH
-    baseline (`lth_num_layers == 0`, :130-139) and the training hooks (:304-316 and the train branch of :370-371)
-    are outside the accelerated path and raise NotImplementedError instead of silently running something else;
-    the recall statistic (:319-398, eval branch) is built on the selection kernel (`usa_local_compute`).
+  * the LSH baseline (`lth_num_layers == 0`, :130-139) is not built, and `CENTER` normalisation (:163-167) exists
+    only in soft mode: the bit-cache keeps codes of keys hashed once, which a statistic over all cached keys would
+    invalidate at every step;
+  * the training side - soft mode (`hard=False`: tanh / sigmoid, :174-176, 197-198), `train_step` (:304-316) and the train
+    branch of `usa_local_compute` (:356-371) - is differentiable torch code batched over heads (one baddbmm per MLP layer
+    instead of a Python loop over heads); the recall statistic (:372-398) runs on the selection kernel.
 """
 from __future__ import annotations
 
 import math
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -49,6 +52,7 @@ class USA(nn.Module):
             raise NotImplementedError("lth_num_layers must be 1, 2 or 3 (the LSH baseline, 0, is not part of this build)")
         if self.lth_final_dim not in (32, 64):
             raise NotImplementedError("lth_final_dim must be 32 or 64: codes are packed in one or two 32-bit words")
+        self.center = bool(os.environ.get("CENTER", 0))      # as the reference reads it (:34, :98): any non-empty value is on
 
         def mlp():
             if self.num_layers == 3:
@@ -75,9 +79,29 @@ class USA(nn.Module):
         """A module kept in bf16 computes with bf16 roundings after every layer; anything else in fp32."""
         return _ops.HA_ARITH_BF16 if self.dtype == torch.bfloat16 else _ops.HA_ARITH_F32
 
-    def _embed(self, vectors: torch.Tensor, side: str, hard: bool) -> torch.Tensor:
+    def _stacked(self, side: str) -> List[Tuple[torch.Tensor, torch.Tensor]]:
+        """Per layer (W [heads, out, in], b [heads, out]) stacked from the per-head modules; gradients reach the modules."""
+        heads = self.layers(side)
+        return [(torch.stack([h[l][0] for h in heads]), torch.stack([h[l][1] for h in heads])) for l in range(self.num_layers)]
+
+    def _soft_logits(self, vectors: torch.Tensor, side: str) -> torch.Tensor:
+        """[b, heads, s, d] -> MLP outputs [b, heads, s, D], all heads in one baddbmm per layer (differentiable)."""
+        b, a, s, d = vectors.shape
+        if a != self.num_heads:
+            raise ValueError(f"expected {self.num_heads} heads, got {a}")
+        x = vectors.transpose(0, 1).reshape(a, b * s, d)
+        stacked = self._stacked(side)
+        for l, (w, bias) in enumerate(stacked):
+            x = torch.baddbmm(bias.unsqueeze(1), x, w.transpose(1, 2))
+            if l + 1 < len(stacked):
+                x = torch.nn.functional.silu(x)
+        return x.view(a, b, s, -1).transpose(0, 1)
+
+    def _embed(self, vectors: torch.Tensor, side: str, hard: bool):
         if not hard:
-            raise NotImplementedError("soft (tanh) embeddings are a training feature outside this build")
+            return torch.tanh(self._soft_logits(vectors.to(self.dtype), side)), None
+        if self.center:
+            raise NotImplementedError("CENTER normalisation is available in soft mode only: the bit-cache hashes every key once")
         b, a, s, d = vectors.shape
         if a != self.num_heads:
             raise ValueError(f"expected {self.num_heads} heads, got {a}")
@@ -88,25 +112,36 @@ class USA(nn.Module):
         return torch.sign(logits), codes
 
     def k_embedding(self, vectors: torch.Tensor, hard: bool = False) -> torch.Tensor:
-        """[b, heads, s, d] -> sign embeddings [b, heads, s, D] in fp32 (reference :204-214)."""
-        return self._embed(vectors, "k", hard)[0]
+        """[b, heads, s, d] -> embeddings [b, heads, s, D] in fp32: signs (hard) or tanh (soft) (reference :204-214)."""
+        return self._embed(vectors, "k", hard)[0].float()
 
     def q_embedding(self, vectors: torch.Tensor, hard: bool = False) -> torch.Tensor:
-        return self._embed(vectors, "q", hard)[0]
+        return self._embed(vectors, "q", hard)[0].float()
 
     def forward(self, K: torch.Tensor, Q: torch.Tensor, hard: bool = False):
-        """span[b, h, t, s] = <sign q_t, sign k_s> = D - 2 * Hamming, non-causal entries at finfo.min; returns
-        (span, sign(K embeddings)) as the reference (:151-200).  Diagnostic API: the decode path does not call it."""
-        ksign, kcodes = self._embed(K, "k", hard)
-        _, qcodes = self._embed(Q, "q", hard)
+        """hard: span[b, h, t, s] = <sign q_t, sign k_s> = D - 2 * Hamming, non-causal entries at finfo.min; soft (the
+        default, differentiable): sigmoid(<tanh q_t, tanh k_s> - lth_thold), non-causal entries 0.  Returns
+        (span, K embeddings) as the reference (:151-200).  The decode path does not call it."""
         b, a, s, _ = K.shape
         t = Q.shape[2]
+        causal = torch.tril(torch.ones(t, s, device=K.device), diagonal=s - t).bool()
+        if not hard:
+            if self.center:     # per head: keys and queries standardised with the statistics of the keys (:163-167)
+                mean = K.mean(dim=(0, 2), keepdim=True)
+                std = K.std(dim=(0, 2), keepdim=True)
+                K, Q = (K - mean) / (std + 1e-6), (Q - mean) / (std + 1e-6)
+            kt, _ = self._embed(K, "k", False)
+            qt, _ = self._embed(Q, "q", False)
+            span = torch.matmul(qt, kt.transpose(2, 3))
+            span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
+            return torch.sigmoid(span - self.lth_thold), kt
+        ksign, kcodes = self._embed(K, "k", hard)
+        _, qcodes = self._embed(Q, "q", hard)
         D = self.lth_final_dim
         span = torch.empty(b, a, t, s, dtype=K.dtype, device=K.device)
         for i in range(t):
             ham = _ops.hamming_score(kcodes, qcodes[:, :, i].contiguous(), s)
             span[:, :, i] = (D - 2 * ham.to(torch.int32)).to(K.dtype)
-        causal = torch.tril(torch.ones(t, s, device=K.device), diagonal=s - t).bool()
         span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
         return span, ksign.to(K.dtype)
 
@@ -137,6 +172,11 @@ class HeavyHitterMixin:
         self.tr_loss_func = None
         self.tr_optimizer = None
         self.overlaps = {}
+        self.last_train_loss = None
+        self.print_offloading_flag = False
+        # KV cache to host memory beyond this many tokens (reference :286, :495-511: 24000, sized for 80 GB parts).  Off by
+        # default here: 288 GB of HBM hold the caches this path is built for; set a length to get the reference's policy.
+        self.offloading_length = None
         self.flash_forward = None
         self._hash_layer: Optional[HashDecodeLayer] = None
 
@@ -147,8 +187,30 @@ class HeavyHitterMixin:
     def _reset_state(self):
         """A new example starts (reference :298-301): drop the cached codes."""
         self.past_key_signatures = None
+        self.print_offloading_flag = False
         if self._hash_layer is not None:
             self._hash_layer.reset()
+
+    # ---- KV offload policy (reference :495-511), on the installed cache classes (`cache.layers[i].keys / .values`)
+    def _cache_layer(self, cache):
+        if cache is None or not hasattr(cache, "layers") or len(cache.layers) <= self.layer_idx:
+            return None
+        layer = cache.layers[self.layer_idx]
+        return layer if getattr(layer, "keys", None) is not None else None
+
+    def ensure_gpu(self, cache, device):
+        layer = self._cache_layer(cache)
+        if layer is not None and not layer.keys.is_cuda:
+            layer.keys, layer.values = layer.keys.to(device), layer.values.to(device)
+
+    def offload_if_necessary_cpu(self, cache):
+        layer = self._cache_layer(cache)
+        if layer is None or self.offloading_length is None or layer.keys.shape[2] < self.offloading_length:
+            return
+        if not self.print_offloading_flag and self.layer_idx == 0:
+            print("OFFLOADING ENABLED >>")
+            self.print_offloading_flag = True
+        layer.keys, layer.values = layer.keys.cpu(), layer.values.cpu()
 
     # ---- bit-cache plumbing
     def _ensure_hash_layer(self, batch: int, seq_len: int, device) -> HashDecodeLayer:
@@ -220,14 +282,15 @@ class HeavyHitterMixin:
 
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
         bsz, q_len, _ = hidden_states.shape
+        self.ensure_gpu(cache, hidden_states.device)
         if q_len > DECODE_MAX_Q_LEN or self.train_usa:
-            if self.train_usa:
-                raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
-            # prefill: the original dense forward (reference :529-550); its keys are hashed lazily at the first decode step
+            # prefill, and every step while the hash is being trained: the original dense forward (reference :529-550);
+            # its keys are hashed lazily at the first decode step
             ret = self.flash_forward(hidden_states=hidden_states, position_embeddings=position_embeddings,
                                      attention_mask=attention_mask, past_key_values=cache, **kwargs)
-            if self.collect_stats:
+            if self.collect_stats or self.train_usa:
                 self.usa_local_compute(hidden_states, attention_mask, None, cache, position_embeddings)
+            self.offload_if_necessary_cpu(cache)
             return ret
         hidden_shape = (bsz, q_len, -1, self.head_dim)
         query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
@@ -243,7 +306,9 @@ class HeavyHitterMixin:
             key_states, value_states = key_states.contiguous(), value_states.contiguous()
         attn = self._sparse_attention(query_states.contiguous(), key_states, value_states)
         attn = attn.transpose(1, 2).reshape(bsz, q_len, -1).contiguous()
-        return self.o_proj(attn), None
+        out = self.o_proj(attn)
+        self.offload_if_necessary_cpu(cache)
+        return out, None
 
     # ---- reference API kept for callers; outside the accelerated path
     def compute_mask_multi(self, key_states, query_states):
@@ -279,8 +344,26 @@ class HeavyHitterMixin:
         assert query_states.shape[-2] == 1
         return self.compute_mask_multi(key_states, query_states)
 
-    def train_step(self, *a, **k):
-        raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
+    @torch.inference_mode(False)
+    def train_step(self, K, Q, target, target_mask):
+        """One optimizer step of the hash module on this layer's keys and queries (reference :304-316): soft scores of
+        Q [b, H, q, d] against K [b, H, S, d] (KV heads already repeated), entries outside `target_mask` zeroed, the
+        installed loss against `target`, backward, optimizer step.  The loss is kept in `last_train_loss`."""
+        if self.tr_loss_func is None or self.tr_optimizer is None:
+            raise RuntimeError("set_train_usa_mode(model, loss_func, optimizer) must install a loss and an optimizer first")
+        with torch.enable_grad():
+            K, Q, target = K.clone(), Q.clone(), target.clone()      # tensors of their own for the backward pass
+            span, _ = self.usa_module(K, Q)
+            span = span.masked_fill(torch.logical_not(target_mask), 0)
+            loss = self.tr_loss_func(span, target)
+            self.tr_optimizer.zero_grad()
+            loss.backward()
+            self.tr_optimizer.step()
+        self.last_train_loss = loss.detach()
+        if self._hash_layer is not None:       # the packed weights and the cached codes belong to the old parameters
+            self._hash_layer = None
+        if self.layer_idx == 5:
+            print(self.layer_idx, K.shape[2], "Train Loss:", loss.item(), flush=True)
 
     def usa_local_compute(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None,
                           position_embeddings=None):
@@ -292,8 +375,6 @@ class HeavyHitterMixin:
         The hash side runs on the selection kernel: all rows of the chunk in one ha_select call against the same codes
         (batch stride 0), each row with its own length.  Ties of the hash score go to the lowest index (the reference's
         torch.topk leaves them open); rows with fewer than 32 candidates count only real candidates as targets."""
-        if self.train_usa:
-            raise NotImplementedError("USA training runs on the reference implementation; this build is inference-only")
         cache = past_key_value
         if cache is None or len(cache.layers) <= self.layer_idx:
             return
@@ -311,6 +392,19 @@ class HeavyHitterMixin:
         q = q.contiguous()
         keys = keys if keys.stride(-1) == 1 else keys.contiguous()
         dev = q.device
+        if self.train_usa:
+            # train branch (:356-371): per row, the 32 highest true logits among the candidates [init, pos - recent] are the
+            # positives; the hash module takes one optimizer step on them.  Logits in fp32 (the reference: model dtype).
+            kk = keys.repeat_interleave(self.num_key_value_groups, dim=1)                       # [b, H, S, d]
+            w = torch.matmul(q.float(), kk.float().transpose(2, 3)) / math.sqrt(d)
+            cand = torch.tril(torch.ones(q_len, S, device=dev), diagonal=S - q_len - self.recent_budget).bool()
+            cand[:, :self.init_budget] = False
+            w.masked_fill_(torch.logical_not(cand), torch.finfo(w.dtype).min)
+            target = torch.zeros(w.shape, dtype=self.usa_module.dtype, device=dev)
+            target.scatter_(-1, torch.topk(w, k=32, dim=-1).indices, 1.0)
+            del w
+            self.train_step(kk.to(self.usa_module.dtype), q.to(self.usa_module.dtype), target, cand)
+            return
 
         # ---- hash side: codes of all keys and of every query row, one selection per row
         hl = self._ensure_hash_layer(bsz, S, dev)

@@ -38,7 +38,6 @@ class LlamaAttention_heavy_hitter(HeavyHitterMixin, nn.Module):
         self.v_proj = nn.Linear(config.hidden_size, config.num_key_value_heads * self.head_dim, bias=bias)
         self.o_proj = nn.Linear(config.num_attention_heads * self.head_dim, config.hidden_size, bias=bias)
         self._init_heavy_hitter(config)
-        self.offloading_length = 24000       # reference :286; KV offload to the host is not part of this build
 
     @staticmethod
     def _apply_rope(q, k, cos, sin):

@@ -29,7 +29,6 @@ class MistralAttention_heavy_hitter(HeavyHitterMixin, nn.Module):
         self.v_proj = nn.Linear(config.hidden_size, config.num_key_value_heads * self.head_dim, bias=False)
         self.o_proj = nn.Linear(config.num_attention_heads * self.head_dim, config.hidden_size, bias=False)
         self._init_heavy_hitter(config)
-        self.offloading_length = 25000       # reference mistral:230
 
     @staticmethod
     def _apply_rope(q, k, cos, sin):

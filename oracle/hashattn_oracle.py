@@ -19,6 +19,9 @@ Stages
                             helpers the reference imports (hashattention_llama.py:18); the reference
                             holds no test at that boundary: parity unpinned there.
   reference_decode_attention  the whole emulated layer-step (used as the timed CPU baseline)
+  usa_forward_soft          tanh embeddings, sigmoid(span - thold)  hashattention_llama.py:151-200 (hard=False)
+  recall_targets            true-logit top-32 target + candidate mask of the train branch  hashattention_llama.py:356-371
+  weighted_bce / train_step the training script's loss and one optimizer step  train_hashattention.py:88-95, hashattention_llama.py:304-316
 
 Tie-break.  The reference sorts with `span.sort(descending=True)` without
 `stable=True` (hashattention_llama.py:430), so which of the equal-score tokens
@@ -335,3 +338,62 @@ def recall_overlap(q: torch.Tensor, k: torch.Tensor, k_heads, q_heads, init_budg
                 pred = set(int(js[t]) for t in order)
                 out[bb, h, i] = sum(1 for j in true_top.tolist() if j in pred) / float(top_true)
     return out
+
+
+# --------------------------------------------------------------------------- training side
+
+def usa_forward_soft(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads, thold: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """`USA.forward(K, Q, hard=False)`: tanh of both embeddings, span = <tanh q, tanh k>, non-causal entries set to
+    finfo.min, then sigmoid(span - thold) (so non-causal entries come out as exactly 0).  Returns (scores, tanh K).
+
+    reference: hashattention_llama.py:151-200 (:174-176 tanh, :184-185 baddbmm, :190-194 causal fill, :196-197 sigmoid).
+    Differentiable: built from torch ops on whatever tensors the head lists hold.
+    """
+    kt = torch.tanh(usa_logits(K, k_heads))
+    qt = torch.tanh(usa_logits(Q, q_heads))
+    span = torch.einsum("bhtd,bhsd->bhts", qt, kt)
+    t, s = Q.shape[-2], K.shape[-2]
+    causal = torch.tril(torch.ones(t, s), diagonal=s - t).bool()
+    span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype))
+    return torch.sigmoid(span - thold), kt
+
+
+def recall_targets(q: torch.Tensor, k: torch.Tensor, init_budget: int, recent_budget: int, top_true: int = 32):
+    """What the train branch of `usa_local_compute` hands to `train_step` (hashattention_llama.py:356-371): the candidate
+    mask [q_len, S] (causal, minus the recent window, minus the sink) and the 0/1 target [b, H, q_len, S] marking each
+    row's `top_true` highest true logits q.k/sqrt(d) after non-candidates were set to finfo.min.  q [b, H, q_len, d] are
+    the rotated queries of the last q_len positions, k [b, Hkv, S, d] the cached keys."""
+    b, H, q_len, d = q.shape
+    S = k.shape[2]
+    kk = repeat_kv(k, H // k.shape[1])
+    w = torch.matmul(q, kk.transpose(2, 3)) / math.sqrt(d)                                    # :358
+    cand = torch.tril(torch.ones(q_len, S), diagonal=S - q_len - recent_budget).bool()        # :360
+    cand[:, :init_budget] = False                                                              # :361
+    w = w.masked_fill(torch.logical_not(cand), torch.finfo(w.dtype).min)                       # :363
+    idx = torch.topk(w, k=top_true, dim=-1).indices                                            # :365
+    target = torch.zeros_like(w)
+    target.scatter_(-1, idx, 1.0)                                                              # :366-368
+    return target, cand
+
+
+def weighted_bce(alpha: float, beta: float):
+    """The loss the training script installs (train_hashattention.py:88-95): binary cross entropy with positives weighted
+    by S * beta + alpha, mean over all entries."""
+    def loss(yhat: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+        w = y.shape[-1] * beta + alpha
+        weight = y * (w - 1) + torch.ones_like(y)
+        return F.binary_cross_entropy(yhat.reshape(-1), y.reshape(-1), weight=weight.reshape(-1))
+    return loss
+
+
+def train_step(K, Q, target, target_mask, k_heads, q_heads, loss_fn, optimizer, thold: float = 0.0) -> float:
+    """One `train_step` (hashattention_llama.py:304-316): soft scores, entries outside `target_mask` zeroed, loss against
+    the target, zero_grad / backward / step.  The head lists must hold the leaf tensors the optimizer updates.
+    Returns the loss before the update."""
+    span, _ = usa_forward_soft(K.clone(), Q.clone(), k_heads, q_heads, thold)
+    span = span.masked_fill(torch.logical_not(target_mask), 0)
+    loss = loss_fn(span, target.clone())
+    optimizer.zero_grad()
+    loss.backward()
+    optimizer.step()
+    return float(loss.item())

@@ -47,9 +47,9 @@ def test_config0_inputs_are_reproducible_and_golden_holds():
         assert (np.abs(kl.numpy())[bits] < 1e-4).all()
 
 
-def _usa_heads(g):
+def _usa_heads(g, prefix="w", leaf=False):
     keys = [str(k) for k in g["state_keys"]]
-    sd = {k: torch.from_numpy(g[f"w{i}"]) for i, k in enumerate(keys)}
+    sd = {k: torch.from_numpy(g[f"{prefix}{i}"]).clone().requires_grad_(leaf) for i, k in enumerate(keys)}
     heads = {"k": [], "q": []}
     for side in ("k", "q"):
         h = 0
@@ -132,3 +132,53 @@ def test_usa_state_dict_layout_matches_the_reference_checkpoints():
     # and the ModuleList wrapping of load_usa gives the "{layer}." prefix of the shipped checkpoints
     ml = torch.nn.ModuleList([usa])
     assert list(ml.state_dict().keys())[0] == "0." + keys[0]
+
+
+def test_training_side_of_the_oracle_matches_vectors_recorded_from_the_reference():
+    """Soft-mode USA.forward, three train_step calls (weighted BCE, Adam) and the train branch's targets, as recorded
+    from the reference's own code by tests/golden/make_reference_train_vectors.py."""
+    g = np.load(os.path.join(HERE, "reference_train_vectors.npz"))
+    K, Q = torch.from_numpy(g["K"]), torch.from_numpy(g["Q"])
+    heads = _usa_heads(g)
+    span, kt = orc.usa_forward_soft(K, Q, heads["k"], heads["q"], 0.0)
+    assert (span - torch.from_numpy(g["soft_span"])).abs().max().item() < 1e-6
+    assert (kt - torch.from_numpy(g["soft_k"])).abs().max().item() < 1e-6
+    q_len, S = Q.shape[2], K.shape[2]
+    assert (span[0, 0, 0, S - q_len + 1:] == 0).all()                  # non-causal entries: sigmoid(finfo.min) = 0 exactly
+    # three optimizer steps from the recorded start
+    leaf = _usa_heads(g, leaf=True)
+    params = [t for side in ("k", "q") for head in leaf[side] for wb in head for t in wb]
+    alpha, beta = g["bce_alpha_beta"]
+    loss_fn = orc.weighted_bce(float(alpha), float(beta))
+    opt = torch.optim.Adam(params, lr=0.001)
+    target = torch.from_numpy(g["target"].astype(np.float32))
+    mask = torch.from_numpy(g["target_mask"])
+    losses = [orc.train_step(K, Q, target, mask, leaf["k"], leaf["q"], loss_fn, opt) for _ in range(3)]
+    assert np.abs(np.array(losses) - g["losses"]).max() < 1e-5 and losses[2] < losses[0]
+    after = _usa_heads(g, prefix="w_after")
+    for side in ("k", "q"):
+        for mine, ref in zip(leaf[side], after[side]):
+            for (w, b), (wr, br) in zip(mine, ref):
+                assert (w.detach() - wr).abs().max().item() < 2e-6 and (b.detach() - br).abs().max().item() < 2e-6
+    assert (leaf["k"][0][0][0].detach() - heads["k"][0][0][0]).abs().max().item() > 1e-4       # the weights did move
+    # the loss alone, from its definition: mean of -w [y log p + (1 - y) log(1 - p)], positives weighted S * beta + alpha
+    p0 = span.masked_fill(~mask, 0).double()
+    y = target.double()
+    wgt = torch.where(y > 0, torch.tensor(S * float(beta) + float(alpha), dtype=torch.float64), torch.tensor(1.0, dtype=torch.float64))
+    by_hand = -(wgt * (y * torch.log(p0).clamp(min=-100) + (1 - y) * torch.log(1 - p0).clamp(min=-100))).mean().item()
+    assert abs(by_hand - g["losses"][0]) < 1e-5
+    # targets of the train branch
+    d = 128
+    hs = torch.from_numpy(g["lc_hidden"])
+    qw = torch.from_numpy(g["lc_q_weight"])
+    keys = torch.from_numpy(g["lc_keys"].astype(np.float32))
+    cos, sin = torch.from_numpy(g["lc_cos"]), torch.from_numpy(g["lc_sin"])
+    q = (hs @ qw.t()).view(1, hs.shape[1], -1, d).transpose(1, 2)
+    q, _ = orc.apply_rotary_pos_emb(q, q, cos, sin)
+    assert (q - torch.from_numpy(g["lc_Q"])).abs().max().item() < 1e-5
+    init, recent = (int(x) for x in g["lc_params"])
+    tgt, cand = orc.recall_targets(q, keys, init, recent)
+    S2 = keys.shape[2]
+    assert np.array_equal(np.packbits(cand.numpy(), axis=-1), g["lc_mask"])
+    assert np.array_equal(np.packbits(tgt.numpy().astype(bool), axis=-1), g["lc_target"])
+    assert int(tgt.sum()) == 32 * q.shape[1] * q.shape[2] and not tgt[..., ~cand[-1]].bool()[..., -1, :].any() and S2 == 1024

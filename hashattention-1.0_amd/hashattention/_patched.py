@@ -30,6 +30,32 @@ from . import _ops
 from .decode import HashDecodeLayer
 
 DECODE_MAX_Q_LEN = 128   # reference: `if q_len > 128 or self.train_usa` routes to the original forward (:529)
+DEFAULT_USA_CFG = {"lth_int_dim": 128, "lth_final_dim": 32, "lth_thold": 0}     # reference :68-72
+
+
+def memory_efficient_softmax(x: torch.Tensor, dim: int) -> torch.Tensor:
+    """Max-subtracted softmax in the input's dtype (reference :37-44; its `use_softmax_maxtrick` switch).  The kernels of
+    this build always subtract the running maximum; the function is kept for callers of the module API."""
+    e = torch.exp(x - x.amax(dim=dim, keepdim=True))
+    return e / e.sum(dim=dim, keepdim=True)
+
+
+class SignSTE(torch.autograd.Function):
+    """sign(x) whose gradient is that of tanh(x) (reference :51-63)."""
+
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return torch.sign(x)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        return grad_output * (1 - torch.tanh(x).square())
+
+
+def ste_sign(x: torch.Tensor) -> torch.Tensor:
+    return SignSTE.apply(x)
 
 
 class USA(nn.Module):
@@ -40,7 +66,7 @@ class USA(nn.Module):
     so reference checkpoints load unchanged.
     """
 
-    def __init__(self, num_heads: int, head_dim: int, usa_params: dict):
+    def __init__(self, num_heads: int, head_dim: int, usa_params: dict = DEFAULT_USA_CFG):
         super().__init__()
         self.head_dim = head_dim
         self.num_heads = num_heads

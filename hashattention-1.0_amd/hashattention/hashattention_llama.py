@@ -15,10 +15,11 @@ import torch
 from torch import nn
 from transformers.models.llama.modeling_llama import LlamaAttention, apply_rotary_pos_emb
 
-from ._patched import USA, HeavyHitterMixin, build_usa_modules, convert_modules, walk
+from ._patched import (DEFAULT_USA_CFG, USA, HeavyHitterMixin, SignSTE, build_usa_modules, convert_modules,
+                       memory_efficient_softmax, ste_sign, walk)
 
 __all__ = ["USA", "LlamaAttention_heavy_hitter", "load_usa", "convert_usa", "reset_usa", "set_train_usa_mode",
-           "set_eval_usa_mode", "print_stats"]
+           "set_eval_usa_mode", "print_stats", "SignSTE", "ste_sign", "memory_efficient_softmax", "DEFAULT_USA_CFG"]
 
 
 class LlamaAttention_heavy_hitter(HeavyHitterMixin, nn.Module):

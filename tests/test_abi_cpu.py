@@ -188,3 +188,21 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_ops, "lib_path", lambda: str(tmp_path / "libhashattn.so"))
     with pytest.raises(ImportError):
         _ops.load_library()
+
+
+def test_module_api_helpers_of_the_reference_are_present():
+    """Small pieces of the reference's module surface that need no kernel: `ste_sign` (sign forward, tanh-derivative
+    backward, hashattention_llama.py:51-66), `memory_efficient_softmax` (:37-44), `DEFAULT_USA_CFG` (:68-72)."""
+    import torch
+    from hashattention import hashattention_llama as hl, hashattention_mistral as hm
+    x = torch.tensor([-2.0, -0.0, 0.0, 0.3, 5.0], requires_grad=True)
+    y = hl.ste_sign(x)
+    assert y.tolist() == [-1.0, 0.0, 0.0, 1.0, 1.0]
+    (y * torch.arange(1.0, 6.0)).sum().backward()
+    assert torch.allclose(x.grad, torch.arange(1.0, 6.0) * (1 - torch.tanh(x.detach()) ** 2))
+    z = torch.randn(3, 7) * 30
+    assert torch.allclose(hl.memory_efficient_softmax(z, dim=-1), torch.softmax(z, dim=-1), atol=1e-6)
+    assert hl.DEFAULT_USA_CFG == {"lth_int_dim": 128, "lth_final_dim": 32, "lth_thold": 0}
+    for api in (hl, hm):
+        for name in ("USA", "load_usa", "convert_usa", "reset_usa", "set_train_usa_mode", "set_eval_usa_mode", "print_stats"):
+            assert callable(getattr(api, name))

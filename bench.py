@@ -84,6 +84,43 @@ def cpu_baseline(w, torch, budget_s=12.0):
                       f"{torch.get_num_threads()} torch threads), {sum(times):.2f} s measured, scaled x{scale:.2f} by cached tokens"}
 
 
+def cpu_sparse_stages(w, torch):
+    """The same stages as the GPU step (codes cached, encode the new token, select, gather-attend), run by the C oracle
+    (OpenMP) on the host for the first sequence of the workload and scaled linearly by cached tokens to the batch.  The
+    codes of the cached keys are made beforehand, un-timed, as on the GPU."""
+    import numpy as np
+    from hashattention.synthetic import Workload, make_problem
+    from oracle import c_oracle, hashattn_oracle as orc
+    w1 = Workload(**{**w.__dict__, "name": w.name + "-cpu", "batch": 1, "seq_lens": [w.seq_lens[0]], "seed": w.seed})
+    p = make_problem(w1)
+    S, H, Hkv, d = w1.seq_lens[0], w.n_q_heads, w.n_kv_heads, w.head_dim
+    Hc, W = len(p.usa.k), w.lth_final_dim // 32
+    np_layers = lambda head: [(Wt.numpy(), b.numpy()) for Wt, b in head]
+    kf = p.k.float()
+    kcodes = np.empty((1, Hc, S, W), dtype=np.uint32)
+    for hc in range(Hc):
+        kcodes[0, hc] = c_oracle.encode(kf[0, hc * Hkv // Hc].numpy(), np_layers(p.usa.k[hc]))[1]
+    t0 = time.perf_counter()
+    qcodes = np.empty((1, H, W), dtype=np.uint32)
+    for hc in range(Hc):        # the new key's code (already in kcodes: timed for the work, result identical)
+        c_oracle.encode(kf[0, hc * Hkv // Hc, S - 1:S].numpy(), np_layers(p.usa.k[hc]))
+    for h in range(H):
+        qcodes[0, h] = c_oracle.encode(p.q[0, h].float().numpy(), np_layers(p.usa.q[h]))[1][0]
+    t1 = time.perf_counter()
+    cap = min(S, w.init_budget + w.recent_budget + orc.heavy_count(S, w.heavy_budget))
+    idx, counts = c_oracle.select(kcodes, qcodes, [S], w.init_budget, w.recent_budget, w.heavy_budget, cap)
+    t2 = time.perf_counter()
+    c_oracle.sparse_attend(p.q[:, :, 0], p.k, p.v, idx, counts, 1.0 / math.sqrt(d))
+    t3 = time.perf_counter()
+    scale = sum(w.seq_lens) / S
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count()))
+    enc, sel, att = (t1 - t0) * 1e6 * w.batch, (t2 - t1) * 1e6 * scale, (t3 - t2) * 1e6 * scale
+    return {"value": enc + sel + att, "unit": "us/layer", "cores": threads, "kind": "port",
+            "stages_us": {"encode_new_k_and_q": enc, "score_select_full_sort": sel, "gather_attend": att},
+            "sample": f"sequence 0 of {w.batch} ({S} tokens, C oracle with OpenMP, {threads} threads), {t3 - t0:.2f} s measured; "
+                      f"encode scaled x{w.batch} by sequences, select and attend x{scale:.2f} by cached tokens"}
+
+
 def traffic_probe(torch, layer, q3, k, v, out, fused_attend=None):
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain copy of known size, then the gather-attend
     kernel, three launches each.  The copy gives the scale of the counter (bytes per reported KiB)."""
@@ -361,6 +398,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)
+        res["cpu_sparse_port"] = cpu_sparse_stages(w, torch)
     print(json.dumps(res))
 
 

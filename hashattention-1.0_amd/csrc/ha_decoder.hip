@@ -39,17 +39,33 @@ template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
-template <int NWAVE, int XCH, int R, int MM>
+// FUSE bit 0: RMSNorm of x in front (x <- bf16(x * rsqrt(mean x^2 + eps) * norm_w), the rounding of a separate norm
+// launch): every workgroup holds all of x, so it norms it itself.  FUSE bit 1: SwiGLU behind (W = [gate rows; up rows],
+// N = 2 F): a workgroup owns RB / 2 gate rows and the RB / 2 up rows of the same columns and writes
+// bf16(bf16(silu(bf16 gate)) * bf16 up) to out [M, F], the roundings of a separate activation launch.
+template <int NWAVE, int XCH, int R, int MM, int FUSE>
 __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *__restrict__ x, int64_t x_sm,
                                                                const uint16_t *__restrict__ w, int64_t w_sn,
                                                                const uint16_t *__restrict__ res, int64_t res_sm,
-                                                               uint16_t *__restrict__ out, int64_t out_sm, int M, int N, int K, int RB) {
+                                                               uint16_t *__restrict__ out, int64_t out_sm, int M, int N, int K, int RB,
+                                                               const uint16_t *__restrict__ norm_w, float eps) {
     constexpr int NV = R * MM;       // sums per lane and row group: 8 or 16
     constexpr int NP = NWAVE * 4;    // partials per sum: one per 16-lane row of every wave
+    constexpr bool kNorm = FUSE & 1, kGlu = FUSE & 2;
     extern __shared__ float s_part[];  // [RB * MM][NP]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int n0 = blockIdx.x * RB;
-    const int nrows = min(RB, N - n0);
+    const int half = RB / 2, F = N / 2;                      // SwiGLU: rows [0, half) of the workgroup are gate rows
+    const int n0 = kGlu ? blockIdx.x * half : blockIdx.x * RB;
+    const int nrows = kGlu ? RB : min(RB, N - n0);
+    // row of W behind local row r, or -1
+    auto w_row = [&](int r) {
+        if constexpr (kGlu) {
+            const int c = n0 + (r < half ? r : r - half);
+            return c < F ? (r < half ? c : F + c) : -1;
+        } else {
+            return r < nrows ? n0 + r : -1;
+        }
+    };
     const int kbase = wave * XCH * 512 + lane * 8;  // first element of this lane's 16 bytes in chunk 0 of its slice
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
 
@@ -69,10 +85,64 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
 #pragma unroll
             for (int c = 0; c < XCH; ++c) {
                 const int k = kbase + c * 512;
-                wv[r][c] = (r0 + r < nrows && k < K) ? *reinterpret_cast<const uint4 *>(w + (int64_t)(n0 + r0 + r) * w_sn + k) : zero;
+                const int n = w_row(r0 + r);
+                wv[r][c] = (n >= 0 && k < K) ? *reinterpret_cast<const uint4 *>(w + (int64_t)n * w_sn + k) : zero;
             }
     };
-    fetch(0, wc);
+    if constexpr (kNorm) {
+        // the first weight rows are requested before the norm is worked out
+        fetch(0, wc);
+        uint4 gw[XCH];
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) {
+            const int k = kbase + c * 512;
+            gw[c] = k < K ? *reinterpret_cast<const uint4 *>(norm_w + k) : zero;
+        }
+        float ss[MM];
+#pragma unroll
+        for (int m = 0; m < MM; ++m) {
+            float a = 0.f;
+#pragma unroll
+            for (int c = 0; c < XCH; ++c) {
+                const uint32_t *p = reinterpret_cast<const uint32_t *>(&xr[c][m]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = __uint_as_float(p[i] << 16), hi = __uint_as_float(p[i] & 0xffff0000u);
+                    a = fmaf(lo, lo, fmaf(hi, hi, a));
+                }
+            }
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) a += __shfl_xor(a, o);
+            ss[m] = a;
+        }
+        if (lane == 0)
+#pragma unroll
+            for (int m = 0; m < MM; ++m) s_part[wave * MM + m] = ss[m];
+        __syncthreads();
+        float rstd[MM];
+#pragma unroll
+        for (int m = 0; m < MM; ++m) {
+            float a = 0.f;
+            for (int wv = 0; wv < NWAVE; ++wv) a += s_part[wv * MM + m];
+            rstd[m] = rsqrtf(a / (float)K + eps);
+        }
+        __syncthreads();  // s_part is written again by the main loop
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) {
+            const uint32_t *g = reinterpret_cast<const uint32_t *>(&gw[c]);
+#pragma unroll
+            for (int m = 0; m < MM; ++m) {
+                uint32_t *p = reinterpret_cast<uint32_t *>(&xr[c][m]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = __uint_as_float(p[i] << 16) * rstd[m] * __uint_as_float(g[i] << 16);
+                    const float hi = __uint_as_float(p[i] & 0xffff0000u) * rstd[m] * __uint_as_float(g[i] & 0xffff0000u);
+                    p[i] = ha_f32_to_bf16_bits(lo) | (ha_f32_to_bf16_bits(hi) << 16);
+                }
+            }
+        }
+    }
+    if constexpr (!kNorm) fetch(0, wc);
     for (int r0 = 0; r0 < nrows; r0 += R) {
         if (r0 + R < nrows) fetch(r0 + R, wn);
         float v[NV];
@@ -119,14 +189,28 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
             for (int c = 0; c < XCH; ++c) wc[r][c] = wn[r][c];
     }
     __syncthreads();
-    for (int o = tid; o < nrows * M; o += NWAVE * 64) {
-        const int m = o / nrows, r = o % nrows;  // consecutive threads write consecutive columns of y
+    auto total = [&](int r, int m) {
         const float *pp = s_part + (r * MM + m) * NP;
         float y = 0.f;
 #pragma unroll 8
         for (int p = 0; p < NP; ++p) y += pp[p];
-        if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + r] << 16);
-        out[(int64_t)m * out_sm + n0 + r] = (uint16_t)ha_f32_to_bf16_bits(y);
+        return y;
+    };
+    if constexpr (kGlu) {
+        const int ncols = min(half, F - n0);
+        for (int o = tid; o < ncols * M; o += NWAVE * 64) {
+            const int m = o / ncols, r = o % ncols;
+            const float g = ha_round_bf16(total(r, m)), u = ha_round_bf16(total(r + half, m));
+            const float y = ha_round_bf16(g / (1.0f + __expf(-g))) * u;
+            out[(int64_t)m * out_sm + n0 + r] = (uint16_t)ha_f32_to_bf16_bits(y);
+        }
+    } else {
+        for (int o = tid; o < nrows * M; o += NWAVE * 64) {
+            const int m = o / nrows, r = o % nrows;  // consecutive threads write consecutive columns of y
+            float y = total(r, m);
+            if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + r] << 16);
+            out[(int64_t)m * out_sm + n0 + r] = (uint16_t)ha_f32_to_bf16_bits(y);
+        }
     }
 }
 
@@ -266,28 +350,46 @@ int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, i
     return HA_OK;
 }
 
-int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
-                     int64_t residual_stride_m, void *out, int64_t out_stride_m, int M, int N, int K, void *stream) {
+}  // extern "C"
+
+static int linear_skinny_impl(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
+                              int64_t residual_stride_m, const void *norm_weight, float eps, int act, void *out, int64_t out_stride_m,
+                              int M, int N, int K, void *stream) {
     HA_REQUIRE(x && w && out, HA_ERR_NULL_POINTER, "x/w/out is NULL");
     HA_REQUIRE(M >= 1 && M <= 16 && N >= 1 && K >= 32 && K % 32 == 0, HA_ERR_BAD_SHAPE, "need 1 <= M <= 16, N >= 1, K a multiple of 32");
-    HA_REQUIRE(x_stride_m >= K && w_stride_n >= K && out_stride_m >= N && (!residual || residual_stride_m >= N), HA_ERR_BAD_SHAPE,
+    HA_REQUIRE(act == HA_ACT_NONE || act == HA_ACT_SWIGLU, HA_ERR_BAD_SHAPE, "unknown activation %d", act);
+    const int n_out = act == HA_ACT_SWIGLU ? N / 2 : N;
+    HA_REQUIRE(act != HA_ACT_SWIGLU || (N % 2 == 0 && !residual), HA_ERR_BAD_SHAPE, "SwiGLU needs an even number of weight rows and no residual");
+    HA_REQUIRE(x_stride_m >= K && w_stride_n >= K && out_stride_m >= n_out && (!residual || residual_stride_m >= N), HA_ERR_BAD_SHAPE,
                "strides smaller than the rows they span");
     HA_REQUIRE(ha_aligned(x, 16) && ha_aligned(w, 16) && x_stride_m % 8 == 0 && w_stride_n % 8 == 0, HA_ERR_MISALIGNED,
                "x and W rows must be 16-byte aligned");
+    const bool fused = norm_weight || act != HA_ACT_NONE;
+    HA_REQUIRE(!fused || (M <= 8 && K <= 16384), HA_ERR_BAD_SHAPE, "the fused norm / activation forms need M <= 8 and K <= 16384");
+    HA_REQUIRE(!norm_weight || (ha_aligned(norm_weight, 16) && eps >= 0.f), HA_ERR_MISALIGNED, "norm weight must be 16-byte aligned, eps >= 0");
     int st = ha_require_device();
     if (st) return st;
     const uint16_t *xp = (const uint16_t *)x, *wp = (const uint16_t *)w, *rp = (const uint16_t *)residual;
+    const uint16_t *gp = (const uint16_t *)norm_weight;
     uint16_t *op = (uint16_t *)out;
     hipStream_t s = (hipStream_t)stream;
     if (M <= 8 && K <= 16384) {
         // rows per workgroup: enough workgroups for two per CU, but at least 16 rows so that the slice of x a wave keeps
         // is paid for
         const int RB = (int64_t)N >= 64 * 1024 ? 64 : (int64_t)N >= 32 * 512 ? 32 : 16;
-        const dim3 g2((N + RB - 1) / RB);
+        const dim3 g2(act == HA_ACT_SWIGLU ? (N / 2 + RB / 2 - 1) / (RB / 2) : (N + RB - 1) / RB);
         const int chunks = (K + 511) / 512;
-#define HA_GEMV(NW_, XCH_, R_, MM_)                                                                                          \
-    hipLaunchKernelGGL((gemv_rows_kernel<NW_, XCH_, R_, MM_>), g2, dim3(NW_ * 64), (size_t)RB * MM_ * NW_ * 4 * sizeof(float), s, \
-                       xp, x_stride_m, wp, w_stride_n, rp, residual_stride_m, op, out_stride_m, M, N, K, RB)
+        const int fuse = (norm_weight ? 1 : 0) | (act == HA_ACT_SWIGLU ? 2 : 0);
+#define HA_GEMV_F(NW_, XCH_, R_, MM_, F_)                                                                                     \
+    hipLaunchKernelGGL((gemv_rows_kernel<NW_, XCH_, R_, MM_, F_>), g2, dim3(NW_ * 64), (size_t)RB * MM_ * NW_ * 4 * sizeof(float), s, \
+                       xp, x_stride_m, wp, w_stride_n, rp, residual_stride_m, op, out_stride_m, M, N, K, RB, gp, eps)
+#define HA_GEMV(NW_, XCH_, R_, MM_)                                  \
+    do {                                                             \
+        if (fuse == 0) HA_GEMV_F(NW_, XCH_, R_, MM_, 0);             \
+        else if (fuse == 1) HA_GEMV_F(NW_, XCH_, R_, MM_, 1);        \
+        else if (fuse == 2) HA_GEMV_F(NW_, XCH_, R_, MM_, 2);        \
+        else HA_GEMV_F(NW_, XCH_, R_, MM_, 3);                       \
+    } while (0)
         if (chunks <= 8) {
             if (M <= 4) HA_GEMV(8, 1, 4, 4);
             else HA_GEMV(8, 1, 2, 8);
@@ -299,6 +401,7 @@ int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w
             else HA_GEMV(16, 2, 1, 8);
         }
 #undef HA_GEMV
+#undef HA_GEMV_F
         HA_CHECK_LAUNCH("gemv_rows_kernel");
         return HA_OK;
     }
@@ -314,6 +417,21 @@ int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w
                            M, N, K);
     HA_CHECK_LAUNCH("skinny_linear_kernel");
     return HA_OK;
+}
+
+extern "C" {
+
+int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
+                     int64_t residual_stride_m, void *out, int64_t out_stride_m, int M, int N, int K, void *stream) {
+    return linear_skinny_impl(x, x_stride_m, w, w_stride_n, residual, residual_stride_m, nullptr, 0.f, HA_ACT_NONE, out, out_stride_m, M, N,
+                              K, stream);
+}
+
+int ha_linear_skinny_fused(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
+                           int64_t residual_stride_m, const void *norm_weight, float eps, int act, void *out, int64_t out_stride_m,
+                           int M, int N, int K, void *stream) {
+    return linear_skinny_impl(x, x_stride_m, w, w_stride_n, residual, residual_stride_m, norm_weight, eps, act, out, out_stride_m, M, N, K,
+                              stream);
 }
 
 }  // extern "C"

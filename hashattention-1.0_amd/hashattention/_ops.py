@@ -71,6 +71,8 @@ def load_library() -> C.CDLL:
     lib.ha_rope_append.argtypes = [vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]
     lib.ha_linear_skinny.restype = i32
     lib.ha_linear_skinny.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
+    lib.ha_linear_skinny_fused.restype = i32
+    lib.ha_linear_skinny_fused.argtypes = [vp, i64, vp, i64, vp, i64, vp, C.c_float, i32, vp, i64, i32, i32, i32, vp]
     lib.ha_swiglu.restype = i32
     lib.ha_swiglu.argtypes = [vp, i64, i32, i32, i32, vp, vp]
     lib.ha_select_prepare.restype = i32
@@ -392,15 +394,28 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _check(load_library().ha_swiglu(_ptr(gate_up), gate_up.stride(0), _DTYPE[gate_up.dtype], B, F, _ptr(out), _stream(gate_up)), "ha_swiglu")
 
 
-def linear_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out [M, N] = x [M, K] @ w[N, K]^T (+ residual [M, N]); bf16, M <= 16.  Streams w once."""
-    _require_cuda(x, w, out, residual)
+HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1
+
+
+def linear_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                  norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5, swiglu: bool = False) -> torch.Tensor:
+    """out [M, N] = x [M, K] @ w[N, K]^T (+ residual [M, N]); bf16, M <= 16.  Streams w once.
+    norm_weight [K]: x is RMS-normalised first (M <= 8, K <= 16384).  swiglu: w = [gate rows; up rows], out [M, N / 2] =
+    silu(gate) * up (M <= 8, K <= 16384, no residual)."""
+    _require_cuda(x, w, out, residual, norm_weight)
     assert x.dtype == w.dtype == out.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2 and out.dim() == 2
     assert x.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1 and (residual is None or (residual.stride(1) == 1 and residual.dtype == x.dtype))
     M, K = x.shape
     N = w.shape[0]
-    assert w.shape[1] == K and out.shape == (M, N) and (residual is None or residual.shape == (M, N))
-    _check(load_library().ha_linear_skinny(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual),
-                                           residual.stride(0) if residual is not None else 0, _ptr(out), out.stride(0), M, N, K,
-                                           _stream(x)), "ha_linear_skinny")
+    n_out = N // 2 if swiglu else N
+    assert w.shape[1] == K and out.shape == (M, n_out) and (residual is None or residual.shape == (M, N))
+    res_stride = residual.stride(0) if residual is not None else 0
+    if norm_weight is None and not swiglu:
+        _check(load_library().ha_linear_skinny(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual), res_stride, _ptr(out),
+                                               out.stride(0), M, N, K, _stream(x)), "ha_linear_skinny")
+        return out
+    assert norm_weight is None or (norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous())
+    _check(load_library().ha_linear_skinny_fused(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual), res_stride, _ptr(norm_weight),
+                                                 float(eps), HA_ACT_SWIGLU if swiglu else HA_ACT_NONE, _ptr(out), out.stride(0), M, N, K,
+                                                 _stream(x)), "ha_linear_skinny_fused")
     return out

@@ -127,8 +127,10 @@ class LlamaShapedDecoder:
         step can be replayed (HIP graph) at a fixed context length.  dense=True attends to the whole cache with the
         dense flash-decode kernel instead (the baseline the sparse step is compared with).
 
-        Per layer: RMSNorm, QKV GEMM, ha_rope_append, the attention step, output GEMM with the residual folded in
-        (addmm), RMSNorm, gate/up GEMM, ha_swiglu, down GEMM with the residual folded in."""
+        Per layer (bf16, up to 8 sequences): QKV projection with its RMSNorm folded in, ha_rope_append, the attention
+        step, output projection with the residual folded in, gate/up projection with its RMSNorm and SwiGLU folded in,
+        down GEMM with the residual folded in (addmm).  Other dtypes and batches: the same steps as library calls plus
+        ha_swiglu."""
         B, H, Hkv, d = self.B, self.H, self.Hkv, self.d
         pos = self.seq_len
         S = pos + 1
@@ -137,8 +139,10 @@ class LlamaShapedDecoder:
         # (2.6 -> 3.3, 1.8 -> 3.0, 4.0 -> 4.4 TB/s at B = 4) and slower for the down projection and the lm_head
         skinny = self.use_skinny and self.dtype == torch.bfloat16 and B <= 8
         for l, p in enumerate(self.layers):
-            h = F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps)
-            qkv = _ops.linear_skinny(h, p["wqkv"], self.qkv) if skinny else F.linear(h, p["wqkv"])
+            if skinny:      # RMSNorm rides in the projection that consumes it
+                qkv = _ops.linear_skinny(x, p["wqkv"], self.qkv, norm_weight=p["attn_norm"], eps=self.eps)
+            else:
+                qkv = F.linear(F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps), p["wqkv"])
             _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
             hl = self.hash[l]
             if dense:
@@ -148,10 +152,12 @@ class LlamaShapedDecoder:
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
             if skinny:
                 x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn, residual=x)
+                # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
+                _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             else:
                 x = torch.addmm(x, self.attn_out.view(B, H * d), p["wo"].t())
-            h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
-            _ops.swiglu(_ops.linear_skinny(h, p["w13"], self.gate_up) if skinny else F.linear(h, p["w13"]), self.ffn_act)
+                h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
+                _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
             x = torch.addmm(x, self.ffn_act, p["w2"].t())
         if advance:
             self.seq_len = S

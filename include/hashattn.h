@@ -271,6 +271,19 @@ int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, i
 int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n,
                      const void *residual, int64_t residual_stride_m, void *out, int64_t out_stride_m,
                      int M, int N, int K, void *stream);
+/*
+ * The same product with the neighbouring elementwise steps of the decoder layer folded in (efficiency/model.py:88-96
+ * RMSNorm, :261 feed-forward `w2(silu(w1 x) * w3 x)`):
+ *   norm_weight != NULL  x is RMS-normalised first: x <- bf16(x * rsqrt(mean_k x^2 + eps) * norm_weight[k]);
+ *   act == HA_ACT_SWIGLU w holds F gate rows followed by F up rows (N = 2 F); out [M, F] = silu(gate) * up with the
+ *                        roundings of ha_swiglu on a bf16 gate/up buffer; no residual.
+ * Both need M <= 8 and K <= 16384 (the row-streaming kernel).  With norm_weight == NULL and act == HA_ACT_NONE this is
+ * ha_linear_skinny.
+ */
+enum { HA_ACT_NONE = 0, HA_ACT_SWIGLU = 1 };
+int ha_linear_skinny_fused(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
+                           int64_t residual_stride_m, const void *norm_weight, float eps, int act, void *out,
+                           int64_t out_stride_m, int M, int N, int K, void *stream);
 
 #ifdef __cplusplus
 }

@@ -168,6 +168,12 @@ def test_arguments_are_validated_before_any_device_work(lib):
                                               for k in ("x", "xs", "w", "ws", "r", "rs", "o", "os", "M", "N", "K", "st")])
     assert lin(w=null) == HA_ERR_NULL and lin(M=17) == HA_ERR_SHAPE and lin(K=100) == HA_ERR_SHAPE and lin(ws=100) == HA_ERR_SHAPE
     assert lin(x=odd) == HA_ERR_ALIGN and lin(xs=4100) == HA_ERR_ALIGN and lin(r=p, rs=10) == HA_ERR_SHAPE
+    linf = lambda **kw: lib.ha_linear_skinny_fused(*[{**dict(x=p, xs=4096, w=p, ws=4096, r=null, rs=0, g=p, eps=C.c_float(1e-5), act=1, o=p, os=4096,
+                                                            M=4, N=4096, K=4096, st=null), **kw}[k]
+                                                     for k in ("x", "xs", "w", "ws", "r", "rs", "g", "eps", "act", "o", "os", "M", "N", "K", "st")])
+    assert linf(act=5) == HA_ERR_SHAPE and linf(N=4095) == HA_ERR_SHAPE and linf(r=p, rs=4096) == HA_ERR_SHAPE      # SwiGLU: even rows, no residual
+    assert linf(M=9) == HA_ERR_SHAPE and linf(K=32768, xs=32768, ws=32768) == HA_ERR_SHAPE and linf(g=odd) == HA_ERR_ALIGN
+    assert linf(os=1000) == HA_ERR_SHAPE and linf(eps=C.c_float(-1.0)) == HA_ERR_ALIGN
     assert lib.ha_swiglu(null, 64, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_NULL
     assert lib.ha_swiglu(p, 63, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_SHAPE and lib.ha_swiglu(p, 64, 9, 1, 32, p, null) == HA_ERR_DTYPE
 

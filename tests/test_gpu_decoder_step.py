@@ -161,3 +161,52 @@ def test_decoder_step_on_the_fused_attention_path_matches_the_two_launch_path():
     torch.cuda.synchronize()
     assert torch.isfinite(a).all()
     assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
+
+
+@pytest.mark.parametrize("M,N,K", [(4, 6144, 4096), (1, 512, 1024), (8, 1000, 4096), (3, 96, 8192), (4, 200, 16384), (5, 64, 64)])
+def test_linear_skinny_with_rmsnorm_in_front(M, N, K):
+    # against F.rms_norm followed by the fp32 product of the bf16-rounded normalised rows
+    print(f"\n[case] linear_skinny + RMSNorm {M}x{N}x{K}", flush=True)
+    from hashattention import _ops
+    g = torch.Generator(device=DEV).manual_seed(M + N + K)
+    x = (torch.randn(M, K, generator=g, device=DEV) * 3).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device=DEV) * K ** -0.5).to(torch.bfloat16)
+    gamma = (1 + 0.2 * torch.randn(K, generator=g, device=DEV)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g, device=DEV).to(torch.bfloat16)
+    h = torch.nn.functional.rms_norm(x, (K,), gamma, 1e-5)
+    want = h.float() @ w.float().t()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    _ops.linear_skinny(x, w, out, norm_weight=gamma, eps=1e-5)
+    assert (out.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+    _ops.linear_skinny(x, w, out, residual=res, norm_weight=gamma, eps=1e-5)
+    want2 = want + res.float()
+    assert (out.float() - want2).abs().max().item() <= 2e-2 * max(1.0, want2.abs().max().item())
+    # the normalised rows themselves: an identity weight returns them
+    if K <= 1024:
+        eye = torch.eye(K, dtype=torch.bfloat16, device=DEV)
+        hn = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_skinny(x, eye, hn, norm_weight=gamma, eps=1e-5)
+        assert (hn.float() - h.float()).abs().max().item() <= 2 ** -6 * max(1.0, h.float().abs().max().item())
+
+
+@pytest.mark.parametrize("M,F,K", [(4, 14336, 4096), (1, 100, 512), (8, 777, 4096), (2, 48, 8192), (4, 40, 64)])
+def test_linear_skinny_with_swiglu_behind(M, F, K):
+    # against the unfused pair: ha_linear_skinny into a bf16 gate/up buffer, then ha_swiglu - same roundings, same sums
+    print(f"\n[case] linear_skinny + SwiGLU {M}x{F}x{K}", flush=True)
+    from hashattention import _ops
+    g = torch.Generator(device=DEV).manual_seed(M + F + K)
+    x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * F, K, generator=g, device=DEV) * K ** -0.5).to(torch.bfloat16)
+    gamma = (1 + 0.2 * torch.randn(K, generator=g, device=DEV)).to(torch.bfloat16)
+    for norm in (None, gamma):
+        gu = torch.empty(M, 2 * F, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_skinny(x, w, gu, norm_weight=norm, eps=1e-5)
+        want = torch.empty(M, F, dtype=torch.bfloat16, device=DEV)
+        _ops.swiglu(gu, want)
+        out = torch.full((M, F + 8), 7.0, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_skinny(x, w, out[:, :F], norm_weight=norm, eps=1e-5, swiglu=True)
+        assert (out[:, F:] == 7.0).all()
+        # the two kernels group the rows of W differently, so a sum can differ in its last bf16 digit
+        ref = torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()
+        assert (out[:, :F].float() - ref).abs().max().item() <= 2e-2 * max(1.0, ref.abs().max().item())
+        assert (out[:, :F].float() - want.float()).abs().max().item() <= 2 ** -6 * max(1.0, want.float().abs().max().item())

@@ -87,7 +87,7 @@ class LlamaShapedDecoder:
         self.q_rot = torch.empty(B, self.H, self.d, dtype=self.dtype, device=self.device)
         self.ffn_act = torch.empty(B, self.ffn, dtype=self.dtype, device=self.device)
         self.qkv = torch.empty(B, (self.H + 2 * self.Hkv) * self.d, dtype=self.dtype, device=self.device)
-        self.x_attn = torch.empty(B, self.hidden, dtype=self.dtype, device=self.device)
+        self.x_attn = [torch.empty(B, self.hidden, dtype=self.dtype, device=self.device) for _ in range(2)]
         self.gate_up = torch.empty(B, 2 * self.ffn, dtype=self.dtype, device=self.device)
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
@@ -151,14 +151,15 @@ class LlamaShapedDecoder:
                 hl.n_cached = pos
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
             if skinny:
-                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn, residual=x)
+                # x lives in one of two buffers from here on (the down projection below adds in place)
+                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn[(l + 1) % 2], residual=x)
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             else:
-                x = torch.addmm(x, self.attn_out.view(B, H * d), p["wo"].t())
+                x = x.addmm_(self.attn_out.view(B, H * d), p["wo"].t())
                 h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
                 _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
-            x = torch.addmm(x, self.ffn_act, p["w2"].t())
+            x = x.addmm_(self.ffn_act, p["w2"].t())      # in place: the out-of-place form first copies x into its result
         if advance:
             self.seq_len = S
         x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)

@@ -3,10 +3,11 @@
 The reference measures end-to-end decode throughput with a gpt-fast fork (efficiency/generate.py:386-434,
 efficiency/model.py:98-345: RMSNorm, rotary embedding, SwiGLU feed-forward, static KV cache).  That fork is not
 runnable as shipped and drives Double-Sparsity labels, not hashes; this module is the same decoder shape with
-the HashAttention step in every layer.  Outside attention: RMSNorm, the down projection and the lm_head are library
-calls (`F.rms_norm`, hipBLASLt); the QKV, output and gate/up projections go through `ha_linear_skinny` when the batch
-is at most 8 rows of bf16; RoPE + cache append and SwiGLU are one launch each (`ha_rope_append`, `ha_swiglu`); the
-residual adds ride in the projections: the point is to time the whole step, and to check the plumbing around the op
+the HashAttention step in every layer.  Outside attention, for up to 8 sequences of bf16: the QKV projection with its
+RMSNorm folded in and the gate/up projection with its RMSNorm in front and SwiGLU behind (`ha_linear_skinny_fused`), the
+output projection with the residual folded in (`ha_linear_skinny`), RoPE + cache append in one launch (`ha_rope_append`);
+the down projection and the lm_head are library GEMMs (hipBLASLt), the final norm `F.rms_norm`.  Other dtypes and batches
+take library calls plus `ha_swiglu`.  The point is to time the whole step, and to check the plumbing around the op
 (rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
 
 Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no

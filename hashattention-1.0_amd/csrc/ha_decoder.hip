@@ -35,6 +35,14 @@ __device__ __forceinline__ float dot8(const uint4 &a, const uint4 &b, float c) {
     c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), c, false);
     return c;
 }
+// A guarded 128-bit load as a load under the execution mask.  Written as `ok ? *p : zero` with `zero` a variable, the
+// compiler selects between two addresses (global memory and the private copy of `zero`) and loads through a generic
+// pointer: flat loads, which also occupy the LDS path and its counter.
+__device__ __forceinline__ uint4 load16_or_zero(const void *p, bool ok) {
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (ok) v = *reinterpret_cast<const uint4 *>(p);
+    return v;
+}
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
@@ -67,7 +75,6 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
         }
     };
     const int kbase = wave * XCH * 512 + lane * 8;  // first element of this lane's 16 bytes in chunk 0 of its slice
-    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
 
     uint4 xr[XCH][MM];
 #pragma unroll
@@ -75,7 +82,7 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
 #pragma unroll
         for (int m = 0; m < MM; ++m) {
             const int k = kbase + c * 512;
-            xr[c][m] = (m < M && k < K) ? *reinterpret_cast<const uint4 *>(x + (int64_t)m * x_sm + k) : zero;
+            xr[c][m] = load16_or_zero(x + (int64_t)m * x_sm + k, m < M && k < K);
         }
 
     uint4 wc[R][XCH], wn[R][XCH];
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
             for (int c = 0; c < XCH; ++c) {
                 const int k = kbase + c * 512;
                 const int n = w_row(r0 + r);
-                wv[r][c] = (n >= 0 && k < K) ? *reinterpret_cast<const uint4 *>(w + (int64_t)n * w_sn + k) : zero;
+                wv[r][c] = load16_or_zero(w + (int64_t)n * w_sn + k, n >= 0 && k < K);
             }
     };
     if constexpr (kNorm) {
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
 #pragma unroll
         for (int c = 0; c < XCH; ++c) {
             const int k = kbase + c * 512;
-            gw[c] = k < K ? *reinterpret_cast<const uint4 *>(norm_w + k) : zero;
+            gw[c] = load16_or_zero(norm_w + k, k < K);
         }
         float ss[MM];
 #pragma unroll
@@ -230,15 +237,14 @@ __global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_
     const uint4 *wp = reinterpret_cast<const uint4 *>(w + (int64_t)n * w_sn) + g;
     const uint4 *xp = reinterpret_cast<const uint4 *>(x + (int64_t)min(r, M - 1) * x_sm) + g;
     const bool x_ok = r < M;
-    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     uint4 wc[PF], xc[PF], wn[PF], xn[PF];
     auto fetch = [&](int s0, uint4 (&wv)[PF], uint4 (&xv)[PF]) {
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
             const bool ok = s0 + i < s_end;
-            wv[i] = ok ? wp[(int64_t)(s0 + i) * 4] : zero;
-            xv[i] = (ok && x_ok) ? xp[(int64_t)(s0 + i) * 4] : zero;
+            wv[i] = load16_or_zero(wp + (int64_t)(s0 + i) * 4, ok);
+            xv[i] = load16_or_zero(xp + (int64_t)(s0 + i) * 4, ok && x_ok);
         }
     };
     if (s_beg < s_end) fetch(s_beg, wc, xc);
@@ -374,13 +380,14 @@ static int linear_skinny_impl(const void *x, int64_t x_stride_m, const void *w, 
     uint16_t *op = (uint16_t *)out;
     hipStream_t s = (hipStream_t)stream;
     if (M <= 8 && K <= 16384) {
-        // rows per workgroup, measured at M = 4.  Plain product: 8 rows for K <= 4096 (output projection 10.0 us against
-        // 11.1 with 16 rows), 16 for longer rows (down projection 28.8 us against 32.1 with 8), 64 for the vocabulary
-        // projection; counts that are not multiples of 8 were always slower.  With the norm in front every workgroup
-        // repeats the norm of x, so fewer, larger workgroups win (whole decoder step 6.5 ms against 7.0 ms with 8 rows).
+        // rows per workgroup, measured at M = 4.  Plain product: 8 rows for K <= 4096 (QKV 11.6 us against 14.2 with 16
+        // rows, output projection 9.6 against 10.3, gate/up 41.1 against 43.6), 16 for the vocabulary projection (174.8
+        // us against 178.3 with 8 and 182.1 with 64) and for longer rows (down projection 24.8 us against 26.0 with 8);
+        // counts that are not multiples of 8 were always slower.  With the norm in front every workgroup repeats the
+        // norm of x, so fewer, larger workgroups win (whole decoder step 6.3 ms against 6.8 ms with 8 rows everywhere).
         const int chunks = (K + 511) / 512;
         const int fuse = (norm_weight ? 1 : 0) | (act == HA_ACT_SWIGLU ? 2 : 0);
-        const int RB = (int64_t)N >= 64 * 1024 ? 64 : (fuse & 1) ? ((int64_t)N >= 32 * 512 ? 32 : 16) : chunks <= 8 ? 8 : 16;
+        const int RB = (fuse & 1) ? ((int64_t)N >= 64 * 1024 ? 64 : (int64_t)N >= 32 * 512 ? 32 : 16) : (chunks <= 8 && (int64_t)N < 64 * 1024) ? 8 : 16;
         const dim3 g2(act == HA_ACT_SWIGLU ? (N / 2 + RB / 2 - 1) / (RB / 2) : (N + RB - 1) / RB);
 #define HA_GEMV_F(NW_, XCH_, R_, MM_, F_)                                                                                     \
     hipLaunchKernelGGL((gemv_rows_kernel<NW_, XCH_, R_, MM_, F_>), g2, dim3(NW_ * 64), (size_t)RB * MM_ * NW_ * 4 * sizeof(float), s, \

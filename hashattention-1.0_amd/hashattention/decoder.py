@@ -3,11 +3,11 @@
 The reference measures end-to-end decode throughput with a gpt-fast fork (efficiency/generate.py:386-434,
 efficiency/model.py:98-345: RMSNorm, rotary embedding, SwiGLU feed-forward, static KV cache).  That fork is not
 runnable as shipped and drives Double-Sparsity labels, not hashes; this module is the same decoder shape with
-the HashAttention step in every layer.  Outside attention, for up to 8 sequences of bf16: the QKV projection with its
-RMSNorm folded in and the gate/up projection with its RMSNorm in front and SwiGLU behind (`ha_linear_skinny_fused`), the
-output projection with the residual folded in (`ha_linear_skinny`), RoPE + cache append in one launch (`ha_rope_append`);
-the down projection and the lm_head are library GEMMs (hipBLASLt), the final norm `F.rms_norm`.  Other dtypes and batches
-take library calls plus `ha_swiglu`.  The point is to time the whole step, and to check the plumbing around the op
+the HashAttention step in every layer.  Outside attention, for up to 8 sequences of bf16, every projection is the
+row-streaming kernel: QKV with its RMSNorm folded in, gate/up with its RMSNorm in front and SwiGLU behind, lm_head with
+the final norm in front (`ha_linear_skinny_fused`), output and down projection with the residual folded in
+(`ha_linear_skinny`); RoPE + cache append is one launch (`ha_rope_append`).  Other dtypes and batches take library calls
+(`F.rms_norm`, hipBLASLt) plus `ha_swiglu`.  The point is to time the whole step, and to check the plumbing around the op
 (rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
 
 Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no
@@ -32,7 +32,8 @@ class LlamaShapedDecoder:
         self.L, self.hidden, self.ffn, self.H, self.Hkv, self.d, self.vocab = n_layers, hidden, ffn, n_heads, n_kv_heads, head_dim, vocab
         self.theta, self.eps, self.dtype, self.device = rope_theta, rms_eps, dtype, torch.device(device)
         self.Hc = n_code_heads
-        self.use_skinny = True   # ha_linear_skinny for the projections it is faster for (bf16, batch <= 8)
+        self.use_skinny = True   # ha_linear_skinny for the projections (bf16, batch <= 8) ...
+        self.skinny_all = True   # ... including the down projection and the lm_head (False: library GEMMs for these two)
         self.usa_shape = (lth_num_layers, lth_int_dim, lth_final_dim)
         self.budgets = (init_budget, recent_budget, heavy_budget)
         g = torch.Generator(device=device).manual_seed(seed)
@@ -90,6 +91,7 @@ class LlamaShapedDecoder:
         self.qkv = torch.empty(B, (self.H + 2 * self.Hkv) * self.d, dtype=self.dtype, device=self.device)
         self.x_attn = [torch.empty(B, self.hidden, dtype=self.dtype, device=self.device) for _ in range(2)]
         self.gate_up = torch.empty(B, 2 * self.ffn, dtype=self.dtype, device=self.device)
+        self.logits = torch.empty(B, self.vocab, dtype=self.dtype, device=self.device)
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
@@ -136,8 +138,8 @@ class LlamaShapedDecoder:
         pos = self.seq_len
         S = pos + 1
         x = self.embed[tokens]                                            # [B, hidden]
-        # the row-streaming kernel measured faster than the library GEMM for the QKV, output and gate/up projections
-        # (2.6 -> 3.3, 1.8 -> 3.0, 4.0 -> 4.4 TB/s at B = 4) and slower for the down projection and the lm_head
+        # the row-streaming kernel against the library GEMM at B = 4: QKV 11.3 us (19.3), output projection 9.5 (19.1),
+        # gate/up 40.9 (59.8), down projection 24.7 (25.1), lm_head 174.8 (184.7)
         skinny = self.use_skinny and self.dtype == torch.bfloat16 and B <= 8
         for l, p in enumerate(self.layers):
             if skinny:      # RMSNorm rides in the projection that consumes it
@@ -153,16 +155,21 @@ class LlamaShapedDecoder:
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
             if skinny:
                 # x lives in one of two buffers from here on (the down projection below adds in place)
-                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn[(l + 1) % 2], residual=x)
+                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn[0 if self.skinny_all else (l + 1) % 2], residual=x)
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             else:
                 x = x.addmm_(self.attn_out.view(B, H * d), p["wo"].t())
                 h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
                 _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
-            x = x.addmm_(self.ffn_act, p["w2"].t())      # in place: the out-of-place form first copies x into its result
+            if skinny and self.skinny_all:
+                x = _ops.linear_skinny(self.ffn_act, p["w2"], self.x_attn[1], residual=x)
+            else:
+                x = x.addmm_(self.ffn_act, p["w2"].t())      # in place: the out-of-place form first copies x into its result
         if advance:
             self.seq_len = S
+        if skinny and self.skinny_all:
+            return _ops.linear_skinny(x, self.lm_head, self.logits, norm_weight=self.final_norm, eps=self.eps)
         x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)
         return F.linear(x, self.lm_head)
 

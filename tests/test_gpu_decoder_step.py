@@ -134,10 +134,13 @@ def test_bf16_decoder_step_with_and_without_the_skinny_projections():
     tokens = torch.tensor([5, 17], device=DEV)
     with torch.no_grad():
         a = dec.decode_step(tokens, advance=False).float()
+        dec.skinny_all = False                      # library GEMMs for the down projection and the lm_head
+        c = dec.decode_step(tokens, advance=False).float()
         dec.use_skinny = False
         b = dec.decode_step(tokens, advance=False).float()
     assert torch.isfinite(a).all()
     assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
+    assert (c - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
 
 
 def test_decoder_step_on_the_fused_attention_path_matches_the_two_launch_path():

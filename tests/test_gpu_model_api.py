@@ -123,8 +123,10 @@ def test_usa_forward_and_mask_api():
     span_ref, ksign_ref = orc.usa_forward_hard(K.cpu(), Q.cpu(), k_heads, q_heads)
     assert torch.equal(span.cpu(), span_ref) and torch.equal(ksign.cpu(), ksign_ref)
     assert torch.equal(usa.k_embedding(K, hard=True).cpu(), ksign_ref)
-    with pytest.raises(NotImplementedError):
-        usa(K, Q, hard=False)
+    with torch.no_grad():
+        soft, ktanh = usa(K, Q, hard=False)                   # soft mode: probabilities, zero beyond the causal edge
+    soft_ref, ktanh_ref = orc.usa_forward_soft(K.cpu(), Q.cpu(), k_heads, q_heads, cfg.lth_thold)
+    assert (soft.cpu() - soft_ref).abs().max().item() < 1e-5 and (ktanh.cpu() - ktanh_ref).abs().max().item() < 1e-5
 
     layer = hl.LlamaAttention_heavy_hitter(cfg, 0).to(DEV)
     layer.usa_module = usa

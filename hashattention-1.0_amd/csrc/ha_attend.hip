@@ -522,9 +522,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
         for (int u = 0; u < U; ++u) j_next[u] = list_index(base + STEP, u);
 #pragma unroll
-        for (int u = 0; u < U; ++u) kr[u] = EL::load8(kb + j0[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) kr[u] = EL::load8s(kb + j0[u] * row_bytes, sub);
 #pragma unroll
-        for (int u = 0; u < U; ++u) vr[u] = EL::load8(vb + j0[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) vr[u] = EL::load8s(vb + j0[u] * row_bytes, sub);
     };
     // consumes list entries [base, base + STEP); needs entries up to base + 3 STEP
     auto step = [&]() {
@@ -532,9 +532,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         Raw8<E> kn[U], vn[U];
         int32_t j_after[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) kn[u] = EL::load8(kb + j_next[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) kn[u] = EL::load8s(kb + j_next[u] * row_bytes, sub);
 #pragma unroll
-        for (int u = 0; u < U; ++u) vn[u] = EL::load8(vb + j_next[u] * row_bytes, sub);
+        for (int u = 0; u < U; ++u) vn[u] = EL::load8s(vb + j_next[u] * row_bytes, sub);
 #pragma unroll
         for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
 
@@ -758,10 +758,10 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
         for (int u = 0; u < kUnroll; ++u) {
             const int r = base + u * kStreams;
             ok[u] = r < r1;
-            kr[u] = EL::load8(kb + token(ok[u] ? r : base) * row_bytes, sub);
+            kr[u] = EL::load8s(kb + token(ok[u] ? r : base) * row_bytes, sub);
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8(vb + token(ok[u] ? base + u * kStreams : base) * row_bytes, sub);
+        for (int u = 0; u < kUnroll; ++u) vr[u] = EL::load8s(vb + token(ok[u] ? base + u * kStreams : base) * row_bytes, sub);
 
         float sc[G][kUnroll];
 #pragma unroll

@@ -43,6 +43,12 @@ __device__ __forceinline__ uint4 load16_or_zero(const void *p, bool ok) {
     if (ok) v = *reinterpret_cast<const uint4 *>(p);
     return v;
 }
+// the same for weights: read once per launch, so with the non-temporal hint (x and the norm weight stay in L2)
+__device__ __forceinline__ uint4 stream16_or_zero(const void *p, bool ok) {
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (ok) v = ha_load16_stream(reinterpret_cast<const uint4 *>(p));
+    return v;
+}
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
@@ -94,7 +100,7 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
             for (int c = 0; c < XCH; ++c) {
                 const int k = kbase + c * 512;
                 const int n = w_row(n0, r0 + r);
-                wv[r][c] = load16_or_zero(w + (int64_t)n * w_sn + k, n >= 0 && k < K);
+                wv[r][c] = stream16_or_zero(w + (int64_t)n * w_sn + k, n >= 0 && k < K);
             }
     };
     int blk = blockIdx.x;
@@ -254,7 +260,7 @@ __global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
             const bool ok = s0 + i < s_end;
-            wv[i] = load16_or_zero(wp + (int64_t)(s0 + i) * 4, ok);
+            wv[i] = stream16_or_zero(wp + (int64_t)(s0 + i) * 4, ok);
             xv[i] = load16_or_zero(xp + (int64_t)(s0 + i) * 4, ok && x_ok);
         }
     };

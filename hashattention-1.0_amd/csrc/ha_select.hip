@@ -33,6 +33,20 @@ __global__ __launch_bounds__(256) void hamming_score_kernel(const uint32_t *__re
     scores[((int64_t)b * H + h) * max_S + j] = (uint8_t)load_code<W>(kc, j).dist(q);
 }
 
+// Workgroups go to the 8 XCDs round-robin in launch order.  Walking a grid (chunk, code head, sequence) code head fastest
+// puts every chunk of a (sequence, code head) row on XCD = code head % 8 when the code heads come in multiples of 8:
+// with 8 code heads that is the XCD on which the attention launch places the query heads of the KV group, so the codes
+// a later pass or launch scans again are already in that L2 (whole step at B = 16, 64K tokens: 120.4 -> 118.9 us).
+__device__ __forceinline__ void walk_code_head_fastest(int &c, int &hc, int &b) {
+    c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
+    if (gridDim.y % 8 == 0) {
+        const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        hc = lin % (int)gridDim.y;
+        c = (lin / (int)gridDim.y) % (int)gridDim.x;
+        b = lin / (int)(gridDim.y * gridDim.x);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Pass 1.  grid (nchunk, Hc, B).  hist[b, h, chunk, level] = #candidates of the chunk at that distance.
 // The LDS histogram is replicated REP times (replica = lane % REP, which is also the bank) so that the
@@ -44,7 +58,8 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
                                                                   int blocks, int nchunk, int vec, uint32_t *__restrict__ hist) {
     constexpr int NL = 32 * W + 1;
     __shared__ uint32_t lh[GQ * NL * REP];
-    const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
+    int c, hc, b;
+    walk_code_head_fastest(c, hc, b);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;
@@ -200,7 +215,8 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
     constexpr int CPL = 4 * kMaxBlocks;  // codes per lane at most
     __shared__ uint32_t s_wtot[kSelWaves][GQ];
 
-    const int c = blockIdx.x, hc = blockIdx.y, b = blockIdx.z;
+    int c, hc, b;
+    walk_code_head_fastest(c, hc, b);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;

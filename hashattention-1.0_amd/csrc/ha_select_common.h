@@ -48,6 +48,8 @@ template <int W> __device__ __forceinline__ Code<W> load_code(const uint32_t *p,
 // indices inside [beg, end).  Codes outside [beg, end) are returned as zero and must be masked by the caller.
 template <int W>
 __device__ __forceinline__ void load_code4(const uint32_t *kc, int j0, int beg, int end, bool vec, Code<W> (&k)[4]) {
+    // plain loads on purpose: the codes are scanned again by a later pass or launch, and with the non-temporal hint the
+    // step measured 4 - 8 us slower
     if (vec) {
         if constexpr (W == 1) {
             const uint4 v = reinterpret_cast<const uint4 *>(kc)[j0 >> 2];

@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the gather-attend kernel, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
 # summarised in profiles/decode_step_config2_hbm_traffic.md, each scaled on a 1 GiB copy (fetch x2.0, write x1.0).
-MEASURED_ATTEND_TRAFFIC_BYTES = {("config2", True): 580.1e6, ("config2", False): 551.4e6}   # key: (workload, selection fused)
+MEASURED_ATTEND_TRAFFIC_BYTES = {("config2", True): 588.6e6, ("config2", False): 551.4e6}   # key: (workload, selection fused)
 
 
 def algorithmic_bytes(w, n_sel_rows):

@@ -239,6 +239,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="config2")
+    ap.add_argument("--batch", type=int, default=None, help="override the number of sequences of a uniform configuration (a variant, not the named workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
@@ -268,6 +269,10 @@ def main():
         return
     dev = "cuda:0"
     w = named_workload(args.config)
+    if args.batch is not None:
+        if len(set(w.seq_lens)) > 1:
+            sys.exit("--batch applies to configurations whose sequences have one length")
+        w.batch, w.seq_lens, w.name = args.batch, [w.seq_lens[0]] * args.batch, f"{w.name} with batch {args.batch}"
     p = make_problem_on_device(w, dev)
     B, H, Hkv, d, S = w.batch, w.n_q_heads, w.n_kv_heads, w.head_dim, w.max_seq_len
     ragged = len(set(w.seq_lens)) > 1

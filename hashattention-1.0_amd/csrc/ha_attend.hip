@@ -121,6 +121,10 @@ struct FusedSel {
 };
 constexpr int kFusedLocalChunks = 64;
 constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
+// a batch of equal lengths is cut into this many workgroups (one per CU): measured against 512 at 64K tokens, B = 6: 76.6
+// against 82.3 us, B = 8: 76.7 against 81.2, B = 12: 107.1 against 125.5; B = 1 at 32K: 39.2 against 40.9; B = 4 at 128K: 84.1
+// against 87.0 - the pieces are setup-bound, so fewer and larger ones win
+constexpr int kFusedUniformPieces = 256;
 constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
 
 // NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.
@@ -938,13 +942,13 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
                               max_seq_len, stream);
 }
 
-// chunks per workgroup of the fused path: whole rows when the rows alone fill the GPU, else enough splits for ~512 workgroups
-// Workgroups per row: enough for two 512-thread workgroups on each of the 256 CUs.  With lengths on the device the
-// kernel decides per row how many of them own chunks, so the grid offers up to four times as many (at most one per
-// kFusedResident / H rows, the count a single sequence would get).
+// Chunks per workgroup of the fused path.  A batch of equal lengths: whole rows when there are at least
+// kFusedUniformPieces rows, else that many workgroups in all.  With lengths on the device the kernel decides per row how
+// many workgroups own chunks (kFusedResident in all), so the grid offers up to four times the uniform count per row (at
+// most kFusedResident / H, the count a single sequence would get).
 static int fused_chunks_per_split(int B, int H, int nchunk, bool ragged) {
     const int64_t rows = (int64_t)B * H;
-    int64_t want = (kFusedResident + rows - 1) / rows;
+    int64_t want = ((ragged && B > 1 ? kFusedResident : kFusedUniformPieces) + rows - 1) / rows;
     if (ragged && B > 1 && B <= kFusedSortBatch && rows < kFusedResident) want = std::min<int64_t>(4 * want, (kFusedResident + H - 1) / H);
     if (want > nchunk) want = nchunk;
     if (want < 1) want = 1;

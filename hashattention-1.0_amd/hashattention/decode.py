@@ -83,7 +83,7 @@ class HashDecodeLayer:
         self.ws_select = _ops.workspace(_ops.select_workspace_bytes(B, self.H, self.Hc, self.W, S_cap), dev)
         self.ws_attend = _ops.workspace(_ops.sparse_decode_workspace_bytes(B, self.H, self.idx_cap), dev)
         # measured: with the thresholds derived in the attention launch the fused path is ahead from 32 rows on (a row
-        # is then cut into up to 16 pieces: 40.3 against 45.2 us at B = 1, 32K tokens; 84.1 against 86.5 us at B = 4, 128K)
+        # is then cut into up to 8 pieces: 39.2 against 45 us at B = 1, 32K tokens; 84.1 against 86.5 us at B = 4, 128K)
         self.fused_ok = B * self.H >= self.fused_min_rows and _ops.fused_applies(B, self.H, self.Hc, self.W, S_cap, self.init_budget,
                                                                  self.recent_budget, self.heavy_budget, self.mode)
         # rows of up to 64 chunks: the attention launch derives the thresholds itself, the step is three launches

@@ -395,6 +395,10 @@ def main():
         "dense_hbm_gbps": ab["dense"] / (ms_dense * 1e-3) / 1e9,
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
+        # the scoring stream (XOR + popcount over every cached code, histogrammed on the fly) as its own launch
+        **({"score_roofline": {"kernel": "select_hist_kernel", "bound": "hbm", "achieved": ab["score"] / (ms_prepare * 1e-3) / 1e9,
+                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["score"] / (ms_prepare * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                               "algorithmic_bytes": ab["score"], "us": ms_prepare * 1e3}} if fused and layer.local_thresholds else {}),
         "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm",
                      "achieved": attend_bytes / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": attend_bytes / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,

@@ -176,3 +176,32 @@ def test_fused_path_equals_two_launch_path_on_unsplit_rows(dtype):
     out_c = torch.empty_like(out_b)
     _ops.sparse_decode_fused(q3, k, v, kc, qc, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws, sm, out_c, wf)
     assert torch.equal(out_b, out_c)
+
+
+def _random_workload(rng, i):
+    H, Hkv = [(8, 2), (4, 4), (8, 8), (16, 2), (32, 8), (4, 1)][rng.integers(6)]
+    Hc = [Hkv, H][rng.integers(2)]
+    B = int(rng.integers(1, 10))
+    top = int(rng.choice([40, 700, 3000, 9000, 20000]))
+    if rng.integers(2):
+        lens = [int(rng.integers(max(1, top // 8), top + 1)) for _ in range(B)]
+    else:
+        lens = [int(rng.integers(max(1, top // 2), top + 1))] * B
+    wide = bool(rng.integers(2))
+    heavy = float(rng.choice([0.0, 1.0 / 32, 0.125, 0.5, 1.0, 37.0, 300.0]))
+    return small_workload(name=f"random{i}", batch=B, seq_lens=lens, n_q_heads=H, n_kv_heads=Hkv, n_code_heads=Hc,
+                          lth_num_layers=2 if wide else 3, lth_final_dim=64 if wide else 32,
+                          init_budget=int(rng.choice([0, 4, 16, 128])), recent_budget=int(rng.choice([0, 1, 16, 128])),
+                          heavy_budget=heavy, dtype=[torch.bfloat16, torch.float16, torch.float32][rng.integers(3)], seed=100 + i)
+
+
+@pytest.mark.parametrize("block", range(8))
+def test_random_shapes_every_stage_against_the_oracle(block):
+    # seeded sweep over batch sizes, head layouts, ragged and equal lengths, code widths, budgets and dtypes: every
+    # stage of every case against the oracle, the fused launch with its in-kernel plan included
+    rng = np.random.default_rng(2024 + block)
+    for i in range(8):
+        w = _random_workload(rng, block * 8 + i)
+        print(f"\n[case] {w.name}: B={w.batch} H={w.n_q_heads}/{w.n_kv_heads}/{w.n_code_heads} S={w.seq_lens} bits={w.lth_final_dim} "
+              f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget} {w.dtype}", flush=True)
+        run_decode_case(w, check_encode=False, check_dense=False)

@@ -141,7 +141,8 @@ def run_decode_case(w: Workload, check_encode: bool = True, mode: str = "simple"
         err3 = float(np.abs(out3.float().cpu().numpy() - ref).max())
         assert err3 <= ATOL[w.dtype], f"fused select+attend max-abs error {err3} > {ATOL[w.dtype]}"
         same = float((out3.float() - out.float()).abs().max().item())
-        assert same <= (2e-6 if w.dtype == torch.float32 else 1e-2), f"fused vs two-launch output differ by {same}"
+        # the two paths add the same rows in different orders: accumulation-order noise in fp32, one rounding of the output in bf16/fp16
+        assert same <= (1e-5 if w.dtype == torch.float32 else 1e-2), f"fused vs two-launch output differ by {same}"
         report.update(fused_err=err3, fused_vs_unfused=same)
         if len(set(w.seq_lens)) == 1:      # equal lengths given on the host (no length array): the same pieces, the same output
             out5 = torch.empty_like(out)

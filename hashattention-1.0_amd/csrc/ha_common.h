@@ -146,4 +146,16 @@ __device__ __forceinline__ float ha_load_elem(const void *p, int64_t i, int dtyp
     return __half2float(reinterpret_cast<const __half *>(p)[i]);
 }
 
+// single element store from float, and the value such a store leaves behind
+__device__ __forceinline__ void ha_store_elem(void *p, int64_t i, float x, int dtype) {
+    if (dtype == HA_F32) reinterpret_cast<float *>(p)[i] = x;
+    else if (dtype == HA_BF16) reinterpret_cast<uint16_t *>(p)[i] = (uint16_t)ha_f32_to_bf16_bits(x);
+    else reinterpret_cast<__half *>(p)[i] = __float2half(x);
+}
+__device__ __forceinline__ float ha_round_to(float x, int dtype) {
+    if (dtype == HA_F32) return x;
+    if (dtype == HA_BF16) return ha_round_bf16(x);
+    return __half2float(__float2half(x));
+}
+
 #endif  // __HIPCC__

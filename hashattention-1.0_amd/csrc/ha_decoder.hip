@@ -291,17 +291,6 @@ __global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_
     }
 }
 
-__device__ __forceinline__ void store_elem(void *p, int64_t i, float x, int dtype) {
-    if (dtype == HA_F32) reinterpret_cast<float *>(p)[i] = x;
-    else if (dtype == HA_BF16) reinterpret_cast<uint16_t *>(p)[i] = (uint16_t)ha_f32_to_bf16_bits(x);
-    else reinterpret_cast<__half *>(p)[i] = __float2half(x);
-}
-__device__ __forceinline__ float round_to(float x, int dtype) {
-    if (dtype == HA_F32) return x;
-    if (dtype == HA_BF16) return ha_round_bf16(x);
-    return __half2float(__float2half(x));
-}
-
 // grid (H + 2 Hkv, B), 64 threads: thread i owns the pair (i, i + 64) of one head vector.
 __global__ __launch_bounds__(64) void rope_append_kernel(const void *__restrict__ qkv, int64_t qkv_sb, int dtype, int H, int Hkv, int pos,
                                                          const int32_t *__restrict__ pos_dev, const float *__restrict__ inv_freq,
@@ -313,22 +302,22 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const void *__restrict_
     const float x0 = ha_load_elem(qkv, src + i, dtype), x1 = ha_load_elem(qkv, src + i + 64, dtype);
     if (head >= H + Hkv) {  // value: copied as it is
         const int64_t dst = b * kv_sb + (int64_t)(head - H - Hkv) * kv_sh + (int64_t)p * kv_ss;
-        store_elem(v_cache, dst + i, x0, dtype);
-        store_elem(v_cache, dst + i + 64, x1, dtype);
+        ha_store_elem(v_cache, dst + i, x0, dtype);
+        ha_store_elem(v_cache, dst + i + 64, x1, dtype);
         return;
     }
     // the angle in fp32, the table rounded to the model dtype: as transformers' rotary embedding builds it
     const float ang = (float)p * inv_freq[i];
-    const float c = round_to(cosf(ang), dtype), s = round_to(sinf(ang), dtype);
+    const float c = ha_round_to(cosf(ang), dtype), s = ha_round_to(sinf(ang), dtype);
     const float y0 = x0 * c - x1 * s, y1 = x1 * c + x0 * s;
     if (head < H) {
         const int64_t dst = ((int64_t)b * H + head) * HA_HEAD_DIM;
-        store_elem(q_out, dst + i, y0, dtype);
-        store_elem(q_out, dst + i + 64, y1, dtype);
+        ha_store_elem(q_out, dst + i, y0, dtype);
+        ha_store_elem(q_out, dst + i + 64, y1, dtype);
     } else {
         const int64_t dst = b * kv_sb + (int64_t)(head - H) * kv_sh + (int64_t)p * kv_ss;
-        store_elem(k_cache, dst + i, y0, dtype);
-        store_elem(k_cache, dst + i + 64, y1, dtype);
+        ha_store_elem(k_cache, dst + i, y0, dtype);
+        ha_store_elem(k_cache, dst + i + 64, y1, dtype);
     }
 }
 
@@ -337,7 +326,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const void *__restrict__ ga
     const int b = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
     if (i >= F) return;
     const float g = ha_load_elem(gate_up, b * gu_sb + i, dtype), u = ha_load_elem(gate_up, b * gu_sb + F + i, dtype);
-    store_elem(out, (int64_t)b * F + i, round_to(g / (1.0f + __expf(-g)), dtype) * u, dtype);
+    ha_store_elem(out, (int64_t)b * F + i, ha_round_to(g / (1.0f + __expf(-g)), dtype) * u, dtype);
 }
 
 }  // namespace

@@ -37,10 +37,24 @@ struct EncSide {
 };
 // Up to two sides share one launch (the new keys and the queries of a decode step): blockIdx.y runs over
 // the heads of side 0, then those of side 1.
+// Optional front end of a decode step (T = 1, 128-wide heads): side 0 / side 1 read the raw key / query rows of a fused
+// QKV projection, rotate them (rotate-half RoPE at the sequence's position), write the rotated key and the value row
+// into the caches and the rotated query to q_out, and hash what they wrote.
+struct EncRope {
+    const float *inv_freq;  // [64]; nullptr: no front end, the sides read finished rows
+    const void *v_src;      // raw value rows [B, Hkv, 128], batch stride v_sb
+    int64_t v_sb;
+    void *q_out;            // [B, H, 128]
+    void *k_cache, *v_cache;
+    int64_t kv_sb, kv_sh, kv_ss;
+    int pos;
+    const int32_t *pos_dev;
+};
 struct EncArgs {
     EncSide side[2];
     int B, T, n_layers, d_in, d_int, d_out, arith;
     int64_t per_head;
+    EncRope rope;
 };
 
 // NL_/DIN_/DINT_/DOUT_ fix the MLP shape at compile time (0 = read it from the arguments).  The usual
@@ -103,16 +117,45 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
     // needs only them and its own weights, not the whole weight prefetch
     constexpr int kXIter = (kRows * kMaxDim + kEncThreads - 1) / kEncThreads;
     float xs[kXIter];
+    const EncRope &rp = a.rope;
+    float xpair[kXIter];  // rope: the other element of the rotation pair
 #pragma unroll
     for (int it = 0; it < kXIter; ++it) {
         const int i = tid + it * kEncThreads;
         xs[it] = 0.f;
+        xpair[it] = 0.f;
         if (i < kRows * d_in) {
             const int r = i / d_in, e = i % d_in;
             const int row = row0 + r;
             if (row < n_rows) {
                 const int b = row / T, t = row % T;
                 xs[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
+                if (rp.inv_freq) xpair[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + (e ^ 64), x_dtype);
+            }
+        }
+    }
+    if (rp.inv_freq) {
+        // rotate-half RoPE of the row this thread element belongs to (T = 1, d_in = 128): the angle in fp32, the table
+        // rounded to the element type as transformers builds it, the result rounded as the cache stores it.  The first
+        // code head of a KV head writes the key and copies the value row; every query head writes its query.
+        const bool writes_kv = !second && head % (n_heads / sd.x_heads) == 0;
+#pragma unroll
+        for (int it = 0; it < kXIter; ++it) {
+            const int i = tid + it * kEncThreads;
+            if (i >= kRows * d_in) continue;
+            const int r = i / d_in, e = i % d_in, b = row0 + r;
+            if (b >= n_rows) continue;
+            const int p = rp.pos_dev ? rp.pos_dev[b] : rp.pos;
+            const float ang = (float)p * rp.inv_freq[e & 63];
+            const float c = ha_round_to(cosf(ang), x_dtype), sn = ha_round_to(sinf(ang), x_dtype);
+            const float y = ha_round_to(e < 64 ? xs[it] * c - xpair[it] * sn : xs[it] * c + xpair[it] * sn, x_dtype);
+            xs[it] = y;
+            if (second) {
+                ha_store_elem(rp.q_out, ((int64_t)b * n_heads + head) * HA_HEAD_DIM + e, y, x_dtype);
+            } else if (writes_kv) {
+                const int64_t dst = b * rp.kv_sb + (int64_t)in_head * rp.kv_sh + (int64_t)p * rp.kv_ss + e;
+                ha_store_elem(rp.k_cache, dst, y, x_dtype);
+                ha_store_elem(rp.v_cache, dst, ha_load_elem(rp.v_src, b * rp.v_sb + (int64_t)in_head * HA_HEAD_DIM + e, x_dtype), x_dtype);
             }
         }
     }
@@ -315,6 +358,42 @@ int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, in
                         0, nullptr, nullptr};
     a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);
+    return launch_encode(a, dim3(tiles, Hc + H), (hipStream_t)stream);
+}
+
+int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                        const int32_t *pos_dev, const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
+                        int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, const float *weights_k,
+                        const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim, int arith, uint32_t *kcodes,
+                        int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream) {
+    HA_REQUIRE(qkv && inv_freq && q_out && k_cache && v_cache, HA_ERR_NULL_POINTER, "qkv/inv_freq/q_out/k_cache/v_cache is NULL");
+    HA_REQUIRE(H > 0 && Hkv > 0 && Hc > 0, HA_ERR_BAD_SHAPE, "H, Hkv, Hc must be positive");
+    int st = validate_encode(qkv, B, Hkv, Hc, 1, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b, kc_stride_h,
+                             pos_dev ? 0 : pos);
+    if (st) return st;
+    HA_REQUIRE(weights_q && qcodes, HA_ERR_NULL_POINTER, "weights_q/qcodes is NULL");
+    HA_REQUIRE(head_dim == HA_HEAD_DIM, HA_ERR_BAD_SHAPE, "the rotary front end needs 128-wide heads");
+    HA_REQUIRE(H + Hc <= 65535, HA_ERR_BAD_SHAPE, "H + Hc <= 65535");
+    HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
+    HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
+    HA_REQUIRE(qkv_stride_b >= (int64_t)(H + 2 * Hkv) * HA_HEAD_DIM, HA_ERR_BAD_SHAPE, "qkv row stride shorter than (H + 2 Hkv) * 128");
+    HA_REQUIRE(cache_len > 0 && (pos_dev || (pos >= 0 && pos < cache_len)), HA_ERR_BAD_SHAPE, "position %d outside the cache of %lld tokens",
+               pos, (long long)cache_len);
+    HA_REQUIRE(kv_stride_s >= HA_HEAD_DIM && kv_stride_h > 0 && kv_stride_b > 0, HA_ERR_BAD_SHAPE, "cache strides smaller than a row");
+    if ((st = ha_require_device())) return st;
+    const int W = final_dim / 32;
+    const int64_t eb = x_dtype == HA_F32 ? 4 : 2;
+    EncArgs a = {};
+    // raw rows of the fused projection: queries at column 0, keys behind the H query heads, values behind the keys
+    a.side[0] = EncSide{(const char *)qkv + (int64_t)H * HA_HEAD_DIM * eb, x_dtype, qkv_stride_b, (int64_t)HA_HEAD_DIM, (int64_t)HA_HEAD_DIM, Hkv, Hc,
+                        weights_k, kcodes, kc_stride_b, kc_stride_h, pos, pos_dev, nullptr};
+    a.side[1] = EncSide{qkv, x_dtype, qkv_stride_b, (int64_t)HA_HEAD_DIM, (int64_t)HA_HEAD_DIM, H, H, weights_q, qcodes, (int64_t)H * W,
+                        (int64_t)W, 0, nullptr, nullptr};
+    a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
+    a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    a.rope = EncRope{inv_freq, (const char *)qkv + (int64_t)(H + Hkv) * HA_HEAD_DIM * eb, qkv_stride_b, q_out, k_cache, v_cache, kv_stride_b,
+                     kv_stride_h, kv_stride_s, pos, pos_dev};
     const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);
     return launch_encode(a, dim3(tiles, Hc + H), (hipStream_t)stream);
 }

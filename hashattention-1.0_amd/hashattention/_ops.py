@@ -69,6 +69,9 @@ def load_library() -> C.CDLL:
                               vp, i64, vp, vp, sz, vp]
     lib.ha_rope_append.restype = i32
     lib.ha_rope_append.argtypes = [vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]
+    lib.ha_rope_encode_step.restype = i32
+    lib.ha_rope_encode_step.argtypes = [vp, i64, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp, vp,
+                                        i32, i32, i32, i32, i32, vp, i64, i64, vp, vp]
     lib.ha_linear_skinny.restype = i32
     lib.ha_linear_skinny.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
     lib.ha_linear_skinny_fused.restype = i32
@@ -384,6 +387,28 @@ def rope_append(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, pos: int, in
     _check(load_library().ha_rope_append(_ptr(qkv), qkv.stride(0), _DTYPE[qkv.dtype], B, n_q_heads, n_kv_heads, int(pos), _ptr(pos_dev),
                                          _ptr(inv_freq), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
                                          k_cache.stride(1), k_cache.stride(2), k_cache.shape[2], _stream(qkv)), "ha_rope_append")
+
+
+def rope_encode_step(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, pos: int, inv_freq: torch.Tensor, q_out: torch.Tensor,
+                     k_cache: torch.Tensor, v_cache: torch.Tensor, wk: torch.Tensor, wq: torch.Tensor, n_layers: int, int_dim: int,
+                     final_dim: int, kcodes: torch.Tensor, qcodes: torch.Tensor, pos_dev: Optional[torch.Tensor] = None,
+                     arith: int = HA_ARITH_F32) -> None:
+    """`rope_append` and `encode_step` of a decode step in one launch: the rows of qkv [B, (H + 2 Hkv) * 128] are rotated,
+    written to q_out / the caches at position pos (or pos_dev[b]), and what was written is hashed into kcodes (at the same
+    position) and qcodes."""
+    _require_cuda(qkv, inv_freq, q_out, k_cache, v_cache, wk, wq, kcodes, qcodes, pos_dev)
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and q_out.is_contiguous() and q_out.dtype == qkv.dtype == k_cache.dtype == v_cache.dtype
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == 64 and inv_freq.is_contiguous()
+    assert k_cache.stride() == v_cache.stride() and k_cache.stride(3) == 1
+    assert kcodes.stride(3) == 1 and kcodes.stride(2) == kcodes.shape[3] and qcodes.is_contiguous()
+    B = qkv.shape[0]
+    assert kcodes.dtype == torch.int32 and qcodes.dtype == torch.int32 and qcodes.numel() == B * n_q_heads * (final_dim // 32)
+    assert pos_dev is not None or int(pos) < kcodes.shape[2]
+    _check(load_library().ha_rope_encode_step(
+        _ptr(qkv), qkv.stride(0), _DTYPE[qkv.dtype], B, n_q_heads, n_kv_heads, wk.shape[0], int(pos), _ptr(pos_dev), _ptr(inv_freq),
+        _ptr(q_out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), k_cache.shape[2],
+        _ptr(wk), _ptr(wq), n_layers, 128, int_dim, final_dim, arith, _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes),
+        _stream(qkv)), "ha_rope_encode_step")
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:

@@ -165,6 +165,9 @@ class HashDecodeLayer:
             newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
             _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
                              self.qcodes, pos_dev=pos, arith=self.arith)
+        return self._select_attend(q3, k_cache, v_cache, seq_len, out, seq_lens, main)
+
+    def _select_attend(self, q3, k_cache, v_cache, seq_len, out, seq_lens, main=None):
         if self.use_fused and self.fused_ok and not self.overlap_windows:
             self.select_prepare(seq_len, seq_lens)
             self.attend_fused(q3, k_cache, v_cache, out, seq_len, seq_lens)
@@ -177,3 +180,17 @@ class HashDecodeLayer:
         else:
             self.attend(q3, k_cache, v_cache, out)
         return out
+
+    def step_from_qkv(self, qkv: torch.Tensor, pos: int, inv_freq: torch.Tensor, q_rot: torch.Tensor, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """The decode step of a uniform batch straight from the fused QKV projection of the new token, qkv [B, (H + 2 Hkv) * 128]:
+        rotary embedding at position `pos`, cache append, hashing of the new key and of the query in ONE launch
+        (ha_rope_encode_step), then selection and attention as in `step`.  q_rot [B, H, 128] receives the rotated query."""
+        if self.overlap_windows:
+            raise RuntimeError("step_from_qkv does not run the second-stream window partial: use rope_append + step")
+        if self.n_cached != pos:
+            raise RuntimeError(f"bit-cache holds {self.n_cached} tokens, the new token sits at position {pos}")
+        _ops.rope_encode_step(qkv, self.H, self.Hkv, pos, inv_freq, q_rot, k_cache, v_cache, self.wk, self.wq, self.num_layers,
+                              self.int_dim, self.final_dim, self.codes, self.qcodes, arith=self.arith)
+        self.n_cached = pos + 1
+        return self._select_attend(q_rot, k_cache, v_cache, pos + 1, out, None)

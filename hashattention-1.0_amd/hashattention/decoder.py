@@ -34,6 +34,7 @@ class LlamaShapedDecoder:
         self.Hc = n_code_heads
         self.use_skinny = True   # ha_linear_skinny for the projections (bf16, batch <= 8) ...
         self.skinny_all = True   # ... including the down projection and the lm_head (False: library GEMMs for these two)
+        self.fuse_rope = True    # ha_rope_encode_step instead of ha_rope_append + ha_encode_step
         self.usa_shape = (lth_num_layers, lth_int_dim, lth_final_dim)
         self.budgets = (init_budget, recent_budget, heavy_budget)
         g = torch.Generator(device=device).manual_seed(seed)
@@ -146,11 +147,15 @@ class LlamaShapedDecoder:
                 qkv = _ops.linear_skinny(x, p["wqkv"], self.qkv, norm_weight=p["attn_norm"], eps=self.eps)
             else:
                 qkv = F.linear(F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps), p["wqkv"])
-            _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
             hl = self.hash[l]
             if dense:
+                _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
                 _ops.dense_decode(self.q_rot, self.k_cache[l], self.v_cache[l], S, None, hl.sm_scale, self.attn_out, self.ws_dense)
+            elif self.fuse_rope and d == 128:
+                hl.n_cached = pos       # rotary embedding, cache append and both hashes in one launch
+                hl.step_from_qkv(qkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l], self.attn_out)
             else:
+                _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
                 hl.n_cached = pos
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
             if skinny:

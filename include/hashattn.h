@@ -263,6 +263,18 @@ int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int 
                    int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, void *stream);
 int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, int F, void *out, void *stream);
 /*
+ * ha_rope_append followed by ha_encode_step, in one launch: the workgroup that hashes a head also rotates it.  qkv as for
+ * ha_rope_append; the rotated query goes to q_out, the rotated key and the value into the caches at position pos (or
+ * pos_dev[b]); the key written is hashed by the Hc key-side MLPs into kcodes at the same position, the query written
+ * by the H query-side MLPs into qcodes [B, H, W] (hashattention_llama.py:567-579 rotary + cache update, :204-226 and
+ * :411-414 the embeddings of the new key and the query).  Bit for bit what the two launches produce.  128-wide heads.
+ */
+int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                        const int32_t *pos_dev, const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
+                        int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len,
+                        const float *weights_k, const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim,
+                        int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream);
+/*
  * out[m, n] = sum_k x[m, k] * w[n, k] (+ residual[m, n]): a Linear layer (weight [N, K] as nn.Linear keeps it) applied to
  * M <= 16 rows, bf16 in and out, fp32 accumulation.  The decode step's projections (efficiency/model.py:236, 261,
  * 304-305: wqkv, wo, w1/w3, w2, and the lm_head of :158) are this shape: they stream every weight once per token, so

@@ -134,6 +134,9 @@ def test_bf16_decoder_step_with_and_without_the_skinny_projections():
     tokens = torch.tensor([5, 17], device=DEV)
     with torch.no_grad():
         a = dec.decode_step(tokens, advance=False).float()
+        dec.fuse_rope = False                       # ha_rope_append + ha_encode_step instead of the one launch: the same bits
+        assert torch.equal(dec.decode_step(tokens, advance=False).float(), a)
+        dec.fuse_rope = True
         dec.skinny_all = False                      # library GEMMs for the down projection and the lm_head
         c = dec.decode_step(tokens, advance=False).float()
         dec.use_skinny = False
@@ -213,3 +216,40 @@ def test_linear_skinny_with_swiglu_behind(M, F, K):
         ref = torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()
         assert (out[:, :F].float() - ref).abs().max().item() <= 2e-2 * max(1.0, ref.abs().max().item())
         assert (out[:, :F].float() - want.float()).abs().max().item() <= 2 ** -6 * max(1.0, want.float().abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("code_heads", ["kv", "q"])
+def test_rope_encode_step_equals_rope_append_then_encode_step(dtype, code_heads):
+    # one launch against the two it replaces: rotated query, both caches and both code buffers bit for bit
+    print(f"\n[case] rope_encode_step {dtype} code heads per {code_heads} head", flush=True)
+    from hashattention import _ops
+    from hashattention.synthetic import layer_dims
+    g = torch.Generator(device=DEV).manual_seed(11)
+    gc = torch.Generator().manual_seed(12)
+    B, H, Hkv, d, cap = 5, 8, 2, 128, 50
+    Hc = Hkv if code_heads == "kv" else H
+    heads = lambda n: [[(torch.randn(fo, fi, generator=gc) * fi ** -0.5, torch.randn(fo, generator=gc) * 0.01)
+                        for fi, fo in layer_dims(d, 128, 32, 3)] for _ in range(n)]
+    wk, wq = _ops.pack_usa_weights(heads(Hc), DEV), _ops.pack_usa_weights(heads(H), DEV)
+    qkv = torch.randn(B, (H + 2 * Hkv) * d + 32, generator=g, device=DEV).to(dtype)[:, :(H + 2 * Hkv) * d]
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    for pos, pos_dev in ((17, None), (0, torch.tensor([3, 49, 0, 21, 8], dtype=torch.int32, device=DEV))):
+        outs = []
+        for fused in (False, True):
+            k_cache = torch.zeros(B, Hkv, cap, d, dtype=dtype, device=DEV)
+            v_cache = torch.zeros_like(k_cache)
+            q_out = torch.zeros(B, H, d, dtype=dtype, device=DEV)
+            kcodes = torch.zeros(B, Hc, cap, 1, dtype=torch.int32, device=DEV)
+            qcodes = torch.zeros(B, H, 1, dtype=torch.int32, device=DEV)
+            if fused:
+                _ops.rope_encode_step(qkv, H, Hkv, pos, inv_freq, q_out, k_cache, v_cache, wk, wq, 3, 128, 32, kcodes, qcodes, pos_dev)
+            else:
+                _ops.rope_append(qkv, H, Hkv, pos, inv_freq, q_out, k_cache, v_cache, pos_dev)
+                p = pos_dev.long() if pos_dev is not None else torch.full((B,), pos, device=DEV)
+                k_new = torch.gather(k_cache, 2, p.view(B, 1, 1, 1).expand(B, Hkv, 1, d))
+                _ops.encode_step(k_new, q_out, wk, wq, 3, 128, 32, kcodes, qcodes, pos0=pos, pos_dev=pos_dev)
+            outs.append((q_out, k_cache, v_cache, kcodes, qcodes))
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
+        assert outs[1][3].ne(0).any() and outs[1][1].ne(0).any()

@@ -164,6 +164,21 @@ def test_arguments_are_validated_before_any_device_work(lib):
 
     assert rope(f=null) == HA_ERR_NULL and rope(dt=7) == HA_ERR_DTYPE
     assert rope(sb=512) == HA_ERR_SHAPE and rope(pos=100) == HA_ERR_SHAPE and rope(pos=-1) == HA_ERR_SHAPE and rope(kss=64) == HA_ERR_SHAPE
+    import ctypes as _C
+    lib.ha_rope_encode_step.restype = _C.c_int
+    i64 = _C.c_int64
+
+    def rope_enc(**kw):
+        a = dict(qkv=p, sb=i64(48 * 128), dt=_ops.HA_BF16, B=1, H=32, Hkv=8, Hc=8, pos=3, pd=null, f=p, q=p, k=p, v=p, ksb=i64(8 * 100 * 128),
+                 ksh=i64(100 * 128), kss=i64(128), cl=i64(100), wk=p, wq=p, nl=3, hd=128, idim=128, fd=32, ar=0, kc=p, csb=i64(800), csh=i64(100),
+                 qc=p, st=null)
+        a.update(kw)
+        return lib.ha_rope_encode_step(*[a[k] for k in ("qkv", "sb", "dt", "B", "H", "Hkv", "Hc", "pos", "pd", "f", "q", "k", "v", "ksb", "ksh",
+                                                        "kss", "cl", "wk", "wq", "nl", "hd", "idim", "fd", "ar", "kc", "csb", "csh", "qc", "st")])
+
+    assert rope_enc(f=null) == HA_ERR_NULL and rope_enc(qc=null) == HA_ERR_NULL and rope_enc(dt=7) == HA_ERR_DTYPE
+    assert rope_enc(hd=64) == HA_ERR_SHAPE and rope_enc(pos=100) == HA_ERR_SHAPE and rope_enc(sb=i64(512)) == HA_ERR_SHAPE
+    assert rope_enc(fd=48) == HA_ERR_SHAPE and rope_enc(Hc=3) == HA_ERR_SHAPE
     lin = lambda **kw: lib.ha_linear_skinny(*[{**dict(x=p, xs=4096, w=p, ws=4096, r=null, rs=0, o=p, os=4096, M=4, N=4096, K=4096, st=null), **kw}[k]
                                               for k in ("x", "xs", "w", "ws", "r", "rs", "o", "os", "M", "N", "K", "st")])
     assert lin(w=null) == HA_ERR_NULL and lin(M=17) == HA_ERR_SHAPE and lin(K=100) == HA_ERR_SHAPE and lin(ws=100) == HA_ERR_SHAPE

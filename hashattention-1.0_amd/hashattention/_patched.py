@@ -10,9 +10,10 @@ What differs from the reference on purpose
   * ties at the top-k boundary go to the lowest token index (the reference's `sort` at :430 is unstable);
   * softmax and the value product are fp32 throughout (the reference rounds probabilities to the query
     dtype at :613);
-  * the LSH baseline (`lth_num_layers == 0`, :130-139) is not built, and `CENTER` normalisation (:163-167) exists
-    only in soft mode: the bit-cache keeps codes of keys hashed once, which a statistic over all cached keys would
-    invalidate at every step;
+  * the LSH baseline (`lth_num_layers == 0`, :75-84, :130-139) and `CENTER` normalisation (:163-167) hash inputs that
+    depend on a statistic over ALL cached keys (their largest norm; their mean and deviation), so a key's code changes
+    as the cache grows: in these two modes the bit-cache is rebuilt at every step, as the reference re-hashes every
+    step, and only selection and attention keep their speed;
   * the training side - soft mode (`hard=False`: tanh / sigmoid, :174-176, 197-198), `train_step` (:304-316) and the train
     branch of `usa_local_compute` (:356-371) - is differentiable torch code batched over heads (one baddbmm per MLP layer
     instead of a Python loop over heads); the recall statistic (:372-398) runs on the selection kernel.
@@ -58,6 +59,31 @@ def ste_sign(x: torch.Tensor) -> torch.Tensor:
     return SignSTE.apply(x)
 
 
+LSH_PAD = 3     # zero coordinates after the lifted one: the encode kernels take input widths that are multiples of 4
+
+
+def lift_to_sphere(x: torch.Tensor, pad: int = 0) -> torch.Tensor:
+    """[b, heads, s, d] -> [b, heads, s, d + 1 + pad]: the coordinate sqrt(M^2 - |x|^2) that gives every vector of a head
+    the same length M = (largest norm in that head) + 1e-3, so that sign random projections rank by inner product;
+    `pad` zeros follow.  Arithmetic as the reference's `IpToCS` (:75-84) per head: the norm in the input's dtype, M^2 in
+    double rounded to fp32, the difference rounded to the input's dtype before relu and sqrt."""
+    norm = torch.linalg.vector_norm(x, dim=-1, keepdim=True)
+    big = norm.amax(dim=(0, 2), keepdim=True).double() + 1e-3
+    gap = ((big * big).float() - norm.square().float()).to(x.dtype)
+    parts = [x, torch.sqrt(torch.relu(gap))]
+    if pad:
+        parts.append(x.new_zeros(*x.shape[:-1], pad))
+    return torch.cat(parts, dim=-1)
+
+
+class IpToCS(nn.Module):
+    """First stage of an LSH-baseline head (reference :75-84): x [..., s, d] of ONE head -> [..., s, d + 1]."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        flat = x.reshape(1, 1, -1, x.shape[-1])
+        return lift_to_sphere(flat).reshape(*x.shape[:-1], x.shape[-1] + 1)
+
+
 class USA(nn.Module):
     """Per-head learned hash: `num_heads` independent MLPs for keys and for queries.
 
@@ -74,8 +100,8 @@ class USA(nn.Module):
         self.lth_final_dim = usa_params["lth_final_dim"]
         self.lth_thold = usa_params["lth_thold"]
         self.num_layers = usa_params.get("lth_num_layers", 3)   # the Mistral variant has no such key (mistral:566-570)
-        if self.num_layers not in (1, 2, 3):
-            raise NotImplementedError("lth_num_layers must be 1, 2 or 3 (the LSH baseline, 0, is not part of this build)")
+        if self.num_layers not in (0, 1, 2, 3):
+            raise NotImplementedError("lth_num_layers must be 0 (LSH baseline), 1, 2 or 3")
         if self.lth_final_dim not in (32, 64):
             raise NotImplementedError("lth_final_dim must be 32 or 64: codes are packed in one or two 32-bit words")
         self.center = bool(os.environ.get("CENTER", 0))      # as the reference reads it (:34, :98): any non-empty value is on
@@ -88,6 +114,17 @@ class USA(nn.Module):
                 return nn.Sequential(nn.Linear(head_dim, self.int_dim), nn.SiLU(), nn.Linear(self.int_dim, self.lth_final_dim))
             return nn.Sequential(nn.Linear(head_dim, self.lth_final_dim))
 
+        if self.num_layers == 0:
+            # LSH baseline (:130-139): one random projection of the lifted vector per head, shared by keys and queries
+            # (the same modules under three names, so a state dict holds each tensor under all three prefixes)
+            print("Implementing LSH for baseline")
+            self.learning_to_hash_transformation = nn.ModuleList(
+                [nn.Sequential(IpToCS(), nn.Linear(head_dim + 1, self.lth_final_dim)) for _ in range(num_heads)])
+            for seq in self.learning_to_hash_transformation:
+                nn.init.normal_(seq[1].weight)
+            self.learning_to_hash_transformation_k = self.learning_to_hash_transformation
+            self.learning_to_hash_transformation_q = self.learning_to_hash_transformation
+            return
         self.learning_to_hash_transformation_k = nn.ModuleList([mlp() for _ in range(num_heads)])
         self.learning_to_hash_transformation_q = nn.ModuleList([mlp() for _ in range(num_heads)])
 
@@ -95,6 +132,38 @@ class USA(nn.Module):
     def layers(self, side: str) -> List[List[Tuple[torch.Tensor, torch.Tensor]]]:
         mods = self.learning_to_hash_transformation_k if side == "k" else self.learning_to_hash_transformation_q
         return [[(m.weight, m.bias) for m in seq if isinstance(m, nn.Linear)] for seq in mods]
+
+    @property
+    def kernel_num_layers(self) -> int:
+        """Linear layers per head as the encode kernels count them (the LSH baseline is one layer on the lifted input)."""
+        return max(1, self.num_layers)
+
+    def kernel_layers(self, side: str) -> List[List[Tuple[torch.Tensor, torch.Tensor]]]:
+        """`layers(side)` in the shape the kernels take: the LSH projection gets zero columns for the padding
+        coordinates of `hash_inputs`."""
+        heads = self.layers(side)
+        if self.num_layers != 0:
+            return heads
+        return [[(torch.nn.functional.pad(w, (0, LSH_PAD)), b) for (w, b) in h] for h in heads]
+
+    @property
+    def rehash_every_step(self) -> bool:
+        """True when a key's code depends on the other cached keys (LSH lift, CENTER statistics): no code can be kept."""
+        return self.center or self.num_layers == 0
+
+    def hash_inputs(self, K: torch.Tensor, Q: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        """What the encode kernels are fed in hard mode for keys K [b, Hx, S, d] (Hx = KV heads or query heads) and
+        queries Q [b, H, t, d]: unchanged for the learned hashes; with CENTER, both standardised per head with the mean
+        and deviation of that head's keys over batch and positions (:163-167); for the LSH baseline, both lifted
+        (`lift_to_sphere`, each with its own largest norm) and zero-padded to a width the kernels take."""
+        if self.center:
+            rep = Q.shape[1] // K.shape[1]
+            mean, std = K.mean(dim=(0, 2), keepdim=True), K.std(dim=(0, 2), keepdim=True)
+            K = (K - mean) / (std + 1e-6)
+            Q = (Q - mean.repeat_interleave(rep, dim=1)) / (std.repeat_interleave(rep, dim=1) + 1e-6)
+        if self.num_layers == 0:
+            K, Q = lift_to_sphere(K, LSH_PAD), lift_to_sphere(Q, LSH_PAD)
+        return K, Q
 
     @property
     def dtype(self) -> torch.dtype:
@@ -108,14 +177,16 @@ class USA(nn.Module):
     def _stacked(self, side: str) -> List[Tuple[torch.Tensor, torch.Tensor]]:
         """Per layer (W [heads, out, in], b [heads, out]) stacked from the per-head modules; gradients reach the modules."""
         heads = self.layers(side)
-        return [(torch.stack([h[l][0] for h in heads]), torch.stack([h[l][1] for h in heads])) for l in range(self.num_layers)]
+        return [(torch.stack([h[l][0] for h in heads]), torch.stack([h[l][1] for h in heads])) for l in range(len(heads[0]))]
 
     def _soft_logits(self, vectors: torch.Tensor, side: str) -> torch.Tensor:
         """[b, heads, s, d] -> MLP outputs [b, heads, s, D], all heads in one baddbmm per layer (differentiable)."""
         b, a, s, d = vectors.shape
         if a != self.num_heads:
             raise ValueError(f"expected {self.num_heads} heads, got {a}")
-        x = vectors.transpose(0, 1).reshape(a, b * s, d)
+        if self.num_layers == 0:
+            vectors = lift_to_sphere(vectors)
+        x = vectors.transpose(0, 1).reshape(a, b * s, -1)
         stacked = self._stacked(side)
         for l, (w, bias) in enumerate(stacked):
             x = torch.baddbmm(bias.unsqueeze(1), x, w.transpose(1, 2))
@@ -123,17 +194,19 @@ class USA(nn.Module):
                 x = torch.nn.functional.silu(x)
         return x.view(a, b, s, -1).transpose(0, 1)
 
-    def _embed(self, vectors: torch.Tensor, side: str, hard: bool):
+    def _embed(self, vectors: torch.Tensor, side: str, hard: bool, prepared: bool = False):
+        """hard: (signs of the logits, packed codes) from the encode kernel; soft: (tanh of the logits, None).
+        `prepared`: the vectors already went through `hash_inputs`."""
         if not hard:
             return torch.tanh(self._soft_logits(vectors.to(self.dtype), side)), None
-        if self.center:
-            raise NotImplementedError("CENTER normalisation is available in soft mode only: the bit-cache hashes every key once")
+        if self.num_layers == 0 and not prepared:
+            vectors = lift_to_sphere(vectors, LSH_PAD)
         b, a, s, d = vectors.shape
         if a != self.num_heads:
             raise ValueError(f"expected {self.num_heads} heads, got {a}")
-        w = _ops.pack_usa_weights(self.layers(side), vectors.device)
+        w = _ops.pack_usa_weights(self.kernel_layers(side), vectors.device)
         codes = torch.empty(b, a, s, self.lth_final_dim // 32, dtype=torch.int32, device=vectors.device)
-        logits = _ops.encode_pack(vectors, w, self.num_layers, self.int_dim, self.lth_final_dim, codes,
+        logits = _ops.encode_pack(vectors, w, self.kernel_num_layers, self.int_dim, self.lth_final_dim, codes,
                                   arith=self.arith, want_logits=True)
         return torch.sign(logits), codes
 
@@ -161,8 +234,9 @@ class USA(nn.Module):
             span = torch.matmul(qt, kt.transpose(2, 3))
             span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
             return torch.sigmoid(span - self.lth_thold), kt
-        ksign, kcodes = self._embed(K, "k", hard)
-        _, qcodes = self._embed(Q, "q", hard)
+        Kh, Qh = self.hash_inputs(K, Q)
+        ksign, kcodes = self._embed(Kh.contiguous(), "k", True, prepared=True)
+        _, qcodes = self._embed(Qh.contiguous(), "q", True, prepared=True)
         D = self.lth_final_dim
         span = torch.empty(b, a, t, s, dtype=K.dtype, device=K.device)
         for i in range(t):
@@ -245,8 +319,8 @@ class HeavyHitterMixin:
         hl = self._hash_layer
         if hl is None:
             usa = self.usa_module
-            hl = HashDecodeLayer(usa.layers("k"), usa.layers("q"), self.num_heads, self.num_key_value_heads, self.head_dim,
-                                 usa.num_layers, usa.int_dim, usa.lth_final_dim, self.init_budget, self.recent_budget,
+            hl = HashDecodeLayer(usa.kernel_layers("k"), usa.kernel_layers("q"), self.num_heads, self.num_key_value_heads,
+                                 self.head_dim, usa.kernel_num_layers, usa.int_dim, usa.lth_final_dim, self.init_budget, self.recent_budget,
                                  self.heavy_budget, self.usa_eval_mode, self.usa_retrieve_depth, usa.arith, device)
             self._hash_layer = hl
         if hl.B != batch or hl.S_cap < seq_len:
@@ -258,17 +332,28 @@ class HeavyHitterMixin:
                 hl.n_cached = n
         return hl
 
+    def _hash_inputs(self, key_states, query_states):
+        """The tensors the encode kernels read for these keys [b, Hkv, S, d] and queries [b, H, q, d]: the states
+        themselves for a learned hash; their standardised / lifted form (`USA.hash_inputs`, computed in the hash
+        module's dtype as the reference casts, :406) when codes depend on the whole cache."""
+        usa = self.usa_module
+        if usa is None or not usa.rehash_every_step:
+            return key_states, query_states
+        kh, qh = usa.hash_inputs(key_states.to(usa.dtype), query_states.to(usa.dtype))
+        return kh.contiguous(), qh.contiguous()
+
     def _sparse_attention(self, query_states, key_states, value_states):
         """query [b, H, q, d] (q <= 128), key/value [b, Hkv, S, d] holding the whole cache including the new tokens.
         Returns [b, H, q, d].  Row i attends as query at absolute position S - q + i (reference :423-428)."""
         b, H, q_len, d = query_states.shape
         S = key_states.shape[2]
         hl = self._ensure_hash_layer(b, S, query_states.device)
-        if hl.n_cached > S - q_len:          # the cache was rewound (new prompt without reset_usa): start over
-            hl.reset()
+        key_hash, query_hash = self._hash_inputs(key_states, query_states)
+        if hl.n_cached > S - q_len or self.usa_module.rehash_every_step:
+            hl.reset()                       # the cache was rewound (new prompt without reset_usa), or no code can be kept
         if hl.n_cached < S - q_len:          # keys cached by a prefill (or by dense steps): encode them in bulk
             lo = hl.n_cached
-            bulk = key_states[:, :, lo:S - q_len]
+            bulk = key_hash[:, :, lo:S - q_len]
             hl.encode_keys(bulk, pos0=lo, use_mfma=(hl.arith == _ops.HA_ARITH_BF16 and bulk.dtype == torch.bfloat16
                                                     and hl.wk_bf16 is not None))
             hl.n_cached = S - q_len
@@ -280,14 +365,15 @@ class HeavyHitterMixin:
             saved = hl.heavy_budget
             hl.heavy_budget = heavy_abs
             try:
-                hl.step(query_states, key_states, value_states, S, out[:, :, 0])
+                hl.step(query_states, key_states, value_states, S, out[:, :, 0],
+                        hash_inputs=None if key_hash is key_states else (key_hash, query_hash))
             finally:
                 hl.heavy_budget = saved
             return out
         # a chunk of q_len rows: the new keys join the bit-cache, then every row is one "sequence" of the kernels - same
         # codes and K/V (batch stride 0), its own query code and its own length S - q_len + i + 1 (reference :423-428)
         dev = query_states.device
-        hl.encode_keys(key_states[:, :, S - q_len:S], pos0=S - q_len)
+        hl.encode_keys(key_hash[:, :, S - q_len:S], pos0=S - q_len)
         hl.n_cached = S
         lens = torch.arange(S - q_len + 1, S + 1, dtype=torch.int32, device=dev)
         cap = S if hl.mode != _ops.HA_SELECT_SIMPLE else min(S, hl.init_budget + hl.recent_budget + heavy)
@@ -298,7 +384,7 @@ class HeavyHitterMixin:
         ws_a = _ops.workspace(_ops.sparse_decode_workspace_bytes(q_len, H, cap), dev)
         o_b = torch.empty(q_len, H, d, dtype=query_states.dtype, device=dev)
         for bi in range(b):
-            _ops.encode_pack(query_states[bi:bi + 1], hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
+            _ops.encode_pack(query_hash[bi:bi + 1], hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
             _ops.select(hl.codes[bi:bi + 1].expand(q_len, -1, -1, -1), qc[0].transpose(0, 1).contiguous(), S, lens, hl.init_budget,
                         hl.recent_budget, heavy_abs, idx, cnt, ws_s, hl.mode, hl.depth)
             _ops.sparse_decode(query_states[bi].transpose(0, 1).contiguous(), key_states[bi:bi + 1].expand(q_len, -1, -1, -1),
@@ -344,6 +430,7 @@ class HeavyHitterMixin:
         S = key_states.shape[2]
         kv = key_states[:, ::self.num_key_value_groups].contiguous() if key_states.shape[1] == H else key_states
         hl = self._ensure_hash_layer(b, S, query_states.device)
+        kv, query_hash = self._hash_inputs(kv, query_states)
         hl.reset()
         hl.encode_keys(kv, pos0=0)
         hl.n_cached = S
@@ -356,7 +443,7 @@ class HeavyHitterMixin:
             ar = torch.arange(hl.idx_cap, device=mask.device)
             for i in range(q_len):
                 s_i = S - q_len + i + 1
-                hl.encode_query(query_states[:, :, i:i + 1].contiguous())
+                hl.encode_query(query_hash[:, :, i:i + 1].contiguous())
                 hl.select(s_i, None)
                 valid = ar[None, None, :] < hl.counts[:, :, None]
                 where = torch.where(valid, hl.idx.long(), torch.full_like(hl.idx, S, dtype=torch.long))
@@ -434,10 +521,11 @@ class HeavyHitterMixin:
 
         # ---- hash side: codes of all keys and of every query row, one selection per row
         hl = self._ensure_hash_layer(bsz, S, dev)
+        key_hash, query_hash = self._hash_inputs(keys, q)
         kc = torch.zeros(bsz, hl.Hc, S, hl.W, dtype=torch.int32, device=dev)
-        _ops.encode_pack(keys, hl.wk, hl.num_layers, hl.int_dim, hl.final_dim, kc, 0, None, hl.arith)
+        _ops.encode_pack(key_hash, hl.wk, hl.num_layers, hl.int_dim, hl.final_dim, kc, 0, None, hl.arith)
         qc = torch.zeros(bsz, H, q_len, hl.W, dtype=torch.int32, device=dev)
-        _ops.encode_pack(q, hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
+        _ops.encode_pack(query_hash, hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
         n_pred = S // 16
         if n_pred < 2:                                  # a heavy budget <= 1 would be read as a fraction
             return

@@ -18,7 +18,7 @@ All buffers are allocated once per (batch, capacity) and reused: the step itself
 from __future__ import annotations
 
 import math
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -53,7 +53,7 @@ class HashDecodeLayer:
         self.wk = _ops.pack_usa_weights(k_layers, self.device)
         self.wq = _ops.pack_usa_weights(q_layers, self.device)
         self.wk_bf16 = None
-        if head_dim == 128 and int_dim == 128:
+        if head_dim == 128 and int_dim == 128 and k_layers[0][0][0].shape[1] == 128:
             self.wk_bf16 = _ops.pack_usa_weights_bf16(k_layers, self.device)
         self.sm_scale = 1.0 / math.sqrt(head_dim)
         self.B = self.S_cap = 0
@@ -135,14 +135,20 @@ class HashDecodeLayer:
 
     # ------------------------------------------------------------------ one decode step
     def step(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, seq_len: int, out: torch.Tensor,
-             seq_lens: Optional[torch.Tensor] = None, n_new: int = 1) -> torch.Tensor:
+             seq_lens: Optional[torch.Tensor] = None, n_new: int = 1,
+             hash_inputs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
         """q [B, H, 1, d]; k_cache/v_cache [B, Hkv, >=seq_len, d] already holding the new token(s) at the end.
 
         Uniform batches: the last `n_new` tokens (positions seq_len - n_new ..) are encoded and appended to the
         bit-cache; everything before must already be there (`encode_keys` at prefill).  Ragged batches pass
         `seq_lens` (int32 [B], lengths including the new token) and `seq_len` = their maximum.
+        `hash_inputs` = (keys [B, Hkv, >=seq_len, d'], queries [B, H, 1, d']): what the hash MLPs read when that is not the
+        cache and the query themselves (standardised or lifted vectors; uniform batches only).
         """
         q3 = q[:, :, 0, :]
+        k_hash, q_hash3 = (k_cache, q3) if hash_inputs is None else (hash_inputs[0], hash_inputs[1][:, :, 0, :])
+        if hash_inputs is not None and seq_lens is not None:
+            raise ValueError("hash_inputs are supported for uniform batches only")
         main = torch.cuda.current_stream(self.device)
         if self.overlap_windows:
             # fork: the sink and recent windows need no selection, so their share of the attention runs on a second
@@ -155,8 +161,8 @@ class HashDecodeLayer:
             if self.n_cached + n_new != seq_len:
                 raise RuntimeError(f"bit-cache holds {self.n_cached} tokens, step at length {seq_len} appends {n_new}")
             if n_new > 1:       # a short multi-token append: older tokens first, the newest rides with the query
-                self.encode_keys(k_cache[:, :, seq_len - n_new:seq_len - 1], pos0=seq_len - n_new)
-            _ops.encode_step(k_cache[:, :, seq_len - 1:seq_len], q3, self.wk, self.wq, self.num_layers, self.int_dim,
+                self.encode_keys(k_hash[:, :, seq_len - n_new:seq_len - 1], pos0=seq_len - n_new)
+            _ops.encode_step(k_hash[:, :, seq_len - 1:seq_len], q_hash3, self.wk, self.wq, self.num_layers, self.int_dim,
                              self.final_dim, self.codes, self.qcodes, pos0=seq_len - 1, arith=self.arith)
             self.n_cached = seq_len
         else:

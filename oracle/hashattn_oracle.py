@@ -8,6 +8,8 @@ CPU-baseline leg may.  Every function names the lines of the reference
 Stages
   usa_mlp / usa_logits      hash MLP of one head / all heads       hashattention/hashattention_llama.py:99-128, 159-169
   usa_forward_hard          ternary sign, span = <sign q, sign k>  hashattention_llama.py:151-200, 51-55
+  standardise_by_keys       CENTER: (x - mean_k) / (std_k + 1e-6) per head      hashattention_llama.py:163-167
+  lift_one_head             LSH baseline: extra coordinate sqrt(M^2 - |x|^2)     hashattention_llama.py:75-84, 130-139
   pack_codes                bit i = logit_i > 0, LSB = dim 0       efficiency/kernels/torchatt.py:55-56, 159, 183-184
   hamming                   popcount(q ^ k)                        efficiency/kernels/bit_count_uint32.py:4-12, torchatt.py:58-62
   compute_mask_multi        sink | recent | top-k heavy mask       hashattention_llama.py:401-446
@@ -68,12 +70,47 @@ def usa_logits(x: torch.Tensor, heads: Sequence[Sequence[Tuple[torch.Tensor, tor
     return torch.stack(outs, dim=1)
 
 
-def usa_forward_hard(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads) -> Tuple[torch.Tensor, torch.Tensor]:
+def standardise_by_keys(K: torch.Tensor, Q: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """CENTER switch of `USA.forward` (hashattention_llama.py:163-167): inside the loop over heads, the keys of head i
+    (all batch entries, all positions) give a mean and an unbiased deviation per feature; keys AND queries of that head
+    are shifted and scaled with them, `1e-6` added to the deviation.  K, Q [b, H, s|t, d] with equal head counts."""
+    Ko, Qo = torch.empty_like(K), torch.empty_like(Q)
+    for i in range(K.shape[1]):
+        k = K[:, i]
+        flat = k.reshape(-1, k.shape[-1])
+        mu, sd = flat.mean(dim=0), flat.std(dim=0)
+        Ko[:, i] = (k - mu) / (sd + 1e-6)
+        Qo[:, i] = (Q[:, i] - mu) / (sd + 1e-6)
+    return Ko, Qo
+
+
+def lift_one_head(x: torch.Tensor) -> torch.Tensor:
+    """`IpToCS` (hashattention_llama.py:75-84), the first stage of every head of the LSH baseline (:130-139): with
+    M = (largest norm among ALL vectors handed in) + 1e-3, append sqrt(max(M^2 - |x|^2, 0)), so that every lifted vector
+    has norm M and the angle between lifted vectors orders them by inner product.  M is a Python float (double), as
+    `.item()` makes it in the reference."""
+    lengths = torch.linalg.vector_norm(x, dim=-1, keepdim=True)
+    M = float(lengths.max()) + 1e-3
+    return torch.cat([x, torch.sqrt(torch.clamp_min(M ** 2 - lengths ** 2, 0))], dim=-1)
+
+
+def lift_heads(X: torch.Tensor) -> torch.Tensor:
+    """The lift applied head by head, as the per-head `Sequential(IpToCS(), Linear)` sees its slice X[:, i]."""
+    return torch.stack([lift_one_head(X[:, i]) for i in range(X.shape[1])], dim=1)
+
+
+def usa_forward_hard(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads, center: bool = False,
+                     lsh: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """`USA.forward(K, Q, hard=True)`: span[b,h,t,s] = sum_i sign(q)_i sign(k)_i, non-causal -> finfo.min.
 
     reference: hashattention_llama.py:151-200.  K, Q are [b, H, s|t, d] (K already repeat_kv'd).
     torch.sign maps 0 to 0 (:55), so an exactly-zero logit contributes nothing to the span.
+    `center`: the CENTER switch (:163-167); `lsh`: heads are `[(W [D, d + 1], b)]` applied to lifted vectors (:130-139).
     """
+    if center:
+        K, Q = standardise_by_keys(K, Q)
+    if lsh:
+        K, Q = lift_heads(K), lift_heads(Q)
     kl = usa_logits(K, k_heads)
     ql = usa_logits(Q, q_heads)
     ks, qs = torch.sign(kl), torch.sign(ql)
@@ -280,22 +317,30 @@ def dense_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor) -> torch.
 
 
 def reference_decode_attention(Q, K, V, k_heads, q_heads, init_budget, recent_budget, heavy_budget,
-                               mode="simple", retrieve_depth=0.0, stable=True, usa_dtype=None):
+                               mode="simple", retrieve_depth=0.0, stable=True, usa_dtype=None, center=False, lsh=False):
     """The reference's emulated decode step between RoPE/cache update and o_proj.
 
     reference: hashattention_llama.py:578-623 with compute_mask_multi :401-446: repeat K/V over the
     group, dense QK^T, re-hash every key, full sort, masked fp32 softmax, AV.
     Q [b,H,q,d]; K,V [b,Hkv,S,d].  Returns (attn_output [b,H,q,d], keep mask [b,H,q,S]).
+    `center` / `lsh` (one K head per query head): the hash reads standardised / lifted vectors, as `usa_forward_hard`.
     """
     H, Hkv = Q.shape[1], K.shape[1]
     Kr, Vr = repeat_kv(K, H // Hkv), repeat_kv(V, H // Hkv)
     ud = usa_dtype or Q.dtype
     # the K MLP list has either one entry per query head or one per KV head
     Kin = Kr if len(k_heads) == H else K
-    kl = usa_logits(Kin.to(ud), k_heads)
+    Kin, Qin = Kin.to(ud), Q.to(ud)
+    if center or lsh:
+        assert len(k_heads) == H
+        if center:
+            Kin, Qin = standardise_by_keys(Kin, Qin)
+        if lsh:
+            Kin, Qin = lift_heads(Kin), lift_heads(Qin)
+    kl = usa_logits(Kin, k_heads)
     if kl.shape[1] != H:
         kl = repeat_kv(kl, H // kl.shape[1])
-    ql = usa_logits(Q.to(ud), q_heads)
+    ql = usa_logits(Qin, q_heads)
     span = torch.einsum("bhtd,bhsd->bhts", torch.sign(ql), torch.sign(kl))
     t, s = Q.shape[-2], K.shape[-2]
     causal = torch.tril(torch.ones(t, s), diagonal=s - t).bool()
@@ -342,13 +387,18 @@ def recall_overlap(q: torch.Tensor, k: torch.Tensor, k_heads, q_heads, init_budg
 
 # --------------------------------------------------------------------------- training side
 
-def usa_forward_soft(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads, thold: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor]:
+def usa_forward_soft(K: torch.Tensor, Q: torch.Tensor, k_heads, q_heads, thold: float = 0.0, center: bool = False,
+                     lsh: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """`USA.forward(K, Q, hard=False)`: tanh of both embeddings, span = <tanh q, tanh k>, non-causal entries set to
     finfo.min, then sigmoid(span - thold) (so non-causal entries come out as exactly 0).  Returns (scores, tanh K).
 
     reference: hashattention_llama.py:151-200 (:174-176 tanh, :184-185 baddbmm, :190-194 causal fill, :196-197 sigmoid).
-    Differentiable: built from torch ops on whatever tensors the head lists hold.
+    Differentiable: built from torch ops on whatever tensors the head lists hold.  `center`, `lsh` as in `usa_forward_hard`.
     """
+    if center:
+        K, Q = standardise_by_keys(K, Q)
+    if lsh:
+        K, Q = lift_heads(K), lift_heads(Q)
     kt = torch.tanh(usa_logits(K, k_heads))
     qt = torch.tanh(usa_logits(Q, q_heads))
     span = torch.einsum("bhtd,bhsd->bhts", qt, kt)

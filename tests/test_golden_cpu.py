@@ -182,3 +182,108 @@ def test_training_side_of_the_oracle_matches_vectors_recorded_from_the_reference
     assert np.array_equal(np.packbits(cand.numpy(), axis=-1), g["lc_mask"])
     assert np.array_equal(np.packbits(tgt.numpy().astype(bool), axis=-1), g["lc_target"])
     assert int(tgt.sum()) == 32 * q.shape[1] * q.shape[2] and not tgt[..., ~cand[-1]].bool()[..., -1, :].any() and S2 == 1024
+
+
+def _center_heads(g):
+    keys = [str(k) for k in g["center_keys"]]
+    sd = {k: torch.from_numpy(g[f"center_w{i}"]) for i, k in enumerate(keys)}
+    return {side: [[(sd[f"learning_to_hash_transformation_{side}.{h}.{l}.weight"], sd[f"learning_to_hash_transformation_{side}.{h}.{l}.bias"])
+                    for l in (0, 2, 4)] for h in range(3)] for side in ("k", "q")}
+
+
+def _lsh_heads(g):
+    return [[(torch.from_numpy(g[f"lsh_w{2 * h}"]), torch.from_numpy(g[f"lsh_w{2 * h + 1}"]))] for h in range(3)]
+
+
+def _span_mismatches(mine, want):
+    """Entries of two hard spans that differ: a logit within round-off of zero may change one sign, i.e. 2 in the span."""
+    diff = (mine - want).abs()
+    assert diff.max().item() <= 2.0
+    return int((diff > 0).sum())
+
+
+def test_center_and_lsh_variants_of_the_oracle_match_vectors_recorded_from_the_reference():
+    """The CENTER switch and the LSH baseline, hard and soft mode, as recorded from the reference's own code by
+    tests/golden/make_reference_lsh_center_vectors.py (two batch entries: pins that the statistics run over batch and
+    positions of one head)."""
+    g = np.load(os.path.join(HERE, "reference_lsh_center_vectors.npz"))
+    K, Q = torch.from_numpy(g["K"]), torch.from_numpy(g["Q"])
+    ch = _center_heads(g)
+    span, ks = orc.usa_forward_hard(K, Q, ch["k"], ch["q"], center=True)
+    want = torch.from_numpy(g["center_hard_span"])
+    assert _span_mismatches(span, want) == 0
+    assert torch.equal(ks.to(torch.int8), torch.from_numpy(g["center_hard_k"]))
+    # the switch matters on these inputs, and leaving it out reproduces the recorded plain spans
+    plain, _ = orc.usa_forward_hard(K, Q, ch["k"], ch["q"])
+    assert _span_mismatches(plain, torch.from_numpy(g["plain_hard_span"])) == 0
+    assert (plain != span).float().mean().item() > 0.5
+    soft, kt = orc.usa_forward_soft(K, Q, ch["k"], ch["q"], 0.0, center=True)
+    assert (soft - torch.from_numpy(g["center_soft_span"])).abs().max().item() < 1e-5
+    assert (kt - torch.from_numpy(g["center_soft_k"])).abs().max().item() < 1e-5
+    # a plausible mistake - statistics per batch entry instead of over the batch - does not reproduce the vectors
+    wrong = torch.cat([orc.usa_forward_hard(K[i:i + 1], Q[i:i + 1], ch["k"], ch["q"], center=True)[0] for i in range(2)])
+    assert (wrong != want).any()
+
+    # ---- LSH baseline: state-dict layout (three prefixes over the same tensors), lift, shared projection
+    keys = [str(k) for k in g["lsh_keys"]]
+    assert keys[:2] == ["learning_to_hash_transformation.0.1.weight", "learning_to_hash_transformation.0.1.bias"]
+    assert len(keys) == 18 and keys[6].startswith("learning_to_hash_transformation_k.") and keys[12].startswith("learning_to_hash_transformation_q.")
+    lh = _lsh_heads(g)
+    assert lh[0][0][0].shape == (32, 129)
+    span, ks = orc.usa_forward_hard(K, Q, lh, lh, lsh=True)
+    want = torch.from_numpy(g["lsh_hard_span"])
+    assert _span_mismatches(span, want) == 0
+    assert torch.equal(ks.to(torch.int8), torch.from_numpy(g["lsh_hard_k"]))
+    assert torch.equal(torch.from_numpy(g["lsh_k_embedding_hard"]), torch.from_numpy(g["lsh_hard_k"]))
+    soft, kt = orc.usa_forward_soft(K, Q, lh, lh, 0.0, lsh=True)
+    assert (soft - torch.from_numpy(g["lsh_soft_span"])).abs().max().item() < 1e-5
+    assert (kt - torch.from_numpy(g["lsh_soft_k"])).abs().max().item() < 1e-4
+    # the lift by its definition: every lifted vector of a head has the same norm, the head's largest norm + 1e-3
+    lifted = orc.lift_heads(K)
+    top = K.norm(dim=-1).amax(dim=(0, 2)) + 1e-3
+    assert (lifted.norm(dim=-1) - top[None, :, None]).abs().max().item() < 1e-4
+    assert torch.equal(lifted[..., :128], K)
+    # a plausible mistake - one largest norm for all heads - does not reproduce the vectors
+    flat = orc.lift_one_head(K)
+    wrong_logits = orc.usa_logits(flat, lh)
+    right_logits = orc.usa_logits(lifted, lh)
+    assert (torch.sign(wrong_logits) != torch.sign(right_logits)).any()
+
+
+def test_module_variants_expose_the_reference_layout_and_soft_scores():
+    """The shipped `USA` in its LSH and CENTER variants: state-dict keys of the reference, a recorded state dict loads, and
+    the soft mode (torch code, runs without a GPU) reproduces the recorded scores."""
+    from hashattention._patched import USA, lift_to_sphere
+    g = np.load(os.path.join(HERE, "reference_lsh_center_vectors.npz"))
+    K, Q = torch.from_numpy(g["K"]), torch.from_numpy(g["Q"])
+    lsh = USA(3, 128, {"lth_int_dim": 128, "lth_final_dim": 32, "lth_thold": 0, "lth_num_layers": 0})
+    lsh.center = False
+    keys = [str(k) for k in g["lsh_keys"]]
+    assert list(lsh.state_dict().keys()) == keys
+    lsh.load_state_dict({k: torch.from_numpy(g[f"lsh_w{i % 6}"]) for i, k in enumerate(keys)})
+    assert lsh.rehash_every_step and lsh.kernel_num_layers == 1
+    assert lsh.kernel_layers("k")[0][0][0].shape == (32, 132) and (lsh.kernel_layers("q")[2][0][0][:, 129:] == 0).all()
+    with torch.no_grad():
+        soft, kt = lsh(K, Q)
+    assert (soft - torch.from_numpy(g["lsh_soft_span"])).abs().max().item() < 1e-5
+    assert (kt - torch.from_numpy(g["lsh_soft_k"])).abs().max().item() < 1e-4
+    # the batched lift equals the oracle's head-by-head one, padding aside
+    mine = lift_to_sphere(K, 3)
+    assert torch.equal(mine[..., :129], orc.lift_heads(K)) and (mine[..., 129:] == 0).all()
+
+    usa = USA(3, 128, {"lth_int_dim": 32, "lth_final_dim": 32, "lth_thold": 0, "lth_num_layers": 3})
+    ckeys = [str(k) for k in g["center_keys"]]
+    usa.load_state_dict({k: torch.from_numpy(g[f"center_w{i}"]) for i, k in enumerate(ckeys)})
+    usa.center = True
+    assert usa.rehash_every_step
+    with torch.no_grad():
+        soft, kt = usa(K, Q)
+        Kh, Qh = usa.hash_inputs(K, Q)
+    assert (soft - torch.from_numpy(g["center_soft_span"])).abs().max().item() < 1e-5
+    Ko, Qo = orc.standardise_by_keys(K, Q)
+    assert (Kh - Ko).abs().max().item() < 1e-5 and (Qh - Qo).abs().max().item() < 1e-5
+    # keys of KV heads against queries of more heads: statistics of KV head i // group
+    Kg, Qg = K[:, :1], Q
+    Kh, Qh = usa.hash_inputs(Kg, Qg)
+    Ko, Qo = orc.standardise_by_keys(Kg.expand(-1, 3, -1, -1), Qg)
+    assert (Qh - Qo).abs().max().item() < 1e-5 and (Kh - Ko[:, :1]).abs().max().item() < 1e-5

@@ -28,8 +28,9 @@ def _config(cls, **kw):
     return cfg
 
 
-def _oracle_forward(layer, usa, cfg, apply_rope):
-    """CPU restatement of the reference's patched forward, bound to an unpatched attention layer."""
+def _oracle_forward(layer, usa, cfg, apply_rope, **variant):
+    """CPU restatement of the reference's patched forward, bound to an unpatched attention layer.  `variant`: center=True
+    or lsh=True for the hash variants whose inputs depend on the whole cache."""
     orig = layer.forward
     k_heads = [[(m.weight.detach().float().cpu(), m.bias.detach().float().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
                for seq in usa.learning_to_hash_transformation_k]
@@ -48,7 +49,8 @@ def _oracle_forward(layer, usa, cfg, apply_rope):
         cos, sin = position_embeddings
         q, k = apply_rope(q, k, cos, sin)
         k, v = past_key_values.update(k, v, self.layer_idx)
-        out, _ = orc.reference_decode_attention(q, k, v, k_heads, q_heads, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget)
+        out, _ = orc.reference_decode_attention(q, k, v, k_heads, q_heads, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget,
+                                                **variant)
         return self.o_proj(out.transpose(1, 2).reshape(b, q_len, -1)), None
 
     layer.forward = types.MethodType(forward, layer)

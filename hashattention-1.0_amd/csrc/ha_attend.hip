@@ -119,6 +119,13 @@ struct FusedSel {
     double heavy_budget;
     int32_t *out_counts;
 };
+// Additive attention mask of a list-fed launch: values [B, len] fp32 (row stride stride_b), indexed by the token position
+// of a list entry, or by the entry's place in the list (by_slot).
+struct AttnMask {
+    const float *values;
+    int64_t stride_b;
+    int len, by_slot;
+};
 constexpr int kFusedLocalChunks = 64;
 constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
 // a batch of equal lengths is cut into this many workgroups (one per CU): measured against 512 at 64K tokens, B = 6: 76.6
@@ -364,7 +371,9 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // ------------------------------------------------------------------------------------------------
 // grid (nsplit_max, H, B).  Workgroup s of row (b, h) attends to idx[b, h, s*split_rows : (s+1)*split_rows).
 // NT threads = NT/16 row streams; U rows per stream per step.
-template <typename E, int NT, int U, int FW>
+// MK: an additive term per list entry (AttnMask), natural-log units, added to the scaled score before the softmax; list-fed
+// launches only.
+template <typename E, int NT, int U, int FW, bool MK = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
@@ -373,8 +382,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                                                            int nsplit_max, float *__restrict__ part_acc,
                                                            float *__restrict__ part_ml, void *__restrict__ out,
                                                            const float *__restrict__ win_part, int win_init, int win_recent,
-                                                           const int32_t *__restrict__ seq_lens, int max_S, const FusedSel fsel) {
+                                                           const int32_t *__restrict__ seq_lens, int max_S, const FusedSel fsel,
+                                                           const AttnMask amask) {
     using EL = Elem<E>;
+    static_assert(!MK || FW == 0, "the additive mask exists for list-fed launches only");
     constexpr int NS = NT / 16;  // row streams
     __shared__ float s_m[NS], s_l[NS];
     __shared__ float s_acc[NS * HA_HEAD_DIM];
@@ -518,6 +529,14 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     int32_t j_next[U];   // indices of the step after the one in flight
     Raw8<E> kr[U], vr[U];
     int base = r0;
+    // MK: the additive term of list position (step base, u), token j, in the log2 units of the scores.  The index is
+    // clamped to the mask row, so a list entry beyond it reads the row's last value instead of a wild address.
+    [[maybe_unused]] float mk[U], mk_next[U];
+    [[maybe_unused]] auto mask_term = [&](int base_, int u, int32_t j) {
+        const int r = base_ + stream + u * NS;
+        const int64_t e = amask.by_slot ? (r < r1 ? r : r0) : j;
+        return amask.values[b * amask.stride_b + min(max(e, (int64_t)0), (int64_t)amask.len - 1)] * kLog2e;
+    };
     // needs list entries [base, base + 2 STEP)
     auto prime = [&]() {
         int32_t j0[U];
@@ -525,6 +544,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int u = 0; u < U; ++u) j0[u] = list_index(base, u);
 #pragma unroll
         for (int u = 0; u < U; ++u) j_next[u] = list_index(base + STEP, u);
+        if constexpr (MK) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) mk[u] = mask_term(base, u, j0[u]);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) kr[u] = EL::load8s(kb + j0[u] * row_bytes, sub);
 #pragma unroll
@@ -541,6 +564,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int u = 0; u < U; ++u) vn[u] = EL::load8s(vb + j_next[u] * row_bytes, sub);
 #pragma unroll
         for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
+        if constexpr (MK) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) mk_next[u] = mask_term(base + STEP, u, j_next[u]);
+        }
 
         // ---- reduce the current step
         float sc[U], mloc = -INFINITY;
@@ -551,6 +578,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
             d = row16_sum(d);
+            if constexpr (MK) d += mk[u];
             sc[u] = (base + stream + u * NS < r1) ? d : -INFINITY;
             mloc = fmaxf(mloc, sc[u]);
         }
@@ -576,6 +604,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             kr[u] = kn[u];
             vr[u] = vn[u];
             j_next[u] = j_after[u];
+            if constexpr (MK) mk[u] = mk_next[u];
         }
         base += STEP;
     };
@@ -877,7 +906,7 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
                               int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv,
                               const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace,
                               size_t workspace_bytes, const float *win_part, int win_init, int win_recent, const int32_t *seq_lens,
-                              int max_seq_len, void *stream) {
+                              int max_seq_len, const AttnMask amask, void *stream) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(idx && counts, HA_ERR_NULL_POINTER, "idx/counts is NULL");
@@ -896,12 +925,12 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
     const dim3 grid(plan.nsplit_max, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-#define HA_SPARSE_LAUNCH(E_, NT_, U_)                                                                                             \
+#define HA_SPARSE_LAUNCH(E_, NT_, U_, MK_)                                                                                           \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,        \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0, MK_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,   \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
                            plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len,        \
-                           FusedSel{});                                                                                           \
+                           FusedSel{}, amask);                                                                                    \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
         if (plan.nsplit_max > 1) {                                                                                                \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
@@ -909,10 +938,13 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
         }                                                                                                                         \
     } while (0)
-#define HA_SPARSE_DISPATCH(E_, U_)                       \
-    do {                                                 \
-        if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_); \
-        else HA_SPARSE_LAUNCH(E_, 256, U_);              \
+#define HA_SPARSE_DISPATCH(E_, U_)                                            \
+    do {                                                                      \
+        if (amask.values) {                                                   \
+            if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_, true);     \
+            else HA_SPARSE_LAUNCH(E_, 256, U_, true);                         \
+        } else if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_, false); \
+        else HA_SPARSE_LAUNCH(E_, 256, U_, false);                            \
     } while (0)
     if (kv_dtype == HA_BF16) HA_SPARSE_DISPATCH(ElemBF16, 4);
     else if (kv_dtype == HA_F16) HA_SPARSE_DISPATCH(ElemF16, 4);
@@ -927,7 +959,22 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, cons
                      int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace, size_t workspace_bytes,
                      void *stream) {
     return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
-                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0, stream);
+                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0, AttnMask{}, stream);
+}
+
+int ha_sparse_decode_masked(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                            int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv, const int32_t *idx,
+                            int64_t idx_cap, const int32_t *counts, float sm_scale, const float *mask, int64_t mask_stride_b,
+                            int mask_len, int mask_by_slot, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    HA_REQUIRE(mask, HA_ERR_NULL_POINTER, "mask is NULL");
+    HA_REQUIRE(mask_len > 0 && mask_stride_b >= 0, HA_ERR_BAD_SHAPE, "mask_len must be positive and mask_stride_b non-negative");
+    HA_REQUIRE(mask_by_slot == 0 || mask_by_slot == 1, HA_ERR_BAD_SHAPE, "mask_by_slot must be 0 or 1");
+    HA_REQUIRE(!mask_by_slot || mask_len >= idx_cap, HA_ERR_BAD_SHAPE, "a mask by list slot needs idx_cap=%lld values per row, got %d",
+               (long long)idx_cap, mask_len);
+    HA_REQUIRE(ha_aligned(mask, 4), HA_ERR_MISALIGNED, "mask misaligned");
+    return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
+                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0,
+                              AttnMask{mask, mask_stride_b, mask_len, mask_by_slot}, stream);
 }
 
 int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
@@ -939,7 +986,7 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
     HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && max_seq_len > 0, HA_ERR_BAD_SHAPE, "bad window budgets or max_seq_len");
     return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
                               counts, sm_scale, out, workspace, workspace_bytes, window_partial, init_budget, recent_budget, seq_lens,
-                              max_seq_len, stream);
+                              max_seq_len, AttnMask{}, stream);
 }
 
 // Chunks per workgroup of the fused path.  A batch of equal lengths: whole rows when there are at least
@@ -1035,7 +1082,7 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
         hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b,                       \
                            q_stride_h, k, v,                                                                                      \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
-                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f);                                      \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{});                          \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \

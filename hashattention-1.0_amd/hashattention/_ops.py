@@ -96,6 +96,9 @@ def load_library() -> C.CDLL:
     lib.ha_sparse_decode.restype = i32
     lib.ha_sparse_decode.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
                                      vp, vp, sz, vp]
+    lib.ha_sparse_decode_masked.restype = i32
+    lib.ha_sparse_decode_masked.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
+                                            vp, i64, i32, i32, vp, vp, sz, vp]
     lib.ha_window_partial_bytes.restype = sz
     lib.ha_window_partial_bytes.argtypes = [i32, i32]
     lib.ha_window_partial.restype = i32
@@ -326,12 +329,21 @@ def _kv_args(q, k, v):
 
 
 def sparse_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor,
-                  sm_scale: float, out: torch.Tensor, ws: torch.Tensor) -> None:
-    """q [B,H,128]; k,v [B,Hkv,S_cap,128]; idx [B,H,idx_cap] int32; counts [B,H] int32; out [B,H,128] (in place)."""
-    _require_cuda(q, k, v, idx, counts, out, ws)
+                  sm_scale: float, out: torch.Tensor, ws: torch.Tensor, mask: Optional[torch.Tensor] = None,
+                  mask_by_slot: bool = False) -> None:
+    """q [B,H,128]; k,v [B,Hkv,S_cap,128]; idx [B,H,idx_cap] int32; counts [B,H] int32; out [B,H,128] (in place).
+    mask: optional fp32 [B, n] (or [1, n] expanded: row stride 0) added to the scaled scores, indexed by token position,
+    or by the place in the list when mask_by_slot."""
+    _require_cuda(q, k, v, idx, counts, out, ws, mask)
     lib = load_library()
     B, H, _ = q.shape
     assert out.is_contiguous() and out.dtype == q.dtype and idx.is_contiguous() and counts.is_contiguous()
+    if mask is not None:
+        assert mask.dtype == torch.float32 and mask.dim() == 2 and mask.shape[0] == B and mask.stride(1) == 1
+        _check(lib.ha_sparse_decode_masked(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
+                                           float(sm_scale), _ptr(mask), mask.stride(0), mask.shape[1], 1 if mask_by_slot else 0,
+                                           _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_sparse_decode_masked")
+        return
     _check(lib.ha_sparse_decode(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
                                 float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _stream(q)), "ha_sparse_decode")
 

@@ -22,6 +22,7 @@ from __future__ import annotations
 
 import math
 import os
+import weakref
 from typing import List, Optional, Tuple
 
 import torch
@@ -58,6 +59,8 @@ class SignSTE(torch.autograd.Function):
 def ste_sign(x: torch.Tensor) -> torch.Tensor:
     return SignSTE.apply(x)
 
+
+_MASK_PROBE = [None, None, False]   # last attention mask examined: weak reference, (version, length), "changes something"
 
 LSH_PAD = 3     # zero coordinates after the lifted one: the encode kernels take input widths that are multiples of 4
 
@@ -342,11 +345,38 @@ class HeavyHitterMixin:
         kh, qh = usa.hash_inputs(key_states.to(usa.dtype), query_states.to(usa.dtype))
         return kh.contiguous(), qh.contiguous()
 
-    def _sparse_attention(self, query_states, key_states, value_states):
+    def _additive_mask(self, attention_mask, b: int, q_len: int, S: int):
+        """The reference adds `attention_mask` [b, 1, q, S] to the scores before the keep-mask and the softmax (:593-598).
+        Returns it as fp32 [b, q, S], or None when it changes nothing for any row's causal part (the kernels apply the
+        causal structure themselves), which is the case for every unpadded batch.  A boolean mask (True = attend) is
+        accepted as well.  Deciding costs one device-to-host read per forward pass, not per layer: the layers of a model
+        are handed the same tensor object."""
+        if attention_mask is None:
+            return None
+        if attention_mask.dim() != 4 or attention_mask.shape[1] != 1 or attention_mask.shape[2] != q_len \
+                or attention_mask.shape[3] < S or attention_mask.shape[0] not in (1, b):
+            raise ValueError(f"Attention mask should be of size {(b, 1, q_len, S)}, but is {tuple(attention_mask.size())}")
+        probe = _MASK_PROBE
+        hit = probe[0] is not None and probe[0]() is attention_mask and probe[1] == (attention_mask._version, S)
+        if not hit:
+            m = attention_mask[:, 0, :, :S]
+            causal = torch.tril(torch.ones(q_len, S, dtype=torch.bool, device=m.device), diagonal=S - q_len)
+            blocked = torch.logical_not(m) if m.dtype == torch.bool else m != 0
+            probe[0], probe[1], probe[2] = weakref.ref(attention_mask), (attention_mask._version, S), \
+                bool((blocked & causal).any().item())
+        if not probe[2]:
+            return None
+        m = attention_mask[:, 0, :, :S]
+        if m.dtype == torch.bool:
+            m = torch.zeros(m.shape, dtype=torch.float32, device=m.device).masked_fill_(torch.logical_not(m), float("-inf"))
+        return m.float().expand(b, q_len, S).contiguous()
+
+    def _sparse_attention(self, query_states, key_states, value_states, attention_mask=None):
         """query [b, H, q, d] (q <= 128), key/value [b, Hkv, S, d] holding the whole cache including the new tokens.
         Returns [b, H, q, d].  Row i attends as query at absolute position S - q + i (reference :423-428)."""
         b, H, q_len, d = query_states.shape
         S = key_states.shape[2]
+        amask = self._additive_mask(attention_mask, b, q_len, S)
         hl = self._ensure_hash_layer(b, S, query_states.device)
         key_hash, query_hash = self._hash_inputs(key_states, query_states)
         if hl.n_cached > S - q_len or self.usa_module.rehash_every_step:
@@ -366,7 +396,8 @@ class HeavyHitterMixin:
             hl.heavy_budget = heavy_abs
             try:
                 hl.step(query_states, key_states, value_states, S, out[:, :, 0],
-                        hash_inputs=None if key_hash is key_states else (key_hash, query_hash))
+                        hash_inputs=None if key_hash is key_states else (key_hash, query_hash),
+                        attn_mask=None if amask is None else amask[:, 0])
             finally:
                 hl.heavy_budget = saved
             return out
@@ -388,7 +419,8 @@ class HeavyHitterMixin:
             _ops.select(hl.codes[bi:bi + 1].expand(q_len, -1, -1, -1), qc[0].transpose(0, 1).contiguous(), S, lens, hl.init_budget,
                         hl.recent_budget, heavy_abs, idx, cnt, ws_s, hl.mode, hl.depth)
             _ops.sparse_decode(query_states[bi].transpose(0, 1).contiguous(), key_states[bi:bi + 1].expand(q_len, -1, -1, -1),
-                               value_states[bi:bi + 1].expand(q_len, -1, -1, -1), idx, cnt, hl.sm_scale, o_b, ws_a)
+                               value_states[bi:bi + 1].expand(q_len, -1, -1, -1), idx, cnt, hl.sm_scale, o_b, ws_a,
+                               mask=None if amask is None else amask[bi])
             out[bi] = o_b.transpose(0, 1)
         return out
 
@@ -416,7 +448,7 @@ class HeavyHitterMixin:
             key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
         if key_states.stride(-1) != 1 or value_states.stride() != key_states.stride():
             key_states, value_states = key_states.contiguous(), value_states.contiguous()
-        attn = self._sparse_attention(query_states.contiguous(), key_states, value_states)
+        attn = self._sparse_attention(query_states.contiguous(), key_states, value_states, attention_mask)
         attn = attn.transpose(1, 2).reshape(bsz, q_len, -1).contiguous()
         out = self.o_proj(attn)
         self.offload_if_necessary_cpu(cache)

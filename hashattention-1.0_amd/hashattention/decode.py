@@ -130,13 +130,15 @@ class HashDecodeLayer:
                                  self.init_budget, self.recent_budget, self.heavy_budget, self.ws_select, self.sm_scale, out,
                                  self.ws_fused, thresholds_ready=not self.local_thresholds, out_counts=self.counts)
 
-    def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor) -> None:
-        _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend)
+    def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
+               attn_mask: Optional[torch.Tensor] = None) -> None:
+        _ops.sparse_decode(q3, k, v, self.idx, self.counts, self.sm_scale, out, self.ws_attend, mask=attn_mask)
 
     # ------------------------------------------------------------------ one decode step
     def step(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, seq_len: int, out: torch.Tensor,
              seq_lens: Optional[torch.Tensor] = None, n_new: int = 1,
-             hash_inputs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+             hash_inputs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+             attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         """q [B, H, 1, d]; k_cache/v_cache [B, Hkv, >=seq_len, d] already holding the new token(s) at the end.
 
         Uniform batches: the last `n_new` tokens (positions seq_len - n_new ..) are encoded and appended to the
@@ -144,6 +146,8 @@ class HashDecodeLayer:
         `seq_lens` (int32 [B], lengths including the new token) and `seq_len` = their maximum.
         `hash_inputs` = (keys [B, Hkv, >=seq_len, d'], queries [B, H, 1, d']): what the hash MLPs read when that is not the
         cache and the query themselves (standardised or lifted vectors; uniform batches only).
+        `attn_mask` fp32 [B, >= seq_len]: added to the scaled score of the token at each position before the softmax (the
+        padding mask of a batch); the selection does not see it.  Takes the list-fed attention launch.
         """
         q3 = q[:, :, 0, :]
         k_hash, q_hash3 = (k_cache, q3) if hash_inputs is None else (hash_inputs[0], hash_inputs[1][:, :, 0, :])
@@ -171,9 +175,15 @@ class HashDecodeLayer:
             newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
             _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
                              self.qcodes, pos_dev=pos, arith=self.arith)
-        return self._select_attend(q3, k_cache, v_cache, seq_len, out, seq_lens, main)
+        return self._select_attend(q3, k_cache, v_cache, seq_len, out, seq_lens, main, attn_mask)
 
-    def _select_attend(self, q3, k_cache, v_cache, seq_len, out, seq_lens, main=None):
+    def _select_attend(self, q3, k_cache, v_cache, seq_len, out, seq_lens, main=None, attn_mask=None):
+        if attn_mask is not None:
+            if self.overlap_windows:
+                raise RuntimeError("an attention mask is not supported together with the second-stream window partial")
+            self.select(seq_len, seq_lens)
+            self.attend(q3, k_cache, v_cache, out, attn_mask)
+            return out
         if self.use_fused and self.fused_ok and not self.overlap_windows:
             self.select_prepare(seq_len, seq_lens)
             self.attend_fused(q3, k_cache, v_cache, out, seq_len, seq_lens)

@@ -174,6 +174,26 @@ int ha_sparse_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
                      float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * ha_sparse_decode with an additive mask: out[b, h] = softmax(q . K[idx] * sm_scale + mask term) V[idx].
+ * mask is fp32 [B, mask_len] (row stride mask_stride_b, in elements; 0 shares one row), in natural-log
+ * units, one row per sequence shared by its heads; entries of -inf (or the dtype's most negative value,
+ * as the reference fills them) remove a list entry from the softmax.
+ *   mask_by_slot = 0: the term of a list entry is mask[b, token position] - the `attention_mask` the
+ *                     patched layer adds before its softmax (hashattention_llama.py:593-598: padding of a
+ *                     batch, on top of the selection); mask_len >= the largest position in the lists
+ *                     (positions beyond it read the row's last value);
+ *   mask_by_slot = 1: the term is mask[b, place in the list], the `Mask` argument of fwd_sparse
+ *                     (efficiency/kernels/sparse.py:14, 46-58, 190-212); mask_len >= idx_cap.
+ * A row whose entries are all removed gives a zero output.
+ */
+int ha_sparse_decode_masked(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                            const void *k, const void *v, int kv_dtype,
+                            int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                            int B, int H, int Hkv, const int32_t *idx, int64_t idx_cap, const int32_t *counts,
+                            float sm_scale, const float *mask, int64_t mask_stride_b, int mask_len, int mask_by_slot,
+                            void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * The same attention in two launches that may overlap in time.  The sink [0, init) and recent [S - recent, S)
  * windows are known before any selection is made and are shared by the query heads of a KV group:
  * ha_window_partial attends to them alone (each row read once per KV head) and leaves an unnormalised partial

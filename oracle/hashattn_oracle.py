@@ -275,26 +275,34 @@ def apply_rotary_pos_emb(q, k, cos, sin):
     return q * cos + rotate_half(q) * sin, k * cos + rotate_half(k) * sin
 
 
-def masked_decode_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-    """Dense scores, mask to finfo.min, softmax in fp32 cast back to Q's dtype, times V.
+def masked_decode_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, mask: torch.Tensor,
+                            attention_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense scores, (+ the additive attention mask,) keep-mask to finfo.min, softmax in fp32 cast back to Q's dtype, times V.
 
-    reference: hashattention_llama.py:585, 606, 613, 615.  Q [b,H,q,d]; K,V [b,H,S,d]; mask [b,H,q,S].
+    reference: hashattention_llama.py:585, 593-598 (`attn_weights + attention_mask`, [b, 1, q, S]), 606, 613, 615.
+    Q [b,H,q,d]; K,V [b,H,S,d]; mask [b,H,q,S].
     """
     w = torch.matmul(Q, K.transpose(2, 3)) / math.sqrt(Q.shape[-1])
+    if attention_mask is not None:
+        assert attention_mask.shape == (Q.shape[0], 1, Q.shape[2], K.shape[2])
+        w = w + attention_mask
     w = w.masked_fill(~mask, torch.finfo(w.dtype).min)
     w = F.softmax(w, dim=-1, dtype=torch.float32).to(Q.dtype)
     return torch.matmul(w, V)
 
 
-def sparse_attend(q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, idx: Sequence[int], sm_scale: float) -> torch.Tensor:
-    """One (batch, head): softmax(q . K[idx] * scale) @ V[idx] in fp32.
+def sparse_attend(q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, idx: Sequence[int], sm_scale: float,
+                  slot_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One (batch, head): softmax(q . K[idx] * scale + slot_mask) @ V[idx] in fp32.
 
-    reference: `torch_fwd_sparse`, efficiency/kernels/sparse.py:190-214 (fp32 softmax, zero mask).
-    q [d]; K, V [S, d].
+    reference: `torch_fwd_sparse`, efficiency/kernels/sparse.py:190-214 (fp32 softmax; `att_value += Mask[b]`, :207, one
+    term per place in the list).  q [d]; K, V [S, d]; slot_mask [len(idx)] or None.
     """
     ii = torch.as_tensor(np.asarray(idx), dtype=torch.long)
     k, v = K[ii].float(), V[ii].float()
     a = (k @ q.float()) * sm_scale
+    if slot_mask is not None:
+        a = a + slot_mask[:len(ii)].float()
     p = torch.softmax(a, dim=0)
     return p @ v
 
@@ -317,13 +325,15 @@ def dense_attention(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor) -> torch.
 
 
 def reference_decode_attention(Q, K, V, k_heads, q_heads, init_budget, recent_budget, heavy_budget,
-                               mode="simple", retrieve_depth=0.0, stable=True, usa_dtype=None, center=False, lsh=False):
+                               mode="simple", retrieve_depth=0.0, stable=True, usa_dtype=None, center=False, lsh=False,
+                               attention_mask=None):
     """The reference's emulated decode step between RoPE/cache update and o_proj.
 
     reference: hashattention_llama.py:578-623 with compute_mask_multi :401-446: repeat K/V over the
     group, dense QK^T, re-hash every key, full sort, masked fp32 softmax, AV.
     Q [b,H,q,d]; K,V [b,Hkv,S,d].  Returns (attn_output [b,H,q,d], keep mask [b,H,q,S]).
     `center` / `lsh` (one K head per query head): the hash reads standardised / lifted vectors, as `usa_forward_hard`.
+    `attention_mask` [b, 1, q, S]: added to the scores before the keep-mask (:593-598); the selection does not see it.
     """
     H, Hkv = Q.shape[1], K.shape[1]
     Kr, Vr = repeat_kv(K, H // Hkv), repeat_kv(V, H // Hkv)
@@ -346,7 +356,7 @@ def reference_decode_attention(Q, K, V, k_heads, q_heads, init_budget, recent_bu
     causal = torch.tril(torch.ones(t, s), diagonal=s - t).bool()
     span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype))
     mask = compute_mask_multi(span, init_budget, recent_budget, heavy_budget, mode, retrieve_depth, stable)
-    return masked_decode_attention(Q, Kr, Vr, mask), mask
+    return masked_decode_attention(Q, Kr, Vr, mask, attention_mask), mask
 
 
 def recall_overlap(q: torch.Tensor, k: torch.Tensor, k_heads, q_heads, init_budget: int, recent_budget: int,

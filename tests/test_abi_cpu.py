@@ -109,6 +109,19 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert sparse(Hkv=3) == HA_ERR_SHAPE and sparse(ss=64) == HA_ERR_SHAPE
     assert sparse(k=odd) == HA_ERR_ALIGN and sparse(ss=132) == HA_ERR_ALIGN     # rows would not stay 16-byte aligned
     assert sparse(wsb=8) == HA_ERR_WS
+
+    def masked(**kw):
+        a = dict(mask=p, msb=400, mlen=400, slot=0, cap=300, Hkv=2, wsb=1 << 16)
+        a.update(kw)
+        return lib.ha_sparse_decode_masked(p, 512, 128, p, p, _ops.HA_BF16, 128000, 128000, 128, 1, 4, a["Hkv"], p, a["cap"], p,
+                                           C.c_float(0.088), a["mask"], a["msb"], a["mlen"], a["slot"], p, p, a["wsb"], null)
+
+    assert masked(mask=null) == HA_ERR_NULL
+    assert masked(mlen=0) == HA_ERR_SHAPE and masked(msb=-1) == HA_ERR_SHAPE and masked(slot=2) == HA_ERR_SHAPE
+    assert masked(slot=1, mlen=299) == HA_ERR_SHAPE              # a mask by list slot must cover the whole list
+    assert masked(mask=odd) == HA_ERR_ALIGN
+    assert masked(Hkv=3) == HA_ERR_SHAPE and masked(wsb=8) == HA_ERR_WS      # the checks of ha_sparse_decode apply
+    assert masked() == HA_ERR_NODEV and masked(slot=1) == HA_ERR_NODEV
     assert lib.ha_dense_decode(p, 512, 128, p, p, _ops.HA_F32, 128000, 128000, 128, 1, 4, 2, 0, null, C.c_float(0.1), p, p, 1 << 16,
                                null) == HA_ERR_SHAPE           # max_seq_len must be positive
 

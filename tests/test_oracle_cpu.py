@@ -255,3 +255,34 @@ def test_recall_overlap_is_pinned_by_its_special_cases_and_a_verbatim_restatemen
     full = ncand <= S // 16
     want = torch.clamp(ncand, max=3).float() / 3
     assert torch.allclose(few[0, :, full], want[full].expand(4, -1))
+
+
+def test_additive_masks_of_the_oracle():
+    """`attention_mask` of the dense formulation (hashattention_llama.py:593-598) and the slot mask of the gather formulation
+    (sparse.py:207), pinned by what the mathematics fixes: -inf removes an entry (equals attending without it), a constant
+    changes nothing, the dense form equals torch's scaled_dot_product_attention with the summed masks, and the two
+    formulations agree when the slot mask is the position mask gathered through the list."""
+    g = torch.Generator().manual_seed(5)
+    b, H, S, d = 2, 3, 50, 16
+    Q, K, V = torch.randn(b, H, 1, d, generator=g), torch.randn(b, H, S, d, generator=g), torch.randn(b, H, S, d, generator=g)
+    keep = torch.rand(b, H, 1, S, generator=g) < 0.6
+    keep[..., 0] = True
+    am = torch.randn(b, 1, 1, S, generator=g)
+    am[:, :, :, 5:9] = float("-inf")
+    out = orc.masked_decode_attention(Q, K, V, keep, am)
+    sdpa = torch.nn.functional.scaled_dot_product_attention(Q, K, V, attn_mask=am.expand(b, H, 1, S).masked_fill(~keep, float("-inf")))
+    assert (out - sdpa).abs().max().item() < 1e-5
+    # the gather formulation with the position mask gathered through the list
+    for bi in range(b):
+        for h in range(H):
+            idx = torch.nonzero(keep[bi, h, 0]).flatten()
+            got = orc.sparse_attend(Q[bi, h, 0], K[bi, h], V[bi, h], idx.numpy(), 1 / d ** 0.5, slot_mask=am[bi, 0, 0, idx])
+            assert (got - out[bi, h, 0]).abs().max().item() < 1e-5
+            # -inf on a slot == the list without that slot; a constant shift == no mask
+            live = torch.isfinite(am[bi, 0, 0, idx])
+            short = orc.sparse_attend(Q[bi, h, 0], K[bi, h], V[bi, h], idx[live].numpy(), 1 / d ** 0.5, slot_mask=am[bi, 0, 0, idx[live]])
+            assert (short - got).abs().max().item() < 1e-6
+            plain = orc.sparse_attend(Q[bi, h, 0], K[bi, h], V[bi, h], idx.numpy(), 1 / d ** 0.5)
+            shifted = orc.sparse_attend(Q[bi, h, 0], K[bi, h], V[bi, h], idx.numpy(), 1 / d ** 0.5, slot_mask=torch.full((len(idx),), 1.5))
+            assert (plain - shifted).abs().max().item() < 1e-6
+            assert (plain - got).abs().max().item() > 1e-3          # and the random mask does change the result

@@ -147,3 +147,30 @@ def test_left_padded_batch_through_the_patched_model():
     plain = _run(model, ids.to(DEV), torch.ones_like(am).to(DEV), steps)
     assert (plain[-1][1] - got[-1][1]).abs().max().item() > 1e-3
     assert (plain[-1][0] - got[-1][0]).abs().max().item() < 1e-4
+
+
+def test_generate_with_a_left_padded_batch():
+    """`model.generate` end to end (greedy): prefill of 150 tokens through the original forward, then single-token steps
+    through the HIP path with the padding mask, against the oracle-driven model on the CPU: the same tokens."""
+    print("\n[case] generate, left-padded batch", flush=True)
+    torch.manual_seed(8)
+    cfg = _config(LlamaConfig)
+    cfg.pad_token_id = 0
+    model = LlamaForCausalLM(cfg).bfloat16().float()
+    ref = copy.deepcopy(model)
+    usa = hl.load_usa(cfg, None)
+    model = hl.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False).float()
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    for li, layer in enumerate(ref.model.layers):
+        _oracle_forward_masked(layer.self_attn, usa[li], cfg, apply_rotary_pos_emb)
+    ids = torch.randint(1, cfg.vocab_size, (2, 150), generator=torch.Generator().manual_seed(4))
+    am = torch.ones(2, 150, dtype=torch.long)
+    am[0, :23] = 0
+    ids[0, :23] = 0
+    kw = dict(max_new_tokens=6, do_sample=False, use_cache=True, pad_token_id=0)
+    with torch.no_grad():
+        got = model.generate(input_ids=ids.to(DEV), attention_mask=am.to(DEV), **kw).cpu()
+        want = ref.generate(input_ids=ids, attention_mask=am, **kw)
+    print("  new tokens:", got[:, 150:].tolist(), flush=True)
+    assert got.shape == (2, 156) and torch.equal(got, want)
+    assert model.model.layers[0].self_attn._hash_layer.n_cached == 155      # the last token is sampled, not fed back

@@ -21,6 +21,7 @@ OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_lsh_ce
 
 
 def main():
+    sys.dont_write_bytecode = True      # the reference tree is read-only: no __pycache__ beside its sources
     sys.path.insert(0, REF)
     from hashattention import hashattention_llama as ref   # prints "CENTER 0"
 

@@ -31,6 +31,7 @@ def bce_loss(alpha, beta):
 
 
 def main():
+    sys.dont_write_bytecode = True      # the reference tree is read-only: no __pycache__ beside its sources
     sys.path.insert(0, REF)
     from hashattention import hashattention_llama as ref   # prints "CENTER 0"
 

@@ -181,6 +181,8 @@ class HashDecodeLayer:
         if attn_mask is not None:
             if self.overlap_windows:
                 raise RuntimeError("an attention mask is not supported together with the second-stream window partial")
+            if attn_mask.dim() != 2 or attn_mask.shape[0] != self.B or attn_mask.shape[1] < seq_len:
+                raise ValueError(f"attn_mask must be [B={self.B}, >= {seq_len}], got {tuple(attn_mask.shape)}")
             self.select(seq_len, seq_lens)
             self.attend(q3, k_cache, v_cache, out, attn_mask)
             return out

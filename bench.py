@@ -206,22 +206,42 @@ def decoder_bench(args, torch):
         attend_alone = lambda: hl0.attend(q[:, :, 0, :], dec.k_cache[0], dec.v_cache[0], out)
     ms_attend = time_gpu(attend_alone, args.steps, args.warmup, torch)
     n_sel_rows = int(hl0.counts.sum().item())
+    # the generation loop proper: greedy tokens at advancing positions, one captured graph replayed per token with the
+    # position on the device (the last `n_gen` slots of the synthetic cache are written again by the generated tokens)
+    n_gen = max(8, min(args.steps, S - 2))
+    def rewind():
+        dec.seq_len = S - 1 - n_gen
+        for hl in dec.hash:
+            hl.n_cached = dec.seq_len
+    with torch.no_grad():
+        rewind()
+        dec.generate(tokens, 4)                       # capture + a few replays
+        rewind()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gen_tokens = dec.generate(tokens, n_gen)
+        e1.record()
+        torch.cuda.synchronize()
+    ms_gen = e0.elapsed_time(e1) / n_gen
     ab = algorithmic_bytes(w, n_sel_rows)
     n_params = sum(t.numel() for p in dec.layers for t in p.values()) + dec.lm_head.numel()
     step_bytes = 2 * n_params + dec.L * (ab["score"] + ab["select"] + ab["gather"])
     res = {
-        "metric": "decode_tokens_per_s", "value": B / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
-        "step_launch": {"value_is": "graph" if ms_graph <= ms_eager else "eager", "hip_graph_replay_ms": ms_graph,
-                        "eager_launches_from_python_ms": ms_eager},
+        "metric": "decode_tokens_per_s", "value": B / (min(ms_step, ms_gen) * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": min(ms_step, ms_gen),
+        "step_launch": {"value_is": "generation_loop" if ms_gen <= ms_step else ("graph" if ms_graph <= ms_eager else "eager"),
+                        "hip_graph_replay_ms": ms_graph, "eager_launches_from_python_ms": ms_eager, "generation_loop_ms": ms_gen},
         "graph_replay_matches_eager": graph_ok,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config3: {dec.L}-layer Llama-3.1-8B-shaped decoder step, B={B} context={S} H={dec.H} Hkv={dec.Hkv} "
                                f"d={dec.d} hidden={dec.hidden} ffn={dec.ffn} vocab={dec.vocab} code_heads={dec.Hc} "
                                f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g} n_sel={n_sel_rows // (B * dec.H)}"},
-        "dense_attention_step_ms": ms_dense, "speedup_vs_dense_attention": ms_dense / ms_step,
+        "generation_loop": {"tokens_per_sequence": n_gen, "ms_per_token_step": ms_gen, "tokens_per_s": B / (ms_gen * 1e-3),
+                            "how": "greedy, positions on the device, one HIP graph replayed per token + arg-max",
+                            "distinct_tokens": int(gen_tokens.unique().numel())},
+        "dense_attention_step_ms": ms_dense, "speedup_vs_dense_attention": ms_dense / min(ms_step, ms_gen),
         "dense_tokens_per_s": B / (ms_dense * 1e-3),
-        "attention_step_us_per_layer": ms_layer * 1e3, "attention_share_of_step": dec.L * ms_layer / ms_step,
+        "attention_step_us_per_layer": ms_layer * 1e3, "attention_share_of_step": dec.L * ms_layer / min(ms_step, ms_gen),
         "prefill_encode_ms_per_layer": ms_prefill_encode,
         "prefill_encode_tflops": 2 * B * dec.Hc * (S - 1) * (128 * 128 * 2 + 128 * 32) / (ms_prefill_encode * 1e-3) / 1e12,
         "cache_fill_seconds": fill_s,

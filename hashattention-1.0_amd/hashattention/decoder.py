@@ -56,6 +56,7 @@ class LlamaShapedDecoder:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.B = self.S_cap = self.seq_len = 0
+        self._gen_graph = None
         inv = 1.0 / (rope_theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
         self.inv_freq = inv
 
@@ -93,6 +94,12 @@ class LlamaShapedDecoder:
         self.x_attn = [torch.empty(B, self.hidden, dtype=self.dtype, device=self.device) for _ in range(2)]
         self.gate_up = torch.empty(B, 2 * self.ffn, dtype=self.dtype, device=self.device)
         self.logits = torch.empty(B, self.vocab, dtype=self.dtype, device=self.device)
+        # a step whose position lives on the device (`decode_step(..., device_pos=True)`, `generate`): token, position and
+        # length of every sequence
+        self.tok_dev = torch.zeros(B, dtype=torch.int64, device=self.device)
+        self.pos_dev = torch.zeros(B, dtype=torch.int32, device=self.device)
+        self.len_dev = torch.ones(B, dtype=torch.int32, device=self.device)
+        self._gen_graph = None
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
@@ -126,10 +133,13 @@ class LlamaShapedDecoder:
         self.seq_len = S
 
     # ------------------------------------------------------------------ one decode step
-    def decode_step(self, tokens: torch.Tensor, advance: bool = True, dense: bool = False) -> torch.Tensor:
+    def decode_step(self, tokens: torch.Tensor, advance: bool = True, dense: bool = False, device_pos: bool = False) -> torch.Tensor:
         """tokens [B] int64 -> logits [B, vocab].  The new token sits at position `seq_len`; with advance=False the
         step can be replayed (HIP graph) at a fixed context length.  dense=True attends to the whole cache with the
         dense flash-decode kernel instead (the baseline the sparse step is compared with).
+        device_pos=True: the position is read from `pos_dev` / `len_dev` on the device instead (every kernel of the step
+        takes it from there and sizes its work for the cache capacity), so ONE captured graph serves successive tokens;
+        `generate` drives it.  bf16 with 128-wide heads, sparse attention only; `seq_len` is left alone.
 
         Per layer (bf16, up to 8 sequences): QKV projection with its RMSNorm folded in, ha_rope_append, the attention
         step, output projection with the residual folded in, gate/up projection with its RMSNorm and SwiGLU folded in,
@@ -148,7 +158,13 @@ class LlamaShapedDecoder:
             else:
                 qkv = F.linear(F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps), p["wqkv"])
             hl = self.hash[l]
-            if dense:
+            if device_pos:
+                if dense or d != 128:
+                    raise RuntimeError("device_pos steps run the sparse attention on 128-wide heads")
+                _ops.rope_encode_step(qkv, H, Hkv, 0, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l], hl.wk, hl.wq,
+                                      hl.num_layers, hl.int_dim, hl.final_dim, hl.codes, hl.qcodes, pos_dev=self.pos_dev, arith=hl.arith)
+                hl._select_attend(self.q_rot, self.k_cache[l], self.v_cache[l], self.S_cap, self.attn_out, self.len_dev)
+            elif dense:
                 _ops.rope_append(qkv, H, Hkv, pos, self.inv_freq, self.q_rot, self.k_cache[l], self.v_cache[l])
                 _ops.dense_decode(self.q_rot, self.k_cache[l], self.v_cache[l], S, None, hl.sm_scale, self.attn_out, self.ws_dense)
             elif self.fuse_rope and d == 128:
@@ -171,12 +187,56 @@ class LlamaShapedDecoder:
                 x = _ops.linear_skinny(self.ffn_act, p["w2"], self.x_attn[1], residual=x)
             else:
                 x = x.addmm_(self.ffn_act, p["w2"].t())      # in place: the out-of-place form first copies x into its result
-        if advance:
+        if advance and not device_pos:
             self.seq_len = S
         if skinny and self.skinny_all:
             return _ops.linear_skinny(x, self.lm_head, self.logits, norm_weight=self.final_norm, eps=self.eps)
         x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)
         return F.linear(x, self.lm_head)
+
+    # ------------------------------------------------------------------ greedy generation, one graph for all tokens
+    def generate(self, tokens: torch.Tensor, n_new: int, use_graph: bool = True) -> torch.Tensor:
+        """Greedy decoding: `tokens` [B] are fed at position `seq_len`, then each step's arg-max, `n_new` steps in all;
+        returns the [B, n_new] tokens produced.  The protocol of the reference's harness (efficiency/generate.py:68-96,
+        `decode_n_tokens`, its step compiled at :340-348): the step is captured ONCE as a HIP graph whose kernels read the position
+        from device memory, and replayed per token; between replays only the arg-max and the position increment are
+        launched, and nothing waits for the host."""
+        B = self.B
+        if tokens.shape != (B,):
+            raise ValueError(f"tokens must be [{B}]")
+        if self.seq_len + n_new > self.S_cap:
+            raise ValueError(f"{n_new} more tokens do not fit the cache ({self.seq_len} of {self.S_cap} used)")
+        self.tok_dev.copy_(tokens)
+        self.pos_dev.fill_(self.seq_len)
+        self.len_dev.fill_(self.seq_len + 1)
+        out = torch.empty(B, n_new, dtype=torch.int64, device=self.device)
+        step = lambda: self.decode_step(self.tok_dev, device_pos=True)
+        if use_graph:
+            if self._gen_graph is None:     # captured once per allocation: the buffers it names do not change
+                # two eager passes on a side stream, as graph capture wants them; they write the slots of the current
+                # position, which the first replay writes again with the same values
+                side, main = torch.cuda.Stream(device=self.device), torch.cuda.current_stream(self.device)
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    step()
+                    step()
+                main.wait_stream(side)
+                self._gen_graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self._gen_graph):
+                    step()
+            run = self._gen_graph.replay
+        else:
+            run = step
+        for i in range(n_new):
+            run()
+            torch.argmax(self.logits, dim=-1, out=self.tok_dev)
+            out[:, i].copy_(self.tok_dev)
+            self.pos_dev.add_(1)
+            self.len_dev.add_(1)
+        self.seq_len += n_new
+        for hl in self.hash:
+            hl.n_cached = self.seq_len
+        return out
 
     # ------------------------------------------------------------------ weights from a transformers Llama
     def load_hf_llama(self, model) -> None:

@@ -253,3 +253,43 @@ def test_rope_encode_step_equals_rope_append_then_encode_step(dtype, code_heads)
         for a, b in zip(*outs):
             assert torch.equal(a, b)
         assert outs[1][3].ne(0).any() and outs[1][1].ne(0).any()
+
+
+@pytest.mark.parametrize("n_heads,batch", [(8, 4), (4, 2)])
+def test_generate_replays_one_graph_for_successive_tokens(n_heads, batch):
+    # positions on the device: one captured graph serves every token.  Against the same steps launched one by one with the
+    # position on the host (8 heads x 4 sequences: the fused attention launch; 4 x 2: the list-fed launches)
+    print(f"\n[case] decoder generate, graph replay per token, H={n_heads} B={batch}", flush=True)
+    mk = lambda: LlamaShapedDecoder(n_layers=2, hidden=512, ffn=1024, n_heads=n_heads, n_kv_heads=2, head_dim=128, vocab=512,
+                                    n_code_heads=2, init_budget=8, recent_budget=8, heavy_budget=0.125, dtype=torch.bfloat16,
+                                    device=DEV, seed=6)
+    n_new, ctx = 12, 1500
+    first = torch.arange(3, 3 + batch, device=DEV)
+    decs = [mk() for _ in range(3)]
+    for dec in decs:
+        dec.allocate(batch, 2000)
+        dec.fill_cache_synthetic(ctx, seed=1)
+    assert all(hl.fused_ok for hl in decs[0].hash) == (n_heads * batch >= 32)
+    with torch.no_grad():
+        host, tok = [], first
+        first_logits = None
+        for _ in range(n_new):
+            logits = decs[0].decode_step(tok)
+            first_logits = logits.float().clone() if first_logits is None else first_logits
+            tok = logits.argmax(-1)
+            host.append(tok)
+        host = torch.stack(host, dim=1)
+        graph = decs[1].generate(first, n_new, use_graph=True)
+        eager = decs[2].generate(first, n_new, use_graph=False)
+    torch.cuda.synchronize()
+    assert graph.shape == (batch, n_new) and decs[1].seq_len == ctx + n_new and decs[1].hash[0].n_cached == ctx + n_new
+    assert torch.equal(graph, eager)                       # the replayed graph and the same launches made eagerly: the same bits
+    for l in range(2):                                     # the caches and the bit-caches grew identically
+        assert torch.equal(decs[1].k_cache[l], decs[2].k_cache[l]) and torch.equal(decs[1].hash[l].codes, decs[2].hash[l].codes)
+    # positions on the host: the rows are cut into other pieces, so the attention output may differ in its last bit
+    same = (graph == host).float().mean().item()
+    print(f"  tokens equal to the host-position loop: {same:.3f}", flush=True)
+    assert torch.equal(graph[:, 0], host[:, 0]) and same >= 0.9
+    assert torch.equal(decs[0].k_cache[0][:, :, :ctx + 1], decs[1].k_cache[0][:, :, :ctx + 1])
+    with pytest.raises(ValueError):
+        decs[1].generate(first, 2000)

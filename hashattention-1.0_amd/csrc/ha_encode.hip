@@ -34,6 +34,8 @@ struct EncSide {
     int pos0;
     const int32_t *pos_dev;
     float *logits;
+    int pos_bias;  // added to pos_dev[b] (-1 when pos_dev holds sequence lengths and the row is the last one)
+    int x_at_pos;  // T = 1: x is a cache and the row to hash sits at the position the code is written to
 };
 // Up to two sides share one launch (the new keys and the queries of a decode step): blockIdx.y runs over
 // the heads of side 0, then those of side 1.
@@ -129,7 +131,9 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
             const int row = row0 + r;
             if (row < n_rows) {
                 const int b = row / T, t = row % T;
-                xs[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + e, x_dtype);
+                int64_t at = t;
+                if (sd.x_at_pos) at = max(pos_dev ? pos_dev[b] + sd.pos_bias : pos0, 0);  // an empty sequence hashes row 0, written nowhere
+                xs[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + at * x_st + e, x_dtype);
                 if (rp.inv_freq) xpair[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + (e ^ 64), x_dtype);
             }
         }
@@ -259,10 +263,10 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
         const bool bit = tid < d_out && s_act[cur][r][tid] > 0.0f;
         const uint64_t bal = __ballot(bit);
         if (logits && tid < d_out) logits[(((int64_t)b * n_heads + head) * T + t) * d_out + tid] = s_act[cur][r][tid];
-        const int64_t pos = (int64_t)(pos_dev ? pos_dev[b] : pos0) + t;
+        const int64_t pos = (int64_t)(pos_dev ? pos_dev[b] + sd.pos_bias : pos0) + t;
         uint32_t *c = codes + b * c_sb + head * c_sh + pos * W;
-        if (lane == 0 && wave * 2 < W) c[wave * 2] = (uint32_t)bal;
-        if (lane == 32 && wave * 2 + 1 < W) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
+        if (lane == 0 && wave * 2 < W && pos >= 0) c[wave * 2] = (uint32_t)bal;
+        if (lane == 32 && wave * 2 + 1 < W && pos >= 0) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
     }
 }
 
@@ -356,6 +360,33 @@ int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, in
                         pos0, pos_dev, nullptr};
     a.side[1] = EncSide{q, x_dtype, q_stride_b, q_stride_h, (int64_t)head_dim, H, H, weights_q, qcodes, (int64_t)H * W, (int64_t)W,
                         0, nullptr, nullptr};
+    a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
+    a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
+    const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);
+    return launch_encode(a, dim3(tiles, Hc + H), (hipStream_t)stream);
+}
+
+int ha_encode_step_cached(const void *k_cache, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s, const void *q,
+                          int64_t q_stride_b, int64_t q_stride_h, int x_dtype, int B, int Hkv, int Hc, int H,
+                          const int32_t *seq_lens, const float *weights_k, const float *weights_q, int n_layers, int head_dim,
+                          int int_dim, int final_dim, int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h,
+                          uint32_t *qcodes, void *stream) {
+    int st = validate_encode(k_cache, B, Hkv, Hc, 1, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b,
+                             kc_stride_h, 0);
+    if (st) return st;
+    HA_REQUIRE(q && weights_q && qcodes && seq_lens, HA_ERR_NULL_POINTER, "q/weights_q/qcodes/seq_lens is NULL");
+    HA_REQUIRE(H > 0 && H + Hc <= 65535, HA_ERR_BAD_SHAPE, "H must be positive and H + Hc <= 65535");
+    HA_REQUIRE(k_stride_s >= head_dim, HA_ERR_BAD_SHAPE, "cache rows overlap: k_stride_s=%lld < head_dim=%d", (long long)k_stride_s,
+               head_dim);
+    HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
+    HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
+    if ((st = ha_require_device())) return st;
+    const int W = final_dim / 32;
+    EncArgs a = {};
+    a.side[0] = EncSide{k_cache, x_dtype, k_stride_b, k_stride_h, k_stride_s, Hkv, Hc, weights_k, kcodes, kc_stride_b, kc_stride_h,
+                        0, seq_lens, nullptr, -1, 1};
+    a.side[1] = EncSide{q, x_dtype, q_stride_b, q_stride_h, (int64_t)head_dim, H, H, weights_q, qcodes, (int64_t)H * W, (int64_t)W,
+                        0, nullptr, nullptr, 0, 0};
     a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
     const unsigned tiles = (unsigned)((B + kRows - 1) / kRows);

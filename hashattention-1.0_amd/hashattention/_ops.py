@@ -57,6 +57,9 @@ def load_library() -> C.CDLL:
     lib.ha_encode_step.restype = i32
     lib.ha_encode_step.argtypes = [vp, i64, i64, i64, vp, i64, i64, i32, i32, i32, i32, i32, i32, vp, vp,
                                    i32, i32, i32, i32, i32, vp, i64, i64, i32, vp, vp, vp]
+    lib.ha_encode_step_cached.restype = i32
+    lib.ha_encode_step_cached.argtypes = [vp, i64, i64, i64, vp, i64, i64, i32, i32, i32, i32, i32, vp, vp, vp,
+                                          i32, i32, i32, i32, i32, vp, i64, i64, vp, vp]
     lib.ha_encode_pack_prefill.restype = i32
     lib.ha_encode_pack_prefill.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32,
                                            vp, i64, i64, i32, vp, vp]
@@ -203,6 +206,25 @@ def encode_step(k_new: torch.Tensor, q3: torch.Tensor, wk: torch.Tensor, wq: tor
                               _DTYPE[k_new.dtype], B, Hkv, wk.shape[0], H, 1, _ptr(wk), _ptr(wq), n_layers, d, int_dim, final_dim,
                               arith, _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), pos0, _ptr(pos_dev), _ptr(qcodes),
                               _stream(q3)), "ha_encode_step")
+
+
+def encode_step_cached(k_cache: torch.Tensor, q3: torch.Tensor, wk: torch.Tensor, wq: torch.Tensor, n_layers: int, int_dim: int,
+                       final_dim: int, kcodes: torch.Tensor, qcodes: torch.Tensor, seq_lens: torch.Tensor,
+                       arith: int = HA_ARITH_F32) -> None:
+    """`encode_step` for lengths on the device: the newest key of sequence b is row seq_lens[b] - 1 of k_cache [B, Hkv, S_cap, d],
+    its code goes to the same position of kcodes; q3 [B, H, d] -> qcodes [B, H, W]."""
+    _require_cuda(k_cache, q3, wk, wq, kcodes, qcodes, seq_lens)
+    lib = load_library()
+    B, Hkv, _, d = k_cache.shape
+    H = q3.shape[1]
+    assert k_cache.stride(3) == 1 and q3.stride(2) == 1 and k_cache.dtype == q3.dtype
+    assert kcodes.stride(3) == 1 and kcodes.stride(2) == kcodes.shape[3] and qcodes.is_contiguous()
+    assert kcodes.dtype == torch.int32 and qcodes.dtype == torch.int32 and qcodes.numel() == B * H * (final_dim // 32)
+    assert seq_lens.dtype == torch.int32 and seq_lens.numel() == B and seq_lens.is_contiguous()
+    _check(lib.ha_encode_step_cached(_ptr(k_cache), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), _ptr(q3), q3.stride(0),
+                                     q3.stride(1), _DTYPE[k_cache.dtype], B, Hkv, wk.shape[0], H, _ptr(seq_lens), _ptr(wk), _ptr(wq),
+                                     n_layers, d, int_dim, final_dim, arith, _ptr(kcodes), kcodes.stride(0), kcodes.stride(1),
+                                     _ptr(qcodes), _stream(q3)), "ha_encode_step_cached")
 
 
 def encode_pack_prefill(x: torch.Tensor, weights_bf16: torch.Tensor, n_layers: int, int_dim: int, final_dim: int,

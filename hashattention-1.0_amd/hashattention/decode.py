@@ -170,11 +170,9 @@ class HashDecodeLayer:
                              self.final_dim, self.codes, self.qcodes, pos0=seq_len - 1, arith=self.arith)
             self.n_cached = seq_len
         else:
-            # ragged: the new key of sequence b sits at seq_lens[b] - 1
-            pos = (seq_lens - 1).to(torch.int32)
-            newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, self.Hkv, 1, self.d).long())
-            _ops.encode_step(newk, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
-                             self.qcodes, pos_dev=pos, arith=self.arith)
+            # ragged: the new key of sequence b sits at seq_lens[b] - 1 and is read from the cache in place
+            _ops.encode_step_cached(k_cache, q3, self.wk, self.wq, self.num_layers, self.int_dim, self.final_dim, self.codes,
+                                    self.qcodes, seq_lens, arith=self.arith)
         return self._select_attend(q3, k_cache, v_cache, seq_len, out, seq_lens, main, attn_mask)
 
     def _select_attend(self, q3, k_cache, v_cache, seq_len, out, seq_lens, main=None, attn_mask=None):

@@ -107,6 +107,19 @@ int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, in
                    uint32_t *qcodes, void *stream);
 
 /*
+ * ha_encode_step for a batch whose lengths live on the device: the newest key of sequence b is read from the
+ * cache itself, row seq_lens[b] - 1 of k_cache [B, Hkv, ., head_dim] (strides k_stride_{b,h,s}), and its code is
+ * written to the same position of the bit-cache; no host-side gather of the new rows.  A sequence of length 0
+ * writes nothing.  Same reference lines as ha_encode_step (hashattention_llama.py:411-414).
+ */
+int ha_encode_step_cached(const void *k_cache, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                          const void *q, int64_t q_stride_b, int64_t q_stride_h, int x_dtype,
+                          int B, int Hkv, int Hc, int H, const int32_t *seq_lens,
+                          const float *weights_k, const float *weights_q,
+                          int n_layers, int head_dim, int int_dim, int final_dim, int arith,
+                          uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream);
+
+/*
  * Bulk (prefill) encode on the matrix cores: the same mapping as ha_encode_pack in HA_ARITH_BF16
  * arithmetic, computed as three chained bf16 MFMA GEMMs per 128-token tile.  x must be bf16,
  * head_dim == int_dim == 128.  `weights_bf16` is the blob of ha_usa_packed_floats() elements per

@@ -134,6 +134,16 @@ def test_arguments_are_validated_before_any_device_work(lib):
                                   a["idim"], a["fd"], a["ar"], a["codes"], a["csb"], a["csh"], a["pos0"], a["pd"], a["lg"], a["st"])
 
     assert enc(w=null) == HA_ERR_NULL
+
+    def enc_cached(**kw):
+        a = dict(k=p, ss=128, q=p, lens=p, H=4, hd=128, dt=_ops.HA_BF16)
+        a.update(kw)
+        return lib.ha_encode_step_cached(a["k"], 128000, 64000, a["ss"], a["q"], 512, 128, a["dt"], 1, 2, 2, a["H"], a["lens"], p, p, 3,
+                                         a["hd"], 128, 32, 0, p, 4000, 1000, p, null)
+
+    assert enc_cached(k=null) == HA_ERR_NULL and enc_cached(lens=null) == HA_ERR_NULL and enc_cached(q=null) == HA_ERR_NULL
+    assert enc_cached(ss=64) == HA_ERR_SHAPE and enc_cached(H=0) == HA_ERR_SHAPE and enc_cached(dt=7) == HA_ERR_DTYPE
+    assert enc_cached() == HA_ERR_NODEV
     assert enc(fd=48) == HA_ERR_SHAPE and enc(nl=4) == HA_ERR_SHAPE and enc(nh=3) == HA_ERR_SHAPE and enc(hd=300) == HA_ERR_SHAPE
     assert enc(dt=5) == HA_ERR_DTYPE and enc(ar=2) == HA_ERR_DTYPE
     assert lib.ha_encode_pack_prefill(p, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 64, 32, p, 64, 16, 0, null, null) == HA_ERR_SHAPE

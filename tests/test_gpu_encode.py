@@ -121,3 +121,36 @@ def test_encode_step_equals_two_encode_packs():
         torch.cuda.synchronize()
         assert torch.equal(a, b) and torch.equal(qa.view(5, 8, 1), qb)
         assert int((a != 7).sum()) == 5 * 2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_encode_step_cached_reads_the_new_keys_in_place(dtype):
+    # lengths on the device: the key of sequence b is read from cache row seq_lens[b] - 1; the same bits as a gather of those
+    # rows followed by ha_encode_step, and nothing else in the bit-cache is touched.  A length of 0 writes nothing.
+    print(f"\n[case] encode_step_cached {dtype}", flush=True)
+    g = torch.Generator().manual_seed(31)
+    B, H, Hkv, Hc, cap, W = 5, 8, 2, 4, 300, 1
+    w = small_workload(batch=1, seq_lens=[64], seed=33)
+    p = make_problem(w)
+    k_layers = (p.usa.k * 4)[:Hc]
+    q_layers = (p.usa.q * 4)[:H]
+    wk, wq = _ops.pack_usa_weights(k_layers, DEV), _ops.pack_usa_weights(q_layers, DEV)
+    k_cache = torch.randn(B, Hkv, cap, 128, generator=g).to(dtype).to(DEV)
+    q3 = torch.randn(B, H, 128, generator=g).to(dtype).to(DEV)
+    lens = torch.tensor([300, 1, 0, 137, 42], dtype=torch.int32, device=DEV)
+    arith = _ops.HA_ARITH_BF16 if dtype == torch.bfloat16 else _ops.HA_ARITH_F32
+    got = torch.full((B, Hc, cap, W), 777, dtype=torch.int32, device=DEV)
+    got_q = torch.zeros(B, H, W, dtype=torch.int32, device=DEV)
+    _ops.encode_step_cached(k_cache, q3, wk, wq, 3, 128, 32, got, got_q, lens, arith=arith)
+    want = torch.full((B, Hc, cap, W), 777, dtype=torch.int32, device=DEV)
+    want_q = torch.zeros(B, H, W, dtype=torch.int32, device=DEV)
+    live = [0, 1, 3, 4]
+    pos = (lens - 1).clamp(min=0)
+    newk = torch.gather(k_cache, 2, pos.view(-1, 1, 1, 1).expand(-1, Hkv, 1, 128).long())
+    _ops.encode_step(newk, q3, wk, wq, 3, 128, 32, want, want_q, pos_dev=pos.to(torch.int32), arith=arith)
+    torch.cuda.synchronize()
+    assert torch.equal(got_q, want_q)
+    assert torch.equal(got[live], want[live])
+    assert (got[2] == 777).all()                                   # the empty sequence wrote nothing
+    touched = (got != 777).sum().item()
+    assert touched <= len(live) * Hc * W and touched >= len(live) * Hc * W - 2       # a code may happen to equal the filler

@@ -28,7 +28,8 @@ from .synthetic import UsaWeights, layer_dims
 class LlamaShapedDecoder:
     def __init__(self, n_layers=32, hidden=4096, ffn=14336, n_heads=32, n_kv_heads=8, head_dim=128, vocab=128256,
                  rope_theta=500000.0, rms_eps=1e-5, n_code_heads=8, lth_num_layers=3, lth_int_dim=128, lth_final_dim=32,
-                 init_budget=128, recent_budget=128, heavy_budget=1.0 / 32, dtype=torch.bfloat16, device="cuda:0", seed=0):
+                 init_budget=128, recent_budget=128, heavy_budget=1.0 / 32, dtype=torch.bfloat16, device="cuda:0", seed=0,
+                 random_init=True):
         self.L, self.hidden, self.ffn, self.H, self.Hkv, self.d, self.vocab = n_layers, hidden, ffn, n_heads, n_kv_heads, head_dim, vocab
         self.theta, self.eps, self.dtype, self.device = rope_theta, rms_eps, dtype, torch.device(device)
         self.Hc = n_code_heads
@@ -40,6 +41,8 @@ class LlamaShapedDecoder:
         g = torch.Generator(device=device).manual_seed(seed)
 
         def w(*shape, fan_in):
+            if not random_init:                    # the weights come from a model (`from_hf`): no 16 GB of noise first
+                return torch.empty(0, dtype=dtype, device=device)
             return (torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * fan_in ** -0.5).to(dtype)
 
         q_out, kv_out = n_heads * head_dim, n_kv_heads * head_dim
@@ -56,7 +59,7 @@ class LlamaShapedDecoder:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.B = self.S_cap = self.seq_len = 0
-        self._gen_graph = None
+        self._gen_graph = self._gen_logits = None
         inv = 1.0 / (rope_theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
         self.inv_freq = inv
 
@@ -99,7 +102,7 @@ class LlamaShapedDecoder:
         self.tok_dev = torch.zeros(B, dtype=torch.int64, device=self.device)
         self.pos_dev = torch.zeros(B, dtype=torch.int32, device=self.device)
         self.len_dev = torch.ones(B, dtype=torch.int32, device=self.device)
-        self._gen_graph = None
+        self._gen_graph = self._gen_logits = None
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
@@ -128,7 +131,10 @@ class LlamaShapedDecoder:
         for l in range(self.L):
             self.k_cache[l][:, :, :S] = keys[l]
             self.v_cache[l][:, :, :S] = values[l]
-            self.hash[l].encode_keys(self.k_cache[l][:, :, :S], pos0=0)
+            # as the patched layer hashes a prefilled cache: the MFMA encoder for a bf16 hash, the exact kernel otherwise
+            self.hash[l].encode_keys(self.k_cache[l][:, :, :S], pos0=0,
+                                     use_mfma=self.dtype == torch.bfloat16 and self.hash[l].arith == _ops.HA_ARITH_BF16
+                                     and self.hash[l].wk_bf16 is not None)
             self.hash[l].n_cached = S
         self.seq_len = S
 
@@ -223,13 +229,14 @@ class LlamaShapedDecoder:
                 main.wait_stream(side)
                 self._gen_graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(self._gen_graph):
-                    step()
+                    self._gen_logits = step()      # the graph's own output buffer: every replay leaves its logits there
             run = self._gen_graph.replay
         else:
-            run = step
+            def run():
+                self._gen_logits = step()
         for i in range(n_new):
             run()
-            torch.argmax(self.logits, dim=-1, out=self.tok_dev)
+            torch.argmax(self._gen_logits, dim=-1, out=self.tok_dev)
             out[:, i].copy_(self.tok_dev)
             self.pos_dev.add_(1)
             self.len_dev.add_(1)
@@ -239,6 +246,42 @@ class LlamaShapedDecoder:
         return out
 
     # ------------------------------------------------------------------ weights from a transformers Llama
+    @classmethod
+    def from_hf(cls, model, usa_modules, batch: int, cache_len: int, dtype=torch.bfloat16, device="cuda:0") -> "LlamaShapedDecoder":
+        """The decoder for a `transformers` LlamaForCausalLM and the hash modules `load_usa` returned for it (one `USA` per
+        layer): same weights, budgets from the model's config (`init_budget`, `heavy_budget`, `recent_budget`, as
+        `convert_usa` reads them), caches for `batch` sequences of up to `cache_len` tokens.  Follow with
+        `prefill_from_hf` and `generate`."""
+        cfg, usa0 = model.config, usa_modules[0]
+        if usa0.rehash_every_step:
+            raise NotImplementedError("the LSH baseline and CENTER re-hash the whole cache every step: use the patched layer")
+        head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
+        dec = cls(n_layers=cfg.num_hidden_layers, hidden=cfg.hidden_size, ffn=cfg.intermediate_size, n_heads=cfg.num_attention_heads,
+                  n_kv_heads=cfg.num_key_value_heads, head_dim=head_dim, vocab=cfg.vocab_size, rms_eps=cfg.rms_norm_eps,
+                  n_code_heads=usa0.num_heads, lth_num_layers=usa0.num_layers, lth_int_dim=usa0.int_dim, lth_final_dim=usa0.lth_final_dim,
+                  init_budget=cfg.init_budget, recent_budget=cfg.recent_budget, heavy_budget=cfg.heavy_budget, dtype=dtype,
+                  device=device, random_init=False)
+        dec.load_hf_llama(model)
+        lin = lambda seqs: [[(m.weight.detach().float().cpu(), m.bias.detach().float().cpu()) for m in seq if isinstance(m, torch.nn.Linear)]
+                            for seq in seqs]
+        dec.allocate(batch, cache_len, [UsaWeights(k=lin(u.learning_to_hash_transformation_k), q=lin(u.learning_to_hash_transformation_q))
+                                        for u in usa_modules])
+        return dec
+
+    def prefill_from_hf(self, model, input_ids: torch.Tensor) -> torch.Tensor:
+        """Prefill with the `transformers` model itself (its dense attention: the reference's `q_len > 128` branch,
+        hashattention_llama.py:529-550), take over its KV cache and hash the keys.  Unpadded prompts of equal length,
+        input_ids [B, S].  Returns the first generated token of every sequence [B] (greedy)."""
+        from transformers import DynamicCache
+        if input_ids.shape[0] != self.B or input_ids.shape[1] + 1 > self.S_cap:
+            raise ValueError(f"prompts must be [{self.B}, < {self.S_cap}]")
+        cache = DynamicCache()
+        with torch.no_grad():
+            logits = model(input_ids.to(self.device), past_key_values=cache, use_cache=True).logits[:, -1]
+        self.load_cache([cache.layers[l].keys.to(self.dtype) for l in range(self.L)],
+                        [cache.layers[l].values.to(self.dtype) for l in range(self.L)])
+        return logits.argmax(-1)
+
     def load_hf_llama(self, model) -> None:
         """Copy the weights of a `transformers` LlamaForCausalLM of the same shape (used by the plumbing test)."""
         sd = model.state_dict()

@@ -293,3 +293,32 @@ def test_generate_replays_one_graph_for_successive_tokens(n_heads, batch):
     assert torch.equal(decs[0].k_cache[0][:, :, :ctx + 1], decs[1].k_cache[0][:, :, :ctx + 1])
     with pytest.raises(ValueError):
         decs[1].generate(first, 2000)
+
+
+def test_decoder_from_hf_prefill_and_generate_match_the_patched_model():
+    # the serving path end to end: a transformers Llama + hash modules -> LlamaShapedDecoder.from_hf, prefill by the model
+    # itself, greedy generation by graph replay; against `generate` of the same model patched with convert_usa
+    print("\n[case] decoder from_hf + prefill_from_hf + generate vs patched model.generate", flush=True)
+    torch.manual_seed(2)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=128, vocab_size=512, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5)
+    for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
+                     recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
+        setattr(cfg, k, v)
+    model = LlamaForCausalLM(cfg).bfloat16().float()
+    usa = hl.load_usa(cfg, None)
+    model = hl.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False).float()
+    B, S0, n_new = 2, 200, 8
+    ids = torch.randint(1, cfg.vocab_size, (B, S0), generator=torch.Generator().manual_seed(5)).to(DEV)
+    with torch.no_grad():
+        want = model.generate(input_ids=ids, max_new_tokens=n_new, do_sample=False, use_cache=True, pad_token_id=0)[:, S0:].cpu()
+    hl.reset_usa(model)
+    dec = LlamaShapedDecoder.from_hf(model, usa, batch=B, cache_len=256, dtype=torch.float32, device=DEV)
+    assert dec.Hc == 4 and dec.budgets == (8, 8, 0.125) and dec.embed.shape == (512, 512)
+    with torch.no_grad():
+        first = dec.prefill_from_hf(model, ids)
+        rest = dec.generate(first, n_new - 1)
+    got = torch.cat([first[:, None], rest], dim=1).cpu()
+    print("  tokens:", got.tolist(), flush=True)
+    assert torch.equal(got, want)
+    assert dec.seq_len == S0 + n_new - 1

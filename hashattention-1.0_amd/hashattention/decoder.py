@@ -285,6 +285,7 @@ class LlamaShapedDecoder:
     def load_hf_llama(self, model) -> None:
         """Copy the weights of a `transformers` LlamaForCausalLM of the same shape (used by the plumbing test)."""
         sd = model.state_dict()
+        self._gen_graph = self._gen_logits = None       # a captured generation step names the old weight buffers
         cast = lambda t: t.detach().to(self.device, self.dtype)
         self.embed = cast(sd["model.embed_tokens.weight"])
         self.lm_head = cast(sd["lm_head.weight"])

@@ -59,6 +59,12 @@ struct EncArgs {
     EncRope rope;
 };
 
+// Position of W[o][k] (k = input, o = output) inside a layer's block of the packed blob: inputs in groups of four,
+// [in / 4][out][4], when the layer has a multiple of 16 inputs; plain W^T [in][out] otherwise.
+__device__ __forceinline__ int64_t weight_index(int in, int out, int k, int o) {
+    return (in & 15) == 0 ? ((int64_t)(k >> 2) * out + o) * 4 + (k & 3) : (int64_t)k * out + o;
+}
+
 // NL_/DIN_/DINT_/DOUT_ fix the MLP shape at compile time (0 = read it from the arguments).  The usual
 // shapes (128 -> 128 [-> 128] -> 32|64) are instantiated: with constant trip counts the weight fetch is
 // 72 plain loads and the kernel is a few hundred instructions, which matters because a decode step is
@@ -170,8 +176,22 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
         const bool active = fits && tid < l_out[l] * kSeg;
         const int out = l < n_layers ? l_out[l] : 1, per = l < n_layers ? l_in[l] / kSeg : 0;
         const int o = tid % out, seg = tid / out;
+        if ((l_in[l] & 15) == 0) {
+            // inputs in groups of four (ha_usa_weight_index): the 64 lanes of a wave, consecutive outputs of one
+            // segment, fetch 1 KiB of consecutive memory per request - a quarter of the requests of a dword walk
+            const float4 *w4 = reinterpret_cast<const float4 *>(wl[l]) + (int64_t)(seg * per / 4) * out + o;
 #pragma unroll
-        for (int i = 0; i < kMaxPerSeg; ++i) wreg[l][i] = (active && i < per) ? wl[l][(int64_t)(seg * per + i) * out + o] : 0.f;
+            for (int i4 = 0; i4 < kMaxPerSeg / 4; ++i4) {
+                const float4 v = (active && 4 * i4 < per) ? w4[(int64_t)i4 * out] : float4{0.f, 0.f, 0.f, 0.f};
+                wreg[l][4 * i4 + 0] = v.x;
+                wreg[l][4 * i4 + 1] = v.y;
+                wreg[l][4 * i4 + 2] = v.z;
+                wreg[l][4 * i4 + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kMaxPerSeg; ++i) wreg[l][i] = (active && i < per) ? wl[l][(int64_t)(seg * per + i) * out + o] : 0.f;
+        }
     }
 #pragma unroll
     for (int it = 0; it < kXIter; ++it) {
@@ -228,7 +248,7 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) p[r] = 0.f;
                 for (int i = 0; i < per; ++i) {
-                    const float wv = Wt[(int64_t)(seg * per + i) * out + o];
+                    const float wv = Wt[weight_index(in, out, seg * per + i, o)];
 #pragma unroll
                     for (int r = 0; r < kRows; ++r) p[r] = fmaf(s_act[cur][r][seg * per + i], wv, p[r]);
                 }
@@ -282,7 +302,7 @@ int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const
     HA_REQUIRE(final_dim == 32 || final_dim == 64, HA_ERR_BAD_SHAPE, "final_dim=%d, must be 32 or 64", final_dim);
     HA_REQUIRE(pos0 >= 0, HA_ERR_BAD_SHAPE, "pos0 must be non-negative");
     HA_REQUIRE(c_sh >= 0 && c_sb >= 0, HA_ERR_BAD_SHAPE, "negative code stride");
-    HA_REQUIRE(ha_aligned(codes, 4) && ha_aligned(weights, 4), HA_ERR_MISALIGNED, "codes/weights misaligned");
+    HA_REQUIRE(ha_aligned(codes, 4) && ha_aligned(weights, 16), HA_ERR_MISALIGNED, "codes must be 4-byte, weights 16-byte aligned");
     return HA_OK;
 }
 

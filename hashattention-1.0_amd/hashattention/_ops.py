@@ -145,12 +145,17 @@ def workspace(nbytes: int, device) -> torch.Tensor:
 # ------------------------------------------------------------------------------------------ encode
 
 def pack_usa_weights(layers_per_head, device=None) -> torch.Tensor:
-    """[[(W [out,in], b [out]), ...] per head] -> fp32 blob [n_heads, per_head]: W^T [in][out] then b, per layer."""
+    """[[(W [out,in], b [out]), ...] per head] -> fp32 blob [n_heads, per_head]: per layer W then b.  W is stored
+    transposed with its inputs in groups of four, [in / 4][out][4], when `in` is a multiple of 16 (the 128-bit
+    coalesced fetch of the encode kernels), as plain W^T [in][out] otherwise."""
     blobs = []
     for layers in layers_per_head:
         parts = []
         for (W, b) in layers:
-            parts.append(W.detach().float().t().contiguous().reshape(-1))
+            wt = W.detach().float().t().contiguous()                      # [in, out]
+            if wt.shape[0] % 16 == 0:
+                wt = wt.view(wt.shape[0] // 4, 4, wt.shape[1]).permute(0, 2, 1).contiguous()
+            parts.append(wt.reshape(-1))
             parts.append(b.detach().float().reshape(-1))
         blobs.append(torch.cat(parts))
     out = torch.stack(blobs).contiguous()

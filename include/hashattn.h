@@ -65,9 +65,12 @@ int ha_device_count(void);
 /* ---------------------------------------------------------------------------------------------
  * Hash-MLP weights.  One head's MLP is 1-3 Linear layers head_dim -> int_dim (-> int_dim) ->
  * final_dim with SiLU between them (USA.__init__, hashattention_llama.py:99-128).  The kernels read
- * a packed fp32 blob per head: for each layer, W transposed to [in][out], then bias [out].
+ * a packed fp32 blob per head, 16-byte aligned: for each layer the weights, then bias [out].  A layer
+ * with a multiple of 16 inputs stores W transposed with its inputs in groups of four, [in / 4][out][4]:
+ * W[o][k] sits at ((k / 4) * out + o) * 4 + k % 4, so that the lanes of a wave (consecutive outputs) fetch
+ * consecutive 16-byte pieces; any other layer stores plain W^T [in][out] (W[o][k] at k * out + o).
  * ha_usa_packed_floats() is the blob length of ONE head; heads are concatenated.
- * Limits: head_dim, int_dim <= 256; final_dim in {32, 64}.
+ * Limits: head_dim, int_dim <= 256 and multiples of 4; final_dim in {32, 64}.
  */
 int64_t ha_usa_packed_floats(int n_layers, int head_dim, int int_dim, int final_dim);
 

@@ -59,6 +59,7 @@ class LlamaShapedDecoder:
         self.k_cache: List[torch.Tensor] = []
         self.v_cache: List[torch.Tensor] = []
         self.B = self.S_cap = self.seq_len = 0
+        self.lengths = None      # per-sequence lengths of a ragged batch (host list); None: every sequence holds seq_len tokens
         self._gen_graph = self._gen_logits = None
         inv = 1.0 / (rope_theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
         self.inv_freq = inv
@@ -77,7 +78,7 @@ class LlamaShapedDecoder:
         return out
 
     def allocate(self, B: int, S_cap: int, usa_per_layer: Optional[List[UsaWeights]] = None) -> None:
-        self.B, self.S_cap, self.seq_len = B, S_cap, 0
+        self.B, self.S_cap, self.seq_len, self.lengths = B, S_cap, 0, None
         nl, idim, fdim = self.usa_shape
         init, recent, heavy = self.budgets
         arith = _ops.HA_ARITH_BF16 if self.dtype == torch.bfloat16 else _ops.HA_ARITH_F32
@@ -125,9 +126,18 @@ class LlamaShapedDecoder:
         self.seq_len = seq_len
         return sum(ms) / len(ms)
 
-    def load_cache(self, keys: List[torch.Tensor], values: List[torch.Tensor]) -> None:
-        """Take over a prefilled cache: per layer keys/values [B, Hkv, S, d] (rotary already applied to the keys)."""
+    def load_cache(self, keys: List[torch.Tensor], values: List[torch.Tensor], lengths: Optional[List[int]] = None) -> None:
+        """Take over a prefilled cache: per layer keys/values [B, Hkv, S, d] (rotary already applied to the keys).
+        `lengths`: tokens of every sequence when the batch is ragged (right-padded to S); what lies beyond a sequence's
+        length is never read and is overwritten as the sequence grows.  A ragged batch decodes through `generate` only."""
         S = keys[0].shape[2]
+        if lengths is not None:
+            lengths = [int(n) for n in lengths]
+            if len(lengths) != self.B or min(lengths) < 1 or max(lengths) > S:
+                raise ValueError(f"lengths must be {self.B} values in 1..{S}")
+            if len(set(lengths)) == 1:       # equal lengths after all: a uniform batch of that length
+                keys, values = [k[:, :, :lengths[0]] for k in keys], [v[:, :, :lengths[0]] for v in values]
+                S, lengths = lengths[0], None
         for l in range(self.L):
             self.k_cache[l][:, :, :S] = keys[l]
             self.v_cache[l][:, :, :S] = values[l]
@@ -136,7 +146,8 @@ class LlamaShapedDecoder:
                                      use_mfma=self.dtype == torch.bfloat16 and self.hash[l].arith == _ops.HA_ARITH_BF16
                                      and self.hash[l].wk_bf16 is not None)
             self.hash[l].n_cached = S
-        self.seq_len = S
+        self.seq_len = S if lengths is None else max(lengths)
+        self.lengths = lengths
 
     # ------------------------------------------------------------------ one decode step
     def decode_step(self, tokens: torch.Tensor, advance: bool = True, dense: bool = False, device_pos: bool = False) -> torch.Tensor:
@@ -152,6 +163,8 @@ class LlamaShapedDecoder:
         down GEMM with the residual folded in (addmm).  Other dtypes and batches: the same steps as library calls plus
         ha_swiglu."""
         B, H, Hkv, d = self.B, self.H, self.Hkv, self.d
+        if self.lengths is not None and not device_pos:
+            raise RuntimeError("a ragged batch keeps its positions on the device: use generate()")
         pos = self.seq_len
         S = pos + 1
         x = self.embed[tokens]                                            # [B, hidden]
@@ -213,8 +226,11 @@ class LlamaShapedDecoder:
         if self.seq_len + n_new > self.S_cap:
             raise ValueError(f"{n_new} more tokens do not fit the cache ({self.seq_len} of {self.S_cap} used)")
         self.tok_dev.copy_(tokens)
-        self.pos_dev.fill_(self.seq_len)
-        self.len_dev.fill_(self.seq_len + 1)
+        if self.lengths is None:
+            self.pos_dev.fill_(self.seq_len)
+        else:       # ragged: every sequence continues at its own length
+            self.pos_dev.copy_(torch.tensor(self.lengths, dtype=torch.int32))
+        torch.add(self.pos_dev, 1, out=self.len_dev)
         out = torch.empty(B, n_new, dtype=torch.int64, device=self.device)
         step = lambda: self.decode_step(self.tok_dev, device_pos=True)
         if use_graph:
@@ -241,6 +257,8 @@ class LlamaShapedDecoder:
             self.pos_dev.add_(1)
             self.len_dev.add_(1)
         self.seq_len += n_new
+        if self.lengths is not None:
+            self.lengths = [n + n_new for n in self.lengths]
         for hl in self.hash:
             hl.n_cached = self.seq_len
         return out
@@ -268,19 +286,32 @@ class LlamaShapedDecoder:
                                         for u in usa_modules])
         return dec
 
-    def prefill_from_hf(self, model, input_ids: torch.Tensor) -> torch.Tensor:
+    def prefill_from_hf(self, model, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Prefill with the `transformers` model itself (its dense attention: the reference's `q_len > 128` branch,
-        hashattention_llama.py:529-550), take over its KV cache and hash the keys.  Unpadded prompts of equal length,
-        input_ids [B, S].  Returns the first generated token of every sequence [B] (greedy)."""
+        hashattention_llama.py:529-550), take over its KV cache and hash the keys.  input_ids [B, S]; prompts of different
+        lengths are RIGHT-padded and described by attention_mask [B, S] (ones, then zeros): every sequence then continues
+        at its own length.  Returns the first generated token of every sequence [B] (greedy)."""
         from transformers import DynamicCache
         if input_ids.shape[0] != self.B or input_ids.shape[1] + 1 > self.S_cap:
             raise ValueError(f"prompts must be [{self.B}, < {self.S_cap}]")
+        lengths = None
+        if attention_mask is not None:
+            am = attention_mask.to(torch.long).cpu()
+            lengths = am.sum(dim=1).tolist()
+            ramp = torch.arange(am.shape[1])[None, :] < am.sum(dim=1, keepdim=True)
+            if not torch.equal(am.bool(), ramp) or min(lengths) < 1:
+                raise ValueError("attention_mask must be ones followed by zeros in every row (right padding), at least one token each")
+            attention_mask = attention_mask.to(self.device)
         cache = DynamicCache()
         with torch.no_grad():
-            logits = model(input_ids.to(self.device), past_key_values=cache, use_cache=True).logits[:, -1]
+            logits = model(input_ids.to(self.device), attention_mask=attention_mask, past_key_values=cache, use_cache=True).logits
+        if lengths is None:
+            last = logits[:, -1]
+        else:
+            last = logits[torch.arange(self.B, device=logits.device), torch.tensor(lengths, device=logits.device) - 1]
         self.load_cache([cache.layers[l].keys.to(self.dtype) for l in range(self.L)],
-                        [cache.layers[l].values.to(self.dtype) for l in range(self.L)])
-        return logits.argmax(-1)
+                        [cache.layers[l].values.to(self.dtype) for l in range(self.L)], lengths)
+        return last.argmax(-1)
 
     def load_hf_llama(self, model) -> None:
         """Copy the weights of a `transformers` LlamaForCausalLM of the same shape (used by the plumbing test)."""

@@ -322,3 +322,39 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model():
     print("  tokens:", got.tolist(), flush=True)
     assert torch.equal(got, want)
     assert dec.seq_len == S0 + n_new - 1
+
+
+def test_ragged_prompts_through_the_decoder_generation_loop():
+    # prompts of different lengths, right-padded: every sequence continues at its own length (positions and lengths on the
+    # device).  Against the same prompts run one by one, unpadded.
+    print("\n[case] decoder generate, ragged prompts", flush=True)
+    torch.manual_seed(4)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=128, vocab_size=512, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5)
+    for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
+                     recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
+        setattr(cfg, k, v)
+    model = LlamaForCausalLM(cfg).float().to(DEV)
+    usa = hl.load_usa(cfg, None).float()
+    lens, S0, n_new = [200, 141, 173], 200, 6
+    ids = torch.randint(1, cfg.vocab_size, (3, S0), generator=torch.Generator().manual_seed(6)).to(DEV)
+    am = (torch.arange(S0)[None, :] < torch.tensor(lens)[:, None]).long().to(DEV)
+    dec = LlamaShapedDecoder.from_hf(model, usa, batch=3, cache_len=256, dtype=torch.float32, device=DEV)
+    with torch.no_grad():
+        first = dec.prefill_from_hf(model, ids, am)
+        assert dec.lengths == lens and dec.seq_len == 200
+        with pytest.raises(RuntimeError):
+            dec.decode_step(first)
+        rest = dec.generate(first, n_new)
+    got = torch.cat([first[:, None], rest], dim=1).cpu()
+    assert dec.lengths == [n + n_new for n in lens]
+    one = LlamaShapedDecoder.from_hf(model, usa, batch=1, cache_len=256, dtype=torch.float32, device=DEV)
+    for b, n in enumerate(lens):
+        with torch.no_grad():
+            f = one.prefill_from_hf(model, ids[b:b + 1, :n])
+            r = one.generate(f, n_new)
+        want = torch.cat([f[:, None], r], dim=1).cpu()[0]
+        print(f"  sequence {b} ({n} tokens): {got[b].tolist()}", flush=True)
+        assert torch.equal(got[b], want), (b, got[b], want)
+    with pytest.raises(ValueError):
+        dec.prefill_from_hf(model, ids, torch.flip(am, dims=[1]))            # left padding is not a ragged batch

@@ -1006,7 +1006,8 @@ int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
                                    int mode) {
     if (B <= 0 || H <= 0 || Hc <= 0 || max_seq_len <= 0 || (W != 1 && W != 2) || H % Hc != 0) return 0;
     if (mode != HA_SELECT_SIMPLE || init_budget < 0 || recent_budget < 0 || heavy_budget < 0.0) return 0;
-    const double heavy = heavy_budget > 1.0 ? heavy_budget : (double)max_seq_len * heavy_budget;
+    // the heavy count as the selection takes it: truncated (int(k) above 1, int(S * fraction) otherwise)
+    const double heavy = std::floor(heavy_budget > 1.0 ? heavy_budget : (double)max_seq_len * heavy_budget);
     return (double)init_budget + (double)recent_budget + heavy <= (double)kFusedListCap ? 1 : 0;
 }
 

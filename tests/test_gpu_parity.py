@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 import torch
 
+from hashattention import _ops
 from tests.parity_util import run_decode_case, small_workload
 
 pytestmark = pytest.mark.gpu
@@ -205,3 +206,15 @@ def test_random_shapes_every_stage_against_the_oracle(block):
         print(f"\n[case] {w.name}: B={w.batch} H={w.n_q_heads}/{w.n_kv_heads}/{w.n_code_heads} S={w.seq_lens} bits={w.lth_final_dim} "
               f"init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget} {w.dtype}", flush=True)
         run_decode_case(w, check_encode=False, check_dense=False)
+
+
+@pytest.mark.parametrize("heavy,fused", [(8000.5, True), (8001.5, False)])
+def test_largest_list_of_the_fused_path(heavy, fused):
+    # the fused launch keeps a row's list in LDS, 8192 entries at most: a selection of exactly that size goes through it
+    # (every stage against the oracle, as in the other cases), one entry more is refused by it and served by the list path
+    print(f"\n[case] list of {int(heavy) + 192} entries", flush=True)
+    w = small_workload(batch=2, seq_lens=[30000, 30000], n_q_heads=4, n_kv_heads=2, n_code_heads=2, init_budget=100, recent_budget=92,
+                       heavy_budget=heavy, seed=91)
+    assert bool(_ops.fused_applies(2, 4, 2, 1, 30000, 100, 92, heavy)) == fused
+    rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
+    assert rep["n_selected"] == int(heavy) + 192 and ("fused_err" in rep) == fused

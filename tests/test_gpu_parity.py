@@ -218,3 +218,18 @@ def test_largest_list_of_the_fused_path(heavy, fused):
     assert bool(_ops.fused_applies(2, 4, 2, 1, 30000, 100, 92, heavy)) == fused
     rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
     assert rep["n_selected"] == int(heavy) + 192 and ("fused_err" in rep) == fused
+
+
+@pytest.mark.parametrize("batch,heads", [(140, 1), (130, 2)])
+def test_ragged_batch_larger_than_the_in_kernel_plan(batch, heads):
+    # the fused launch plans ragged batches of up to 128 sequences inside the kernel; beyond that every row keeps the
+    # pieces the host sized for the longest sequence (with one head per sequence the rows are cut into pieces, with two
+    # they are not).  Every stage against the oracle.
+    print(f"\n[case] ragged batch of {batch} sequences, {heads} head(s)", flush=True)
+    rng = np.random.default_rng(5 + batch)
+    lens = [int(x) for x in rng.integers(700, 5000, batch)]
+    lens[3], lens[7] = 17, 4999                      # one shorter than its windows, one at the top
+    w = small_workload(batch=batch, seq_lens=lens, n_q_heads=heads, n_kv_heads=1, n_code_heads=1, init_budget=16, recent_budget=24,
+                       heavy_budget=0.05, seed=93)
+    rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
+    assert "fused_err" in rep

@@ -154,3 +154,28 @@ def test_encode_step_cached_reads_the_new_keys_in_place(dtype):
     assert (got[2] == 777).all()                                   # the empty sequence wrote nothing
     touched = (got != 777).sum().item()
     assert touched <= len(live) * Hc * W and touched >= len(live) * Hc * W - 2       # a code may happen to equal the filler
+
+
+@pytest.mark.parametrize("int_dim,layers", [(256, 3), (200, 3), (64, 2), (256, 2)])
+def test_generic_mlp_widths_against_the_oracle(int_dim, layers):
+    # hidden widths other than 128: layers wider than 128 outputs stream their weights instead of parking them in
+    # registers, widths that are not multiples of 16 keep the plain weight layout.  fp32 logits against torch, codes exact
+    # wherever a logit is not within round-off of zero
+    print(f"\n[case] hash MLP with hidden width {int_dim}, {layers} layers", flush=True)
+    g = torch.Generator().manual_seed(int_dim + layers)
+    B, Hx, Hn, T, D = 2, 2, 4, 37, 32
+    dims = [(128, int_dim), (int_dim, int_dim), (int_dim, D)] if layers == 3 else [(128, int_dim), (int_dim, D)]
+    heads = [[(torch.randn(o, i, generator=g) * i ** -0.5, torch.randn(o, generator=g) * 0.05) for i, o in dims] for _ in range(Hn)]
+    x = torch.randn(B, Hx, T, 128, generator=g)
+    want = orc.usa_logits(x, heads)                                      # [B, Hn, T, D]
+    w = _ops.pack_usa_weights(heads, DEV)
+    codes = torch.zeros(B, Hn, T, 1, dtype=torch.int32, device=DEV)
+    got = _ops.encode_pack(x.to(DEV), w, layers, int_dim, D, codes, want_logits=True).cpu()
+    torch.cuda.synchronize()
+    err = (got - want).abs().max().item()
+    print(f"  max |logit difference| {err:.2e}", flush=True)
+    assert err < 1e-4
+    want_codes = orc.pack_codes(want).numpy().astype(np.uint32)
+    diff = codes.cpu().numpy().view(np.uint32) ^ want_codes
+    bits = ((diff[..., 0, None] >> np.arange(32, dtype=np.uint32)) & 1).astype(bool)
+    assert (np.abs(want.numpy())[bits] < 1e-4).all()

@@ -218,23 +218,25 @@ def test_linear_skinny_with_swiglu_behind(M, F, K):
         assert (out[:, :F].float() - want.float()).abs().max().item() <= 2 ** -6 * max(1.0, want.float().abs().max().item())
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype,B", [(torch.float32, 5), (torch.bfloat16, 5), (torch.float16, 5), (torch.bfloat16, 40), (torch.float32, 100)])
 @pytest.mark.parametrize("code_heads", ["kv", "q"])
-def test_rope_encode_step_equals_rope_append_then_encode_step(dtype, code_heads):
-    # one launch against the two it replaces: rotated query, both caches and both code buffers bit for bit
-    print(f"\n[case] rope_encode_step {dtype} code heads per {code_heads} head", flush=True)
+def test_rope_encode_step_equals_rope_append_then_encode_step(dtype, B, code_heads):
+    # one launch against the two it replaces: rotated query, both caches and both code buffers bit for bit.  5, 40 and 100
+    # sequences: one, two and four rows per workgroup of the encode launch
+    print(f"\n[case] rope_encode_step {dtype} B={B} code heads per {code_heads} head", flush=True)
     from hashattention import _ops
     from hashattention.synthetic import layer_dims
     g = torch.Generator(device=DEV).manual_seed(11)
     gc = torch.Generator().manual_seed(12)
-    B, H, Hkv, d, cap = 5, 8, 2, 128, 50
+    H, Hkv, d, cap = 8, 2, 128, 50
     Hc = Hkv if code_heads == "kv" else H
     heads = lambda n: [[(torch.randn(fo, fi, generator=gc) * fi ** -0.5, torch.randn(fo, generator=gc) * 0.01)
                         for fi, fo in layer_dims(d, 128, 32, 3)] for _ in range(n)]
     wk, wq = _ops.pack_usa_weights(heads(Hc), DEV), _ops.pack_usa_weights(heads(H), DEV)
     qkv = torch.randn(B, (H + 2 * Hkv) * d + 32, generator=g, device=DEV).to(dtype)[:, :(H + 2 * Hkv) * d]
     inv_freq = (1.0 / (500000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
-    for pos, pos_dev in ((17, None), (0, torch.tensor([3, 49, 0, 21, 8], dtype=torch.int32, device=DEV))):
+    some = torch.tensor([3, 49, 0, 21, 8] + [int(x) for x in torch.randint(0, cap, (B - 5,), generator=gc)], dtype=torch.int32, device=DEV)
+    for pos, pos_dev in ((17, None), (0, some)):
         outs = []
         for fused in (False, True):
             k_cache = torch.zeros(B, Hkv, cap, d, dtype=dtype, device=DEV)

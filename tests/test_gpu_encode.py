@@ -179,3 +179,30 @@ def test_generic_mlp_widths_against_the_oracle(int_dim, layers):
     diff = codes.cpu().numpy().view(np.uint32) ^ want_codes
     bits = ((diff[..., 0, None] >> np.arange(32, dtype=np.uint32)) & 1).astype(bool)
     assert (np.abs(want.numpy())[bits] < 1e-4).all()
+
+
+@pytest.mark.parametrize("B", [3, 20, 60])
+def test_encode_step_rows_per_workgroup(B):
+    # 3, 20 and 60 sequences: the step's encode launch runs one, two and four rows per workgroup; codes of the new keys and
+    # of the queries against the oracle (bits may differ only where a logit is within round-off of zero)
+    print(f"\n[case] encode_step, {B} sequences", flush=True)
+    from tests.parity_util import compare_codes
+    g = torch.Generator().manual_seed(50 + B)
+    H, Hkv, Hc = 8, 2, 2
+    w = small_workload(batch=1, seq_lens=[64], seed=51)
+    p = make_problem(w)
+    k_layers, q_layers = (p.usa.k * 4)[:Hc], (p.usa.q * 4)[:H]
+    wk, wq = _ops.pack_usa_weights(k_layers, DEV), _ops.pack_usa_weights(q_layers, DEV)
+    k_new = torch.randn(B, Hkv, 1, 128, generator=g)
+    q = torch.randn(B, H, 1, 128, generator=g)
+    kcodes = torch.zeros(B, Hc, 8, 1, dtype=torch.int32, device=DEV)
+    qcodes = torch.zeros(B, H, 1, dtype=torch.int32, device=DEV)
+    _ops.encode_step(k_new.to(DEV), q[:, :, 0].to(DEV), wk, wq, 3, 128, 32, kcodes, qcodes, pos0=5)
+    torch.cuda.synchronize()
+    kl, ql = orc.usa_logits(k_new, k_layers), orc.usa_logits(q, q_layers)
+    want_k = orc.pack_codes(kl).numpy().astype(np.uint32)            # [B, Hc, 1, 1]
+    want_q = orc.pack_codes(ql).numpy().astype(np.uint32)            # [B, H, 1, 1]
+    nk = compare_codes("new keys", kcodes[:, :, 5:6].cpu().numpy().view(np.uint32), want_k, kl.numpy())
+    nq = compare_codes("queries", qcodes.view(B, H, 1, 1).cpu().numpy().view(np.uint32), want_q, ql.numpy())
+    print(f"  bits differing at near-zero logits: keys {nk}, queries {nq}", flush=True)
+    assert (kcodes[:, :, :5] == 0).all() and (kcodes[:, :, 6:] == 0).all()

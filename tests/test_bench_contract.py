@@ -1,0 +1,37 @@
+"""The benchmark's command-line contract: more than one GPU is refused with a message (CPU), and one short run prints
+ONE JSON line carrying the agreed keys, the roofline of the dominant kernel and the CPU baseline (GPU)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+@pytest.mark.gpu
+def test_one_json_line_with_roofline_and_cpu_baseline():
+    print("\n[case] bench.py --steps 20 --warmup 3", flush=True)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "3"], capture_output=True, text=True,
+                       timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 20 and d["warmup"] == 3 and d["vs_baseline"] is None and d["higher_is_better"] is False
+    assert d["unit"] == "us/layer" and abs(d["value"] - d["ms_per_step"] * 1e3) < 1e-6 and "config2" in d["config"]["workload"]
+    rf = d["roofline"]
+    assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s" and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
+    assert 0.3 < rf["frac"] < 1.0 and rf["traffic"] is not None
+    cb = d["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > d["value"] and "sample" in cb
+    assert d["graph_replay_matches_eager"] is True

@@ -10,8 +10,8 @@ the final norm in front (`ha_linear_skinny_fused`), output and down projection w
 (`F.rms_norm`, hipBLASLt) plus `ha_swiglu`.  The point is to time the whole step, and to check the plumbing around the op
 (rotate-half RoPE, grouped KV heads, cache append) against `transformers`.
 
-Caches are preallocated per layer, key and value row of a token side by side (`[B, Hkv, S_cap, 2, d]`, handed to the
-kernels as two strided views); a step writes the new key/value in place, so there is no per-step concatenation.
+Caches are preallocated `[B, Hkv, S_cap, d]` per layer; a step writes the new key/value in place, so there is no
+per-step concatenation.
 """
 from __future__ import annotations
 
@@ -84,12 +84,8 @@ class LlamaShapedDecoder:
         arith = _ops.HA_ARITH_BF16 if self.dtype == torch.bfloat16 else _ops.HA_ARITH_F32
         self.k_cache, self.v_cache, self.hash = [], [], []
         for l in range(self.L):
-            # key and value row of a token side by side, [B, Hkv, S_cap, 2, d]: the gather fetches both, and one 512-byte
-            # stretch of memory serves it better than two 256-byte ones (attention launch 65.2 -> 64.1 us at 4 x 128K tokens,
-            # 99.8 -> 96.4 us at 16 x 64K); the kernels only see two views with the same strides
-            kv = torch.zeros(B, self.Hkv, S_cap, 2, self.d, dtype=self.dtype, device=self.device)
-            self.k_cache.append(kv[:, :, :, 0])
-            self.v_cache.append(kv[:, :, :, 1])
+            self.k_cache.append(torch.zeros(B, self.Hkv, S_cap, self.d, dtype=self.dtype, device=self.device))
+            self.v_cache.append(torch.zeros(B, self.Hkv, S_cap, self.d, dtype=self.dtype, device=self.device))
             usa = usa_per_layer[l] if usa_per_layer is not None else self.random_usa(1000 + l)
             hl = HashDecodeLayer(usa.k, usa.q, self.H, self.Hkv, self.d, nl, idim, fdim, init, recent, heavy, arith=arith,
                                  device=self.device)

@@ -282,6 +282,8 @@ class HeavyHitterMixin:
         self.offloading_length = None
         self.flash_forward = None
         self._hash_layer: Optional[HashDecodeLayer] = None
+        self._cache_ref = None       # weak reference to the KV cache object whose keys the bit-cache was made from
+        self._cache_id = None
 
     def __repr__(self):
         return (f"{super().__repr__()}\nSparsification Setting(topk:{self.heavy_budget}  edge:{self.init_budget, self.recent_budget} "
@@ -291,6 +293,7 @@ class HeavyHitterMixin:
         """A new example starts (reference :298-301): drop the cached codes."""
         self.past_key_signatures = None
         self.print_offloading_flag = False
+        self._cache_ref = self._cache_id = None
         if self._hash_layer is not None:
             self._hash_layer.reset()
 
@@ -316,6 +319,43 @@ class HeavyHitterMixin:
         layer.keys, layer.values = layer.keys.cpu(), layer.values.cpu()
 
     # ---- bit-cache plumbing
+    def _cache_len(self, cache) -> int:
+        """Tokens this layer already holds in `cache` (0 for no cache or a layer not yet written)."""
+        if cache is None:
+            return 0
+        if hasattr(cache, "get_seq_length"):
+            try:
+                return int(cache.get_seq_length(self.layer_idx))
+            except (IndexError, KeyError):
+                return 0
+        layer = self._cache_layer(cache)
+        return 0 if layer is None else int(layer.keys.shape[-2])
+
+    def _sync_bit_cache(self, cache) -> None:
+        """Keep the bit-cache in step with the KV cache before a forward pass appends to it.  The reference is stateless
+        here (`past_key_signatures` stays None, :407-408, every key is re-hashed every step), so a caller may start a new
+        prompt without `reset_usa`: codes are kept only while the SAME cache object still holds at least the tokens they
+        were made from.  Another cache object drops them all; a cache that was rewound keeps the codes of its prefix."""
+        if cache is None:
+            same = False
+        elif self._cache_ref is not None:
+            same = self._cache_ref() is cache
+        else:
+            same = self._cache_id is not None and self._cache_id == id(cache)
+        if not same:
+            self._cache_ref, self._cache_id = None, (id(cache) if cache is not None else None)
+            try:
+                self._cache_ref = weakref.ref(cache) if cache is not None else None
+            except TypeError:           # a cache class without weak references: object identities are compared instead
+                pass
+        hl = self._hash_layer
+        if hl is None:
+            return
+        if not same:
+            hl.reset()
+        else:
+            hl.n_cached = min(hl.n_cached, self._cache_len(cache))
+
     def _ensure_hash_layer(self, batch: int, seq_len: int, device) -> HashDecodeLayer:
         if self.usa_module is None:
             raise RuntimeError("convert_usa() must attach a USA module before the decode branch runs")
@@ -427,6 +467,7 @@ class HeavyHitterMixin:
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
         bsz, q_len, _ = hidden_states.shape
         self.ensure_gpu(cache, hidden_states.device)
+        self._sync_bit_cache(cache)
         if q_len > DECODE_MAX_Q_LEN or self.train_usa:
             # prefill, and every step while the hash is being trained: the original dense forward (reference :529-550);
             # its keys are hashed lazily at the first decode step
@@ -482,6 +523,7 @@ class HeavyHitterMixin:
                 mask[:, :, i].scatter_(2, where, True)
         finally:
             hl.heavy_budget = saved
+            hl.reset()      # these codes belong to the keys handed in, not to a KV cache: the next decode step hashes afresh
         mask = mask[..., :S]
         return mask
 
@@ -600,10 +642,11 @@ class HeavyHitterMixin:
 
 # ------------------------------------------------------------------------------------------ module-patch helpers
 
-def build_usa_modules(config, path, default_num_layers=None) -> nn.ModuleList:
-    """Body of `load_usa` (reference :633-646): one USA per decoder layer, optionally loaded from a state dict."""
+def build_usa_modules(config, path, force_num_layers=None) -> nn.ModuleList:
+    """Body of `load_usa` (reference :633-646): one USA per decoder layer, optionally loaded from a state dict.
+    `force_num_layers`: the depth of the hash MLP when the family's reference ignores `config.lth_num_layers` (Mistral)."""
     cfg = {"lth_int_dim": config.lth_init_dim, "lth_final_dim": config.lth_final_dim, "lth_thold": config.lth_thold,
-           "lth_num_layers": getattr(config, "lth_num_layers", default_num_layers or 3)}
+           "lth_num_layers": force_num_layers if force_num_layers is not None else config.lth_num_layers}
     head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
     mods = nn.ModuleList([USA(config.num_attention_heads, head_dim, cfg) for _ in range(config.num_hidden_layers)])
     if path is not None:

@@ -42,7 +42,9 @@ class MistralAttention_heavy_hitter(HeavyHitterMixin, nn.Module):
 
 
 def load_usa(config, path):
-    return build_usa_modules(config, path, default_num_layers=3)
+    """As the Llama `load_usa`, except that `config.lth_num_layers` is not read: the reference's Mistral `USA` has the
+    three-layer MLP only (hashattention_mistral.py:77-88, :566-570)."""
+    return build_usa_modules(config, path, force_num_layers=3)
 
 
 def convert_usa(model, config, usa_modules, collect_stats, train_usa):

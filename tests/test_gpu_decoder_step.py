@@ -360,3 +360,56 @@ def test_ragged_prompts_through_the_decoder_generation_loop():
         assert torch.equal(got[b], want), (b, got[b], want)
     with pytest.raises(ValueError):
         dec.prefill_from_hf(model, ids, torch.flip(am, dims=[1]))            # left padding is not a ragged batch
+
+
+def test_full_width_decoder_step_at_131072_tokens():
+    # The shape the decode throughput is quoted on, two layers deep: hidden 4096, ffn 14336, 32 query / 8 KV heads, four
+    # sequences with 131071 cached tokens each, bf16.  (1) the step on the fused select-attend launch against the same step
+    # on ha_select + ha_sparse_decode; (2) the last layer's attention output against the double-precision oracle on the index
+    # lists the oracle's own selection makes from that layer's codes.
+    import math
+    import numpy as np
+    from oracle import c_oracle
+    print("\n[case] full-width decoder step, B=4, context 131072", flush=True)
+    B, S = 4, 131072
+    dec = LlamaShapedDecoder(n_layers=2, hidden=4096, ffn=14336, n_heads=32, n_kv_heads=8, head_dim=128, vocab=32000, n_code_heads=8,
+                             init_budget=128, recent_budget=128, heavy_budget=1.0 / 32, dtype=torch.bfloat16, device=DEV, seed=11)
+    dec.allocate(B, S)
+    dec.fill_cache_synthetic(S - 1)
+    tokens = torch.tensor([3, 1415, 9265, 31999], device=DEV)
+    assert all(h.use_fused and h.fused_ok for h in dec.hash)
+    last = dec.hash[-1]
+
+    def snapshot():
+        # what the last layer's attention launch read and wrote in the step just made (the new token's row included)
+        return dict(q=dec.q_rot.cpu(), out=dec.attn_out.float().cpu().numpy(),
+                    kc=last.codes[:, :, :S].cpu().numpy().view(np.uint32), qc=last.qcodes.view(B, 32, 1).cpu().numpy().view(np.uint32),
+                    k_new=dec.k_cache[-1][:, :, S - 1].cpu(), v_new=dec.v_cache[-1][:, :, S - 1].cpu())
+
+    with torch.no_grad():
+        fused = dec.decode_step(tokens, advance=False).float().clone()
+        snap_fused = snapshot()
+        for h in dec.hash:
+            h.use_fused = False
+        lists = dec.decode_step(tokens, advance=False).float()
+        snap_lists = snapshot()
+    assert torch.isfinite(fused).all()
+    scale = max(1.0, fused.abs().max().item())
+    err = (fused - lists).abs().max().item()
+    print(f"  logits: fused launch vs index lists in memory, max-abs {err:.2e} (largest logit {scale:.2f})", flush=True)
+    assert err <= 3e-2 * scale, err
+    seq = np.full(B, S, dtype=np.int32)
+    cap = 128 + 128 + S // 32
+    k_cpu, v_cpu = dec.k_cache[-1][:, :, :S].cpu(), dec.v_cache[-1][:, :, :S].cpu()
+    for name, snap in (("fused launch", snap_fused), ("lists in memory", snap_lists)):
+        # the layer's input differs by bf16 noise between the two steps (the first layer's attention adds its rows in another
+        # order), so each step is checked against the oracle on ITS query, codes and new row
+        k_cpu[:, :, S - 1], v_cpu[:, :, S - 1] = snap["k_new"], snap["v_new"]
+        ref_idx, ref_cnt = c_oracle.select(snap["kc"], snap["qc"], seq, 128, 128, 1.0 / 32, cap)
+        assert (ref_cnt == cap).all()
+        if name == "lists in memory":
+            assert np.array_equal(last.counts.cpu().numpy(), ref_cnt) and np.array_equal(last.idx.cpu().numpy()[:, :, :cap], ref_idx)
+        ref = c_oracle.sparse_attend(snap["q"], k_cpu, v_cpu, ref_idx, ref_cnt, 1 / math.sqrt(128))
+        aerr = np.abs(snap["out"] - ref).max()
+        print(f"  last layer's attention output ({name}) vs the oracle: max-abs {aerr:.2e}", flush=True)
+        assert aerr <= 2e-2

@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("name", ["config1", "config2", "config4"])
+@pytest.mark.parametrize("name", ["config1", "config2", "config3", "config4"])
 def test_full_size_configuration(name):
     print(f"\n[case] full size {name}", flush=True)
     w = named_workload(name)

@@ -175,3 +175,54 @@ def test_recall_statistic_matches_the_oracle():
     assert diff.max().item() <= 1 / 32 + 1e-6 and (diff > 0).float().mean().item() < 0.05, (diff.max().item(), (diff > 0).float().mean().item())
     assert 0.0 < attn.overlaps[1024][3] <= 1.0
     hl.print_stats(model)
+
+
+def _greedy(model, prompt, n_new, cache=None):
+    """Greedy continuation with a cache of its own (as `generate` makes one per call) unless one is handed in."""
+    cache = DynamicCache() if cache is None else cache
+    toks = []
+    with torch.no_grad():
+        logits = model(prompt, past_key_values=cache, use_cache=True).logits[:, -1]
+        for _ in range(n_new):
+            nxt = logits.argmax(-1, keepdim=True)
+            toks.append(nxt)
+            logits = model(nxt, past_key_values=cache, use_cache=True).logits[:, -1]
+    return torch.cat(toks, dim=1).cpu(), logits.float().cpu()
+
+
+def test_a_new_prompt_needs_no_reset_usa():
+    # The reference keeps no hash state between calls (past_key_signatures stays None, hashattention_llama.py:407-408), and
+    # its README never calls reset_usa between prompts.  The bit-cache must therefore notice a new prompt by itself: a
+    # longer prompt after a shorter one (the stale codes of the first would otherwise stay in front), a shorter one after a
+    # longer one, a short prompt that goes through the q_len <= 128 branch, and a cache object that is rewound and reused.
+    print("\n[case] prompts back to back without reset_usa", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(LlamaConfig)
+    model = LlamaForCausalLM(cfg).bfloat16().float()
+    usa = hl.load_usa(cfg, None)
+    model = hl.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False).float()
+    g = torch.Generator().manual_seed(9)
+    prompts = [torch.randint(0, cfg.vocab_size, (2, n), generator=g).to(DEV) for n in (200, 500, 150, 60, 300)]
+    want = []
+    for p in prompts:                              # every prompt from a clean state
+        hl.reset_usa(model)
+        want.append(_greedy(model, p, 10))
+    hl.reset_usa(model)
+    for p, (toks, logits) in zip(prompts, want):   # the same prompts back to back, no reset in between
+        got_toks, got_logits = _greedy(model, p, 10)
+        assert torch.equal(got_toks, toks)
+        assert (got_logits - logits).abs().max().item() < 1e-4
+    # one cache object, rewound to a prefix and continued with other tokens: the codes of the prefix stay valid, the rest
+    # is hashed again
+    hl.reset_usa(model)
+    cache = DynamicCache()
+    _greedy(model, prompts[1], 6, cache)
+    assert model.model.layers[0].self_attn._hash_layer.n_cached == 500 + 6
+    cache.crop(-106)                                       # drop the last 106 tokens: 400 are left
+    tail = prompts[4][:, :150]
+    got = _greedy(model, tail, 5, cache)
+    assert model.model.layers[0].self_attn._hash_layer.n_cached == 400 + 150 + 5
+    hl.reset_usa(model)
+    ref = _greedy(model, torch.cat([prompts[1][:, :400], tail], dim=1), 5)
+    assert torch.equal(got[0], ref[0])
+    assert (got[1] - ref[1]).abs().max().item() < 2e-2      # the prefill was chunked differently (500 | 150 against 550 at once)

@@ -13,9 +13,21 @@
 // Both streaming kernels fetch all codes of their chunk before using any (128-bit loads, up to 16 codes
 // per lane), so a workgroup has its whole chunk in flight at once instead of paying one memory round
 // trip per tile.
+#include <mutex>
+
 #include "ha_select_common.h"
 
 using namespace ha_sel;
+
+// Scratch of ha_select_static: the selection's workspace (chunk histograms, row meta, chunk prefixes) for callers that
+// cannot allocate.  Every GPU the library runs on holds its own copy at its own address until the process ends.  In host
+// code the name `scratch` is only a handle: the array's device address on the current GPU comes from
+// hipGetSymbolAddress (static_scratch below, once per device), and that pointer is what the kernels are given.  Nothing
+// in it has to start at zero: the histogram launch writes every counter of every (row, chunk) it is launched for, the
+// threshold launch every meta and prefix entry, before the next launch reads them.  Calls that overlap in time on one
+// GPU (two streams, two threads) would share the array and race.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace {
 
@@ -323,6 +335,28 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
     }
 }
 
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (resolved at the first call on that device).
+int static_scratch(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) HA_FAIL(HA_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    HA_REQUIRE(dev >= 0 && dev < kMaxDevices, HA_ERR_NO_DEVICE, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) HA_FAIL(HA_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return HA_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
 int validate_codes(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, const uint32_t *qcodes, int B, int H, int Hc, int W,
                    int max_seq_len) {
     HA_REQUIRE(kcodes && qcodes, HA_ERR_NULL_POINTER, "kcodes/qcodes is NULL");
@@ -391,7 +425,7 @@ size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
 static int select_impl(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
                        int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
                        int mode, int depth, int algo, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
-                       size_t workspace_bytes, void *stream, bool prepare_only) {
+                       size_t workspace_bytes, void *stream, bool prepare_only, bool use_static_scratch = false) {
     int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len);
     if (st) return st;
     HA_REQUIRE(prepare_only || (out_idx && out_counts), HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
@@ -401,11 +435,22 @@ static int select_impl(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_s
     HA_REQUIRE(mode == HA_SELECT_SIMPLE || mode == HA_SELECT_THRESHOLD, HA_ERR_BAD_SHAPE, "unknown select mode %d", mode);
     HA_REQUIRE(algo >= HA_SELECT_ALGO_AUTO && algo <= HA_SELECT_ALGO_SAMPLED_EXACT_ROWS, HA_ERR_BAD_SHAPE, "unknown select algo %d", algo);
     HA_REQUIRE(idx_cap > 0, HA_ERR_BAD_SHAPE, "idx_cap must be positive");
-    const size_t need = ha_select_workspace_bytes(B, H, Hc, W, max_seq_len);
-    HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "select workspace: need %zu bytes, got %zu", need,
-               workspace ? workspace_bytes : (size_t)0);
-    HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "select workspace must be 256-byte aligned");
-    if ((st = ha_require_device())) return st;
+    if (use_static_scratch) {
+        // the histogram method's own need (the sampled method parks candidates in a far larger workspace)
+        const size_t need = carve_select_ws(nullptr, (int64_t)B * H, select_plan(B, Hc, max_seq_len).nchunk, W).bytes;
+        HA_REQUIRE(need <= kStaticScratchBytes, HA_ERR_WORKSPACE,
+                   "ha_select_static: this shape needs %zu bytes of scratch, the built-in buffer holds %zu: use ha_select with a "
+                   "workspace of ha_select_workspace_bytes()", need, kStaticScratchBytes);
+        if ((st = ha_require_device())) return st;
+        if ((st = static_scratch(&workspace))) return st;
+        algo = HA_SELECT_ALGO_HISTOGRAM;
+    } else {
+        const size_t need = ha_select_workspace_bytes(B, H, Hc, W, max_seq_len);
+        HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "select workspace: need %zu bytes, got %zu", need,
+                   workspace ? workspace_bytes : (size_t)0);
+        HA_REQUIRE(ha_aligned(workspace, 256), HA_ERR_MISALIGNED, "select workspace must be 256-byte aligned");
+        if ((st = ha_require_device())) return st;
+    }
 
     if (prepare_only) algo = HA_SELECT_ALGO_HISTOGRAM;
     if (algo == HA_SELECT_ALGO_AUTO) {
@@ -448,6 +493,16 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
               size_t workspace_bytes, void *stream) {
     return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
                        heavy_budget, mode, depth, algo, out_idx, idx_cap, out_counts, workspace, workspace_bytes, stream, false);
+}
+
+size_t ha_select_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int ha_select_static(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
+                     int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                     int mode, int depth, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *stream) {
+    return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
+                       heavy_budget, mode, depth, HA_SELECT_ALGO_HISTOGRAM, out_idx, idx_cap, out_counts, nullptr, 0, stream, false,
+                       true);
 }
 
 int ha_select_histogram(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,

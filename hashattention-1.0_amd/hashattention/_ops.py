@@ -70,6 +70,9 @@ def load_library() -> C.CDLL:
     lib.ha_select.restype = i32
     lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, i32,
                               vp, i64, vp, vp, sz, vp]
+    lib.ha_select_static_max_bytes.restype = sz
+    lib.ha_select_static.restype = i32
+    lib.ha_select_static.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, vp, i64, vp, vp]
     lib.ha_rope_append.restype = i32
     lib.ha_rope_append.argtypes = [vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]
     lib.ha_rope_encode_step.restype = i32
@@ -283,6 +286,23 @@ def select(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_len
     _check(lib.ha_select(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
                          _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth, algo,
                          _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select")
+
+
+def select_static(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],
+                  init_budget: int, recent_budget: int, heavy_budget: float, out_idx: torch.Tensor, out_counts: torch.Tensor,
+                  mode: int = HA_SELECT_SIMPLE, depth: int = 0) -> None:
+    """`select` without a workspace: the library's built-in device scratch is used and nothing is allocated (shapes whose
+    scratch exceeds ha_select_static_max_bytes() are refused).  Calls on one GPU must not overlap in time."""
+    _require_cuda(kcodes, qcodes, seq_lens, out_idx, out_counts)
+    lib = load_library()
+    B, Hc, _, W = kcodes.shape
+    H = qcodes.shape[1]
+    assert qcodes.is_contiguous() and kcodes.stride(3) == 1 and kcodes.stride(2) == W
+    assert out_idx.is_contiguous() and out_idx.dtype == torch.int32 and out_counts.is_contiguous() and out_counts.dtype == torch.int32
+    assert seq_lens is None or (seq_lens.dtype == torch.int32 and seq_lens.is_contiguous())
+    _check(lib.ha_select_static(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
+                                _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth,
+                                _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _stream(kcodes)), "ha_select_static")
 
 
 def select_prepare(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],

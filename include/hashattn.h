@@ -171,6 +171,23 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
               void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * ha_select without a workspace argument, for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The selection's scratch
+ * (chunk histograms, row thresholds, chunk prefixes: what ha_select keeps in its workspace) lives in a device array of
+ * ha_select_static_max_bytes() = 8 MiB built into the library, one copy per GPU, held until the process ends.  The call
+ * allocates and frees nothing.  Always the histogram method; same lists and counts as ha_select, bit for bit.
+ * Shapes whose scratch would not fit (B * H * ceil(max_seq_len / 4096) * (32 W + 3) * 4 bytes, roughly) are refused
+ * with HA_ERR_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on one GPU (two streams or
+ * threads) race; calls on one stream are ordered.  The first call on a GPU resolves the array's address
+ * (hipGetSymbolAddress): make one call before capturing a graph that contains another.
+ */
+size_t ha_select_static_max_bytes(void);
+int ha_select_static(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                     int B, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                     int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
+                     int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *stream);
+
+/*
  * Gather-only decode attention: out[b, h] = softmax(q[b, h] . K[b, h/G, idx] * sm_scale) V[b, h/G, idx]
  * over the first counts[b, h] entries of idx[b, h]; fp32 online softmax, split over the index list
  * and merged by log-sum-exp.  Replaces flash_fwd_sparse / fwd_sparse

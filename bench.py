@@ -25,9 +25,22 @@ for p in (os.path.join(ROOT, "hashattention-1.0_amd"), ROOT):
 
 HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the gather-attend kernel, from the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
-# summarised in profiles/decode_step_config2_hbm_traffic.md, each scaled on a 1 GiB copy (fetch x2.0, write x1.0).
-MEASURED_ATTEND_TRAFFIC_BYTES = {("config2", True): 588.6e6, ("config2", False): 551.4e6}   # key: (workload, selection fused)
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "decode_step_config2_hbm_traffic.md")
+
+
+def measured_traffic(workload_name, fused, code_heads):
+    """HBM bytes per launch of the step's attention kernel as the two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE, each
+    scaled on a 1 GiB copy) measured them: read from the tracked summary, which names the commit it was measured at in
+    lines of the form `traffic_bytes[config2, fused, code_heads=8] = 588.6e6 (commit abc1234)`.  None when the summary
+    has no line for this workload."""
+    import re
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+    except OSError:
+        return None
+    key = re.escape(f"traffic_bytes[{workload_name}, {'fused' if fused else 'lists'}, code_heads={code_heads}]")
+    m = re.search(key + r"\s*=\s*([0-9.eE+]+)\s*\(commit ([0-9a-f]{7,40})\)", text)
+    return {"bytes": float(m.group(1)), "commit": m.group(2)} if m else None
 
 
 def algorithmic_bytes(w, n_sel_rows):
@@ -54,6 +67,30 @@ def time_gpu(fn, steps, warmup, torch):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / steps
+
+
+def time_rotating(fns, steps, warmup, torch):
+    """`time_gpu` over a rotation: call i runs fns[i % len(fns)], so consecutive launches work on different inputs."""
+    it = [0]
+
+    def fn():
+        fns[it[0] % len(fns)]()
+        it[0] += 1
+    return time_gpu(fn, steps, warmup, torch)
+
+
+def capture_graph(fn, torch):
+    """fn() captured in a HIP graph (after one eager pass on a side stream, as capture wants it)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g
 
 
 def cpu_baseline(w, torch, budget_s=12.0):
@@ -121,28 +158,21 @@ def cpu_sparse_stages(w, torch):
                       f"encode scaled x{w.batch} by sequences, select and attend x{scale:.2f} by cached tokens"}
 
 
-def traffic_probe(torch, layer, q3, k, v, out, fused_attend=None):
-    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain copy of known size, then the gather-attend
-    kernel, three launches each.  The copy gives the scale of the counter (bytes per reported KiB)."""
+def traffic_probe(torch, device, attend_fns):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a plain copy of known size three times, then the step's
+    attention launch three times on every input set in turn.  The copy gives the scale of the counter (bytes per reported KiB)."""
     n = 1 << 30
-    src = torch.empty(n, dtype=torch.uint8, device=q3.device).random_(0, 255)
+    src = torch.empty(n, dtype=torch.uint8, device=device).random_(0, 255)
     dst = torch.empty_like(src)
     torch.cuda.synchronize()
     for _ in range(3):
         dst.copy_(src)
     torch.cuda.synchronize()
-    from hashattention import _ops
-    w = layer
     for _ in range(3):
-        if fused_attend is not None:
-            fused_attend()
-        elif layer.overlap_windows:
-            _ops.sparse_decode_heavy(q3, k, v, w.idx, w.counts, w.sm_scale, out, w.ws_attend, w.win, w.init_budget,
-                                     w.recent_budget, k.shape[2], None)
-        else:
-            layer.attend(q3, k, v, out)
+        for fn in attend_fns:
+            fn()
     torch.cuda.synchronize()
-    print(json.dumps({"probe": "copy 1 GiB x3 (runtime copy kernel), then the step's sparse_attend launch x3"}))
+    print(json.dumps({"probe": f"copy 1 GiB x3 (runtime copy kernel), then the step's sparse_attend launch x3 on each of {len(attend_fns)} input sets in turn"}))
 
 
 def decoder_bench(args, torch):
@@ -253,6 +283,94 @@ def decoder_bench(args, torch):
     print(json.dumps(res))
 
 
+class InputSet:
+    """One attention layer's worth of inputs and state: its own Q/K/V, hash weights, bit-cache, workspaces and output."""
+
+    def __init__(self, w, args, dev, torch, seed_offset, code_heads=None):
+        from hashattention.decode import HashDecodeLayer
+        from hashattention.synthetic import Workload, make_problem_on_device, make_usa_weights
+        self.w = Workload(**{**w.__dict__, "seed": w.seed + seed_offset})
+        self.p = make_problem_on_device(self.w, dev)
+        self.torch, self.dev = torch, dev
+        self.ragged = len(set(w.seq_lens)) > 1
+        self.seq_lens = self.p.seq_lens if self.ragged else None
+        self.S = w.max_seq_len
+        self.q3 = self.p.q[:, :, 0, :]
+        self.layer = self.make_layer(self.p.usa, args)
+        self.out = torch.empty(w.batch, w.n_q_heads, w.head_dim, dtype=w.dtype, device=dev)
+
+    def make_layer(self, usa, args):
+        from hashattention.decode import HashDecodeLayer
+        w, torch = self.w, self.torch
+        layer = HashDecodeLayer(usa.k, usa.q, w.n_q_heads, w.n_kv_heads, w.head_dim, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
+                                w.init_budget, w.recent_budget, w.heavy_budget, device=self.dev)
+        if args.fused_min_rows is not None:
+            layer.fused_min_rows = args.fused_min_rows
+        layer.allocate(w.batch, self.S)
+        layer.select_algo = args.select_algo
+        layer.overlap_windows = args.overlap_windows
+        layer.use_fused = not args.two_launch
+        # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
+        layer.encode_keys(self.p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
+        torch.cuda.synchronize()
+        layer.n_cached = self.S - 1             # the step re-encodes the newest key, as a real decode step does
+        return layer
+
+    def other_code_heads(self, n_code_heads, args):
+        """A second layer over the same K/V with `n_code_heads` key-side hash MLPs (its own weights and bit-cache)."""
+        from hashattention.synthetic import Workload, make_usa_weights
+        w2 = Workload(**{**self.w.__dict__, "n_code_heads": n_code_heads})
+        twin = object.__new__(InputSet)
+        twin.__dict__.update(self.__dict__)
+        twin.w = w2
+        twin.layer = twin.make_layer(make_usa_weights(w2), args)
+        twin.out = self.torch.empty_like(self.out)
+        return twin
+
+    # the launches that are timed
+    def step(self):
+        if self.ragged:
+            self.layer.step(self.p.q, self.p.k, self.p.v, self.S, self.out, seq_lens=self.seq_lens)
+        else:
+            self.layer.n_cached = self.S - 1
+            self.layer.step(self.p.q, self.p.k, self.p.v, self.S, self.out)
+
+    def encode_only(self):
+        from hashattention import _ops
+        l, S = self.layer, self.S
+        _ops.encode_step(self.p.k[:, :, S - 1:S], self.q3, l.wk, l.wq, l.num_layers, l.int_dim, l.final_dim, l.codes, l.qcodes, pos0=S - 1)
+
+    def select(self):
+        self.layer.select(self.S, self.seq_lens)
+
+    def select_prepare(self):
+        self.layer.select_prepare(self.S, self.seq_lens)
+
+    def attend_fused(self):
+        self.layer.attend_fused(self.q3, self.p.k, self.p.v, self.out, self.S, self.seq_lens)
+
+    def attend_lists(self):
+        self.layer.attend(self.q3, self.p.k, self.p.v, self.out)
+
+
+def time_step(sets, steps, warmup, torch):
+    """The whole step over a rotation of input sets: eager launches and one HIP graph holding one pass over all sets,
+    replayed.  Returns (ms eager, ms graph, graph replay reproduces the eager outputs)."""
+    fns = [s.step for s in sets]
+    ms_eager = time_rotating(fns, steps, warmup, torch)
+    torch.cuda.synchronize()
+    ref = [s.out.clone() for s in sets]
+
+    def one_pass():
+        for f in fns:
+            f()
+    graph = capture_graph(one_pass, torch)
+    replays = max(1, (steps + len(sets) - 1) // len(sets))
+    ms_graph = time_gpu(graph.replay, replays, max(1, warmup // len(sets)), torch) / len(sets)
+    ok = all(bool(torch.equal(s.out, r)) for s, r in zip(sets, ref))
+    return ms_eager, ms_graph, ok
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -260,6 +378,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="config2")
     ap.add_argument("--batch", type=int, default=None, help="override the number of sequences of a uniform configuration (a variant, not the named workload)")
+    ap.add_argument("--code-heads", type=int, default=None, help="key-side hash MLPs per layer: 8 (one per KV head, the named workloads) or 32 "
+                    "(one per query head, as the reference's load_usa builds them); a variant, not the named workload")
+    ap.add_argument("--input-sets", type=int, default=4, help="independent (Q, K, V, codes, weights) sets the timed launches rotate over, "
+                    "so that consecutive launches never touch the same rows (as consecutive layers of a model)")
+    ap.add_argument("--no-code-heads-32", action="store_true", help="skip the extra timing of the one-code-per-query-head layout")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
@@ -277,8 +400,7 @@ def main():
 
     import torch
     from hashattention import _ops
-    from hashattention.decode import HashDecodeLayer
-    from hashattention.synthetic import make_problem_on_device, named_workload
+    from hashattention.synthetic import named_workload
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HashAttention path has no CPU fallback", file=sys.stderr)
@@ -293,83 +415,56 @@ def main():
         if len(set(w.seq_lens)) > 1:
             sys.exit("--batch applies to configurations whose sequences have one length")
         w.batch, w.seq_lens, w.name = args.batch, [w.seq_lens[0]] * args.batch, f"{w.name} with batch {args.batch}"
-    p = make_problem_on_device(w, dev)
+    if args.code_heads is not None and args.code_heads != w.n_code_heads:
+        w.n_code_heads, w.name = args.code_heads, f"{w.name} with {args.code_heads} code heads"
+    n_sets = max(1, args.input_sets)
+    sets = [InputSet(w, args, dev, torch, 101 * i) for i in range(n_sets)]
+    s0 = sets[0]
+    layer = s0.layer
     B, H, Hkv, d, S = w.batch, w.n_q_heads, w.n_kv_heads, w.head_dim, w.max_seq_len
-    ragged = len(set(w.seq_lens)) > 1
-    seq_lens = p.seq_lens if ragged else None
-
-    layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, d, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
-                            w.init_budget, w.recent_budget, w.heavy_budget, device=dev)
-    if args.fused_min_rows is not None:
-        layer.fused_min_rows = args.fused_min_rows
-    layer.allocate(B, S)
-    layer.select_algo = args.select_algo
-    layer.overlap_windows = args.overlap_windows
-    layer.use_fused = not args.two_launch
+    ragged = s0.ragged
     fused = layer.use_fused and layer.fused_ok and not layer.overlap_windows
-    # prefill: codes of every cached key (un-timed, as in the reference protocol: efficiency/kernels/torchatt.py:183-184)
-    layer.encode_keys(p.k, use_mfma=(w.dtype == torch.bfloat16 and not args.exact_encode))
-    torch.cuda.synchronize()
-    layer.n_cached = S - 1                      # the step re-encodes the newest key, as a real decode step does
-    out = torch.empty(B, H, d, dtype=w.dtype, device=dev)
-    out_dense = torch.empty_like(out)
-    ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)
-    q3 = p.q[:, :, 0, :]
-
-    def step():
-        if ragged:
-            layer.step(p.q, p.k, p.v, S, out, seq_lens=seq_lens)
-        else:
-            layer.n_cached = S - 1
-            layer.step(p.q, p.k, p.v, S, out)
-
-    def encode_only():
-        _ops.encode_step(p.k[:, :, S - 1:S], q3, layer.wk, layer.wq, layer.num_layers, layer.int_dim, layer.final_dim,
-                         layer.codes, layer.qcodes, pos0=S - 1)
+    rot = lambda name: [getattr(s, name) for s in sets]
 
     if args.traffic_probe:
-        step()
-        traffic_probe(torch, layer, q3, p.k, p.v, out,
-                      (lambda: layer.attend_fused(q3, p.k, p.v, out, S, seq_lens)) if fused else None)
+        for s in sets:
+            s.step()
+        traffic_probe(torch, dev, rot("attend_fused") if fused else rot("attend_lists"))
         return
-    ms_step_eager = time_gpu(step, args.steps, args.warmup, torch)
-    # the same launch sequence captured once in a HIP graph and replayed: the step as a serving loop runs it
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        step()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        step()
-    ref_out = out.clone()
-    ms_step_graph = time_gpu(graph.replay, args.steps, args.warmup, torch)
-    graph_ok = bool(torch.equal(out, ref_out))
+    ms_step_eager, ms_step_graph, graph_ok = time_step(sets, args.steps, args.warmup, torch)
     ms_step = min(ms_step_graph, ms_step_eager)
-    ms_encode = time_gpu(encode_only, args.steps, args.warmup, torch)
-    ms_select = time_gpu(lambda: layer.select(S, seq_lens), args.steps, args.warmup, torch)
+    # the same step replayed on ONE input set, as earlier versions of this benchmark timed it: the rows it gathers (604 MB)
+    # are the same in every launch, so part of them can still sit in the 256 MB memory-side cache
+    ms_single_eager, ms_single_graph, _ = time_step(sets[:1], args.steps, args.warmup, torch)
+    ms_encode = time_rotating(rot("encode_only"), args.steps, args.warmup, torch)
+    ms_select = time_rotating(rot("select"), args.steps, args.warmup, torch)
+    ms_window = 0.0
     if layer.overlap_windows:      # the dominant kernel as the step launches it: heavy tokens only, window partial merged
-        _ops.window_partial(q3, p.k, p.v, S, seq_lens, w.init_budget, w.recent_budget, layer.sm_scale, layer.win)
-        ms_attend = time_gpu(lambda: _ops.sparse_decode_heavy(q3, p.k, p.v, layer.idx, layer.counts, layer.sm_scale, out,
+        p = s0.p
+        _ops.window_partial(s0.q3, p.k, p.v, S, s0.seq_lens, w.init_budget, w.recent_budget, layer.sm_scale, layer.win)
+        ms_attend = time_gpu(lambda: _ops.sparse_decode_heavy(s0.q3, p.k, p.v, layer.idx, layer.counts, layer.sm_scale, s0.out,
                                                               layer.ws_attend, layer.win, w.init_budget, w.recent_budget, S,
-                                                              seq_lens), args.steps, args.warmup, torch)
-        ms_window = time_gpu(lambda: _ops.window_partial(q3, p.k, p.v, S, seq_lens, w.init_budget, w.recent_budget,
+                                                              s0.seq_lens), args.steps, args.warmup, torch)
+        ms_window = time_gpu(lambda: _ops.window_partial(s0.q3, p.k, p.v, S, s0.seq_lens, w.init_budget, w.recent_budget,
                                                          layer.sm_scale, layer.win), args.steps, args.warmup, torch)
-    elif fused:    # the step's dominant launch: list rebuilt from the codes in LDS + gather-attend (thresholds already in the workspace)
-        layer.select(S, seq_lens)              # leaves the same thresholds as select_prepare, plus the lists for the comparison below
-        ms_attend_lists = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
-        ms_prepare = time_gpu(lambda: layer.select_prepare(S, seq_lens), args.steps, args.warmup, torch)
-        ms_attend = time_gpu(lambda: layer.attend_fused(q3, p.k, p.v, out, S, seq_lens), args.steps, args.warmup, torch)
-        ms_window = 0.0
+    elif fused:    # the step's dominant launch: list rebuilt from the codes in LDS + gather-attend
+        for s in sets:
+            s.select()                         # leaves the lists for the comparison below
+        ms_attend_lists = time_rotating(rot("attend_lists"), args.steps, args.warmup, torch)
+        ms_prepare = time_rotating(rot("select_prepare"), args.steps, args.warmup, torch)
+        ms_attend = time_rotating(rot("attend_fused"), args.steps, args.warmup, torch)
+        ms_attend_single = time_gpu(s0.attend_fused, args.steps, args.warmup, torch)
     else:
-        ms_attend = time_gpu(lambda: layer.attend(q3, p.k, p.v, out), args.steps, args.warmup, torch)
-        ms_window = 0.0
-    ms_dense = time_gpu(lambda: _ops.dense_decode(q3, p.k, p.v, S, seq_lens, layer.sm_scale, out_dense, ws_dense),
-                        max(10, args.steps // 4), max(2, args.warmup // 4), torch)
+        ms_attend = time_rotating(rot("attend_lists"), args.steps, args.warmup, torch)
+    out_dense = torch.empty_like(s0.out)
+    ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)
+    dense = [(lambda s=s: _ops.dense_decode(s.q3, s.p.k, s.p.v, S, s.seq_lens, layer.sm_scale, out_dense, ws_dense)) for s in sets]
+    ms_dense = time_rotating(dense, max(10, args.steps // 4), max(2, args.warmup // 4), torch)
+    dense[0]()
 
+    s0.step()
     if fused:
-        layer.select(S, seq_lens)
+        s0.select()
     n_sel_rows = int(layer.counts.sum().item())
     ab = algorithmic_bytes(w, n_sel_rows)
     eb = 2 if w.dtype != torch.float32 else 4
@@ -378,8 +473,15 @@ def main():
         attend_bytes = (n_sel_rows - n_win_rows) * (2 * d * eb + 4) + B * H * (2 * d * eb + 130 * 4)
     else:
         attend_bytes = ab["gather"]
-    sparse_bytes = ab["score"] + ab["select"] + ab["gather"]
-    err = (out.float() - out_dense.float()).abs().max().item()   # informational: sparse vs dense output distance
+    # algorithmic bytes of the step: codes read once, rows gathered; the index lists travel through memory on the two-launch path only
+    sparse_bytes = ab["score"] + ab["gather"] + (0 if fused else ab["select"])
+    err = (s0.out.float() - out_dense.float()).abs().max().item()   # informational: sparse vs dense output distance
+    traffic = measured_traffic(args.config, bool(fused), w.n_code_heads) if args.batch is None else None
+
+    def roofline_obj(kernel, nbytes, ms, **extra):
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        return {"kernel": kernel, "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                "algorithmic_bytes": nbytes, "us": ms * 1e3, **extra}
 
     res = {
         "metric": "sparse_decode_us_per_layer",
@@ -390,7 +492,13 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": ms_step,
         "step_launch": {"value_is": "graph" if ms_step_graph <= ms_step_eager else "eager",
-                        "hip_graph_replay_us": ms_step_graph * 1e3, "eager_launches_from_python_us": ms_step_eager * 1e3},
+                        "hip_graph_replay_us": ms_step_graph * 1e3, "eager_launches_from_python_us": ms_step_eager * 1e3,
+                        "input_sets": n_sets,
+                        "how": f"launches rotate over {n_sets} independent input sets (own Q, K, V, hash weights, bit-cache): no launch "
+                               "touches the rows of the launch before it"},
+        "single_set": {"us_per_layer": min(ms_single_eager, ms_single_graph) * 1e3, "hip_graph_replay_us": ms_single_graph * 1e3,
+                       "eager_launches_from_python_us": ms_single_eager * 1e3,
+                       "how": "the same step replayed on one input set (every launch gathers the same rows)"},
         "graph_replay_matches_eager": graph_ok,
         "higher_is_better": False,
         "scaling": "weak",
@@ -406,6 +514,7 @@ def main():
                 "ha_encode_step + ha_select + " + ("ha_window_partial + ha_sparse_decode_heavy" if layer.overlap_windows else "ha_sparse_decode"),
         "stages_us": {"encode_new_k_and_q": ms_encode * 1e3,
                       **({"select_prepare": ms_prepare * 1e3, "select_attend_fused": ms_attend * 1e3,
+                          "select_attend_fused_single_set": ms_attend_single * 1e3,
                           "two_launch_select": ms_select * 1e3, "two_launch_attend": ms_attend_lists * 1e3} if fused else
                          {"score_select": ms_select * 1e3, "gather_attend": ms_attend * 1e3}),
                       "window_partial_second_stream": ms_window * 1e3, "dense_flash_decode": ms_dense * 1e3},
@@ -416,15 +525,29 @@ def main():
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
         # the scoring stream (XOR + popcount over every cached code, histogrammed on the fly) as its own launch
-        **({"score_roofline": {"kernel": "select_hist_kernel", "bound": "hbm", "achieved": ab["score"] / (ms_prepare * 1e-3) / 1e9,
-                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["score"] / (ms_prepare * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                               "algorithmic_bytes": ab["score"], "us": ms_prepare * 1e3}} if fused and layer.local_thresholds else {}),
-        "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm",
-                     "achieved": attend_bytes / (ms_attend * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": attend_bytes / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_ATTEND_TRAFFIC_BYTES.get((w.name, bool(fused))),
-                     "algorithmic_bytes": attend_bytes, "us": ms_attend * 1e3},
+        **({"score_roofline": roofline_obj("select_hist_kernel", ab["score"], ms_prepare)} if fused and layer.local_thresholds else {}),
+        "roofline": roofline_obj("sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", attend_bytes, ms_attend,
+                                 traffic=traffic["bytes"] if traffic else None,
+                                 traffic_measured_at_commit=traffic["commit"] if traffic else None),
     }
+    # the layout the reference's load_usa builds (one key-side hash MLP per QUERY head, hashattention_llama.py:642): four
+    # times the codes, no code shared inside a KV group; same K/V, rotation and timing protocol
+    if w.n_code_heads != H and not args.no_code_heads_32 and args.batch is None and fused:
+        twins = [s.other_code_heads(H, args) for s in sets]
+        t_eager, t_graph, t_ok = time_step(twins, args.steps, args.warmup, torch)
+        t_fused = twins[0].layer.use_fused and twins[0].layer.fused_ok
+        t_prepare = time_rotating([t.select_prepare for t in twins], args.steps, args.warmup, torch)
+        t_attend = time_rotating([t.attend_fused if t_fused else t.attend_lists for t in twins], args.steps, args.warmup, torch)
+        t_step = min(t_eager, t_graph)
+        ab2 = algorithmic_bytes(twins[0].w, n_sel_rows)
+        bytes2 = ab2["score"] + ab2["gather"] + (0 if t_fused else ab2["select"])
+        res["code_heads_per_query_head"] = {
+            "code_heads": H, "us_per_layer": t_step * 1e3, "hip_graph_replay_us": t_graph * 1e3, "eager_launches_from_python_us": t_eager * 1e3,
+            "graph_replay_matches_eager": t_ok, "hbm_gbps_step": bytes2 / (t_step * 1e-3) / 1e9,
+            "hbm_frac_step": bytes2 / (t_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "speedup_vs_dense": ms_dense / t_step,
+            "score_roofline": roofline_obj("select_hist_kernel", ab2["score"], t_prepare),
+            "roofline": roofline_obj("sparse_attend_kernel (selection fused)" if t_fused else "sparse_attend_kernel", ab2["gather"], t_attend)}
+        del twins
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)
         res["cpu_sparse_port"] = cpu_sparse_stages(w, torch)

@@ -32,11 +32,17 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 constexpr int kMinSplitRows = 64;
 
-// Tuning overrides (read once): HASHATTN_SPARSE_SPLIT_ROWS = rows of the index list per workgroup
-// (0 = whole list, no split merge), HASHATTN_SPARSE_THREADS = 256 or 512.
+// Tuning overrides for experiments, compiled in only with -DHASHATTN_TUNING_ENV (read once): HASHATTN_SPARSE_SPLIT_ROWS =
+// rows of the index list per workgroup (0 = whole list, no split merge), HASHATTN_SPARSE_THREADS = 256 or 512.  The
+// library as shipped reads no environment variable.
 inline int env_int(const char *name, int dflt) {
+#ifdef HASHATTN_TUNING_ENV
     const char *e = getenv(name);
     return (e && *e) ? atoi(e) : dflt;
+#else
+    (void)name;
+    return dflt;
+#endif
 }
 
 struct SparsePlan {

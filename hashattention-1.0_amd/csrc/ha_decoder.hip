@@ -295,12 +295,15 @@ __global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_
 __global__ __launch_bounds__(64) void rope_append_kernel(const void *__restrict__ qkv, int64_t qkv_sb, int dtype, int H, int Hkv, int pos,
                                                          const int32_t *__restrict__ pos_dev, const float *__restrict__ inv_freq,
                                                          void *__restrict__ q_out, void *__restrict__ k_cache,
-                                                         void *__restrict__ v_cache, int64_t kv_sb, int64_t kv_sh, int64_t kv_ss) {
+                                                         void *__restrict__ v_cache, int64_t kv_sb, int64_t kv_sh, int64_t kv_ss,
+                                                         int64_t cache_len) {
     const int head = blockIdx.x, b = blockIdx.y, i = threadIdx.x;
     const int p = pos_dev ? pos_dev[b] : pos;
+    const bool inside = p >= 0 && p < cache_len;  // a device-side position beyond the cache writes no key or value
     const int64_t src = b * qkv_sb + (int64_t)head * HA_HEAD_DIM;
     const float x0 = ha_load_elem(qkv, src + i, dtype), x1 = ha_load_elem(qkv, src + i + 64, dtype);
     if (head >= H + Hkv) {  // value: copied as it is
+        if (!inside) return;
         const int64_t dst = b * kv_sb + (int64_t)(head - H - Hkv) * kv_sh + (int64_t)p * kv_ss;
         ha_store_elem(v_cache, dst + i, x0, dtype);
         ha_store_elem(v_cache, dst + i + 64, x1, dtype);
@@ -314,7 +317,7 @@ __global__ __launch_bounds__(64) void rope_append_kernel(const void *__restrict_
         const int64_t dst = ((int64_t)b * H + head) * HA_HEAD_DIM;
         ha_store_elem(q_out, dst + i, y0, dtype);
         ha_store_elem(q_out, dst + i + 64, y1, dtype);
-    } else {
+    } else if (inside) {
         const int64_t dst = b * kv_sb + (int64_t)(head - H) * kv_sh + (int64_t)p * kv_ss;
         ha_store_elem(k_cache, dst + i, y0, dtype);
         ha_store_elem(k_cache, dst + i + 64, y1, dtype);
@@ -346,7 +349,7 @@ int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int 
     int st = ha_require_device();
     if (st) return st;
     hipLaunchKernelGGL(rope_append_kernel, dim3(H + 2 * Hkv, B), dim3(64), 0, (hipStream_t)stream, qkv, qkv_stride_b, dtype, H, Hkv, pos,
-                       pos_dev, inv_freq, q_out, k_cache, v_cache, kv_stride_b, kv_stride_h, kv_stride_s);
+                       pos_dev, inv_freq, q_out, k_cache, v_cache, kv_stride_b, kv_stride_h, kv_stride_s, cache_len);
     HA_CHECK_LAUNCH("rope_append_kernel");
     return HA_OK;
 }

@@ -36,6 +36,9 @@ struct EncSide {
     float *logits;
     int pos_bias;  // added to pos_dev[b] (-1 when pos_dev holds sequence lengths and the row is the last one)
     int x_at_pos;  // T = 1: x is a cache and the row to hash sits at the position the code is written to
+    // tokens a (sequence, head) row of `codes` can hold, from its strides: a position read from device memory that lies
+    // beyond it is written nowhere instead of into the next row (0: unknown, no check)
+    int64_t pos_cap;
 };
 // Up to two sides share one launch (the new keys and the queries of a decode step): blockIdx.y runs over
 // the heads of side 0, then those of side 1.
@@ -51,6 +54,7 @@ struct EncRope {
     int64_t kv_sb, kv_sh, kv_ss;
     int pos;
     const int32_t *pos_dev;
+    int64_t cache_len;      // tokens a (sequence, head) row of the caches holds: a device-side position beyond it writes nothing
 };
 struct EncArgs {
     EncSide side[2];
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
             xs[it] = y;
             if (second) {
                 ha_store_elem(rp.q_out, ((int64_t)b * n_heads + head) * HA_HEAD_DIM + e, y, x_dtype);
-            } else if (writes_kv) {
+            } else if (writes_kv && p >= 0 && p < rp.cache_len) {
                 const int64_t dst = b * rp.kv_sb + (int64_t)in_head * rp.kv_sh + (int64_t)p * rp.kv_ss + e;
                 ha_store_elem(rp.k_cache, dst, y, x_dtype);
                 ha_store_elem(rp.v_cache, dst, ha_load_elem(rp.v_src, b * rp.v_sb + (int64_t)in_head * HA_HEAD_DIM + e, x_dtype), x_dtype);
@@ -286,8 +290,9 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
         if (logits && tid < d_out) logits[(((int64_t)b * n_heads + head) * T + t) * d_out + tid] = s_act[cur][r][tid];
         const int64_t pos = (int64_t)(pos_dev ? pos_dev[b] + sd.pos_bias : pos0) + t;
         uint32_t *c = codes + b * c_sb + head * c_sh + pos * W;
-        if (lane == 0 && wave * 2 < W && pos >= 0) c[wave * 2] = (uint32_t)bal;
-        if (lane == 32 && wave * 2 + 1 < W && pos >= 0) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
+        const bool inside = pos >= 0 && (sd.pos_cap == 0 || pos < sd.pos_cap);
+        if (lane == 0 && wave * 2 < W && inside) c[wave * 2] = (uint32_t)bal;
+        if (lane == 32 && wave * 2 + 1 < W && inside) c[wave * 2 + 1] = (uint32_t)(bal >> 32);
     }
 }
 
@@ -311,7 +316,14 @@ int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const
 // that path (three layers, back to back: 7.6 us with four rows, 5.0 us with one at 4 sequences); but every workgroup
 // fetches its head's weights, so the grid is kept within 1.5 workgroups per CU (640 workgroups of one row at 16
 // sequences: 9.2 us against 7.1 us for 320 of two).  Bulk encodes keep four rows.
-int launch_encode(const EncArgs &a, int64_t n_rows, int heads, hipStream_t s) {
+int launch_encode(const EncArgs &a_in, int64_t n_rows, int heads, hipStream_t s) {
+    EncArgs a = a_in;
+    // capacity of a code row from its strides (rows of [B, heads, S_cap, W] are c_sh = S_cap * W words apart)
+    const int W = a.d_out / 32;
+    for (int i = 0; i < 2; ++i) {
+        const int64_t span = a.side[i].n_heads > 1 ? a.side[i].c_sh : (a.B > 1 ? a.side[i].c_sb : 0);
+        a.side[i].pos_cap = span > 0 ? span / W : 0;
+    }
     int rows = kMaxRows;
     for (int r = 1; r < kMaxRows; r *= 2)
         if (((n_rows + r - 1) / r) * heads <= 384) {
@@ -456,7 +468,7 @@ int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int 
     a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
     a.rope = EncRope{inv_freq, (const char *)qkv + (int64_t)(H + Hkv) * HA_HEAD_DIM * eb, qkv_stride_b, q_out, k_cache, v_cache, kv_stride_b,
-                     kv_stride_h, kv_stride_s, pos, pos_dev};
+                     kv_stride_h, kv_stride_s, pos, pos_dev, cache_len};
     return launch_encode(a, B, Hc + H, (hipStream_t)stream);
 }
 

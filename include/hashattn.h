@@ -84,7 +84,8 @@ int64_t ha_usa_packed_floats(int n_layers, int head_dim, int int_dim, int final_
  *   weights  packed blob of n_heads heads; MLP head i reads x head i / (n_heads / x_heads)
  *   codes    [B, n_heads, ., W] uint32, strides c_stride_{b,h} in words; token t of sequence b is
  *            written at position pos0 + t, or pos_dev[b] + t when pos_dev (int32 [B]) is given:
- *            this is the append into the per-layer bit-cache
+ *            this is the append into the per-layer bit-cache; a position taken from pos_dev that lies outside the row
+ *            (negative, or beyond the c_stride_h / W tokens a row spans) is written nowhere
  *   logits   optional fp32 [B, n_heads, T, final_dim] contiguous (tests, diagnostics); may be NULL
  */
 int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t,
@@ -255,8 +256,9 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
  * method only: it leaves in the workspace, per (sequence, query head), the threshold distance T, the number of ties
  * taken and the heavy count, and per 1024..4096-token chunk how many selected tokens precede it, and writes
  * out_counts.  ha_sparse_decode_fused then rebuilds each row's ordered index list in LDS straight from the codes
- * (same order as ha_select's list, so the output equals ha_select + ha_sparse_decode bit for bit when rows are not
- * split) and attends to it: the list never travels through memory and the compaction launch disappears.
+ * (the same tokens as ha_select's list in another fixed order, so the output equals that of ha_select + ha_sparse_decode
+ * up to the order of the fp32 additions) and attends to it: the list never travels through memory and the compaction
+ * launch disappears.
  * Budgets, seq_lens and code arguments must be those given to ha_select_prepare; `select_workspace` is the
  * workspace it filled.  With thresholds_ready = 0 the workspace needs only the chunk histograms (ha_select_histogram,
  * the first launch alone): every workgroup of the attention launch derives its row's threshold and prefixes
@@ -308,7 +310,8 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h,
  * q and k are rotated in the rotate-half convention (pairs (i, i + 64), transformers' apply_rotary_pos_emb; not
  * the interleaved pairs of efficiency/model.py:333-345) by the angle pos * inv_freq[i], the cos/sin table rounded
  * to `dtype` as transformers does; q goes to q_out [B, H, 128], k and v into the caches at token position `pos`
- * (or pos_dev[b] when pos_dev is not NULL; the caller guarantees pos_dev[b] < cache_len).  Cache strides in elements.
+ * (or pos_dev[b] when pos_dev is not NULL; a sequence whose pos_dev[b] lies outside [0, cache_len) gets its rotated query
+ * but no key or value is written for it).  Cache strides in elements.
  * ha_swiglu: out[b, i] = silu(gate_up[b, i]) * gate_up[b, F + i], silu rounded to `dtype` before the product.
  */
 int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int H, int Hkv, int pos, const int32_t *pos_dev,
@@ -321,6 +324,7 @@ int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, i
  * pos_dev[b]); the key written is hashed by the Hc key-side MLPs into kcodes at the same position, the query written
  * by the H query-side MLPs into qcodes [B, H, W] (hashattention_llama.py:567-579 rotary + cache update, :204-226 and
  * :411-414 the embeddings of the new key and the query).  Bit for bit what the two launches produce.  128-wide heads.
+ * A sequence whose pos_dev[b] lies outside [0, cache_len) (or beyond its code row) writes no key, value or key code.
  */
 int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
                         const int32_t *pos_dev, const float *inv_freq, void *q_out, void *k_cache, void *v_cache,

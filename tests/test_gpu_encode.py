@@ -206,3 +206,45 @@ def test_encode_step_rows_per_workgroup(B):
     nq = compare_codes("queries", qcodes.view(B, H, 1, 1).cpu().numpy().view(np.uint32), want_q, ql.numpy())
     print(f"  bits differing at near-zero logits: keys {nk}, queries {nq}", flush=True)
     assert (kcodes[:, :, :5] == 0).all() and (kcodes[:, :, 6:] == 0).all()
+
+
+def test_device_side_positions_outside_the_cache_write_nothing():
+    # Positions read from device memory cannot be checked on the host.  A sequence whose position lies outside its cache
+    # row must leave caches and bit-cache untouched (it would otherwise land in a neighbouring head's row or beyond the
+    # buffer); the sequences inside are written as usual.  Every kernel exits normally.
+    print("\n[case] device-side positions beyond the cache", flush=True)
+    w = small_workload(batch=4, seq_lens=[64] * 4, seed=31)
+    p = make_problem(w)
+    B, H, Hkv, Hc, d, cap = 4, w.n_q_heads, w.n_kv_heads, w.n_code_heads, 128, 40
+    wk, wq = _ops.pack_usa_weights(p.usa.k, DEV), _ops.pack_usa_weights(p.usa.q, DEV)
+    g = torch.Generator(device=DEV).manual_seed(2)
+    qkv = torch.randn(B, (H + 2 * Hkv) * d, generator=g, device=DEV).to(torch.bfloat16)
+    inv_freq = (1.0 / (500000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    pos = torch.tensor([7, cap, -3, 100000], dtype=torch.int32, device=DEV)       # inside, one past the end, negative, far out
+
+    def buffers():
+        kc = torch.full((B, Hkv, cap, d), 7.0, dtype=torch.bfloat16, device=DEV)
+        return kc, kc.clone(), torch.full((B, Hc, cap, 1), 12345, dtype=torch.int32, device=DEV)
+    k1, v1, c1 = buffers()
+    q1 = torch.zeros(B, H, d, dtype=torch.bfloat16, device=DEV)
+    qc1 = torch.zeros(B, H, 1, dtype=torch.int32, device=DEV)
+    _ops.rope_encode_step(qkv, H, Hkv, 0, inv_freq, q1, k1, v1, wk, wq, 3, 128, 32, c1, qc1, pos_dev=pos)
+    # the same launch for the first sequence alone, at its host-side position: what "written as usual" means
+    k2, v2, c2 = buffers()
+    q2 = torch.zeros(1, H, d, dtype=torch.bfloat16, device=DEV)
+    qc2 = torch.zeros(1, H, 1, dtype=torch.int32, device=DEV)
+    _ops.rope_encode_step(qkv[:1], H, Hkv, 7, inv_freq, q2, k2[:1], v2[:1], wk, wq, 3, 128, 32, c2[:1], qc2)
+    torch.cuda.synchronize()
+    assert torch.equal(k1[0], k2[0]) and torch.equal(v1[0], v2[0]) and torch.equal(c1[0], c2[0]) and torch.equal(qc1[0], qc2[0])
+    assert (k1[1:] == 7.0).all() and (v1[1:] == 7.0).all() and (c1[1:] == 12345).all()
+    # the two-launch form: ha_rope_append and ha_encode_step with the same positions
+    k3, v3, c3 = buffers()
+    q3 = torch.zeros(B, H, d, dtype=torch.bfloat16, device=DEV)
+    qc3 = torch.zeros(B, H, 1, dtype=torch.int32, device=DEV)
+    _ops.rope_append(qkv, H, Hkv, 0, inv_freq, q3, k3, v3, pos)
+    knew = torch.randn(B, Hkv, 1, d, generator=g, device=DEV).to(torch.bfloat16)
+    _ops.encode_step(knew, q3, wk, wq, 3, 128, 32, c3, qc3, pos_dev=pos)
+    torch.cuda.synchronize()
+    assert torch.equal(k3[0], k2[0]) and torch.equal(v3[0], v2[0]) and torch.equal(q3, q1)
+    assert (k3[1:] == 7.0).all() and (v3[1:] == 7.0).all() and (c3[1:] == 12345).all()
+    assert (c3[0, :, :7] == 12345).all() and (c3[0, :, 8:] == 12345).all() and (c3[0, :, 7] != 12345).all()

@@ -389,7 +389,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                                                            float *__restrict__ part_ml, void *__restrict__ out,
                                                            const float *__restrict__ win_part, int win_init, int win_recent,
                                                            const int32_t *__restrict__ seq_lens, int max_S, const FusedSel fsel,
-                                                           const AttnMask amask) {
+                                                           const AttnMask amask, int rows_per_seq) {
     using EL = Elem<E>;
     static_assert(!MK || FW == 0, "the additive mask exists for list-fed launches only");
     constexpr int NS = NT / 16;  // row streams
@@ -510,8 +510,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         r1 = (int)min((int64_t)r0 + split_rows, skip_front + n);
         ix = idx + row * idx_cap;
     }
-    const char *kb = (const char *)k + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
-    const char *vb = (const char *)v + (b * kv_sb + (h / G) * kv_sh) * EL::bytes;
+    // rows_per_seq consecutive batch entries attend to the cache of one sequence (the rows of a chunk of tokens)
+    const int64_t b_kv = rows_per_seq > 1 ? b / rows_per_seq : b;
+    const char *kb = (const char *)k + (b_kv * kv_sb + (h / G) * kv_sh) * EL::bytes;
+    const char *vb = (const char *)v + (b_kv * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;
     constexpr int STEP = NS * U;  // rows of the list consumed per step by the workgroup
 
@@ -912,9 +914,11 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
                               int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv,
                               const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace,
                               size_t workspace_bytes, const float *win_part, int win_init, int win_recent, const int32_t *seq_lens,
-                              int max_seq_len, const AttnMask amask, void *stream) {
+                              int max_seq_len, const AttnMask amask, void *stream, int rows_per_seq = 1) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
+    HA_REQUIRE(rows_per_seq >= 1 && B % rows_per_seq == 0, HA_ERR_BAD_SHAPE, "rows_per_sequence=%d must divide the %d batch entries",
+               rows_per_seq, B);
     HA_REQUIRE(idx && counts, HA_ERR_NULL_POINTER, "idx/counts is NULL");
     HA_REQUIRE(idx_cap > 0, HA_ERR_BAD_SHAPE, "idx_cap must be positive");
     const size_t need = ha_sparse_decode_workspace_bytes(B, H, idx_cap);
@@ -936,7 +940,7 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
         hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0, MK_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,   \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
                            plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len,        \
-                           FusedSel{}, amask);                                                                                    \
+                           FusedSel{}, amask, rows_per_seq);                                                                      \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
         if (plan.nsplit_max > 1) {                                                                                                \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
@@ -981,6 +985,17 @@ int ha_sparse_decode_masked(const void *q, int64_t q_stride_b, int64_t q_stride_
     return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
                               counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0,
                               AttnMask{mask, mask_stride_b, mask_len, mask_by_slot}, stream);
+}
+
+int ha_sparse_decode_rows(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                          int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int rows_per_sequence, int H, int Hkv,
+                          const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, const float *mask,
+                          int64_t mask_stride_b, int mask_len, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    HA_REQUIRE(!mask || (mask_len > 0 && mask_stride_b >= 0 && ha_aligned(mask, 4)), HA_ERR_BAD_SHAPE,
+               "mask_len must be positive, mask_stride_b non-negative, the mask 4-byte aligned");
+    return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
+                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0,
+                              mask ? AttnMask{mask, mask_stride_b, mask_len, 0} : AttnMask{}, stream, rows_per_sequence);
 }
 
 int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
@@ -1089,7 +1104,7 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
         hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b,                       \
                            q_stride_h, k, v,                                                                                      \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
-                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{});                          \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);                       \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \

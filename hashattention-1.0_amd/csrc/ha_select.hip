@@ -67,7 +67,8 @@ template <int W, int GQ, int REP>
 __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t *__restrict__ kcodes, int64_t kc_sb, int64_t kc_sh,
                                                                   const uint32_t *__restrict__ qcodes, int H, int max_S,
                                                                   const int32_t *__restrict__ seq_lens, int init, int recent,
-                                                                  int blocks, int nchunk, int vec, uint32_t *__restrict__ hist) {
+                                                                  int blocks, int nchunk, int vec, uint32_t *__restrict__ hist,
+                                                                  int rows_per_seq) {
     constexpr int NL = 32 * W + 1;
     __shared__ uint32_t lh[GQ * NL * REP];
     int c, hc, b;
@@ -81,7 +82,9 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const uint32_t
     const int beg = max(lo, c * chunk), end = min(hi, (c + 1) * chunk);
 
     ChunkRegs<W> cr;
-    if (beg < end) load_chunk<W>(kcodes + b * kc_sb + hc * kc_sh, c * chunk, blocks, beg, end, vec != 0, wave, lane, cr);
+    // rows_per_seq consecutive batch entries are queries against the codes of one sequence (the rows of a chunk of tokens)
+    if (beg < end)
+        load_chunk<W>(kcodes + (b / rows_per_seq) * kc_sb + hc * kc_sh, c * chunk, blocks, beg, end, vec != 0, wave, lane, cr);
     for (int i = tid; i < GQ * NL * REP; i += kSelThreads) lh[i] = 0;
     __syncthreads();
 
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
                                                                      const int32_t *__restrict__ seq_lens, int init, int recent,
                                                                      int blocks, int nchunk, int vec, const int32_t *__restrict__ meta,
                                                                      const int32_t *__restrict__ chunk_pre,
-                                                                     int32_t *__restrict__ out_idx, int64_t idx_cap) {
+                                                                     int32_t *__restrict__ out_idx, int64_t idx_cap, int rows_per_seq) {
     constexpr int CPL = 4 * kMaxBlocks;  // codes per lane at most
     __shared__ uint32_t s_wtot[kSelWaves][GQ];
 
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(kSelThreads) void select_compact_kernel(const uint3
 
     const int cpl = 4 * blocks;
     const int j_lane = c * chunk + (wave * HA_WAVE + lane) * cpl;
-    const uint32_t *kc = kcodes + b * kc_sb + hc * kc_sh;
+    const uint32_t *kc = kcodes + (b / rows_per_seq) * kc_sb + hc * kc_sh;
     Code<W> k[CPL];
     uint32_t vmask;  // bit e: code j_lane + e is a candidate of this chunk
     if (vec && blocks == kMaxBlocks && beg == c * chunk && end == (c + 1) * chunk) {
@@ -358,14 +361,14 @@ int static_scratch(void **out) {
 
 // ------------------------------------------------------------------------------------------------
 int validate_codes(const uint32_t *kcodes, int64_t kc_sb, int64_t kc_sh, const uint32_t *qcodes, int B, int H, int Hc, int W,
-                   int max_seq_len) {
+                   int max_seq_len, bool any_group = false) {
     HA_REQUIRE(kcodes && qcodes, HA_ERR_NULL_POINTER, "kcodes/qcodes is NULL");
     HA_REQUIRE(B > 0 && H > 0 && Hc > 0 && max_seq_len > 0, HA_ERR_BAD_SHAPE, "B, H, Hc, max_seq_len must be positive");
     HA_REQUIRE(B <= 65535 && H <= 65535, HA_ERR_BAD_SHAPE, "B and H are limited to 65535");
     HA_REQUIRE(W == 1 || W == 2, HA_ERR_BAD_SHAPE, "code words W=%d, must be 1 or 2", W);
     HA_REQUIRE(H % Hc == 0, HA_ERR_BAD_SHAPE, "H=%d not a multiple of Hc=%d", H, Hc);
     const int gq = H / Hc;
-    HA_REQUIRE(gq == 1 || gq == 2 || gq == 4 || gq == 8, HA_ERR_BAD_SHAPE, "H/Hc=%d, must be 1, 2, 4 or 8", gq);
+    HA_REQUIRE(any_group || gq == 1 || gq == 2 || gq == 4 || gq == 8, HA_ERR_BAD_SHAPE, "H/Hc=%d, must be 1, 2, 4 or 8", gq);
     HA_REQUIRE(kc_sh >= (int64_t)max_seq_len * W && (kc_sb >= kc_sh || kc_sb == 0), HA_ERR_BAD_SHAPE,
                "code strides smaller than the rows they span");
     HA_REQUIRE((int64_t)max_seq_len <= (int64_t)kMaxChunks * kMaxBlocks * kBlock, HA_ERR_BAD_SHAPE, "max_seq_len above %d",
@@ -381,7 +384,7 @@ extern "C" {
 
 int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H,
                      int Hc, int W, int max_seq_len, const int32_t *seq_lens, uint8_t *scores, void *stream) {
-    int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len);
+    int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, true);
     if (st) return st;
     HA_REQUIRE(scores, HA_ERR_NULL_POINTER, "scores is NULL");
     if ((st = ha_require_device())) return st;
@@ -408,7 +411,8 @@ size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
 #define HA_SELECT_LAUNCH(W_, GQ_, REP_)                                                                                           \
     do {                                                                                                                          \
         hipLaunchKernelGGL((select_hist_kernel<W_, GQ_, REP_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,  \
-                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.hist);  \
+                           qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.hist,   \
+                           rows_per_seq);                                                                                         \
         HA_CHECK_LAUNCH("select_hist_kernel");                                                                                    \
         if (!out_counts) break; /* ha_select_histogram: chunk histograms only */                                                  \
         hipLaunchKernelGGL(select_threshold_kernel<W_>, dim3(H, B), dim3(kSelThreads), 0, s, ws.hist, H, max_seq_len, seq_lens,   \
@@ -418,16 +422,22 @@ size_t ha_select_workspace_bytes(int B, int H, int Hc, int W, int max_seq_len) {
         if (!out_idx) break; /* ha_select_prepare: thresholds and offsets only */                                                 \
         hipLaunchKernelGGL((select_compact_kernel<W_, GQ_>), grid, dim3(kSelThreads), 0, s, kcodes, kc_stride_b, kc_stride_h,     \
                            qcodes, H, max_seq_len, seq_lens, init_budget, recent_budget, plan.blocks, plan.nchunk, vec, ws.meta,  \
-                           ws.chunk_pre, out_idx, idx_cap);                                                                       \
+                           ws.chunk_pre, out_idx, idx_cap, rows_per_seq);                                                         \
         HA_CHECK_LAUNCH("select_compact_kernel");                                                                                 \
     } while (0)
 
 static int select_impl(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,
                        int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
                        int mode, int depth, int algo, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
-                       size_t workspace_bytes, void *stream, bool prepare_only, bool use_static_scratch = false) {
+                       size_t workspace_bytes, void *stream, bool prepare_only, bool use_static_scratch = false,
+                       int rows_per_seq = 1) {
     int st = validate_codes(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len);
     if (st) return st;
+    HA_REQUIRE(rows_per_seq >= 1 && B % rows_per_seq == 0, HA_ERR_BAD_SHAPE, "rows_per_sequence=%d must divide the %d batch entries",
+               rows_per_seq, B);
+    HA_REQUIRE(rows_per_seq == 1 || algo == HA_SELECT_ALGO_AUTO || algo == HA_SELECT_ALGO_HISTOGRAM, HA_ERR_BAD_SHAPE,
+               "several rows per sequence take the histogram method");
+    if (rows_per_seq > 1) algo = HA_SELECT_ALGO_HISTOGRAM;
     HA_REQUIRE(prepare_only || (out_idx && out_counts), HA_ERR_NULL_POINTER, "out_idx/out_counts is NULL");
     HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && heavy_budget >= 0.0 && depth >= 0, HA_ERR_BAD_SHAPE,
                "budgets and depth must be non-negative");
@@ -503,6 +513,16 @@ int ha_select_static(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
     return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
                        heavy_budget, mode, depth, HA_SELECT_ALGO_HISTOGRAM, out_idx, idx_cap, out_counts, nullptr, 0, stream, false,
                        true);
+}
+
+int ha_select_rows(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int rows_per_sequence,
+                   int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget,
+                   double heavy_budget, int mode, int depth, int32_t *out_idx, int64_t idx_cap, int32_t *out_counts, void *workspace,
+                   size_t workspace_bytes, void *stream) {
+    HA_REQUIRE(seq_lens, HA_ERR_NULL_POINTER, "ha_select_rows needs one length per row");
+    return select_impl(kcodes, kc_stride_b, kc_stride_h, qcodes, B, H, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget,
+                       heavy_budget, mode, depth, HA_SELECT_ALGO_HISTOGRAM, out_idx, idx_cap, out_counts, workspace, workspace_bytes,
+                       stream, false, false, rows_per_sequence);
 }
 
 int ha_select_histogram(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hc,

@@ -70,6 +70,11 @@ def load_library() -> C.CDLL:
     lib.ha_select.restype = i32
     lib.ha_select.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, i32,
                               vp, i64, vp, vp, sz, vp]
+    lib.ha_select_rows.restype = i32
+    lib.ha_select_rows.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, vp, i64, vp, vp, sz, vp]
+    lib.ha_sparse_decode_rows.restype = i32
+    lib.ha_sparse_decode_rows.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, f32,
+                                          vp, i64, i32, vp, vp, sz, vp]
     lib.ha_select_static_max_bytes.restype = sz
     lib.ha_select_static.restype = i32
     lib.ha_select_static.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, i32, i32, f64, i32, i32, vp, i64, vp, vp]
@@ -286,6 +291,41 @@ def select(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_len
     _check(lib.ha_select(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H, Hc, W, max_seq_len,
                          _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth, algo,
                          _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select")
+
+
+def select_rows(kcodes: torch.Tensor, qcodes: torch.Tensor, rows_per_sequence: int, max_seq_len: int, seq_lens: torch.Tensor,
+                init_budget: int, recent_budget: int, heavy_budget: float, out_idx: torch.Tensor, out_counts: torch.Tensor,
+                ws: torch.Tensor, mode: int = HA_SELECT_SIMPLE, depth: int = 0) -> None:
+    """`select` for chunks of tokens: qcodes [n_rows, H, W], seq_lens [n_rows], lists [n_rows, H, cap]; row n is a query
+    against the codes of sequence n // rows_per_sequence (kcodes [n_seq, Hc, S_cap, W])."""
+    _require_cuda(kcodes, qcodes, seq_lens, out_idx, out_counts, ws)
+    lib = load_library()
+    n_seq, Hc, _, W = kcodes.shape
+    n_rows, H = qcodes.shape[0], qcodes.shape[1]
+    assert n_rows == n_seq * rows_per_sequence and qcodes.is_contiguous() and kcodes.stride(3) == 1 and kcodes.stride(2) == W
+    assert out_idx.is_contiguous() and out_idx.dtype == torch.int32 and out_counts.is_contiguous() and out_counts.dtype == torch.int32
+    assert out_idx.shape[0] == n_rows and seq_lens.dtype == torch.int32 and seq_lens.is_contiguous() and seq_lens.numel() == n_rows
+    _check(lib.ha_select_rows(_ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), n_rows, rows_per_sequence, H, Hc, W,
+                              max_seq_len, _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget), mode, depth,
+                              _ptr(out_idx), out_idx.shape[2], _ptr(out_counts), _ptr(ws), ws.numel(), _stream(kcodes)), "ha_select_rows")
+
+
+def sparse_decode_rows(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rows_per_sequence: int, idx: torch.Tensor,
+                       counts: torch.Tensor, sm_scale: float, out: torch.Tensor, ws: torch.Tensor,
+                       mask: Optional[torch.Tensor] = None) -> None:
+    """`sparse_decode` for chunks of tokens: q, out [n_rows, H, 128], idx [n_rows, H, cap]; row n attends to the cache of
+    sequence n // rows_per_sequence (k, v [n_seq, Hkv, S_cap, 128]).  mask: optional fp32 [n_rows, n], by token position."""
+    _require_cuda(q, k, v, idx, counts, out, ws, mask)
+    lib = load_library()
+    n_rows, H, _ = q.shape
+    assert n_rows == k.shape[0] * rows_per_sequence and out.is_contiguous() and out.dtype == q.dtype and out.shape == q.shape
+    assert idx.is_contiguous() and counts.is_contiguous() and idx.shape[0] == n_rows
+    if mask is not None:
+        assert mask.dtype == torch.float32 and mask.dim() == 2 and mask.shape[0] == n_rows and mask.stride(1) == 1
+    _check(lib.ha_sparse_decode_rows(*_kv_args(q, k, v), n_rows, rows_per_sequence, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
+                                     float(sm_scale), _ptr(mask), mask.stride(0) if mask is not None else 0,
+                                     mask.shape[1] if mask is not None else 0, _ptr(out), _ptr(ws), ws.numel(), _stream(q)),
+           "ha_sparse_decode_rows")
 
 
 def select_static(kcodes: torch.Tensor, qcodes: torch.Tensor, max_seq_len: int, seq_lens: Optional[torch.Tensor],

@@ -207,11 +207,22 @@ class USA(nn.Module):
         b, a, s, d = vectors.shape
         if a != self.num_heads:
             raise ValueError(f"expected {self.num_heads} heads, got {a}")
-        w = _ops.pack_usa_weights(self.kernel_layers(side), vectors.device)
+        w = self._packed_weights(side, vectors.device)
         codes = torch.empty(b, a, s, self.lth_final_dim // 32, dtype=torch.int32, device=vectors.device)
         logits = _ops.encode_pack(vectors, w, self.kernel_num_layers, self.int_dim, self.lth_final_dim, codes,
                                   arith=self.arith, want_logits=True)
         return torch.sign(logits), codes
+
+    def _packed_weights(self, side: str, device) -> torch.Tensor:
+        """The side's weights in the kernels' blob form, repacked only when a parameter changed (tensor versions) or moved."""
+        params = [t for head in self.layers(side) for wb in head for t in wb]
+        key = (str(device),) + tuple((t.data_ptr(), t._version, t.dtype) for t in params)
+        cache = self.__dict__.setdefault("_packed", {})
+        hit = cache.get(side)
+        if hit is None or hit[0] != key:
+            hit = (key, _ops.pack_usa_weights(self.kernel_layers(side), device))
+            cache[side] = hit
+        return hit[1]
 
     def k_embedding(self, vectors: torch.Tensor, hard: bool = False) -> torch.Tensor:
         """[b, heads, s, d] -> embeddings [b, heads, s, D] in fp32: signs (hard) or tanh (soft) (reference :204-214)."""
@@ -241,10 +252,9 @@ class USA(nn.Module):
         ksign, kcodes = self._embed(Kh.contiguous(), "k", True, prepared=True)
         _, qcodes = self._embed(Qh.contiguous(), "q", True, prepared=True)
         D = self.lth_final_dim
-        span = torch.empty(b, a, t, s, dtype=K.dtype, device=K.device)
-        for i in range(t):
-            ham = _ops.hamming_score(kcodes, qcodes[:, :, i].contiguous(), s)
-            span[:, :, i] = (D - 2 * ham.to(torch.int32)).to(K.dtype)
+        # the t query tokens of a head are t "query heads" of its code head: one scoring launch for all of them
+        ham = _ops.hamming_score(kcodes, qcodes.reshape(b, a * t, qcodes.shape[-1]), s).view(b, a, t, s)
+        span = (D - 2 * ham.to(torch.int32)).to(K.dtype)
         span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
         return span, ksign.to(K.dtype)
 
@@ -441,28 +451,13 @@ class HeavyHitterMixin:
             finally:
                 hl.heavy_budget = saved
             return out
-        # a chunk of q_len rows: the new keys join the bit-cache, then every row is one "sequence" of the kernels - same
-        # codes and K/V (batch stride 0), its own query code and its own length S - q_len + i + 1 (reference :423-428)
-        dev = query_states.device
+        # a chunk of q_len rows: the new keys join the bit-cache, then every row of every sequence is one batch entry of ONE
+        # selection and ONE attention launch - the codes and K/V of its sequence, its own query code and its own length
+        # S - q_len + i + 1 (reference :423-428)
         hl.encode_keys(key_hash[:, :, S - q_len:S], pos0=S - q_len)
         hl.n_cached = S
-        lens = torch.arange(S - q_len + 1, S + 1, dtype=torch.int32, device=dev)
-        cap = S if hl.mode != _ops.HA_SELECT_SIMPLE else min(S, hl.init_budget + hl.recent_budget + heavy)
-        qc = torch.zeros(1, H, q_len, hl.W, dtype=torch.int32, device=dev)
-        idx = torch.empty(q_len, H, cap, dtype=torch.int32, device=dev)
-        cnt = torch.empty(q_len, H, dtype=torch.int32, device=dev)
-        ws_s = _ops.workspace(_ops.select_workspace_bytes(q_len, H, hl.Hc, hl.W, S), dev)
-        ws_a = _ops.workspace(_ops.sparse_decode_workspace_bytes(q_len, H, cap), dev)
-        o_b = torch.empty(q_len, H, d, dtype=query_states.dtype, device=dev)
-        for bi in range(b):
-            _ops.encode_pack(query_hash[bi:bi + 1], hl.wq, hl.num_layers, hl.int_dim, hl.final_dim, qc, 0, None, hl.arith)
-            _ops.select(hl.codes[bi:bi + 1].expand(q_len, -1, -1, -1), qc[0].transpose(0, 1).contiguous(), S, lens, hl.init_budget,
-                        hl.recent_budget, heavy_abs, idx, cnt, ws_s, hl.mode, hl.depth)
-            _ops.sparse_decode(query_states[bi].transpose(0, 1).contiguous(), key_states[bi:bi + 1].expand(q_len, -1, -1, -1),
-                               value_states[bi:bi + 1].expand(q_len, -1, -1, -1), idx, cnt, hl.sm_scale, o_b, ws_a,
-                               mask=None if amask is None else amask[bi])
-            out[bi] = o_b.transpose(0, 1)
-        return out
+        return hl.chunk_step(query_states, key_states, value_states, S, out, heavy_abs,
+                             q_hash=None if query_hash is query_states else query_hash, attn_mask=amask)
 
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
         bsz, q_len, _ = hidden_states.shape

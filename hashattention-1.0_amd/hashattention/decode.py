@@ -197,6 +197,53 @@ class HashDecodeLayer:
             self.attend(q3, k_cache, v_cache, out)
         return out
 
+    # ------------------------------------------------------------------ a chunk of several new tokens per sequence
+    def _chunk_buffers(self, n_rows: int, cap: int, s_max: int, dtype: torch.dtype):
+        """Lists, counts, query codes, output rows and workspaces of `chunk_step`, kept between calls and grown when a
+        chunk needs more."""
+        key = (n_rows, dtype)
+        cb = getattr(self, "_chunk", None)
+        if cb is None or cb["key"] != key or cb["cap"] < cap or cb["s_max"] < s_max:
+            dev = self.device
+            cap_a, s_a = max(cap, cb["cap"] if cb and cb["key"] == key else 0), max(s_max, self.S_cap)
+            cb = dict(key=key, cap=cap_a, s_max=s_a,
+                      qc=torch.zeros(self.B, self.H, n_rows // self.B, self.W, dtype=torch.int32, device=dev),
+                      qc_rows=torch.zeros(n_rows, self.H, self.W, dtype=torch.int32, device=dev),
+                      idx=torch.zeros(n_rows, self.H, cap_a, dtype=torch.int32, device=dev),
+                      cnt=torch.zeros(n_rows, self.H, dtype=torch.int32, device=dev),
+                      out=torch.empty(n_rows, self.H, self.d, dtype=dtype, device=dev),
+                      q_rows=torch.empty(n_rows, self.H, self.d, dtype=dtype, device=dev),
+                      lens=torch.zeros(n_rows, dtype=torch.int32, device=dev),
+                      ramp=torch.arange(n_rows, dtype=torch.int32, device=dev) % (n_rows // self.B),
+                      ws_s=_ops.workspace(_ops.select_workspace_bytes(n_rows, self.H, self.Hc, self.W, s_a), dev),
+                      ws_a=_ops.workspace(_ops.sparse_decode_workspace_bytes(n_rows, self.H, cap_a), dev))
+            self._chunk = cb
+        return cb
+
+    def chunk_step(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, seq_len: int, out: torch.Tensor,
+                   heavy_budget: float, q_hash: Optional[torch.Tensor] = None, attn_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q [B, H, T, d]: T new query tokens per sequence (1 < T <= 128) whose keys are already in the caches and in the
+        bit-cache (`encode_keys`); row i attends as the query at position seq_len - T + i with its own causal windows
+        (hashattention_llama.py:423-428).  Three launches for the whole batch: the query codes, ONE selection and ONE
+        attention over the B * T rows (`ha_select_rows`, `ha_sparse_decode_rows`).  out [B, H, T, d].
+        `q_hash`: what the query-side hash MLPs read when that is not q itself; attn_mask fp32 [B, T, >= seq_len]."""
+        B, H, T, d = q.shape
+        S = seq_len
+        n_rows = B * T
+        cap = S if self.mode != _ops.HA_SELECT_SIMPLE else max(1, min(S, self.init_budget + self.recent_budget + self.heavy_count(S)))
+        cb = self._chunk_buffers(n_rows, cap, S, q.dtype)
+        qh = q if q_hash is None else q_hash
+        _ops.encode_pack(qh, self.wq, self.num_layers, self.int_dim, self.final_dim, cb["qc"], 0, None, self.arith)
+        cb["qc_rows"].view(B, T, H, self.W).copy_(cb["qc"].transpose(1, 2))
+        cb["q_rows"].view(B, T, H, d).copy_(q.transpose(1, 2))
+        torch.add(cb["ramp"], S - T + 1, out=cb["lens"])                    # row (b, i) sees keys [0, S - T + i]
+        _ops.select_rows(self.codes, cb["qc_rows"], T, S, cb["lens"], self.init_budget, self.recent_budget, heavy_budget,
+                         cb["idx"], cb["cnt"], cb["ws_s"], self.mode, self.depth)
+        mask = None if attn_mask is None else attn_mask.reshape(n_rows, attn_mask.shape[-1])
+        _ops.sparse_decode_rows(cb["q_rows"], k_cache, v_cache, T, cb["idx"], cb["cnt"], self.sm_scale, cb["out"], cb["ws_a"], mask=mask)
+        out.copy_(cb["out"].view(B, T, H, d).transpose(1, 2))
+        return out
+
     def step_from_qkv(self, qkv: torch.Tensor, pos: int, inv_freq: torch.Tensor, q_rot: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """The decode step of a uniform batch straight from the fused QKV projection of the new token, qkv [B, (H + 2 Hkv) * 128]:

@@ -138,7 +138,8 @@ int ha_encode_pack_prefill(const void *x, int64_t x_stride_b, int64_t x_stride_h
 
 /*
  * Hamming distance of every cached code to the query code: scores[b, h, j] =
- * popcount(kcodes[b, h / (H/Hc), j] ^ qcodes[b, h]) for j < seq_len[b].  Diagnostic/test entry;
+ * popcount(kcodes[b, h / (H/Hc), j] ^ qcodes[b, h]) for j < seq_len[b] (any number of query heads per code head:
+ * the t query tokens of USA.forward are t * H "heads").  Diagnostic/test entry;
  * ha_select fuses this.  Replaces efficiency/kernels/bit_count_uint32.py:4-33, bit_count_long.py:4-33
  * and the xor of torchatt.py:58 (span = final_dim - 2 * distance, hashattention_llama.py:180-187).
  *   kcodes [B, Hc, ., W] strides kc_stride_{b,h} words; qcodes [B, H, W] contiguous;
@@ -170,6 +171,30 @@ int ha_select(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, 
               int init_budget, int recent_budget, double heavy_budget, int mode, int depth, int algo,
               int32_t *out_idx, int64_t idx_cap, int32_t *out_counts,
               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * ha_select and ha_sparse_decode for a chunk of several new tokens per sequence (hashattention_llama.py:423-428: the
+ * decode branch takes up to 128 query tokens, each with its own causal windows and budget).  The B batch entries are
+ * rows: rows_per_sequence consecutive ones belong to one sequence, i.e. entry n reads the codes (the K/V cache) of
+ * sequence n / rows_per_sequence - kc_stride_b and kv_stride_b are strides between SEQUENCES - and has its own query
+ * (qcodes [B, H, W], q [B, H, 128]), its own length seq_lens[n] (required), index list, count, output row and, for the
+ * attention, its own mask row (mask may be NULL; by token position, as ha_sparse_decode_masked with mask_by_slot = 0).
+ * One call serves every row of every sequence: the number of launches of a chunk does not depend on the batch.  The
+ * selection uses the histogram method; workspaces are sized for B rows (ha_select_workspace_bytes(B, ...),
+ * ha_sparse_decode_workspace_bytes(B, ...)).
+ */
+int ha_select_rows(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                   int B, int rows_per_sequence, int H, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                   int init_budget, int recent_budget, double heavy_budget, int mode, int depth,
+                   int32_t *out_idx, int64_t idx_cap, int32_t *out_counts,
+                   void *workspace, size_t workspace_bytes, void *stream);
+int ha_sparse_decode_rows(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                          const void *k, const void *v, int kv_dtype,
+                          int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                          int B, int rows_per_sequence, int H, int Hkv,
+                          const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale,
+                          const float *mask, int64_t mask_stride_b, int mask_len,
+                          void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * ha_select without a workspace argument, for callers that cannot allocate device memory (code under HIP graph capture,

@@ -114,3 +114,46 @@ def test_step_replayed_from_a_hip_graph_matches_eager(fused):
         assert torch.equal(out, want), i
         scratch = torch.randn(1 << 20, device=DEV).sum().item()     # unrelated eager work between replays
         assert scratch == scratch
+
+
+@pytest.mark.parametrize("hc", [2, 8])
+@pytest.mark.parametrize("batch,T,masked", [(3, 7, False), (2, 5, True), (1, 128, False)])
+def test_chunk_of_tokens_in_one_selection_and_one_attention_launch(batch, T, masked, hc):
+    # a chunk of T new tokens per sequence (hashattention_llama.py:423-428): row i of every sequence attends with its own
+    # causal windows and budget.  All B * T rows go through ONE ha_select_rows and ONE ha_sparse_decode_rows call; output
+    # and kept sets against the reference layer's dense restatement (causal + optional padding mask added to the scores)
+    print(f"\n[case] chunk step B={batch} T={T} masked={masked} Hc={hc}", flush=True)
+    S = 700
+    w = small_workload(batch=batch, seq_lens=[S] * batch, n_code_heads=hc, dtype=torch.float32, seed=31 + T)
+    p = make_problem(w)
+    k, v = p.k.to(DEV), p.v.to(DEV)
+    layer = _layer(w, p)
+    layer.allocate(batch, S)
+    layer.encode_keys(k)
+    layer.n_cached = S
+    q = torch.randn(batch, w.n_q_heads, T, w.head_dim, generator=torch.Generator().manual_seed(9))
+    add = torch.zeros(batch, 1, T, S)
+    rows = torch.arange(T).view(T, 1) + S - T
+    add.masked_fill_((torch.arange(S).view(1, S) > rows).view(1, 1, T, S), torch.finfo(torch.float32).min)
+    amask = None
+    if masked:                      # left padding of different lengths, as transformers hands it to the layer
+        for b in range(batch):
+            add[b, :, :, :3 + 2 * b] = torch.finfo(torch.float32).min
+        amask = add[:, 0].contiguous().to(DEV)
+    out = torch.empty(batch, w.n_q_heads, T, w.head_dim, device=DEV)
+    for rep in range(2):            # the second call reuses the buffers of the first
+        heavy = layer.heavy_count(S)            # the reference sizes every row's budget by the cache length (:431-434)
+        layer.chunk_step(q.to(DEV), k, v, S, out, 0.0 if heavy == 0 else heavy + 0.5, attn_mask=amask)
+        ref, mask = orc.reference_decode_attention(q, p.k, p.v, p.usa.k, p.usa.q, w.init_budget, w.recent_budget, w.heavy_budget,
+                                                   attention_mask=add)
+        idx = layer._chunk["idx"].cpu().numpy()
+        cnt = layer._chunk["cnt"].cpu().numpy()
+        causal = (add[0, 0] == 0) if not masked else (torch.arange(S).view(1, S) <= rows)
+        for b in range(batch):
+            for i in range(T):
+                for h in range(w.n_q_heads):
+                    got = np.zeros(S, dtype=bool)
+                    got[idx[b * T + i, h, :cnt[b * T + i, h]]] = True
+                    assert np.array_equal(got, (mask[b, h, i] & causal[i]).numpy()), (b, i, h)
+        err = (out.cpu() - ref).abs().max().item()
+        assert err < 2e-5, err

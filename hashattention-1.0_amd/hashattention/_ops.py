@@ -63,6 +63,9 @@ def load_library() -> C.CDLL:
     lib.ha_encode_pack_prefill.restype = i32
     lib.ha_encode_pack_prefill.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32,
                                            vp, i64, i64, i32, vp, vp]
+    lib.ha_encode_pack_prefill_f32.restype = i32
+    lib.ha_encode_pack_prefill_f32.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i32, i32, i32, i32,
+                                               vp, i64, i64, i32, vp, vp]
     lib.ha_hamming_score.restype = i32
     lib.ha_hamming_score.argtypes = [vp, i64, i64, vp, i32, i32, i32, i32, i32, vp, vp, vp]
     lib.ha_select_workspace_bytes.restype = sz
@@ -255,6 +258,24 @@ def encode_pack_prefill(x: torch.Tensor, weights_bf16: torch.Tensor, n_layers: i
                                       _ptr(weights_bf16), n_layers, d, int_dim, final_dim,
                                       _ptr(codes), codes.stride(0), codes.stride(1), pos0, _ptr(pos_dev), _stream(x)),
            "ha_encode_pack_prefill")
+
+
+def encode_pack_prefill_f32(x: torch.Tensor, weights: torch.Tensor, n_layers: int, int_dim: int, final_dim: int,
+                            codes: torch.Tensor, pos0: int = 0, pos_dev: Optional[torch.Tensor] = None) -> None:
+    """fp32 MFMA bulk encode for fp32 hash modules; tensors as `encode_pack` (weights from `pack_usa_weights`)."""
+    _require_cuda(x, weights, codes, pos_dev)
+    lib = load_library()
+    B, xh, T, d = x.shape
+    n_heads = weights.shape[0]
+    assert weights.dtype == torch.float32 and weights.is_contiguous()
+    assert weights.shape[1] == lib.ha_usa_packed_floats(n_layers, d, int_dim, final_dim)
+    assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3] and codes.dtype == torch.int32
+    if pos_dev is None:
+        assert pos0 + T <= codes.shape[2]
+    _check(lib.ha_encode_pack_prefill_f32(_ptr(x), _DTYPE[x.dtype], x.stride(0), x.stride(1), x.stride(2), B, xh, n_heads, T,
+                                          _ptr(weights), n_layers, d, int_dim, final_dim,
+                                          _ptr(codes), codes.stride(0), codes.stride(1), pos0, _ptr(pos_dev), _stream(x)),
+           "ha_encode_pack_prefill_f32")
 
 
 # ------------------------------------------------------------------------------------------ score / select

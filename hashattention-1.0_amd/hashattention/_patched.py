@@ -434,8 +434,7 @@ class HeavyHitterMixin:
         if hl.n_cached < S - q_len:          # keys cached by a prefill (or by dense steps): encode them in bulk
             lo = hl.n_cached
             bulk = key_hash[:, :, lo:S - q_len]
-            hl.encode_keys(bulk, pos0=lo, use_mfma=(hl.arith == _ops.HA_ARITH_BF16 and bulk.dtype == torch.bfloat16
-                                                    and hl.wk_bf16 is not None))
+            hl.encode_keys_bulk(bulk, pos0=lo)
             hl.n_cached = S - q_len
         out = torch.empty(b, H, q_len, d, dtype=query_states.dtype, device=query_states.device)
         # the reference takes the heavy budget from the full key length for every query row (:431-434)

@@ -107,6 +107,21 @@ class HashDecodeLayer:
         else:
             _ops.encode_pack(k, self.wk, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev, self.arith)
 
+    # from this many keys per sequence on, a bulk encode goes to the matrix cores (below, the latency-built kernel wins)
+    BULK_MIN_TOKENS = 256
+
+    def encode_keys_bulk(self, k: torch.Tensor, pos0: int = 0, pos_dev: Optional[torch.Tensor] = None) -> None:
+        """`encode_keys` for the keys a prefill left behind: on the matrix cores in the arithmetic of the hash module -
+        bf16 MFMA for a module kept in bf16 (bf16 keys), fp32 MFMA for a module kept in fp32 - when the MLP is 128 wide
+        throughout; the scalar kernel otherwise and for a handful of keys."""
+        wide = self.wk_bf16 is not None and k.shape[2] >= self.BULK_MIN_TOKENS     # 128-wide layers: the MFMA shapes
+        if wide and self.arith == _ops.HA_ARITH_BF16 and k.dtype == torch.bfloat16:
+            _ops.encode_pack_prefill(k, self.wk_bf16, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev)
+        elif wide and self.arith == _ops.HA_ARITH_F32:
+            _ops.encode_pack_prefill_f32(k, self.wk, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev)
+        else:
+            _ops.encode_pack(k, self.wk, self.num_layers, self.int_dim, self.final_dim, self.codes, pos0, pos_dev, self.arith)
+
     def encode_query(self, q: torch.Tensor) -> None:
         """q [B, H, 1, d] -> self.qcodes."""
         _ops.encode_pack(q, self.wq, self.num_layers, self.int_dim, self.final_dim, self.qcodes, 0, None, self.arith)

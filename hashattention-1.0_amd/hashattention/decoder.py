@@ -141,10 +141,8 @@ class LlamaShapedDecoder:
         for l in range(self.L):
             self.k_cache[l][:, :, :S] = keys[l]
             self.v_cache[l][:, :, :S] = values[l]
-            # as the patched layer hashes a prefilled cache: the MFMA encoder for a bf16 hash, the exact kernel otherwise
-            self.hash[l].encode_keys(self.k_cache[l][:, :, :S], pos0=0,
-                                     use_mfma=self.dtype == torch.bfloat16 and self.hash[l].arith == _ops.HA_ARITH_BF16
-                                     and self.hash[l].wk_bf16 is not None)
+            # as the patched layer hashes a prefilled cache: on the matrix cores, in the arithmetic of the hash module
+            self.hash[l].encode_keys_bulk(self.k_cache[l][:, :, :S], pos0=0)
             self.hash[l].n_cached = S
         self.seq_len = S if lengths is None else max(lengths)
         self.lengths = lengths

@@ -137,6 +137,20 @@ int ha_encode_pack_prefill(const void *x, int64_t x_stride_b, int64_t x_stride_h
                            void *stream);
 
 /*
+ * Bulk (prefill) encode for hash modules kept in fp32 (what load_usa returns, hashattention_llama.py:640-646; the layer
+ * casts the keys to the module's dtype, :406): the mapping of ha_encode_pack in HA_ARITH_F32, computed as chained fp32
+ * MFMA GEMMs per 256-token tile.  x of x_dtype (bf16 / fp16 rows are widened exactly), head_dim == int_dim == 128,
+ * `weights` the same packed fp32 blob ha_encode_pack reads.  The matrix core sums in its own order, so a sign bit can
+ * differ from ha_encode_pack's where the logit is within fp32 rounding of zero.  Replaces the same un-timed prefill
+ * encode (efficiency/kernels/torchatt.py:183-184) as ha_encode_pack_prefill.
+ */
+int ha_encode_pack_prefill_f32(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_t,
+                               int B, int x_heads, int n_heads, int T,
+                               const float *weights, int n_layers, int head_dim, int int_dim, int final_dim,
+                               uint32_t *codes, int64_t c_stride_b, int64_t c_stride_h, int pos0, const int32_t *pos_dev,
+                               void *stream);
+
+/*
  * Hamming distance of every cached code to the query code: scores[b, h, j] =
  * popcount(kcodes[b, h / (H/Hc), j] ^ qcodes[b, h]) for j < seq_len[b] (any number of query heads per code head:
  * the t query tokens of USA.forward are t * H "heads").  Diagnostic/test entry;

@@ -32,12 +32,59 @@ constexpr int wp_bytes(int out) { return (out / 32) * kKSteps * 64 * 16; }
 
 // SiLU of a Linear output in bf16 arithmetic: the accumulator is rounded to bf16, y * sigmoid(y) is evaluated
 // in fp32 with the hardware exp2 and reciprocal (1 ulp each, far below the bf16 rounding that follows in the
-// caller).  Two of the five operations are quarter-rate transcendentals: with 256 activations per (token,
-// head) against 72 MFMA cycles, this, not the matrix pipe, bounds the kernel.
+// caller).  Evaluated per activation it costs ~13 issue slots, two of them transcendentals, against the 72 MFMA
+// cycles per (token, head) that 256 activations share: three times the matrix work.  The kernel uses it to build
+// the table below.
 __device__ __forceinline__ float silu_bf16(float acc) {
     const float y = (float)(__bf16)acc;
     const float t = __builtin_amdgcn_exp2f(y * -1.4426950408889634f);
     return y * __builtin_amdgcn_rcpf(1.0f + t);
+}
+
+// The activation as a table.  Its input is a bf16 value, so bf16(SiLU(y)) is a function of 16 bits: the workgroup keeps
+// it in LDS for every |y| from 2^-20 up (all larger magnitudes, infinities and NaNs included), one 32-bit entry per
+// magnitude: low half the result for +|y|, high half for -|y|, both computed with silu_bf16 itself, so the table gives
+// what the formula gives.  Magnitudes below 2^-20 read the entry of 2^-20: an absolute error under 2^-21 on a value that
+// is added to sums of order one in fp32.  A pair of activations then costs one packed conversion, a packed clamp, a few
+// integer operations, two LDS reads and one byte permute instead of four transcendentals.
+constexpr uint32_t kTabLo = 107u << 7;                    // bf16 bits of 2^-20
+constexpr int kTabEntries = 0x8000 - (int)kTabLo;        // magnitudes kTabLo .. 0x7fff
+constexpr int kTabBytes = kTabEntries * 4;
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void fill_silu_table(uint32_t *tab, int tid) {
+    for (int i = tid; i < kTabEntries; i += kMfThreads) {
+        const uint32_t mag = kTabLo + (uint32_t)i;
+        uint32_t pos, neg;
+        if (mag >= (134u << 7) && mag <= 0x7f80u) {      // |y| >= 2^7, not NaN: exp2 under- / overflows, SiLU(y) = y or -0
+            pos = mag;
+            neg = 0x8000u;
+        } else {
+            const float y = __uint_as_float(mag << 16);
+            pos = __builtin_bit_cast(unsigned short, (__bf16)silu_bf16(y));
+            neg = __builtin_bit_cast(unsigned short, (__bf16)silu_bf16(-y));
+        }
+        tab[i] = pos | (neg << 16);
+    }
+}
+
+// bf16(SiLU(bf16(a0))) | bf16(SiLU(bf16(a1))) << 16 through the table
+__device__ __forceinline__ uint32_t silu_pair_lut(float a0, float a1, const uint32_t *tab) {
+    f32x2 a;
+    a.x = a0, a.y = a1;
+    const uint32_t p = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, bf16x2));
+    const u16x2 mag = __builtin_bit_cast(u16x2, p & 0x7fff7fffu);
+    u16x2 lo;
+    lo.x = (unsigned short)kTabLo, lo.y = (unsigned short)kTabLo;
+    const uint32_t pc = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(mag, lo));
+    const uint32_t d0 = tab[(int)(pc & 0xffffu) - (int)kTabLo];
+    const uint32_t d1 = tab[(int)(pc >> 16) - (int)kTabLo];
+    // result half k comes from entry k: its high half when activation k is negative, else its low half
+    const uint32_t sel = 0x05040100u + ((p >> 15) & 0x00010001u) * 0x0202u;
+    return __builtin_amdgcn_perm(d1, d0, sel);
 }
 
 // Copy W [out][128] (bf16, global) into the MFMA A-operand order.  c_perm selects the k permutation:
@@ -81,8 +128,8 @@ __device__ __forceinline__ void layer_mfma(const uint4 *Wp, const float *bias, c
     }
 }
 
-// hidden layer: 128 -> 128 with SiLU; output is the next layer's B operand set
-__device__ __forceinline__ void hidden_layer(const uint4 *Wp, const float *bias, const bf16x8 (&Bin)[kKSteps][2],
+// hidden layer: 128 -> 128 with SiLU (through the table); output is the next layer's B operand set
+__device__ __forceinline__ void hidden_layer(const uint4 *Wp, const float *bias, const uint32_t *tab, const bf16x8 (&Bin)[kKSteps][2],
                                              bf16x8 (&Bout)[kKSteps][2], int lane) {
 #pragma unroll
     for (int ob = 0; ob < 4; ++ob) {
@@ -91,10 +138,17 @@ __device__ __forceinline__ void hidden_layer(const uint4 *Wp, const float *bias,
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-            for (int p = 0; p < 2; ++p)
+            for (int p = 0; p < 2; ++p) {
+                uint32_t w[4];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) Bout[2 * ob + p][nb][j] = (__bf16)silu_bf16(acc[0][nb][8 * p + j]);
+                for (int m = 0; m < 4; ++m) w[m] = silu_pair_lut(acc[0][nb][8 * p + 2 * m], acc[0][nb][8 * p + 2 * m + 1], tab);
+                Bout[2 * ob + p][nb] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+            }
     }
+}
+
+template <int NL, int D> constexpr int lds_bytes() {
+    return (NL - 1) * wp_bytes(kDim) + wp_bytes(D) + ((NL - 1) * kDim + D) * 4 + (NL > 1 ? kTabBytes : 0);
 }
 
 // grid (wg_per_seq, n_heads, B).  NL layers, final width D (32 or 64).
@@ -104,16 +158,19 @@ __global__ __launch_bounds__(kMfThreads) void encode_mfma_kernel(const __bf16 *_
                                                                  const __bf16 *__restrict__ wblob, int64_t per_head,
                                                                  uint32_t *__restrict__ codes, int64_t c_sb, int64_t c_sh, int pos0,
                                                                  const int32_t *__restrict__ pos_dev) {
-    extern __shared__ uint4 smem[];
+    // one static LDS block per instantiation: every address in it is a compile-time constant, so a table read needs no
+    // address arithmetic beyond the scaled index (the rest folds into the instruction's offset field)
+    __shared__ __align__(16) unsigned char smem[lds_bytes<NL, D>()];
     constexpr int NOBF = D / 32;
     constexpr int W = D / 32;
-    // LDS: hidden weights (NL-1) x 32 KB | final weights | biases fp32 [(NL-1)*128 + D]
-    char *sp = reinterpret_cast<char *>(smem);
+    // LDS: hidden weights (NL-1) x 32 KB | final weights | biases fp32 [(NL-1)*128 + D] | SiLU table (NL > 1)
+    unsigned char *sp = smem;
     uint4 *wp_hidden[NL > 1 ? NL - 1 : 1];
 #pragma unroll
     for (int l = 0; l < NL - 1; ++l) wp_hidden[l] = reinterpret_cast<uint4 *>(sp + l * wp_bytes(kDim));
     uint4 *wp_final = reinterpret_cast<uint4 *>(sp + (NL - 1) * wp_bytes(kDim));
     float *s_bias = reinterpret_cast<float *>(sp + (NL - 1) * wp_bytes(kDim) + wp_bytes(D));
+    uint32_t *s_tab = reinterpret_cast<uint32_t *>(s_bias + (NL - 1) * kDim + D);
 
     const int head = blockIdx.y, b = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int in_head = head / (n_heads / x_heads);
@@ -128,6 +185,7 @@ __global__ __launch_bounds__(kMfThreads) void encode_mfma_kernel(const __bf16 *_
         }
         fill_weights(reinterpret_cast<uint2 *>(wp_final), w, D, NL > 1, tid);
         for (int i = tid; i < D; i += kMfThreads) s_bias[(NL - 1) * kDim + i] = (float)w[D * kDim + i];
+        if constexpr (NL > 1) fill_silu_table(s_tab, tid);
     }
     __syncthreads();
 
@@ -149,8 +207,8 @@ __global__ __launch_bounds__(kMfThreads) void encode_mfma_kernel(const __bf16 *_
 #pragma unroll
             for (int ks = 0; ks < kKSteps; ++ks) Ba[ks][nb] = __builtin_bit_cast(bf16x8, row[2 * ks + half]);
         }
-        if constexpr (NL >= 2) hidden_layer(wp_hidden[0], s_bias, Ba, Bb, lane);
-        if constexpr (NL >= 3) hidden_layer(wp_hidden[1], s_bias + kDim, Bb, Ba, lane);
+        if constexpr (NL >= 2) hidden_layer(wp_hidden[0], s_bias, s_tab, Ba, Bb, lane);
+        if constexpr (NL >= 3) hidden_layer(wp_hidden[1], s_bias + kDim, s_tab, Bb, Ba, lane);
 
         f32x16 acc[NOBF][2];
         if constexpr (NL == 2) layer_mfma<NOBF>(wp_final, s_bias + (NL - 1) * kDim, Bb, acc, lane);
@@ -172,20 +230,12 @@ __global__ __launch_bounds__(kMfThreads) void encode_mfma_kernel(const __bf16 *_
     }
 }
 
-template <int NL, int D> constexpr int lds_bytes() { return (NL - 1) * wp_bytes(kDim) + wp_bytes(D) + ((NL - 1) * kDim + D) * 4; }
-
 template <int NL, int D>
 int launch_mfma(dim3 grid, hipStream_t s, const __bf16 *x, int64_t x_sb, int64_t x_sh, int64_t x_st, int x_heads, int n_heads, int T,
                 int tiles_per_wg, const __bf16 *w, int64_t per_head, uint32_t *codes, int64_t c_sb, int64_t c_sh, int pos0,
                 const int32_t *pos_dev) {
-    constexpr int lds = lds_bytes<NL, D>();
-    auto kern = encode_mfma_kernel<NL, D>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) HA_FAIL(HA_ERR_HIP, "hipFuncSetAttribute(%d bytes LDS): %s", lds, hipGetErrorString(e));
-    }
-    hipLaunchKernelGGL(kern, grid, dim3(kMfThreads), lds, s, x, x_sb, x_sh, x_st, x_heads, n_heads, T, tiles_per_wg, w, per_head, codes,
-                       c_sb, c_sh, pos0, pos_dev);
+    hipLaunchKernelGGL((encode_mfma_kernel<NL, D>), grid, dim3(kMfThreads), 0, s, x, x_sb, x_sh, x_st, x_heads, n_heads, T, tiles_per_wg, w,
+                       per_head, codes, c_sb, c_sh, pos0, pos_dev);
     HA_CHECK_LAUNCH("encode_mfma_kernel");
     return HA_OK;
 }
@@ -212,9 +262,9 @@ extern "C" int ha_encode_pack_prefill(const void *x, int64_t x_stride_b, int64_t
 
     const int64_t per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
     const int tiles = (T + kTile - 1) / kTile;
-    // enough workgroups to fill 256 CUs a few times over, but several tiles each so the LDS weight fill amortises
+    // enough workgroups to fill 256 CUs a few times over, but several tiles each so the LDS fill (weights, table) amortises
     int tiles_per_wg = 1;
-    while (tiles_per_wg < 8 && (int64_t)B * n_heads * ((tiles + 2 * tiles_per_wg - 1) / (2 * tiles_per_wg)) >= 1024) tiles_per_wg *= 2;
+    while (tiles_per_wg < 16 && (int64_t)B * n_heads * ((tiles + 2 * tiles_per_wg - 1) / (2 * tiles_per_wg)) >= 1024) tiles_per_wg *= 2;
     const dim3 grid((tiles + tiles_per_wg - 1) / tiles_per_wg, n_heads, B);
     hipStream_t s = (hipStream_t)stream;
     const __bf16 *xp = (const __bf16 *)x, *wp = (const __bf16 *)weights_bf16;

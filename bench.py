@@ -353,6 +353,43 @@ class InputSet:
         self.layer.attend(self.q3, self.p.k, self.p.v, self.out)
 
 
+def first_step_probe(s, args, torch):
+    """The first decode step after a prefill, per layer, with one key-side hash MLP per query head (the reference's layout):
+    every cached key is hashed in bulk (`encode_keys_bulk`: bf16 MFMA for a hash module kept in bf16, fp32 MFMA for one kept
+    in fp32) and one decode step follows.  Milliseconds per layer, HIP events; the fp32 module's scalar-kernel time is measured
+    on one sequence's keys and scaled to the batch."""
+    from hashattention import _ops
+    from hashattention.decode import HashDecodeLayer
+    from hashattention.synthetic import make_usa_weights
+    w, S = s.w, s.S
+    usa = make_usa_weights(w)
+    out = {"code_heads": w.n_code_heads, "cached_tokens": S - 1, "sequences": w.batch}
+    for name, arith in (("bf16_module", _ops.HA_ARITH_BF16), ("fp32_module", _ops.HA_ARITH_F32)):
+        layer = HashDecodeLayer(usa.k, usa.q, w.n_q_heads, w.n_kv_heads, w.head_dim, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
+                                w.init_budget, w.recent_budget, w.heavy_budget, arith=arith, device=s.dev)
+        layer.allocate(w.batch, S)
+
+        def first():
+            layer.encode_keys_bulk(s.p.k[:, :, :S - 1])
+            layer.n_cached = S - 1
+            layer.step(s.p.q, s.p.k, s.p.v, S, s.out)
+
+        def bulk():
+            layer.encode_keys_bulk(s.p.k[:, :, :S - 1])
+
+        out[name + "_ms"] = time_gpu(first, 3, 1, torch)
+        out[name + "_bulk_hash_ms"] = time_gpu(bulk, 3, 1, torch)
+        if arith == _ops.HA_ARITH_F32:
+            def scalar():
+                _ops.encode_pack(s.p.k[:1, :, :S - 1], layer.wk, layer.num_layers, layer.int_dim, layer.final_dim, layer.codes, 0, None, arith)
+            out["fp32_module_scalar_kernel_bulk_hash_ms"] = time_gpu(scalar, 1, 1, torch) * w.batch
+        del layer
+    flop = w.batch * w.n_code_heads * (S - 1) * 2 * (w.head_dim * w.lth_int_dim + (w.lth_num_layers - 2) * w.lth_int_dim ** 2
+                                                      + w.lth_int_dim * w.lth_final_dim)
+    out["bulk_hash_tflops"] = {k[:-len("_bulk_hash_ms")]: flop / (out[k] * 1e-3) / 1e12 for k in list(out) if k.endswith("_bulk_hash_ms")}
+    return out
+
+
 def time_step(sets, steps, warmup, torch):
     """The whole step over a rotation of input sets: eager launches and one HIP graph holding one pass over all sets,
     replayed.  Returns (ms eager, ms graph, graph replay reproduces the eager outputs)."""
@@ -384,6 +421,7 @@ def main():
                     "so that consecutive launches never touch the same rows (as consecutive layers of a model)")
     ap.add_argument("--no-code-heads-32", action="store_true", help="skip the extra timing of the one-code-per-query-head layout")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-first-step", action="store_true", help="skip timing the first decode step after a prefill (bulk hash of all cached keys)")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
     ap.add_argument("--fused-min-rows", type=int, default=None, help="take the fused select-attend path from this many (sequence, head) rows on")
@@ -547,6 +585,8 @@ def main():
             "hbm_frac_step": bytes2 / (t_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "speedup_vs_dense": ms_dense / t_step,
             "score_roofline": roofline_obj("select_hist_kernel", ab2["score"], t_prepare),
             "roofline": roofline_obj("sparse_attend_kernel (selection fused)" if t_fused else "sparse_attend_kernel", ab2["gather"], t_attend)}
+        if not args.no_first_step:
+            res["first_step_after_prefill"] = first_step_probe(twins[0], args, torch)
         del twins
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)

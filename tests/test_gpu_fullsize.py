@@ -74,3 +74,33 @@ def test_full_size_configuration(name):
         errd = np.abs(outd.float().cpu().numpy() - refd).max()
         print(f"  dense max-abs error {errd:.2e}", flush=True)
         assert errd <= 2e-2
+
+
+@pytest.mark.parametrize("name,n_seq", [("config1", 1), ("config3", 1), ("config4", 2)])
+def test_full_length_fp32_encoders_against_the_oracle(name, n_seq):
+    # the fp32 hash of every cached key of whole sequences at the benchmark lengths (32K, 128K, ragged with 64-bit codes),
+    # by the exact scalar kernel and by the fp32 matrix-core kernel, against the torch fp32 oracle on the CPU: a sign bit may
+    # differ only where the oracle's |logit| < 1e-4
+    from oracle import hashattn_oracle as orc
+    from tests.parity_util import compare_codes
+    print(f"\n[case] full-length fp32 encoders {name}", flush=True)
+    w = named_workload(name)
+    p = make_problem_on_device(w, DEV)
+    S, W, Hc = w.max_seq_len, w.code_words, w.n_code_heads
+    k = p.k[:n_seq]
+    wk = _ops.pack_usa_weights(p.usa.k, DEV)
+    exact = torch.zeros(n_seq, Hc, S, W, dtype=torch.int32, device=DEV)
+    mfma = torch.zeros(n_seq, Hc, S, W, dtype=torch.int32, device=DEV)
+    _ops.encode_pack(k, wk, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim, exact)
+    _ops.encode_pack_prefill_f32(k, wk, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim, mfma)
+    torch.cuda.synchronize()
+    k_cpu = k.float().cpu()
+    for b in range(n_seq):
+        kl = orc.usa_logits(k_cpu[b:b + 1], p.usa.k)                        # [1, Hc, S, D]
+        want = orc.pack_codes(kl).numpy().astype(np.uint32)
+        valid = np.zeros((1, Hc, S), dtype=bool)
+        valid[:, :, :w.seq_lens[b]] = True
+        n_exact = compare_codes("exact kernel", exact[b:b + 1].cpu().numpy().view(np.uint32), want, kl.numpy(), valid)
+        n_mfma = compare_codes("fp32 mfma kernel", mfma[b:b + 1].cpu().numpy().view(np.uint32), want, kl.numpy(), valid)
+        print(f"  sequence {b}: {w.seq_lens[b]} tokens x {Hc} heads x {w.lth_final_dim} bits, differing from the oracle: "
+              f"exact {n_exact}, mfma {n_mfma}", flush=True)

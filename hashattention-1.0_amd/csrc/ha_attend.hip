@@ -226,8 +226,8 @@ __device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, 
 
 // Setup, second half: threshold, prefixes, list length, the chunk of the r-th tie.
 template <int W, int NTT>
-__device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row, int S, int sp, int *s_cstar, uint32_t *s_h,
-                                                 int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
+__device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row, int S, int sp, int row_pieces, int *s_cstar,
+                                                 uint32_t *s_h, int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
     const int tid = threadIdx.x;
     if (f.hist) {
         local_thresholds<W, NTT>(f, row, S, s_h, s_pre, s_meta);
@@ -243,6 +243,30 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         fr.nheavy = f.meta[row * 4 + 2];
         fr.neq = f.meta[row * 4 + 3];
         fr.pre = f.chunk_pre + row * f.nchunk * 2;
+    }
+    // The pieces of a split row take equal shares of the row's WORK, not of its chunks: with ties broken by the lowest index
+    // the taken part of the tie bucket lies at the front of the sequence, so pieces of equal token ranges gather very
+    // different numbers of rows (B = 4 at 128K tokens: 2750 against 1350 rows, 56 against 43 us).  A piece's work is counted
+    // as its selected rows plus kChunkScanRows per chunk it scans (a chunk's scan takes about as long as gathering that many
+    // rows); piece i starts at the first chunk before which at least i / pieces of the row's work lies.  Every workgroup of
+    // the row derives the same boundaries from the same prefixes, whichever launch derived the thresholds.
+    if (row_pieces > 1 && f.nchunk <= HA_WAVE) {
+        constexpr int kChunkScanRows = 48;
+        if (tid < HA_WAVE) {  // nchunk <= 64: a chunk per lane
+            const int c = tid;
+            const int nc_row = min((S + f.chunk - 1) / f.chunk, f.nchunk);  // chunks that hold tokens of this row
+            const int total = fr.nheavy + kChunkScanRows * nc_row;
+            const int wt = c < nc_row ? fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r) + kChunkScanRows * c : total;
+            const int t0 = (int)((int64_t)sp * total / row_pieces), t1 = (int)((int64_t)(sp + 1) * total / row_pieces);
+            const unsigned long long m0 = __ballot(wt >= t0), m1 = __ballot(wt >= t1);
+            if (tid == 0) {
+                s_meta[4] = sp == 0 ? 0 : min(m0 ? __ffsll((long long)m0) - 1 : f.nchunk, f.nchunk);
+                s_meta[5] = sp == row_pieces - 1 ? f.nchunk : min(m1 ? __ffsll((long long)m1) - 1 : f.nchunk, f.nchunk);
+            }
+        }
+        __syncthreads();
+        fr.c0 = s_meta[4];
+        fr.nc = max(s_meta[5] - fr.c0, 0);
     }
     const int c1 = fr.c0 + fr.nc;
     const int32_t *pre = fr.pre;
@@ -266,9 +290,33 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
 // how many leading list entries are in LDS afterwards.  Two workgroup barriers per round; called by all threads.
 // The gather loop runs between rounds, so the scan's integer work sits in the shadow of the loop's memory waits
 // instead of in front of it.
+// The codes of this wave's group in scan round `round`, requested now and ranked later (fused_round with PRE): a
+// workgroup that has its CU to itself asks for the next round's codes before it goes back to the gather loop, so that
+// they travel under the loop's row loads instead of being waited for with nothing else in flight.  Needs only the row's
+// geometry (fused_windows), not its threshold; `n_groups` as fused_round's, or its value for a row with heavy tokens.
 template <int W, int GS, int NW>
+__device__ __forceinline__ void fused_round_issue(const FusedSel &f, const FusedRow &fr, int b, int h, int round, int n_groups,
+                                                  ha_sel::Code<W> (&k)[GS][4]) {
+    using namespace ha_sel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int GC = GS * HA_WAVE * 4;
+    const int gpc = f.chunk / GC;
+    const int g = round * NW + wave;
+    const bool active = g < n_groups;
+    const int c = fr.c0 + (active ? g / gpc : 0), gi = active ? g % gpc : 0;
+    const int cb = c * f.chunk, j_first = cb + gi * GC;
+    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
+    const bool whole = f.vec && beg == cb && end == cb + f.chunk;
+    if (active && beg < end) {
+        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+        load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
+    }
+}
+
+template <int W, int GS, int NW, bool PRE = false>
 __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, int round, int n_groups,
-                                           uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list) {
+                                           uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list,
+                                           ha_sel::Code<W> (*kpre)[4] = nullptr /* PRE: the round's codes, from fused_round_issue */) {
     using namespace ha_sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int GC = GS * HA_WAVE * 4;  // codes per group
@@ -284,9 +332,16 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
     uint32_t lt = 0, le = 0;  // bit 4 s + e: code (slab s, element e) of this lane has d < T / d <= T
     if (active && beg < end && fr.nheavy > 0) {
         const Code<W> q = load_qcode<W>(f.qcodes, row);
-        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
         Code<W> k[GS][4];
-        load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
+        if constexpr (PRE) {
+#pragma unroll
+            for (int s = 0; s < GS; ++s)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) k[s][e] = kpre[s][e];
+        } else {
+            const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+            load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
+        }
         const int neg_t = -fr.T;
 #pragma unroll
         for (int s = GS - 1; s >= 0; --s)
@@ -379,8 +434,10 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // NT threads = NT/16 row streams; U rows per stream per step.
 // MK: an additive term per list entry (AttnMask), natural-log units, added to the scaled score before the softmax; list-fed
 // launches only.
-template <typename E, int NT, int U, int FW, bool MK = false>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+// PF (fused launches whose grid gives every workgroup a CU of its own): 2 waves per SIMD instead of 4, i.e. 256 registers
+// per lane, of which 32 W hold the codes of the next scan round while the gather loop runs (fused_round_issue).
+template <typename E, int NT, int U, int FW, bool MK = false, bool PF = false>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, PF ? 2 : 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
                                                            const int32_t *__restrict__ idx, int64_t idx_cap,
@@ -402,7 +459,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     // in-kernel thresholds: the row's chunk histograms (+ their totals), chunk prefixes, {T, r, n_heavy, tie bucket}
     __shared__ uint32_t s_h[FW > 0 ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
     __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedLocalChunks : 1];
-    __shared__ int32_t s_meta[4];
+    __shared__ int32_t s_meta[6];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
     // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
@@ -630,10 +687,12 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             prime();
             primed = true;
         }
+        // PF: the codes of a scan round are requested a round ahead
+        [[maybe_unused]] ha_sel::Code<FW> kpf[PF ? GS : 1][4];
         {
             int S = seq_lens ? seq_lens[b] : max_S;
             if (S > max_S) S = max_S;
-            fused_thresholds<FW, NT>(fsel, row, S, sp, &s_cstar, s_h, s_pre, s_meta, fr);
+            fused_thresholds<FW, NT>(fsel, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
         }
         r1 = fr.n;
         if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
@@ -642,7 +701,28 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
         const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
         const int rounds = (n_groups + NW - 1) / NW;
-        for (int k = 0; k < rounds; ++k) {
+        bool scanned = false;
+        if constexpr (PF) {
+            if (wide) {
+                scanned = true;
+                auto after_round = [&](int ready) {
+                    ready = min(ready, r1);
+                    if (!primed && ready >= min(2 * STEP, r1)) {
+                        prime();
+                        primed = true;
+                    }
+                    while (primed && base + 3 * STEP <= ready) step();
+                };
+                if (rounds > 0) fused_round_issue<FW, GS, NW>(fsel, fr, b, h, 0, n_groups, kpf);
+                for (int k = 0; k < rounds; ++k) {
+                    int ready = fused_round<FW, GS, NW, true>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list, kpf);
+                    if (k == rounds - 1) break;
+                    fused_round_issue<FW, GS, NW>(fsel, fr, b, h, k + 1, n_groups, kpf);
+                    after_round(ready);
+                }
+            }
+        }
+        for (int k = 0; k < rounds && !scanned; ++k) {
             int ready = wide ? fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list)
                              : fused_round<FW, 4, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
             if (k == rounds - 1) break;
@@ -1099,12 +1179,20 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     const dim3 grid(nsplit, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
+    // a grid of at most one workgroup per CU: the instantiation that requests its scan codes a round ahead
+    const bool alone = rows * nsplit <= 256;
+
 #define HA_FUSED_LAUNCH(E_, U_, FW_)                                                                                              \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b,                       \
-                           q_stride_h, k, v,                                                                                      \
-                           kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
-                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);                       \
+        if (alone)                                                                                                                \
+            hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_, false, true>), grid, dim3(512), 0, s, q, q_stride_b,      \
+                               q_stride_h, k, v, kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap,    \
+                               nullptr, sl2, 0, nsplit, part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f,          \
+                               AttnMask{}, 1);                                                                                    \
+        else                                                                                                                      \
+            hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,  \
+                               kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0,     \
+                               nsplit, part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);           \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \

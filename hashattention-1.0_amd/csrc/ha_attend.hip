@@ -136,7 +136,8 @@ constexpr int kFusedLocalChunks = 64;
 constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
 // a batch of equal lengths is cut into this many workgroups (one per CU): measured against 512 at 64K tokens, B = 6: 76.6
 // against 82.3 us, B = 8: 76.7 against 81.2, B = 12: 107.1 against 125.5; B = 1 at 32K: 39.2 against 40.9; B = 4 at 128K: 84.1
-// against 87.0 - the pieces are setup-bound, so fewer and larger ones win
+// against 87.0 - the pieces are setup-bound, so fewer and larger ones win (measured again with pieces of equal work, 256 / 384 /
+// 512 pieces: B = 1 at 32K 22.1 / 28.0 / 27.4 us, B = 4 at 128K 60.2 / 69.3 / 63.4, B = 8 at 64K 58.5 / 66.2 / 66.5)
 constexpr int kFusedUniformPieces = 256;
 constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
 

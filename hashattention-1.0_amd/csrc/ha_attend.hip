@@ -569,7 +569,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, 
         ix = idx + row * idx_cap;
     }
     // rows_per_seq consecutive batch entries attend to the cache of one sequence (the rows of a chunk of tokens)
-    const int64_t b_kv = rows_per_seq > 1 ? b / rows_per_seq : b;
+    // (list-fed launches only: in the fused instantiation the extra value would cost it a spilled register)
+    int64_t b_kv = b;
+    if constexpr (FW == 0) b_kv = rows_per_seq > 1 ? b / rows_per_seq : b;
     const char *kb = (const char *)k + (b_kv * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const char *vb = (const char *)v + (b_kv * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;

@@ -233,3 +233,17 @@ def test_ragged_batch_larger_than_the_in_kernel_plan(batch, heads):
                        heavy_budget=0.05, seed=93)
     rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
     assert "fused_err" in rep
+
+
+@pytest.mark.parametrize("lens,heads,bits,heavy", [([70000, 70000], (8, 2, 2), 32, 1.0 / 32), ([131072], (4, 4, 4), 64, 0.002),
+                                                    ([52000, 90000, 33000], (8, 8, 8), 32, 1500.0), ([200000], (16, 4, 4), 32, 7000.0)])
+def test_long_rows_cut_into_pieces_of_equal_work(lens, heads, bits, heavy):
+    # few long rows: the fused launch cuts every row into pieces whose boundaries follow the selected rows and the chunks to
+    # scan (every workgroup of a row derives them from the row's chunk prefixes), with the lengths on the host (one workgroup
+    # per CU, scan codes requested a round ahead) and on the device (in-kernel plan).  Every stage against the oracle.
+    print(f"\n[case] long rows {lens} heads={heads} bits={bits} heavy={heavy}", flush=True)
+    w = small_workload(name="long", batch=len(lens), seq_lens=lens, n_q_heads=heads[0], n_kv_heads=heads[1], n_code_heads=heads[2],
+                       lth_num_layers=2 if bits == 64 else 3, lth_final_dim=bits, init_budget=128, recent_budget=16,
+                       heavy_budget=heavy, dtype=torch.bfloat16, seed=77)
+    rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
+    assert "fused_err" in rep

@@ -141,12 +141,31 @@ constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are plan
 constexpr int kFusedUniformPieces = 256;
 constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
 
-// NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.
+// NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.  `whole` (uniform
+// over the wave: the chunk lies inside the candidate range and its row takes 128-bit loads) is tested ONCE, around all the
+// loads: tested per slab, each load sits in a branch of its own whose join makes the compiler wait for every outstanding
+// load - the slab before it and the K/V rows of the gather loop - before it issues the next one, eight drained round trips
+// per scan round instead of one.
 template <int W, int NSLAB>
 __device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int beg, int end, bool whole, int lane,
                                            ha_sel::Code<W> (&k)[NSLAB][4]) {
+    if (whole) {
 #pragma unroll
-    for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, whole, k[s]);
+        for (int s = 0; s < NSLAB; ++s) {
+            const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
+            if constexpr (W == 1) {
+                const uint4 v = reinterpret_cast<const uint4 *>(kc)[j0 >> 2];
+                k[s][0].w0 = v.x, k[s][1].w0 = v.y, k[s][2].w0 = v.z, k[s][3].w0 = v.w;
+            } else {
+                const uint4 a = reinterpret_cast<const uint4 *>(kc)[j0 >> 1], b = reinterpret_cast<const uint4 *>(kc)[(j0 >> 1) + 1];
+                k[s][0].w0 = a.x, k[s][0].w1 = a.y, k[s][1].w0 = a.z, k[s][1].w1 = a.w;
+                k[s][2].w0 = b.x, k[s][2].w1 = b.y, k[s][3].w0 = b.z, k[s][3].w1 = b.w;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, false, k[s]);
+    }
 }
 
 // A fused workgroup alternates scan rounds (fused_round: its waves place the selected tokens of the next few chunks in

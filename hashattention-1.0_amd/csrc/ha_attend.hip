@@ -133,6 +133,7 @@ struct AttnMask {
     int len, by_slot;
 };
 constexpr int kFusedLocalChunks = 64;
+constexpr int kFusedMaxChunks = 256;  // chunks of a row of the fused path: the row's chunk prefixes are kept in LDS
 constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
 // a batch of equal lengths is cut into this many workgroups (one per CU): measured against 512 at 64K tokens, B = 6: 76.6
 // against 82.3 us, B = 8: 76.7 against 81.2, B = 12: 107.1 against 125.5; B = 1 at 32K: 39.2 against 40.9; B = 4 at 128K: 84.1
@@ -141,31 +142,13 @@ constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are plan
 constexpr int kFusedUniformPieces = 256;
 constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
 
-// NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, all requested at once.  `whole` (uniform
-// over the wave: the chunk lies inside the candidate range and its row takes 128-bit loads) is tested ONCE, around all the
-// loads: tested per slab, each load sits in a branch of its own whose join makes the compiler wait for every outstanding
-// load - the slab before it and the K/V rows of the gather loop - before it issues the next one, eight drained round trips
-// per scan round instead of one.
+// NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, for rows that do not take 128-bit loads
+// (misaligned, or strides that are no multiples of four codes): element loads inside [beg, end), zeros outside.
 template <int W, int NSLAB>
-__device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int beg, int end, bool whole, int lane,
-                                           ha_sel::Code<W> (&k)[NSLAB][4]) {
-    if (whole) {
+__device__ __forceinline__ void load_slabs_by_element(const uint32_t *kc, int j_first, int beg, int end, int lane,
+                                                      ha_sel::Code<W> (&k)[NSLAB][4]) {
 #pragma unroll
-        for (int s = 0; s < NSLAB; ++s) {
-            const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
-            if constexpr (W == 1) {
-                const uint4 v = reinterpret_cast<const uint4 *>(kc)[j0 >> 2];
-                k[s][0].w0 = v.x, k[s][1].w0 = v.y, k[s][2].w0 = v.z, k[s][3].w0 = v.w;
-            } else {
-                const uint4 a = reinterpret_cast<const uint4 *>(kc)[j0 >> 1], b = reinterpret_cast<const uint4 *>(kc)[(j0 >> 1) + 1];
-                k[s][0].w0 = a.x, k[s][0].w1 = a.y, k[s][1].w0 = a.z, k[s][1].w1 = a.w;
-                k[s][2].w0 = b.x, k[s][2].w1 = b.y, k[s][3].w0 = b.z, k[s][3].w1 = b.w;
-            }
-        }
-    } else {
-#pragma unroll
-        for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, false, k[s]);
-    }
+    for (int s = 0; s < NSLAB; ++s) ha_sel::load_code4<W>(kc, j_first + s * (HA_WAVE * 4) + lane * 4, beg, end, false, k[s]);
 }
 
 // A fused workgroup alternates scan rounds (fused_round: its waves place the selected tokens of the next few chunks in
@@ -174,7 +157,10 @@ __device__ __forceinline__ void load_slabs(const uint32_t *kc, int j_first, int 
 // waves, and giving two of eight to the scan cost more than the scan itself.  Building the whole list first costs
 // the scan's ~15 us up front.)
 struct FusedRow {
-    const int32_t *pre;  // {#d < T, #d == T} before each chunk of the row: the workspace's, or the workgroup's own in LDS
+    // {#d < T, #d == T} before each chunk of the row, in LDS: worked out by the workgroup or copied from the workspace.  (Read
+    // from either place through one pointer they would be flat loads, and a flat load in a scan round waits for every
+    // outstanding request of the wave, rows on their way included.)
+    const int32_t *pre;
     int lo, hi, T, r, nheavy, neq, c0, nc, n;
     int nwin;   // window entries at the head of this workgroup's list (sink if it has the first chunk, recent if the last)
     int hbase;  // list position of a heavy token = hbase + (#d < T before it) + min(#d == T before it, r)
@@ -262,7 +248,10 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         fr.r = f.meta[row * 4 + 1];
         fr.nheavy = f.meta[row * 4 + 2];
         fr.neq = f.meta[row * 4 + 3];
-        fr.pre = f.chunk_pre + row * f.nchunk * 2;
+        const int32_t *gp = f.chunk_pre + row * f.nchunk * 2;
+        for (int i = tid; i < 2 * f.nchunk; i += NTT) s_pre[i] = gp[i];
+        __syncthreads();
+        fr.pre = s_pre;
     }
     // The pieces of a split row take equal shares of the row's WORK, not of its chunks: with ties broken by the lowest index
     // the taken part of the tie bucket lies at the front of the sequence, so pieces of equal token ranges gather very
@@ -289,88 +278,143 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         fr.nc = max(s_meta[5] - fr.c0, 0);
     }
     const int c1 = fr.c0 + fr.nc;
-    const int32_t *pre = fr.pre;
     // heavy tokens of the row before chunk c
-    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : pre[c * 2] + min(pre[c * 2 + 1], fr.r); };
+    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r); };
     fr.hbase = fr.nwin - rank(fr.c0);
     fr.n = min(fr.nwin + max(rank(c1) - rank(fr.c0), 0), kFusedListCap);
     if (tid == 0) *s_cstar = -1;
     __syncthreads();
     for (int i = tid; i < fr.nc; i += NTT) {
         const int c = fr.c0 + i;
-        const int eq0 = pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? pre[(c + 1) * 2 + 1] : fr.neq;
+        const int eq0 = fr.pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? fr.pre[(c + 1) * 2 + 1] : fr.neq;
         if (eq0 < fr.r && fr.r < eq1) *s_cstar = c;  // at most one chunk of the row
     }
     __syncthreads();
     fr.cstar = *s_cstar;
 }
 
+// Scan rounds work on staged codes: the codes of a wave's group travel from memory straight into a 4 KiB region of LDS that
+// belongs to the wave (one 16-byte request per lane and instruction, lane l's bytes at l * 16 behind the address in M0), a
+// round ahead, so they occupy no registers while the gather loop runs between the rounds and nobody waits for them when the
+// next round starts.  (Requested inside the round that ranks them, every round waits a memory round trip with nothing else of
+// the wave in flight; held in registers across the loop they cost 16 - 32 of its 128.)  The requests are inline assembly on
+// purpose: the compiler does not see them.  Through the builtin it waits for every outstanding request in front of each LDS
+// access it cannot tell from the staging space, and before each barrier.  Its own `s_waitcnt vmcnt(n)` stay safe, because
+// requests return in order: unseen requests among the n youngest only make a wait cover more than it had to, which is why
+// the codes are requested in front of a step's rows, not behind them.  The wave's own wait for its staged codes is written
+// by hand (staged_codes_arrived): once at least eight later requests have been issued - one gather step or the loop's
+// priming - "at most eight outstanding" means the codes are in LDS.
+constexpr int kStageWaveWords = 1024;  // staging region of one wave: 1024 32-bit codes or 512 64-bit codes
+__device__ __forceinline__ void request_16_bytes_to_lds(const uint32_t *src, const uint32_t *dst /* uniform over the wave */) {
+    const uint32_t lds_byte_address = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)dst);
+    uint32_t saved_m0;  // M0 is the compiler's: handed back as it was
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "v"(src), "s"(lds_byte_address)
+                 : "memory");
+}
+__device__ __forceinline__ void staged_codes_arrived(bool eight_younger_requests) {
+    if (eight_younger_requests) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+// Requests the codes of this wave's group of scan round `round` (geometry as in fused_round).  Lanes past the end of the
+// candidate range ask for the chunk's first codes instead (the range is not empty, so they exist); fused_round masks them.
+// Rows that do not take 128-bit loads are not staged: fused_staged_codes loads their codes itself.
+template <int W, int GS, int NW>
+__device__ __forceinline__ void fused_round_stage(const FusedSel &f, const FusedRow &fr, int b, int h, int round, int n_groups,
+                                                  const uint32_t *s_stage) {
+    static_assert(GS * HA_WAVE * 4 * W == kStageWaveWords, "a group fills the wave's staging region");
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // the wave's number in scalar registers
+    constexpr int GC = GS * HA_WAVE * 4;
+    const int gpc = f.chunk / GC, gpc_log2 = __builtin_ctz((unsigned)gpc);  // a power of two
+    const int g = round * NW + wave;
+    if (g >= n_groups || !f.vec) return;
+    const int c = fr.c0 + (g >> gpc_log2), gi = g & (gpc - 1);
+    const int cb = c * f.chunk, j_first = cb + gi * GC;
+    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
+    if (beg >= end) return;
+    const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
+    const uint32_t *dst = s_stage + wave * kStageWaveWords;
+#pragma unroll
+    for (int s = 0; s < GS; ++s) {
+        const int j0 = j_first + s * (HA_WAVE * 4) + lane * 4;
+        const int64_t j = j0 < end ? j0 : cb;
+        if constexpr (W == 1) {
+            request_16_bytes_to_lds(kc + j, dst + s * 256);
+        } else {
+            request_16_bytes_to_lds(kc + j * 2, dst + s * 512);
+            request_16_bytes_to_lds(kc + j * 2 + 4, dst + s * 512 + 256);
+        }
+    }
+}
+// The codes fused_round_stage requested for this wave, from its staging region into registers.
+template <int W, int GS>
+__device__ __forceinline__ void fused_staged_codes(const uint32_t *s_stage, bool eight_younger_requests, ha_sel::Code<W> (&k)[GS][4]) {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // the wave's number in scalar registers
+    staged_codes_arrived(eight_younger_requests);
+    const uint4 *sw = reinterpret_cast<const uint4 *>(s_stage + wave * kStageWaveWords);
+#pragma unroll
+    for (int s = 0; s < GS; ++s) {
+        if constexpr (W == 1) {
+            const uint4 v = sw[s * HA_WAVE + lane];
+            k[s][0].w0 = v.x, k[s][1].w0 = v.y, k[s][2].w0 = v.z, k[s][3].w0 = v.w;
+        } else {
+            const uint4 a = sw[s * 2 * HA_WAVE + lane], b2 = sw[(s * 2 + 1) * HA_WAVE + lane];
+            k[s][0].w0 = a.x, k[s][0].w1 = a.y, k[s][1].w0 = a.z, k[s][1].w1 = a.w;
+            k[s][2].w0 = b2.x, k[s][2].w1 = b2.y, k[s][3].w0 = b2.z, k[s][3].w1 = b2.w;
+        }
+    }
+}
+
 // One scan round of a fused workgroup: its NW waves take NW consecutive groups of GS slabs (a group is part of one
 // chunk; a chunk's groups never straddle rounds), place the selected tokens of those groups in the list, and return
 // how many leading list entries are in LDS afterwards.  Two workgroup barriers per round; called by all threads.
 // The gather loop runs between rounds, so the scan's integer work sits in the shadow of the loop's memory waits
-// instead of in front of it.
-// The codes of this wave's group in scan round `round`, requested now and ranked later (fused_round with PRE): a
-// workgroup that has its CU to itself asks for the next round's codes before it goes back to the gather loop, so that
-// they travel under the loop's row loads instead of being waited for with nothing else in flight.  Needs only the row's
-// geometry (fused_windows), not its threshold; `n_groups` as fused_round's, or its value for a row with heavy tokens.
+// instead of in front of it.  `q`: the row's query code; `s_stage`, `eight_younger_requests`: see fused_staged_codes.
 template <int W, int GS, int NW>
-__device__ __forceinline__ void fused_round_issue(const FusedSel &f, const FusedRow &fr, int b, int h, int round, int n_groups,
-                                                  ha_sel::Code<W> (&k)[GS][4]) {
+__device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr, int b, int h, const ha_sel::Code<W> &q, int round, int n_groups,
+                                           uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list, const uint32_t *s_stage,
+                                           bool eight_younger_requests) {
     using namespace ha_sel;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    constexpr int GC = GS * HA_WAVE * 4;
-    const int gpc = f.chunk / GC;
-    const int g = round * NW + wave;
-    const bool active = g < n_groups;
-    const int c = fr.c0 + (active ? g / gpc : 0), gi = active ? g % gpc : 0;
-    const int cb = c * f.chunk, j_first = cb + gi * GC;
-    const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
-    const bool whole = f.vec && beg == cb && end == cb + f.chunk;
-    if (active && beg < end) {
-        const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
-        load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
-    }
-}
-
-template <int W, int GS, int NW, bool PRE = false>
-__device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr, int b, int h, int64_t row, int round, int n_groups,
-                                           uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list,
-                                           ha_sel::Code<W> (*kpre)[4] = nullptr /* PRE: the round's codes, from fused_round_issue */) {
-    using namespace ha_sel;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // the wave's number in scalar registers
     constexpr int GC = GS * HA_WAVE * 4;  // codes per group
-    const int gpc = f.chunk / GC;         // groups per chunk: 1, 2 or 4 (divides NW)
+    const int gpc = f.chunk / GC, gpc_log2 = __builtin_ctz((unsigned)gpc);  // groups per chunk: a power of two that divides NW
     const int g = round * NW + wave;
     const bool active = g < n_groups;
-    const int c = fr.c0 + (active ? g / gpc : 0), gi = active ? g % gpc : 0;
+    const int c = fr.c0 + (active ? g >> gpc_log2 : 0), gi = active ? g & (gpc - 1) : 0;
     const int cb = c * f.chunk, j_first = cb + gi * GC;
     const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
     const bool whole = f.vec && beg == cb && end == cb + f.chunk;
-    const int32_t *pre = fr.pre;
 
     uint32_t lt = 0, le = 0;  // bit 4 s + e: code (slab s, element e) of this lane has d < T / d <= T
     if (active && beg < end && fr.nheavy > 0) {
-        const Code<W> q = load_qcode<W>(f.qcodes, row);
         Code<W> k[GS][4];
-        if constexpr (PRE) {
-#pragma unroll
-            for (int s = 0; s < GS; ++s)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) k[s][e] = kpre[s][e];
+        if (f.vec) {
+            fused_staged_codes<W, GS>(s_stage, eight_younger_requests, k);
         } else {
             const uint32_t *kc = f.kcodes + b * f.kc_sb + (h / f.gq) * f.kc_sh;
-            load_slabs<W, GS>(kc, j_first, beg, end, whole, lane, k);
+            load_slabs_by_element<W, GS>(kc, j_first, beg, end, lane, k);
         }
-        const int neg_t = -fr.T;
+        if (c == fr.cstar) {
+            const int neg_t = -fr.T;
 #pragma unroll
-        for (int s = GS - 1; s >= 0; --s)
+            for (int s = GS - 1; s >= 0; --s)
 #pragma unroll
-            for (int e = 3; e >= 0; --e) {
-                const int key = k[s][e].dist(q) + neg_t;  // sign bit: d < T; of key - 1: d <= T
-                lt = __builtin_amdgcn_alignbit(lt, (uint32_t)key, 31);
-                le = __builtin_amdgcn_alignbit(le, (uint32_t)(key - 1), 31);
-            }
+                for (int e = 3; e >= 0; --e) {
+                    const int key = k[s][e].dist(q) + neg_t;  // sign bit: d < T; of key - 1: d <= T
+                    lt = __builtin_amdgcn_alignbit(lt, (uint32_t)key, 31);
+                    le = __builtin_amdgcn_alignbit(le, (uint32_t)(key - 1), 31);
+                }
+        } else {
+            // any other chunk takes all of its ties (those before it do not reach r) or none: one compare per code, against
+            // T + 1 or T, and the chunk counts no ties of its own
+            const int neg_t = -(fr.T + (fr.pre[c * 2 + 1] < fr.r ? 1 : 0));
+#pragma unroll
+            for (int s = GS - 1; s >= 0; --s)
+#pragma unroll
+                for (int e = 3; e >= 0; --e) lt = __builtin_amdgcn_alignbit(lt, (uint32_t)(k[s][e].dist(q) + neg_t), 31);
+            le = lt;
+        }
         if (!whole) {
             uint32_t valid = 0;
 #pragma unroll
@@ -392,7 +436,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 
     // tokens of the row with d < T / d == T before this group: the chunk's prefix plus the chunk's earlier groups,
     // which are the gi waves just below this one
-    int a = pre[c * 2], t = pre[c * 2 + 1];
+    int a = fr.pre[c * 2], t = fr.pre[c * 2 + 1];
     for (int w2 = wave - gi; w2 < wave; ++w2) {
         const uint32_t v = s_cnt[w2];
         a += (int)(v & 0xFFFFu);
@@ -454,10 +498,8 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // NT threads = NT/16 row streams; U rows per stream per step.
 // MK: an additive term per list entry (AttnMask), natural-log units, added to the scaled score before the softmax; list-fed
 // launches only.
-// PF (fused launches whose grid gives every workgroup a CU of its own): 2 waves per SIMD instead of 4, i.e. 256 registers
-// per lane, of which 32 W hold the codes of the next scan round while the gather loop runs (fused_round_issue).
-template <typename E, int NT, int U, int FW, bool MK = false, bool PF = false>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, PF ? 2 : 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
+template <typename E, int NT, int U, int FW, bool MK = false>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
                                                            const int32_t *__restrict__ idx, int64_t idx_cap,
@@ -471,14 +513,22 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, 
     static_assert(!MK || FW == 0, "the additive mask exists for list-fed launches only");
     constexpr int NS = NT / 16;  // row streams
     __shared__ float s_m[NS], s_l[NS];
-    __shared__ float s_acc[NS * HA_HEAD_DIM];
+    // the streams' partial results at the end of the kernel; before that, in a fused launch, the waves' staging regions (and,
+    // for 64-bit codes, the histogram tile of the threshold search, which is over before the first codes are requested)
+    constexpr int kStageWords = FW > 0 ? (NT / HA_WAVE) * kStageWaveWords : 0;
+    constexpr int kRawWords = kStageWords > NS * HA_HEAD_DIM ? kStageWords : NS * HA_HEAD_DIM;
+    constexpr bool kTileInRaw = FW == 2;
+    __shared__ __attribute__((aligned(16))) uint32_t s_raw[kRawWords];
+    float *s_acc = reinterpret_cast<float *>(s_raw);
     __shared__ int32_t s_list[FW > 0 ? kFusedListCap : 1];
     __shared__ uint32_t s_cnt[FW > 0 ? 64 : 1];
     __shared__ int s_cstar;
     __shared__ int s_plan[2];
     // in-kernel thresholds: the row's chunk histograms (+ their totals), chunk prefixes, {T, r, n_heavy, tie bucket}
-    __shared__ uint32_t s_h[FW > 0 ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
-    __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedLocalChunks : 1];
+    static_assert(!kTileInRaw || (kFusedLocalChunks + 1) * (32 * FW + 1) <= kRawWords, "the histogram tile fits the staging space");
+    __shared__ uint32_t s_tile[FW > 0 && !kTileInRaw ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
+    uint32_t *s_h = kTileInRaw ? s_raw : s_tile;
+    __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedMaxChunks : 1];
     __shared__ int32_t s_meta[6];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
@@ -596,13 +646,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, 
     const int64_t row_bytes = kv_ss * EL::bytes;
     constexpr int STEP = NS * U;  // rows of the list consumed per step by the workgroup
 
-    float qf[8];
-    {
-        float t[8];
-        EL::unpack(EL::load8((const char *)q + (b * q_sb + h * q_sh) * EL::bytes, sub), t);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qf[i] = t[i] * scale_log2e;
-    }
+    // the query slice as it lies in memory: the score is dot8(q, k) * scale, two elements per instruction for 16-bit rows
+    const Raw8<E> qraw = EL::load8((const char *)q + (b * q_sb + h * q_sh) * EL::bytes, sub);
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
@@ -660,11 +705,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, 
         float sc[U], mloc = -INFINITY;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            float kf[8], d = 0.f;
-            EL::unpack(kr[u], kf);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
-            d = row16_sum(d);
+            float d = row16_sum(EL::dot8(qraw, kr[u])) * scale_log2e;
             if constexpr (MK) d += mk[u];
             sc[u] = (base + stream + u * NS < r1) ? d : -INFINITY;
             mloc = fmaxf(mloc, sc[u]);
@@ -700,60 +741,63 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(PF ? 2 : 4, 
         // scan rounds and gather steps alternate: after a round the list is complete up to `ready`, and the loop runs
         // as far as its look-ahead (3 steps) allows.  Everything here is uniform over the workgroup.
         constexpr int NW = NT / HA_WAVE;
-        constexpr int GS = FW == 1 ? 8 : 4;  // slabs per wave and round
-        const bool wide = fsel.chunk % (GS * HA_WAVE * 4) == 0;  // else 1024-code chunks (short rows): 4 slabs
-        const int gc = (wide ? GS : 4) * HA_WAVE * 4;
+        constexpr int GS = kStageWaveWords / (HA_WAVE * 4 * FW);  // slabs per wave and round: a staging region's worth
+        constexpr int gc = GS * HA_WAVE * 4;                      // codes per wave and round; divides every chunk size
+        // the row's query code, once and in scalar registers: loaded in a scan round it would be the youngest request of the
+        // wave there, and waiting for it would mean waiting for every row on its way
+        ha_sel::Code<FW> qcode = ha_sel::load_qcode<FW>(fsel.qcodes, row);
+        qcode.w0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w0);
+        if constexpr (FW == 2) qcode.w1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w1);
         // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out
         bool primed = false;
         if (fr.nwin >= 2 * STEP) {
             prime();
             primed = true;
         }
-        // PF: the codes of a scan round are requested a round ahead
-        [[maybe_unused]] ha_sel::Code<FW> kpf[PF ? GS : 1][4];
+        // the codes of the first round are requested before the thresholds are worked out too, when the workgroup's chunks
+        // are known by then (a row in one piece) and the histogram tile has a place of its own
+        bool staged_early = false;
+        if constexpr (!kTileInRaw) {
+            if (row_pieces == 1) {
+                fused_round_stage<FW, GS, NW>(fsel, fr, b, h, 0, fr.nc * (fsel.chunk / gc), s_raw);
+                staged_early = true;
+            }
+        }
         {
             int S = seq_lens ? seq_lens[b] : max_S;
             if (S > max_S) S = max_S;
             fused_thresholds<FW, NT>(fsel, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
         }
         r1 = fr.n;
+        const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
+        const int rounds = (n_groups + NW - 1) / NW;
+        // codes requested for a round that will not take place must not arrive in the partial results later
+        if (staged_early && rounds == 0) staged_codes_arrived(false);
         if (nsplit == 1 && r1 == 0) {  // empty sequence: defined as a zero output (uniform over the workgroup)
             if (tid < HA_HEAD_DIM) EL::store1((char *)out + row * HA_HEAD_DIM * EL::bytes, tid, 0.f);
             return;
         }
-        const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
-        const int rounds = (n_groups + NW - 1) / NW;
-        bool scanned = false;
-        if constexpr (PF) {
-            if (wide) {
-                scanned = true;
-                auto after_round = [&](int ready) {
-                    ready = min(ready, r1);
-                    if (!primed && ready >= min(2 * STEP, r1)) {
-                        prime();
-                        primed = true;
-                    }
-                    while (primed && base + 3 * STEP <= ready) step();
-                };
-                if (rounds > 0) fused_round_issue<FW, GS, NW>(fsel, fr, b, h, 0, n_groups, kpf);
-                for (int k = 0; k < rounds; ++k) {
-                    int ready = fused_round<FW, GS, NW, true>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list, kpf);
-                    if (k == rounds - 1) break;
-                    fused_round_issue<FW, GS, NW>(fsel, fr, b, h, k + 1, n_groups, kpf);
-                    after_round(ready);
-                }
-            }
-        }
-        for (int k = 0; k < rounds && !scanned; ++k) {
-            int ready = wide ? fused_round<FW, GS, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list)
-                             : fused_round<FW, 4, NW>(fsel, fr, b, h, row, k, n_groups, s_cnt, &s_cstar, s_list);
+        if (rounds > 0 && !staged_early) fused_round_stage<FW, GS, NW>(fsel, fr, b, h, 0, n_groups, s_raw);
+        bool covered = false;  // eight row requests have been issued behind the staged codes' requests
+        for (int k = 0; k < rounds; ++k) {
+            int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, qcode, k, n_groups, s_cnt, &s_cstar, s_list, s_raw, covered);
             if (k == rounds - 1) break;
             ready = min(ready, r1);
+            fused_round_stage<FW, GS, NW>(fsel, fr, b, h, k + 1, n_groups, s_raw);
+            covered = false;
             if (!primed && ready >= min(2 * STEP, r1)) {
                 prime();
                 primed = true;
+                covered = true;
             }
-            while (primed && base + 3 * STEP <= ready) step();
+            // Steps two at a time: a step's requests go to the registers its predecessor has just read, so after two
+            // steps every row is where the loop expects it; after one, leaving the loop costs a copy of rows that are
+            // still on their way, i.e. a wait for everything outstanding.
+            while (primed && base + 4 * STEP <= ready) {
+                step();
+                step();
+                covered = true;
+            }
         }
         if (!primed) prime();
         while (base < r1) step();
@@ -1131,6 +1175,7 @@ int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
     if (mode != HA_SELECT_SIMPLE || init_budget < 0 || recent_budget < 0 || heavy_budget < 0.0) return 0;
     // the heavy count as the selection takes it: truncated (int(k) above 1, int(S * fraction) otherwise)
     const double heavy = std::floor(heavy_budget > 1.0 ? heavy_budget : (double)max_seq_len * heavy_budget);
+    if (ha_sel::select_plan(B, Hc, max_seq_len).nchunk > kFusedMaxChunks) return 0;  // a row's chunk prefixes are kept in LDS
     return (double)init_budget + (double)recent_budget + heavy <= (double)kFusedListCap ? 1 : 0;
 }
 
@@ -1158,8 +1203,10 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     HA_REQUIRE(kc_stride_h >= (int64_t)max_seq_len * W && kc_stride_b >= kc_stride_h, HA_ERR_BAD_SHAPE,
                "code strides smaller than the rows they span");
     HA_REQUIRE(ha_sparse_decode_fused_applies(B, H, Hc, W, max_seq_len, init_budget, recent_budget, heavy_budget, HA_SELECT_SIMPLE),
-               HA_ERR_BAD_SHAPE, "selection larger than the %d-entry list of the fused path: use ha_select + ha_sparse_decode",
-               kFusedListCap);
+               HA_ERR_BAD_SHAPE,
+               "selection larger than the %d-entry list, or rows longer than the %d chunks, of the fused path: use ha_select + "
+               "ha_sparse_decode",
+               kFusedListCap, kFusedMaxChunks);
     HA_REQUIRE(select_workspace_bytes >= ha_select_workspace_bytes(B, H, Hc, W, max_seq_len), HA_ERR_WORKSPACE,
                "select workspace smaller than ha_select_workspace_bytes");
     const size_t need = ha_sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len);
@@ -1201,20 +1248,11 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     const dim3 grid(nsplit, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-    // a grid of at most one workgroup per CU: the instantiation that requests its scan codes a round ahead
-    const bool alone = rows * nsplit <= 256;
-
 #define HA_FUSED_LAUNCH(E_, U_, FW_)                                                                                              \
     do {                                                                                                                          \
-        if (alone)                                                                                                                \
-            hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_, false, true>), grid, dim3(512), 0, s, q, q_stride_b,      \
-                               q_stride_h, k, v, kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap,    \
-                               nullptr, sl2, 0, nsplit, part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f,          \
-                               AttnMask{}, 1);                                                                                    \
-        else                                                                                                                      \
-            hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,  \
-                               kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0,     \
-                               nsplit, part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);           \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,      \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);                       \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \

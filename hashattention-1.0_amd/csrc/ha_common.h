@@ -92,6 +92,15 @@ template <> struct Elem<ElemF32> {
         f[0] = __uint_as_float(r.a.x); f[1] = __uint_as_float(r.a.y); f[2] = __uint_as_float(r.a.z); f[3] = __uint_as_float(r.a.w);
         f[4] = __uint_as_float(r.b.x); f[5] = __uint_as_float(r.b.y); f[6] = __uint_as_float(r.b.z); f[7] = __uint_as_float(r.b.w);
     }
+    // sum over the slice of a[i] * b[i]
+    __device__ static __forceinline__ float dot8(const Raw8<ElemF32> &a, const Raw8<ElemF32> &b) {
+        float fa[8], fb[8], d = 0.f;
+        unpack(a, fa);
+        unpack(b, fb);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d = fmaf(fa[i], fb[i], d);
+        return d;
+    }
     __device__ static __forceinline__ void store1(void *row, int i, float x) { reinterpret_cast<float *>(row)[i] = x; }
 };
 template <> struct Elem<ElemBF16> {
@@ -109,6 +118,15 @@ template <> struct Elem<ElemBF16> {
     __device__ static __forceinline__ void unpack(const Raw8<ElemBF16> &r, float (&f)[8]) {
         f[0] = ha_bf16_lo(r.a.x); f[1] = ha_bf16_hi(r.a.x); f[2] = ha_bf16_lo(r.a.y); f[3] = ha_bf16_hi(r.a.y);
         f[4] = ha_bf16_lo(r.a.z); f[5] = ha_bf16_hi(r.a.z); f[6] = ha_bf16_lo(r.a.w); f[7] = ha_bf16_hi(r.a.w);
+    }
+    // sum over the slice of a[i] * b[i]: two elements per instruction (v_dot2c_f32_bf16), products and sums in fp32, nothing
+    // unpacked
+    __device__ static __forceinline__ float dot8(const Raw8<ElemBF16> &a, const Raw8<ElemBF16> &b) {
+        typedef __bf16 ha_bf16x2 __attribute__((ext_vector_type(2)));
+        float d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ha_bf16x2, a.a.x), __builtin_bit_cast(ha_bf16x2, b.a.x), 0.f, false);
+        d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ha_bf16x2, a.a.y), __builtin_bit_cast(ha_bf16x2, b.a.y), d, false);
+        d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ha_bf16x2, a.a.z), __builtin_bit_cast(ha_bf16x2, b.a.z), d, false);
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ha_bf16x2, a.a.w), __builtin_bit_cast(ha_bf16x2, b.a.w), d, false);
     }
     __device__ static __forceinline__ void store1(void *row, int i, float x) {
         reinterpret_cast<uint16_t *>(row)[i] = (uint16_t)ha_f32_to_bf16_bits(x);
@@ -133,6 +151,14 @@ template <> struct Elem<ElemF16> {
             f[2 * i] = __half2float(__ushort_as_half((unsigned short)(w[i] & 0xFFFFu)));
             f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(w[i] >> 16)));
         }
+    }
+    // sum over the slice of a[i] * b[i]: two elements per instruction (v_dot2c_f32_f16)
+    __device__ static __forceinline__ float dot8(const Raw8<ElemF16> &a, const Raw8<ElemF16> &b) {
+        typedef _Float16 ha_f16x2 __attribute__((ext_vector_type(2)));
+        float d = __builtin_amdgcn_fdot2(__builtin_bit_cast(ha_f16x2, a.a.x), __builtin_bit_cast(ha_f16x2, b.a.x), 0.f, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(ha_f16x2, a.a.y), __builtin_bit_cast(ha_f16x2, b.a.y), d, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(ha_f16x2, a.a.z), __builtin_bit_cast(ha_f16x2, b.a.z), d, false);
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(ha_f16x2, a.a.w), __builtin_bit_cast(ha_f16x2, b.a.w), d, false);
     }
     __device__ static __forceinline__ void store1(void *row, int i, float x) {
         reinterpret_cast<__half *>(row)[i] = __float2half_rn(x);

@@ -247,3 +247,25 @@ def test_long_rows_cut_into_pieces_of_equal_work(lens, heads, bits, heavy):
                        heavy_budget=heavy, dtype=torch.bfloat16, seed=77)
     rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
     assert "fused_err" in rep
+
+
+@pytest.mark.parametrize("batch,heads,lens,dtype", [(16, (32, 8, 8), "uniform", torch.bfloat16), (16, (32, 8, 16), "ragged", torch.bfloat16),
+                                                     (64, (8, 4, 4), "ragged", torch.float16), (40, (16, 2, 2), "short", torch.bfloat16)])
+def test_grids_of_512_rows_and_more(batch, heads, lens, dtype):
+    # 512 and more (sequence, head) rows: more fused workgroups than the device holds at once (two per CU), query heads that
+    # share a code head and scan the same codes side by side.  Equal lengths (on the host and on the device), ragged lengths
+    # (in-kernel plan), rows shorter than their windows.  Every stage against the oracle.
+    print(f"\n[case] many rows: B={batch} heads={heads} lengths {lens} {dtype}", flush=True)
+    rng = np.random.default_rng(batch + heads[0])
+    if lens == "uniform":
+        seq_lens = [9000] * batch
+    elif lens == "ragged":
+        seq_lens = [int(x) for x in rng.integers(1500, 9000, batch)]
+    else:
+        seq_lens = [int(x) for x in rng.integers(1, 1300, batch)]
+        seq_lens[0], seq_lens[1] = 1, 40
+    w = small_workload(name="many_rows", batch=batch, seq_lens=seq_lens, n_q_heads=heads[0], n_kv_heads=heads[1], n_code_heads=heads[2],
+                       init_budget=32, recent_budget=48, heavy_budget=1.0 / 16, dtype=dtype, seed=101)
+    assert batch * heads[0] >= 512
+    rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
+    assert "fused_err" in rep

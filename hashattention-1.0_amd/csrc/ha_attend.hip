@@ -141,6 +141,7 @@ constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are plan
 // 512 pieces: B = 1 at 32K 22.1 / 28.0 / 27.4 us, B = 4 at 128K 60.2 / 69.3 / 63.4, B = 8 at 64K 58.5 / 66.2 / 66.5)
 constexpr int kFusedUniformPieces = 256;
 constexpr int kFusedResident = 512;   // 512-thread workgroups resident at once: two on each of 256 CUs
+constexpr int kChunkScanRows = 48;    // a chunk's scan takes about as long as gathering this many rows (pieces of equal work)
 
 // NSLAB slabs of 256 codes of one chunk, four consecutive codes per lane and slab, for rows that do not take 128-bit loads
 // (misaligned, or strides that are no multiples of four codes): element loads inside [beg, end), zeros outside.
@@ -167,15 +168,42 @@ struct FusedRow {
     int cstar;  // the chunk of this workgroup that holds the r-th tie (ties before it are taken, after it not), or -1
 };
 
-// All threads of the workgroup: row constants and the windows.
-// Threshold and chunk prefixes of one row from its chunk histograms, by the workgroup itself (the work of
-// select_threshold_kernel for this row).  s_h: nchunk * NL words, s_pre: 2 * nchunk, s_meta: 4.
+// The row's chunk histograms (ha_select_histogram's), requested when the kernel starts and parked in registers: by the time
+// the threshold search wants them in LDS their round trip is over.
+template <int W, int NTT> struct HistTileRegs {
+    static constexpr int NL = 32 * W + 1;
+    static constexpr int N = (kFusedLocalChunks * NL + NTT - 1) / NTT;
+    uint32_t v[N];
+    __device__ __forceinline__ void request(const FusedSel &f, int64_t row) {
+        const uint32_t *hp = f.hist + row * f.nchunk * NL;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int at = (int)threadIdx.x + i * NTT;
+            v[i] = 0;
+            if (at < f.nchunk * NL) v[i] = hp[at];
+        }
+    }
+    __device__ __forceinline__ void to_lds(const FusedSel &f, uint32_t *s_h) const {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int at = (int)threadIdx.x + i * NTT;
+            if (at < f.nchunk * NL) s_h[at] = v[i];
+        }
+    }
+};
+
+// Setup of a row whose thresholds are derived in the launch (the work of select_threshold_kernel for this row, plus what the
+// workgroup needs of its own piece), three barriers: the histogram tile into LDS; level totals (a level per thread); then ONE
+// wave does the rest without leaving its registers - the threshold T and the tie remainder r (a level per lane: a wave scan
+// of the totals, the first lane whose running total reaches the budget), the chunk prefixes {#d < T, #d == T} (a chunk per
+// lane, two wave scans), the piece's chunk range by work (see fused_thresholds) and the chunk that holds the r-th tie (two
+// ballots) - and leaves s_pre and s_meta = {T, r, n_heavy, #d == T, first chunk, end chunk, tie chunk}.  At most 64 chunks.
 template <int W, int NTT>
-__device__ __forceinline__ void local_thresholds(const FusedSel &f, int64_t row, int S, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
+__device__ __forceinline__ void local_thresholds(const FusedSel &f, const HistTileRegs<W, NTT> &tile, int S, int sp, int row_pieces,
+                                                 int c0_even, int nc_even, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
     constexpr int NL = 32 * W + 1;
     const int tid = threadIdx.x;
-    const uint32_t *hp = f.hist + row * f.nchunk * NL;
-    for (int i = tid; i < f.nchunk * NL; i += NTT) s_h[i] = hp[i];
+    tile.to_lds(f, s_h);
     __syncthreads();
     uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile
     if (tid < NL) {
@@ -184,27 +212,64 @@ __device__ __forceinline__ void local_thresholds(const FusedSel &f, int64_t row,
         s_tot[tid] = t;
     }
     __syncthreads();
-    if (tid == 0) {
-        const ha_sel::RowBudget rb = ha_sel::row_budget(S, f.init, f.recent, f.heavy_budget);
-        int T, r, nheavy;
-        ha_sel::solve_threshold(s_tot, NL - 1, NL, rb.kk, HA_SELECT_SIMPLE, 0, T, r, nheavy);
-        s_meta[0] = T;
-        s_meta[1] = r;
-        s_meta[2] = nheavy;
-        s_meta[3] = T < NL ? (int)s_tot[T] : 0;
-    }
-    __syncthreads();
-    if (tid < HA_WAVE) {  // nchunk <= 64: one wave, one chunk per lane, two scans
-        const int T = s_meta[0];
+    if (tid < HA_WAVE) {
+        const int lane = tid;
+        const int kk = ha_sel::row_budget(S, f.init, f.recent, f.heavy_budget).kk;
+        // ha_sel::solve_threshold, simple mode: T = the first level at which the running total reaches kk, r = what is still
+        // missing in front of it; nothing (0, 0, 0) when the budget is empty
+        const uint32_t mine = lane < NL ? s_tot[lane] : 0u;
+        const uint32_t run = ha_sel::wave_inclusive_scan(mine);
+        int T = 0, r = 0, nheavy = 0;
+        if (kk > 0) {
+            const unsigned long long reached = __ballot(lane < NL && (int)run >= kk);
+            if (reached) {
+                T = __ffsll((long long)reached) - 1;
+                r = kk - __builtin_amdgcn_readlane((int)(run - mine), T);
+                nheavy = kk;
+            } else if (NL > HA_WAVE) {  // 64-bit codes: the one level beyond the lanes
+                const int before = __builtin_amdgcn_readlane((int)run, HA_WAVE - 1);
+                if (before + (int)s_tot[NL - 1] >= kk) {
+                    T = NL - 1;
+                    r = kk - before;
+                    nheavy = kk;
+                }
+            }
+        }
+        const int neq = (int)s_tot[T];
+        // chunk prefixes
         uint32_t lt = 0, eq = 0;
-        if (tid < f.nchunk) {
-            for (int l = 0; l < T && l < NL; ++l) lt += s_h[tid * NL + l];
-            if (T < NL) eq = s_h[tid * NL + T];
+        if (lane < f.nchunk) {
+            for (int l = 0; l < T; ++l) lt += s_h[lane * NL + l];
+            eq = s_h[lane * NL + T];
         }
         const uint32_t ilt = ha_sel::wave_inclusive_scan(lt), ieq = ha_sel::wave_inclusive_scan(eq);
-        if (tid < f.nchunk) {
-            s_pre[tid * 2] = (int32_t)(ilt - lt);
-            s_pre[tid * 2 + 1] = (int32_t)(ieq - eq);
+        const int pre_lt = (int)(ilt - lt), pre_eq = (int)(ieq - eq);
+        if (lane < f.nchunk) {
+            s_pre[lane * 2] = pre_lt;
+            s_pre[lane * 2 + 1] = pre_eq;
+        }
+        // this piece's chunks: an even share of the row's work (fused_thresholds has the rule), or the even share of its chunks
+        int c0 = c0_even, c1 = c0_even + nc_even;
+        if (row_pieces > 1) {
+            const int nc_row = min((S + f.chunk - 1) / f.chunk, f.nchunk);
+            const int total = nheavy + kChunkScanRows * nc_row;
+            const int wt = lane < nc_row ? pre_lt + min(pre_eq, r) + kChunkScanRows * lane : total;
+            const int t0 = (int)((int64_t)sp * total / row_pieces), t1 = (int)((int64_t)(sp + 1) * total / row_pieces);
+            const unsigned long long m0 = __ballot(wt >= t0), m1 = __ballot(wt >= t1);
+            c0 = sp == 0 ? 0 : min(m0 ? __ffsll((long long)m0) - 1 : f.nchunk, f.nchunk);
+            c1 = sp == row_pieces - 1 ? f.nchunk : min(m1 ? __ffsll((long long)m1) - 1 : f.nchunk, f.nchunk);
+            c1 = max(c1, c0);
+        }
+        // the chunk of this piece in which the r-th tie lies: ties before it do not reach r, ties through it pass r
+        const unsigned long long tie = __ballot(lane >= c0 && lane < c1 && lane < f.nchunk && pre_eq < r && r < (int)ieq);
+        if (lane == 0) {
+            s_meta[0] = T;
+            s_meta[1] = r;
+            s_meta[2] = nheavy;
+            s_meta[3] = neq;
+            s_meta[4] = c0;
+            s_meta[5] = c1;
+            s_meta[6] = tie ? __ffsll((long long)tie) - 1 : -1;
         }
     }
     __syncthreads();
@@ -231,17 +296,29 @@ __device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, 
 }
 
 // Setup, second half: threshold, prefixes, list length, the chunk of the r-th tie.
+// The pieces of a split row take equal shares of the row's WORK, not of its chunks: with ties broken by the lowest index
+// the taken part of the tie bucket lies at the front of the sequence, so pieces of equal token ranges gather very
+// different numbers of rows (B = 4 at 128K tokens: 2750 against 1350 rows, 56 against 43 us).  A piece's work is counted
+// as its selected rows plus kChunkScanRows per chunk it scans (a chunk's scan takes about as long as gathering that many
+// rows); piece i starts at the first chunk before which at least i / pieces of the row's work lies.  Every workgroup of
+// the row derives the same boundaries from the same prefixes, whichever launch derived the thresholds.
 template <int W, int NTT>
-__device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row, int S, int sp, int row_pieces, int *s_cstar,
-                                                 uint32_t *s_h, int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
+__device__ __forceinline__ void fused_thresholds(const FusedSel &f, const HistTileRegs<W, NTT> &tile, int64_t row, int S, int sp,
+                                                 int row_pieces, int *s_cstar, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta,
+                                                 FusedRow &fr) {
     const int tid = threadIdx.x;
+    fr.pre = s_pre;
+    // heavy tokens of the row before chunk c
+    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r); };
     if (f.hist) {
-        local_thresholds<W, NTT>(f, row, S, s_h, s_pre, s_meta);
+        local_thresholds<W, NTT>(f, tile, S, sp, row_pieces, fr.c0, fr.nc, s_h, s_pre, s_meta);
         fr.T = s_meta[0];
         fr.r = s_meta[1];
         fr.nheavy = s_meta[2];
         fr.neq = s_meta[3];
-        fr.pre = s_pre;
+        fr.c0 = s_meta[4];
+        fr.nc = s_meta[5] - fr.c0;
+        fr.cstar = s_meta[6];
         if (sp == 0 && tid == 0 && f.out_counts) f.out_counts[row] = fr.lo + fr.nheavy + (S - fr.hi);
     } else {
         fr.T = f.meta[row * 4 + 0];
@@ -250,47 +327,36 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         fr.neq = f.meta[row * 4 + 3];
         const int32_t *gp = f.chunk_pre + row * f.nchunk * 2;
         for (int i = tid; i < 2 * f.nchunk; i += NTT) s_pre[i] = gp[i];
+        if (tid == 0) *s_cstar = -1;
         __syncthreads();
-        fr.pre = s_pre;
-    }
-    // The pieces of a split row take equal shares of the row's WORK, not of its chunks: with ties broken by the lowest index
-    // the taken part of the tie bucket lies at the front of the sequence, so pieces of equal token ranges gather very
-    // different numbers of rows (B = 4 at 128K tokens: 2750 against 1350 rows, 56 against 43 us).  A piece's work is counted
-    // as its selected rows plus kChunkScanRows per chunk it scans (a chunk's scan takes about as long as gathering that many
-    // rows); piece i starts at the first chunk before which at least i / pieces of the row's work lies.  Every workgroup of
-    // the row derives the same boundaries from the same prefixes, whichever launch derived the thresholds.
-    if (row_pieces > 1 && f.nchunk <= HA_WAVE) {
-        constexpr int kChunkScanRows = 48;
-        if (tid < HA_WAVE) {  // nchunk <= 64: a chunk per lane
-            const int c = tid;
-            const int nc_row = min((S + f.chunk - 1) / f.chunk, f.nchunk);  // chunks that hold tokens of this row
-            const int total = fr.nheavy + kChunkScanRows * nc_row;
-            const int wt = c < nc_row ? fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r) + kChunkScanRows * c : total;
-            const int t0 = (int)((int64_t)sp * total / row_pieces), t1 = (int)((int64_t)(sp + 1) * total / row_pieces);
-            const unsigned long long m0 = __ballot(wt >= t0), m1 = __ballot(wt >= t1);
-            if (tid == 0) {
-                s_meta[4] = sp == 0 ? 0 : min(m0 ? __ffsll((long long)m0) - 1 : f.nchunk, f.nchunk);
-                s_meta[5] = sp == row_pieces - 1 ? f.nchunk : min(m1 ? __ffsll((long long)m1) - 1 : f.nchunk, f.nchunk);
+        if (row_pieces > 1 && f.nchunk <= HA_WAVE) {
+            if (tid < HA_WAVE) {  // nchunk <= 64: a chunk per lane
+                const int c = tid;
+                const int nc_row = min((S + f.chunk - 1) / f.chunk, f.nchunk);  // chunks that hold tokens of this row
+                const int total = fr.nheavy + kChunkScanRows * nc_row;
+                const int wt = c < nc_row ? fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r) + kChunkScanRows * c : total;
+                const int t0 = (int)((int64_t)sp * total / row_pieces), t1 = (int)((int64_t)(sp + 1) * total / row_pieces);
+                const unsigned long long m0 = __ballot(wt >= t0), m1 = __ballot(wt >= t1);
+                if (tid == 0) {
+                    s_meta[4] = sp == 0 ? 0 : min(m0 ? __ffsll((long long)m0) - 1 : f.nchunk, f.nchunk);
+                    s_meta[5] = sp == row_pieces - 1 ? f.nchunk : min(m1 ? __ffsll((long long)m1) - 1 : f.nchunk, f.nchunk);
+                }
             }
+            __syncthreads();
+            fr.c0 = s_meta[4];
+            fr.nc = max(s_meta[5] - fr.c0, 0);
+        }
+        for (int i = tid; i < fr.nc; i += NTT) {
+            const int c = fr.c0 + i;
+            const int eq0 = fr.pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? fr.pre[(c + 1) * 2 + 1] : fr.neq;
+            if (eq0 < fr.r && fr.r < eq1) *s_cstar = c;  // at most one chunk of the row
         }
         __syncthreads();
-        fr.c0 = s_meta[4];
-        fr.nc = max(s_meta[5] - fr.c0, 0);
+        fr.cstar = *s_cstar;
     }
     const int c1 = fr.c0 + fr.nc;
-    // heavy tokens of the row before chunk c
-    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r); };
     fr.hbase = fr.nwin - rank(fr.c0);
     fr.n = min(fr.nwin + max(rank(c1) - rank(fr.c0), 0), kFusedListCap);
-    if (tid == 0) *s_cstar = -1;
-    __syncthreads();
-    for (int i = tid; i < fr.nc; i += NTT) {
-        const int c = fr.c0 + i;
-        const int eq0 = fr.pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? fr.pre[(c + 1) * 2 + 1] : fr.neq;
-        if (eq0 < fr.r && fr.r < eq1) *s_cstar = c;  // at most one chunk of the row
-    }
-    __syncthreads();
-    fr.cstar = *s_cstar;
 }
 
 // Scan rounds work on staged codes: the codes of a wave's group travel from memory straight into a 4 KiB region of LDS that
@@ -529,7 +595,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __shared__ uint32_t s_tile[FW > 0 && !kTileInRaw ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
     uint32_t *s_h = kTileInRaw ? s_raw : s_tile;
     __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedMaxChunks : 1];
-    __shared__ int32_t s_meta[6];
+    __shared__ int32_t s_meta[8];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
     // (head in group, group) instead of heads in order puts the query heads of one KV group 8*k apart when
@@ -593,6 +659,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     int r0, r1, nsplit;
     const int32_t *ix = nullptr;
     FusedRow fr = {};
+    [[maybe_unused]] HistTileRegs<(FW > 0 ? FW : 1), NT> hist_tile;
     int j_max = 0;  // fused: last token of the sequence (list entries are clamped to it: a wrong entry must not become a wild address)
     if constexpr (FW > 0) {
         int S = seq_lens ? seq_lens[b] : max_S;
@@ -609,6 +676,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             }
             return;
         }
+        if (fsel.hist) hist_tile.request(fsel, row);
         fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr);
         j_max = max(S - 1, 0);
         r0 = 0;
@@ -766,7 +834,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         {
             int S = seq_lens ? seq_lens[b] : max_S;
             if (S > max_S) S = max_S;
-            fused_thresholds<FW, NT>(fsel, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
+            fused_thresholds<FW, NT>(fsel, hist_tile, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
         }
         r1 = fr.n;
         const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;

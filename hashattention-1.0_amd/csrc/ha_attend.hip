@@ -183,18 +183,22 @@ template <int W, int NTT> struct HistTileRegs {
             if (at < f.nchunk * NL) v[i] = hp[at];
         }
     }
-    __device__ __forceinline__ void to_lds(const FusedSel &f, uint32_t *s_h) const {
+    // the tile into LDS, and every counter added to its level's total (s_tot: NL words, zero)
+    __device__ __forceinline__ void to_lds(const FusedSel &f, uint32_t *s_h, uint32_t *s_tot) const {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int at = (int)threadIdx.x + i * NTT;
-            if (at < f.nchunk * NL) s_h[at] = v[i];
+            if (at < f.nchunk * NL) {
+                s_h[at] = v[i];
+                if (v[i]) atomicAdd(&s_tot[at % NL], v[i]);
+            }
         }
     }
 };
 
 // Setup of a row whose thresholds are derived in the launch (the work of select_threshold_kernel for this row, plus what the
-// workgroup needs of its own piece), three barriers: the histogram tile into LDS; level totals (a level per thread); then ONE
-// wave does the rest without leaving its registers - the threshold T and the tie remainder r (a level per lane: a wave scan
+// workgroup needs of its own piece), two barriers: the histogram tile into LDS, every counter added to its level's total on
+// the way; then ONE wave does the rest without leaving its registers - the threshold T and the tie remainder r (a level per lane: a wave scan
 // of the totals, the first lane whose running total reaches the budget), the chunk prefixes {#d < T, #d == T} (a chunk per
 // lane, two wave scans), the piece's chunk range by work (see fused_thresholds) and the chunk that holds the r-th tie (two
 // ballots) - and leaves s_pre and s_meta = {T, r, n_heavy, #d == T, first chunk, end chunk, tie chunk}.  At most 64 chunks.
@@ -203,14 +207,8 @@ __device__ __forceinline__ void local_thresholds(const FusedSel &f, const HistTi
                                                  int c0_even, int nc_even, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
     constexpr int NL = 32 * W + 1;
     const int tid = threadIdx.x;
-    tile.to_lds(f, s_h);
-    __syncthreads();
-    uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile
-    if (tid < NL) {
-        uint32_t t = 0;
-        for (int c = 0; c < f.nchunk; ++c) t += s_h[c * NL + tid];
-        s_tot[tid] = t;
-    }
+    uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile, zeroed by the caller before its last barrier
+    tile.to_lds(f, s_h, s_tot);
     __syncthreads();
     if (tid < HA_WAVE) {
         const int lane = tid;
@@ -676,7 +674,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             }
             return;
         }
-        if (fsel.hist) hist_tile.request(fsel, row);
+        if (fsel.hist) {
+            hist_tile.request(fsel, row);
+            if (tid < 32 * FW + 1) s_h[fsel.nchunk * (32 * FW + 1) + tid] = 0;  // the level totals (local_thresholds)
+        }
         fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr);
         j_max = max(S - 1, 0);
         r0 = 0;
@@ -816,20 +817,22 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         ha_sel::Code<FW> qcode = ha_sel::load_qcode<FW>(fsel.qcodes, row);
         qcode.w0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w0);
         if constexpr (FW == 2) qcode.w1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w1);
-        // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out
-        bool primed = false;
-        if (fr.nwin >= 2 * STEP) {
-            prime();
-            primed = true;
-        }
-        // the codes of the first round are requested before the thresholds are worked out too, when the workgroup's chunks
-        // are known by then (a row in one piece) and the histogram tile has a place of its own
+        // the codes of the first round are requested before the thresholds are worked out, when the workgroup's chunks are
+        // known by then (a row in one piece) and the histogram tile has a place of its own - and before the window rows:
+        // the compiler's wait for the histogram tile (requested earlier still) counts the requests it knows, so unseen
+        // requests behind the rows would make it wait for as many rows
         bool staged_early = false;
         if constexpr (!kTileInRaw) {
             if (row_pieces == 1) {
                 fused_round_stage<FW, GS, NW>(fsel, fr, b, h, 0, fr.nc * (fsel.chunk / gc), s_raw);
                 staged_early = true;
             }
+        }
+        // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out too
+        bool primed = false;
+        if (fr.nwin >= 2 * STEP) {
+            prime();
+            primed = true;
         }
         {
             int S = seq_lens ? seq_lens[b] : max_S;

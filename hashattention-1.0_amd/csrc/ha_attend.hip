@@ -198,17 +198,16 @@ template <int W, int NTT> struct HistTileRegs {
 
 // Setup of a row whose thresholds are derived in the launch (the work of select_threshold_kernel for this row, plus what the
 // workgroup needs of its own piece), two barriers: the histogram tile into LDS, every counter added to its level's total on
-// the way; then ONE wave does the rest without leaving its registers - the threshold T and the tie remainder r (a level per lane: a wave scan
+// the way (HistTileRegs::to_lds, by the caller); then ONE wave does the rest without leaving its registers - the threshold T and the tie remainder r (a level per lane: a wave scan
 // of the totals, the first lane whose running total reaches the budget), the chunk prefixes {#d < T, #d == T} (a chunk per
 // lane, two wave scans), the piece's chunk range by work (see fused_thresholds) and the chunk that holds the r-th tie (two
 // ballots) - and leaves s_pre and s_meta = {T, r, n_heavy, #d == T, first chunk, end chunk, tie chunk}.  At most 64 chunks.
 template <int W, int NTT>
-__device__ __forceinline__ void local_thresholds(const FusedSel &f, const HistTileRegs<W, NTT> &tile, int S, int sp, int row_pieces,
-                                                 int c0_even, int nc_even, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
+__device__ __forceinline__ void local_thresholds(const FusedSel &f, int S, int sp, int row_pieces, int c0_even, int nc_even,
+                                                 const uint32_t *s_h, int32_t *s_pre, int32_t *s_meta) {
     constexpr int NL = 32 * W + 1;
     const int tid = threadIdx.x;
-    uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile, zeroed by the caller before its last barrier
-    tile.to_lds(f, s_h, s_tot);
+    const uint32_t *s_tot = s_h + f.nchunk * NL;  // NL words behind the tile: the caller has stored the tile and added up the totals
     __syncthreads();
     if (tid < HA_WAVE) {
         const int lane = tid;
@@ -237,8 +236,13 @@ __device__ __forceinline__ void local_thresholds(const FusedSel &f, const HistTi
         // chunk prefixes
         uint32_t lt = 0, eq = 0;
         if (lane < f.nchunk) {
-            for (int l = 0; l < T; ++l) lt += s_h[lane * NL + l];
-            eq = s_h[lane * NL + T];
+            const uint32_t *mine_h = s_h + lane * NL;
+            uint32_t a1 = 0, a2 = 0, a3 = 0;  // four sums: four reads on their way at a time, not one
+            int l = 0;
+            for (; l + 4 <= T; l += 4) lt += mine_h[l], a1 += mine_h[l + 1], a2 += mine_h[l + 2], a3 += mine_h[l + 3];
+            for (; l < T; ++l) lt += mine_h[l];
+            lt += a1 + a2 + a3;
+            eq = mine_h[T];
         }
         const uint32_t ilt = ha_sel::wave_inclusive_scan(lt), ieq = ha_sel::wave_inclusive_scan(eq);
         const int pre_lt = (int)(ilt - lt), pre_eq = (int)(ieq - eq);
@@ -301,15 +305,14 @@ __device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, 
 // rows); piece i starts at the first chunk before which at least i / pieces of the row's work lies.  Every workgroup of
 // the row derives the same boundaries from the same prefixes, whichever launch derived the thresholds.
 template <int W, int NTT>
-__device__ __forceinline__ void fused_thresholds(const FusedSel &f, const HistTileRegs<W, NTT> &tile, int64_t row, int S, int sp,
-                                                 int row_pieces, int *s_cstar, uint32_t *s_h, int32_t *s_pre, int32_t *s_meta,
-                                                 FusedRow &fr) {
+__device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row, int S, int sp, int row_pieces, int *s_cstar,
+                                                 const uint32_t *s_h, int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
     const int tid = threadIdx.x;
     fr.pre = s_pre;
     // heavy tokens of the row before chunk c
     auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r); };
     if (f.hist) {
-        local_thresholds<W, NTT>(f, tile, S, sp, row_pieces, fr.c0, fr.nc, s_h, s_pre, s_meta);
+        local_thresholds<W, NTT>(f, S, sp, row_pieces, fr.c0, fr.nc, s_h, s_pre, s_meta);
         fr.T = s_meta[0];
         fr.r = s_meta[1];
         fr.nheavy = s_meta[2];
@@ -814,9 +817,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         constexpr int gc = GS * HA_WAVE * 4;                      // codes per wave and round; divides every chunk size
         // the row's query code, once and in scalar registers: loaded in a scan round it would be the youngest request of the
         // wave there, and waiting for it would mean waiting for every row on its way
+        // (requested here, moved to the scalar registers behind the threshold search: in front of it the move would wait a
+        // memory round trip before the window rows and the first codes are even requested)
         ha_sel::Code<FW> qcode = ha_sel::load_qcode<FW>(fsel.qcodes, row);
-        qcode.w0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w0);
-        if constexpr (FW == 2) qcode.w1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w1);
         // the codes of the first round are requested before the thresholds are worked out, when the workgroup's chunks are
         // known by then (a row in one piece) and the histogram tile has a place of its own - and before the window rows:
         // the compiler's wait for the histogram tile (requested earlier still) counts the requests it knows, so unseen
@@ -828,18 +831,26 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 staged_early = true;
             }
         }
-        // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out too
+        // the windows alone fill the first two steps: their rows are requested before the thresholds are worked out too.
+        // The histogram tile goes from its registers to LDS behind them, written out in either branch: placed behind the
+        // branch, the compiler's wait for the tile would have to assume that no rows were requested and wait for all but two
+        // of the requests it knows - for the window rows too.
         bool primed = false;
         if (fr.nwin >= 2 * STEP) {
             prime();
             primed = true;
+            if (fsel.hist) hist_tile.to_lds(fsel, s_h, s_h + fsel.nchunk * (32 * FW + 1));
+        } else {
+            if (fsel.hist) hist_tile.to_lds(fsel, s_h, s_h + fsel.nchunk * (32 * FW + 1));
         }
         {
             int S = seq_lens ? seq_lens[b] : max_S;
             if (S > max_S) S = max_S;
-            fused_thresholds<FW, NT>(fsel, hist_tile, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
+            fused_thresholds<FW, NT>(fsel, row, S, sp, row_pieces, &s_cstar, s_h, s_pre, s_meta, fr);
         }
         r1 = fr.n;
+        qcode.w0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w0);
+        if constexpr (FW == 2) qcode.w1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)qcode.w1);
         const int n_groups = fr.nheavy > 0 ? fr.nc * (fsel.chunk / gc) : 0;
         const int rounds = (n_groups + NW - 1) / NW;
         // codes requested for a round that will not take place must not arrive in the partial results later

@@ -133,7 +133,9 @@ struct AttnMask {
     int len, by_slot;
 };
 constexpr int kFusedLocalChunks = 64;
-constexpr int kFusedMaxChunks = 256;  // chunks of a row of the fused path: the row's chunk prefixes are kept in LDS
+// chunk prefixes a workgroup keeps in LDS: those of the whole row up to this many chunks, of its own piece beyond (the host
+// cuts longer rows into pieces of at most this many chunks)
+constexpr int kFusedMaxChunks = 256;
 constexpr int kFusedSortBatch = 128;  // ragged batches up to this size are planned in the kernel (order and piece size)
 // a batch of equal lengths is cut into this many workgroups (one per CU): measured against 512 at 64K tokens, B = 6: 76.6
 // against 82.3 us, B = 8: 76.7 against 81.2, B = 12: 107.1 against 125.5; B = 1 at 32K: 39.2 against 40.9; B = 4 at 128K: 84.1
@@ -162,6 +164,9 @@ struct FusedRow {
     // from either place through one pointer they would be flat loads, and a flat load in a scan round waits for every
     // outstanding request of the wave, rows on their way included.)
     const int32_t *pre;
+    int pre_first;  // the chunk pre[0], pre[1] belong to (0 unless only the piece's prefixes were copied)
+    __device__ __forceinline__ int pre_lt(int c) const { return pre[(c - pre_first) * 2]; }
+    __device__ __forceinline__ int pre_eq(int c) const { return pre[(c - pre_first) * 2 + 1]; }
     int lo, hi, T, r, nheavy, neq, c0, nc, n;
     int nwin;   // window entries at the head of this workgroup's list (sink if it has the first chunk, recent if the last)
     int hbase;  // list position of a heavy token = hbase + (#d < T before it) + min(#d == T before it, r)
@@ -309,8 +314,9 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
                                                  const uint32_t *s_h, int32_t *s_pre, int32_t *s_meta, FusedRow &fr) {
     const int tid = threadIdx.x;
     fr.pre = s_pre;
+    fr.pre_first = 0;
     // heavy tokens of the row before chunk c
-    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r); };
+    auto rank = [&](int c) { return c >= f.nchunk ? fr.nheavy : fr.pre_lt(c) + min(fr.pre_eq(c), fr.r); };
     if (f.hist) {
         local_thresholds<W, NTT>(f, S, sp, row_pieces, fr.c0, fr.nc, s_h, s_pre, s_meta);
         fr.T = s_meta[0];
@@ -327,7 +333,13 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         fr.nheavy = f.meta[row * 4 + 2];
         fr.neq = f.meta[row * 4 + 3];
         const int32_t *gp = f.chunk_pre + row * f.nchunk * 2;
-        for (int i = tid; i < 2 * f.nchunk; i += NTT) s_pre[i] = gp[i];
+        if (f.nchunk <= kFusedMaxChunks) {
+            for (int i = tid; i < 2 * f.nchunk; i += NTT) s_pre[i] = gp[i];
+        } else {  // a long row: this piece's chunks and the one behind them (no more than kFusedMaxChunks + 1: the host sees to it)
+            fr.pre_first = fr.c0;
+            const int n = min(fr.nc + 1, f.nchunk - fr.c0);
+            for (int i = tid; i < 2 * n; i += NTT) s_pre[i] = gp[2 * fr.c0 + i];
+        }
         if (tid == 0) *s_cstar = -1;
         __syncthreads();
         if (row_pieces > 1 && f.nchunk <= HA_WAVE) {
@@ -335,7 +347,7 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
                 const int c = tid;
                 const int nc_row = min((S + f.chunk - 1) / f.chunk, f.nchunk);  // chunks that hold tokens of this row
                 const int total = fr.nheavy + kChunkScanRows * nc_row;
-                const int wt = c < nc_row ? fr.pre[c * 2] + min(fr.pre[c * 2 + 1], fr.r) + kChunkScanRows * c : total;
+                const int wt = c < nc_row ? fr.pre_lt(c) + min(fr.pre_eq(c), fr.r) + kChunkScanRows * c : total;
                 const int t0 = (int)((int64_t)sp * total / row_pieces), t1 = (int)((int64_t)(sp + 1) * total / row_pieces);
                 const unsigned long long m0 = __ballot(wt >= t0), m1 = __ballot(wt >= t1);
                 if (tid == 0) {
@@ -349,7 +361,7 @@ __device__ __forceinline__ void fused_thresholds(const FusedSel &f, int64_t row,
         }
         for (int i = tid; i < fr.nc; i += NTT) {
             const int c = fr.c0 + i;
-            const int eq0 = fr.pre[c * 2 + 1], eq1 = c + 1 < f.nchunk ? fr.pre[(c + 1) * 2 + 1] : fr.neq;
+            const int eq0 = fr.pre_eq(c), eq1 = c + 1 < f.nchunk ? fr.pre_eq(c + 1) : fr.neq;
             if (eq0 < fr.r && fr.r < eq1) *s_cstar = c;  // at most one chunk of the row
         }
         __syncthreads();
@@ -475,7 +487,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
         } else {
             // any other chunk takes all of its ties (those before it do not reach r) or none: one compare per code, against
             // T + 1 or T, and the chunk counts no ties of its own
-            const int neg_t = -(fr.T + (fr.pre[c * 2 + 1] < fr.r ? 1 : 0));
+            const int neg_t = -(fr.T + (fr.pre_eq(c) < fr.r ? 1 : 0));
 #pragma unroll
             for (int s = GS - 1; s >= 0; --s)
 #pragma unroll
@@ -503,7 +515,7 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 
     // tokens of the row with d < T / d == T before this group: the chunk's prefix plus the chunk's earlier groups,
     // which are the gi waves just below this one
-    int a = fr.pre[c * 2], t = fr.pre[c * 2 + 1];
+    int a = fr.pre_lt(c), t = fr.pre_eq(c);
     for (int w2 = wave - gi; w2 < wave; ++w2) {
         const uint32_t v = s_cnt[w2];
         a += (int)(v & 0xFFFFu);
@@ -595,7 +607,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     static_assert(!kTileInRaw || (kFusedLocalChunks + 1) * (32 * FW + 1) <= kRawWords, "the histogram tile fits the staging space");
     __shared__ uint32_t s_tile[FW > 0 && !kTileInRaw ? (kFusedLocalChunks + 1) * (32 * FW + 1) : 1];
     uint32_t *s_h = kTileInRaw ? s_raw : s_tile;
-    __shared__ int32_t s_pre[FW > 0 ? 2 * kFusedMaxChunks : 1];
+    __shared__ int32_t s_pre[FW > 0 ? 2 * (kFusedMaxChunks + 1) : 1];
     __shared__ int32_t s_meta[8];
 
     // Workgroups are handed to the 8 XCDs round-robin in launch order.  Walking blockIdx.y over
@@ -646,6 +658,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 }
                 const unsigned long long ok = __ballot((int64_t)total * H <= kFusedResident);
                 int pick = ok ? (__ffsll((long long)ok)) * cstep : 64 * cstep;
+                pick = min(pick, kFusedMaxChunks);  // the chunk prefixes a workgroup keeps in LDS
                 pick = max(pick, (longest + (int)gridDim.x - 1) / (int)gridDim.x);  // the grid has gridDim.x workgroups per row
                 if (tid == 192) s_plan[1] = pick;
             }
@@ -1248,7 +1261,8 @@ static int fused_chunks_per_split(int B, int H, int nchunk, bool ragged) {
     if (ragged && B > 1 && B <= kFusedSortBatch && rows < kFusedResident) want = std::min<int64_t>(4 * want, (kFusedResident + H - 1) / H);
     if (want > nchunk) want = nchunk;
     if (want < 1) want = 1;
-    return (int)((nchunk + want - 1) / want);
+    // no piece longer than the chunk prefixes a workgroup keeps in LDS
+    return std::min((int)((nchunk + want - 1) / want), kFusedMaxChunks);
 }
 
 int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len, int init_budget, int recent_budget, double heavy_budget,
@@ -1257,7 +1271,6 @@ int ha_sparse_decode_fused_applies(int B, int H, int Hc, int W, int max_seq_len,
     if (mode != HA_SELECT_SIMPLE || init_budget < 0 || recent_budget < 0 || heavy_budget < 0.0) return 0;
     // the heavy count as the selection takes it: truncated (int(k) above 1, int(S * fraction) otherwise)
     const double heavy = std::floor(heavy_budget > 1.0 ? heavy_budget : (double)max_seq_len * heavy_budget);
-    if (ha_sel::select_plan(B, Hc, max_seq_len).nchunk > kFusedMaxChunks) return 0;  // a row's chunk prefixes are kept in LDS
     return (double)init_budget + (double)recent_budget + heavy <= (double)kFusedListCap ? 1 : 0;
 }
 
@@ -1285,10 +1298,8 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     HA_REQUIRE(kc_stride_h >= (int64_t)max_seq_len * W && kc_stride_b >= kc_stride_h, HA_ERR_BAD_SHAPE,
                "code strides smaller than the rows they span");
     HA_REQUIRE(ha_sparse_decode_fused_applies(B, H, Hc, W, max_seq_len, init_budget, recent_budget, heavy_budget, HA_SELECT_SIMPLE),
-               HA_ERR_BAD_SHAPE,
-               "selection larger than the %d-entry list, or rows longer than the %d chunks, of the fused path: use ha_select + "
-               "ha_sparse_decode",
-               kFusedListCap, kFusedMaxChunks);
+               HA_ERR_BAD_SHAPE, "selection larger than the %d-entry list of the fused path: use ha_select + ha_sparse_decode",
+               kFusedListCap);
     HA_REQUIRE(select_workspace_bytes >= ha_select_workspace_bytes(B, H, Hc, W, max_seq_len), HA_ERR_WORKSPACE,
                "select workspace smaller than ha_select_workspace_bytes");
     const size_t need = ha_sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len);

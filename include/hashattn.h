@@ -302,9 +302,8 @@ int ha_sparse_decode_heavy(const void *q, int64_t q_stride_b, int64_t q_stride_h
  * workspace it filled.  With thresholds_ready = 0 the workspace needs only the chunk histograms (ha_select_histogram,
  * the first launch alone): every workgroup of the attention launch derives its row's threshold and prefixes
  * itself and out_counts (may be NULL) is written by that launch - one launch less per step; rows of at most 64
- * chunks (max_seq_len <= 262144, ha_sparse_decode_fused_local_thresholds returns 1).  Only HA_SELECT_SIMPLE, only while
- * init + recent + heavy <= 8192 entries (a row's list is kept in LDS) and only for rows of at most 256 chunks
- * (max_seq_len <= 1048576: a row's chunk prefixes are kept in LDS too) - ha_sparse_decode_fused_applies returns 1;
+ * chunks (max_seq_len <= 262144, ha_sparse_decode_fused_local_thresholds returns 1).  Only HA_SELECT_SIMPLE, and only while
+ * init + recent + heavy <= 8192 entries: a row's list is kept in LDS (ha_sparse_decode_fused_applies returns 1);
  * otherwise use ha_select + ha_sparse_decode.  Replaces the same
  * reference lines as those two (hashattention_llama.py:401-446, 585-615; efficiency/kernels/torchatt.py:52-71).
  */

@@ -269,3 +269,17 @@ def test_grids_of_512_rows_and_more(batch, heads, lens, dtype):
     assert batch * heads[0] >= 512
     rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
     assert "fused_err" in rep
+
+
+@pytest.mark.parametrize("tokens,heads", [(1 << 20, (2, 1, 1)), (300001, (4, 2, 2)), (1 << 19, (8, 8, 8))])
+def test_rows_of_many_chunks_through_the_fused_path(tokens, heads):
+    # rows of more than 256 chunks (few code heads: chunks of 1024 tokens, up to 1024 of them here): a fused workgroup keeps only
+    # the chunk prefixes of its own piece in LDS, pieces hold at most 256 chunks, thresholds come from ha_select_prepare (more
+    # than 64 chunks).  With 8 code heads the same length has 256 chunks and the whole row's prefixes fit.  Every stage against
+    # the oracle.
+    print(f"\n[case] row of {tokens} tokens, heads {heads}", flush=True)
+    w = small_workload(name="many_chunks", batch=1, seq_lens=[tokens], n_q_heads=heads[0], n_kv_heads=heads[1], n_code_heads=heads[2],
+                       init_budget=64, recent_budget=64, heavy_budget=4000.0, dtype=torch.bfloat16, seed=17)
+    assert _ops.fused_applies(1, heads[0], heads[2], 1, tokens, 64, 64, 4000.0)
+    rep = run_decode_case(w, check_encode=False, check_dense=False, verbose=True)
+    assert "fused_err" in rep

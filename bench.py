@@ -352,6 +352,23 @@ class InputSet:
     def attend_lists(self):
         self.layer.attend(self.q3, self.p.k, self.p.v, self.out)
 
+    def attend_fused_paged(self):
+        """The fused launch reading the same cache through a token -> slot table that maps every token to its own row."""
+        from hashattention import _ops
+        l, w = self.layer, self.w
+        if not hasattr(self, "slots"):
+            self.slots = self.torch.arange(self.S, dtype=self.torch.int32, device=self.dev).repeat(w.batch, 1)
+        _ops.sparse_decode_fused(self.q3, self.p.k, self.p.v, l.codes, l.qcodes.view(w.batch, w.n_q_heads, l.W), self.S, self.seq_lens,
+                                 l.init_budget, l.recent_budget, l.heavy_budget, l.ws_select, l.sm_scale, self.out, l.ws_fused,
+                                 thresholds_ready=not l.local_thresholds, out_counts=l.counts, slots=self.slots)
+
+    def attend_lists_paged(self):
+        from hashattention import _ops
+        l = self.layer
+        if not hasattr(self, "slots"):
+            self.slots = self.torch.arange(self.S, dtype=self.torch.int32, device=self.dev).repeat(self.w.batch, 1)
+        _ops.sparse_decode(self.q3, self.p.k, self.p.v, l.idx, l.counts, l.sm_scale, self.out, l.ws_attend, slots=self.slots)
+
 
 def first_step_probe(s, args, torch):
     """The first decode step after a prefill, per layer, with one key-side hash MLP per query head (the reference's layout):
@@ -492,6 +509,13 @@ def main():
         ms_prepare = time_rotating(rot("select_prepare"), args.steps, args.warmup, torch)
         ms_attend = time_rotating(rot("attend_fused"), args.steps, args.warmup, torch)
         ms_attend_single = time_gpu(s0.attend_fused, args.steps, args.warmup, torch)
+        # the same launches through a token -> slot table (identity: every token at its own row), timed right behind the plain
+        # ones; outputs must be the same bits
+        ref_out = s0.out.clone()
+        s0.attend_fused_paged()
+        paged_ok = bool(torch.equal(s0.out, ref_out))
+        ms_attend_paged = time_rotating(rot("attend_fused_paged"), args.steps, args.warmup, torch)
+        ms_lists_paged = time_rotating(rot("attend_lists_paged"), args.steps, args.warmup, torch)
     else:
         ms_attend = time_rotating(rot("attend_lists"), args.steps, args.warmup, torch)
     out_dense = torch.empty_like(s0.out)
@@ -562,6 +586,11 @@ def main():
         "dense_hbm_gbps": ab["dense"] / (ms_dense * 1e-3) / 1e9,
         "tokens_per_s_layer": B / (ms_step * 1e-3),
         "sparse_vs_dense_max_abs": err,
+        **({"paged_cache_identity_table": {"select_attend_fused_us": ms_attend_paged * 1e3, "vs_unpaged": ms_attend_paged / ms_attend,
+                                           "two_launch_attend_us": ms_lists_paged * 1e3, "two_launch_vs_unpaged": ms_lists_paged / ms_attend_lists,
+                                           "same_bits_as_unpaged": paged_ok,
+                                           "how": "ha_sparse_decode_fused_paged / ha_sparse_decode_paged with slot_of_token[b, j] = j on the same cache"}}
+           if fused else {}),
         # the scoring stream (XOR + popcount over every cached code, histogrammed on the fly) as its own launch
         **({"score_roofline": roofline_obj("select_hist_kernel", ab["score"], ms_prepare)} if fused and layer.local_thresholds else {}),
         "roofline": roofline_obj("sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", attend_bytes, ms_attend,

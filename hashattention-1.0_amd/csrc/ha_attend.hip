@@ -132,6 +132,13 @@ struct AttnMask {
     int64_t stride_b;
     int len, by_slot;
 };
+// Token -> slot map of a paged cache (the `Req_to_tokens` table of efficiency/kernels/flash_fwd_sparse.py:396-470): the K/V
+// row of token j of sequence b is row slots[b * stride_b + j] of the cache.  slots == nullptr: the identity.
+struct SlotMap {
+    const int32_t *slots;
+    int64_t stride_b;
+    int max_slot;  // n_slots - 1: entries of the fused launch's LDS list are clamped to it
+};
 constexpr int kFusedLocalChunks = 64;
 // chunk prefixes a workgroup keeps in LDS: those of the whole row up to this many chunks, of its own piece beyond (the host
 // cuts longer rows into pieces of at most this many chunks)
@@ -285,7 +292,8 @@ __device__ __forceinline__ void local_thresholds(const FusedSel &f, int S, int s
 // Setup, first half: what is known without any threshold - the row's window geometry, this workgroup's chunks, and the
 // window entries at the head of its list (the loop can be primed on them while the second half runs).
 template <int NTT>
-__device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, int cps, int row_pieces, int32_t *s_list, FusedRow &fr) {
+__device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, int cps, int row_pieces, int32_t *s_list, FusedRow &fr,
+                                              const int32_t *slot_row /* this sequence's token -> slot map, or nullptr */) {
     const int tid = threadIdx.x;
     fr.lo = min(f.init, S);
     fr.hi = max(S - f.recent, fr.lo);
@@ -296,9 +304,10 @@ __device__ __forceinline__ void fused_windows(const FusedSel &f, int S, int sp, 
     // sink: first workgroup; recent: last workgroup of the row
     const int n_sink = sp == 0 ? fr.lo : 0, n_recent = sp == row_pieces - 1 ? S - fr.hi : 0;
     fr.nwin = min(n_sink + n_recent, kFusedListCap);
-    for (int i = tid; i < n_sink && i < fr.nwin; i += NTT) s_list[i] = i;
+    // with a slot map the list holds slots: the window entries are translated here, the heavy ones by fused_round
+    for (int i = tid; i < n_sink && i < fr.nwin; i += NTT) s_list[i] = slot_row ? slot_row[i] : i;
     for (int i = tid; i < n_recent; i += NTT)
-        if (n_sink + i < fr.nwin) s_list[n_sink + i] = fr.hi + i;
+        if (n_sink + i < fr.nwin) s_list[n_sink + i] = slot_row ? slot_row[fr.hi + i] : fr.hi + i;
     __syncthreads();
 }
 
@@ -392,6 +401,15 @@ __device__ __forceinline__ void request_16_bytes_to_lds(const uint32_t *src, con
                  : "v"(src), "s"(lds_byte_address)
                  : "memory");
 }
+// One 4-byte request per active lane: lane l's word lands at dst + l (dst uniform over the wave); inactive lanes write nothing.
+__device__ __forceinline__ void request_4_bytes_to_lds(const int32_t *src, const int32_t *dst /* uniform over the wave */) {
+    const uint32_t lds_byte_address = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)dst);
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "v"(src), "s"(lds_byte_address)
+                 : "memory");
+}
 __device__ __forceinline__ void staged_codes_arrived(bool eight_younger_requests) {
     if (eight_younger_requests) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -453,7 +471,7 @@ __device__ __forceinline__ void fused_staged_codes(const uint32_t *s_stage, bool
 template <int W, int GS, int NW>
 __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr, int b, int h, const ha_sel::Code<W> &q, int round, int n_groups,
                                            uint32_t *s_cnt /* [NW] */, int *s_ready, int32_t *s_list, const uint32_t *s_stage,
-                                           bool eight_younger_requests) {
+                                           bool eight_younger_requests, const int32_t *slot_row) {
     using namespace ha_sel;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // the wave's number in scalar registers
     constexpr int GC = GS * HA_WAVE * 4;  // codes per group
@@ -465,6 +483,10 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
     const int beg = max(fr.lo, cb), end = min(fr.hi, cb + f.chunk);
     const bool whole = f.vec && beg == cb && end == cb + f.chunk;
 
+    // Slot map: the entries the previous round placed are being translated in place (below); those requests are older than
+    // the staged codes' and every wave waits for its own here, so behind this round's first barrier the previous round's
+    // entries hold slots for everybody.
+    if (slot_row) staged_codes_arrived(eight_younger_requests);
     uint32_t lt = 0, le = 0;  // bit 4 s + e: code (slab s, element e) of this lane has d < T / d <= T
     if (active && beg < end && fr.nheavy > 0) {
         Code<W> k[GS][4];
@@ -565,6 +587,19 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
             }
         }
     }
+    // Slot map: the tokens this wave has just placed - one contiguous stretch of the list - are replaced by their slots, in
+    // place and without a register: lane l asks for the map entry of the token at stretch position l, the answer lands on
+    // that list entry (memory -> LDS).  The wave's LDS operations complete in order, so the tokens read back here are the
+    // ones written above, and each request is issued after the read of the entry it overwrites.
+    if (slot_row && active && tot != 0) {
+        const int first = fr.hbase + a + min(t, r);
+        const int p0 = max(first, 0);
+        const int p1 = min(first - min(t, r) + (int)(tot & 0xFFFFu) + min(t + (int)(tot >> 16), r), fr.n);
+        for (int pb = p0; pb < p1; pb += HA_WAVE) {
+            const int p = pb + lane;
+            if (p < p1) request_4_bytes_to_lds(slot_row + s_list[p], s_list + pb);
+        }
+    }
     // the last group of the round knows where the placed prefix ends
     const int last = min(n_groups - 1 - round * NW, NW - 1);
     if (wave == last && lane == 0) *s_ready = fr.hbase + a + (int)(tot & 0xFFFFu) + min(t + (int)(tot >> 16), r);
@@ -587,9 +622,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                                                            float *__restrict__ part_ml, void *__restrict__ out,
                                                            const float *__restrict__ win_part, int win_init, int win_recent,
                                                            const int32_t *__restrict__ seq_lens, int max_S, const FusedSel fsel,
-                                                           const AttnMask amask, int rows_per_seq) {
+                                                           const AttnMask amask, int rows_per_seq, const SlotMap smap) {
     using EL = Elem<E>;
     static_assert(!MK || FW == 0, "the additive mask exists for list-fed launches only");
+    // staged_codes_arrived(true) waits with vmcnt(8): a gather step (and the loop's priming) must put at least eight
+    // vector-memory loads per wave behind the staged codes' requests - U key rows and U value rows of 8 elements, one
+    // 128-bit load per 16 bytes
+    static_assert(FW == 0 || 2 * U * (Elem<E>::bytes * 8 / 16) >= 8, "fewer than eight row loads per gather step: vmcnt(8) would not cover the staged codes");
     constexpr int NS = NT / 16;  // row streams
     __shared__ float s_m[NS], s_l[NS];
     // the streams' partial results at the end of the kernel; before that, in a fused launch, the waves' staging regions (and,
@@ -694,8 +733,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             hist_tile.request(fsel, row);
             if (tid < 32 * FW + 1) s_h[fsel.nchunk * (32 * FW + 1) + tid] = 0;  // the level totals (local_thresholds)
         }
-        fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr);
-        j_max = max(S - 1, 0);
+        fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr, smap.slots ? smap.slots + b * smap.stride_b : nullptr);
+        j_max = smap.slots ? smap.max_slot : max(S - 1, 0);
         r0 = 0;
         r1 = fr.nwin;  // until the thresholds are known the list is its windows
     } else {
@@ -730,6 +769,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const char *vb = (const char *)v + (b_kv * kv_sb + (h / G) * kv_sh) * EL::bytes;
     const int64_t row_bytes = kv_ss * EL::bytes;
     constexpr int STEP = NS * U;  // rows of the list consumed per step by the workgroup
+    // this sequence's token -> slot map (nullptr: rows lie at their token positions)
+    const int32_t *slot_row = smap.slots ? smap.slots + b_kv * smap.stride_b : nullptr;
 
     // the query slice as it lies in memory: the score is dot8(q, k) * scale, two elements per instruction for 16-bit rows
     const Raw8<E> qraw = EL::load8((const char *)q + (b * q_sb + h * q_sh) * EL::bytes, sub);
@@ -744,6 +785,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         else return ix[r < r1 ? r : r0];
     };
     int32_t j_next[U];   // indices of the step after the one in flight
+    // list-fed launch with a slot map: j_next holds slots; the tokens of the step behind that one are loaded a step earlier
+    // still, so that their map entries can be requested without waiting for them (t_after), and a mask by token position
+    // keeps the tokens of the step after the one in flight (tok_next)
+    [[maybe_unused]] int32_t t_after[U], tok_next[U];
     Raw8<E> kr[U], vr[U];
     int base = r0;
     // MK: the additive term of list position (step base, u), token j, in the log2 units of the scores.  The index is
@@ -765,6 +810,17 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
             for (int u = 0; u < U; ++u) mk[u] = mask_term(base, u, j0[u]);
         }
+        if constexpr (FW == 0) {
+            if (slot_row) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    t_after[u] = list_index(base + 2 * STEP, u);
+                    if constexpr (MK) tok_next[u] = j_next[u];
+                    j0[u] = slot_row[j0[u]];
+                    j_next[u] = slot_row[j_next[u]];
+                }
+            }
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) kr[u] = EL::load8s(kb + j0[u] * row_bytes, sub);
 #pragma unroll
@@ -779,11 +835,27 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int u = 0; u < U; ++u) kn[u] = EL::load8s(kb + j_next[u] * row_bytes, sub);
 #pragma unroll
         for (int u = 0; u < U; ++u) vn[u] = EL::load8s(vb + j_next[u] * row_bytes, sub);
+        [[maybe_unused]] int32_t tok_after[U];
+        bool translated = false;
+        if constexpr (FW == 0) {
+            if (slot_row) {  // uniform: tokens of step + 2 arrived a step ago -> their slots; tokens of step + 3 requested
+                translated = true;
 #pragma unroll
-        for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
+                for (int u = 0; u < U; ++u) {
+                    const int32_t t = t_after[u];
+                    j_after[u] = slot_row[t];
+                    if constexpr (MK) tok_after[u] = t;
+                    t_after[u] = list_index(base + 3 * STEP, u);
+                }
+            }
+        }
+        if (!translated) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
+        }
         if constexpr (MK) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) mk_next[u] = mask_term(base + STEP, u, j_next[u]);
+            for (int u = 0; u < U; ++u) mk_next[u] = mask_term(base + STEP, u, translated ? tok_next[u] : j_next[u]);
         }
 
         // ---- reduce the current step
@@ -817,7 +889,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             kr[u] = kn[u];
             vr[u] = vn[u];
             j_next[u] = j_after[u];
-            if constexpr (MK) mk[u] = mk_next[u];
+            if constexpr (MK) {
+                mk[u] = mk_next[u];
+                if (translated) tok_next[u] = tok_after[u];
+            }
         }
         base += STEP;
     };
@@ -874,8 +949,18 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
         if (rounds > 0 && !staged_early) fused_round_stage<FW, GS, NW>(fsel, fr, b, h, 0, n_groups, s_raw);
         bool covered = false;  // eight row requests have been issued behind the staged codes' requests
+        // Slot map: a round's entries are translated in place behind the round and hold slots for every wave once the next
+        // round's first barrier has passed, so the loop runs one round behind the scan: `usable` = the entries placed by the
+        // rounds before the last one (the windows were translated when they were written).
+        int usable = fr.nwin, placed = fr.nwin;
         for (int k = 0; k < rounds; ++k) {
-            int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, qcode, k, n_groups, s_cnt, &s_cstar, s_list, s_raw, covered);
+            int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, qcode, k, n_groups, s_cnt, &s_cstar, s_list, s_raw, covered, slot_row);
+            if (slot_row) {
+                usable = placed;
+                placed = min(ready, r1);
+                ready = usable;
+                if (k == rounds - 1) covered = false;  // the youngest requests are now this round's translations
+            }
             if (k == rounds - 1) break;
             ready = min(ready, r1);
             fused_round_stage<FW, GS, NW>(fsel, fr, b, h, k + 1, n_groups, s_raw);
@@ -893,6 +978,22 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 step();
                 covered = true;
             }
+        }
+        if (slot_row && rounds > 0) {
+            // the last round's entries: run what the earlier rounds allow, then every wave waits for its own translations
+            // and the waves meet
+            if (!primed && usable >= min(2 * STEP, r1)) {
+                prime();
+                primed = true;
+                covered = true;
+            }
+            while (primed && base + 4 * STEP <= usable) {
+                step();
+                step();
+                covered = true;
+            }
+            staged_codes_arrived(covered);
+            __syncthreads();
         }
         if (!primed) prime();
         while (base < r1) step();
@@ -1155,7 +1256,8 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
                               int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int H, int Hkv,
                               const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, void *out, void *workspace,
                               size_t workspace_bytes, const float *win_part, int win_init, int win_recent, const int32_t *seq_lens,
-                              int max_seq_len, const AttnMask amask, void *stream, int rows_per_seq = 1) {
+                              int max_seq_len, const AttnMask amask, void *stream, int rows_per_seq = 1,
+                              const SlotMap smap = SlotMap{}) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(rows_per_seq >= 1 && B % rows_per_seq == 0, HA_ERR_BAD_SHAPE, "rows_per_sequence=%d must divide the %d batch entries",
@@ -1181,7 +1283,7 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
         hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0, MK_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,   \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
                            plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len,        \
-                           FusedSel{}, amask, rows_per_seq);                                                                      \
+                           FusedSel{}, amask, rows_per_seq, smap);                                                                \
         HA_CHECK_LAUNCH("sparse_attend_kernel");                                                                                  \
         if (plan.nsplit_max > 1) {                                                                                                \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, counts, 0, idx_cap, H, \
@@ -1285,12 +1387,12 @@ size_t ha_sparse_decode_fused_workspace_bytes(int B, int H, int Hc, int max_seq_
     return part_bytes((int64_t)B * H, plan.nchunk);
 }
 
-int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
                            int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes, int64_t kc_stride_b,
                            int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W, int max_seq_len,
                            const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
                            const void *select_workspace, size_t select_workspace_bytes, int thresholds_ready, int32_t *out_counts,
-                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream, const SlotMap smap) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(kcodes && qcodes && select_workspace, HA_ERR_NULL_POINTER, "kcodes/qcodes/select_workspace is NULL");
@@ -1345,7 +1447,7 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     do {                                                                                                                          \
         hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,      \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
-                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1);                       \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1, smap);                 \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \
@@ -1364,6 +1466,61 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
     }
 #undef HA_FUSED_LAUNCH
     return HA_OK;
+}
+
+int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes, int64_t kc_stride_b,
+                           int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W, int max_seq_len,
+                           const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                           const void *select_workspace, size_t select_workspace_bytes, int thresholds_ready, int32_t *out_counts,
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    return sparse_decode_fused_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, kcodes, kc_stride_b,
+                                    kc_stride_h, qcodes, B, H, Hkv, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget, heavy_budget,
+                                    select_workspace, select_workspace_bytes, thresholds_ready, out_counts, sm_scale, out, workspace,
+                                    workspace_bytes, stream, SlotMap{});
+}
+
+static int validate_slot_map(const int32_t *slot_of_token, int64_t slot_stride_b, int64_t n_slots) {
+    HA_REQUIRE(slot_of_token, HA_ERR_NULL_POINTER, "slot_of_token is NULL");
+    HA_REQUIRE(slot_stride_b >= 0, HA_ERR_BAD_SHAPE, "slot_stride_b must not be negative");
+    HA_REQUIRE(n_slots > 0 && n_slots <= 2147483647LL, HA_ERR_BAD_SHAPE, "n_slots=%lld, must be in 1..2^31-1", (long long)n_slots);
+    HA_REQUIRE(ha_aligned(slot_of_token, 4), HA_ERR_MISALIGNED, "slot_of_token misaligned");
+    return HA_OK;
+}
+
+int ha_sparse_decode_paged(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int B, int rows_per_sequence, int H, int Hkv,
+                           const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale, const float *mask,
+                           int64_t mask_stride_b, int mask_len, int mask_by_slot, const int32_t *slot_of_token, int64_t slot_stride_b,
+                           int64_t n_slots, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    int st = validate_slot_map(slot_of_token, slot_stride_b, n_slots);
+    if (st) return st;
+    if (mask) {
+        HA_REQUIRE(mask_len > 0 && mask_stride_b >= 0, HA_ERR_BAD_SHAPE, "mask_len must be positive and mask_stride_b non-negative");
+        HA_REQUIRE(mask_by_slot == 0 || mask_by_slot == 1, HA_ERR_BAD_SHAPE, "mask_by_slot must be 0 or 1");
+        HA_REQUIRE(!mask_by_slot || mask_len >= idx_cap, HA_ERR_BAD_SHAPE, "a mask by list slot needs idx_cap=%lld values per row, got %d",
+                   (long long)idx_cap, mask_len);
+        HA_REQUIRE(ha_aligned(mask, 4), HA_ERR_MISALIGNED, "mask misaligned");
+    }
+    return sparse_decode_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, idx, idx_cap,
+                              counts, sm_scale, out, workspace, workspace_bytes, nullptr, 0, 0, nullptr, 0,
+                              mask ? AttnMask{mask, mask_stride_b, mask_len, mask_by_slot} : AttnMask{}, stream, rows_per_sequence,
+                              SlotMap{slot_of_token, slot_stride_b, (int)(n_slots - 1)});
+}
+
+int ha_sparse_decode_fused_paged(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                                 int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes,
+                                 int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W,
+                                 int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
+                                 const void *select_workspace, size_t select_workspace_bytes, int thresholds_ready,
+                                 int32_t *out_counts, const int32_t *slot_of_token, int64_t slot_stride_b, int64_t n_slots,
+                                 float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    int st = validate_slot_map(slot_of_token, slot_stride_b, n_slots);
+    if (st) return st;
+    return sparse_decode_fused_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, kcodes, kc_stride_b,
+                                    kc_stride_h, qcodes, B, H, Hkv, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget, heavy_budget,
+                                    select_workspace, select_workspace_bytes, thresholds_ready, out_counts, sm_scale, out, workspace,
+                                    workspace_bytes, stream, SlotMap{slot_of_token, slot_stride_b, (int)(n_slots - 1)});
 }
 
 size_t ha_window_partial_bytes(int B, int H) {

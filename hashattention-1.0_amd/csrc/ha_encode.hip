@@ -297,7 +297,8 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
 }
 
 int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const void *weights, int n_layers, int head_dim,
-                    int int_dim, int final_dim, const uint32_t *codes, int64_t c_sb, int64_t c_sh, int pos0) {
+                    int int_dim, int final_dim, const uint32_t *codes, int64_t c_sb, int64_t c_sh, int pos0,
+                    const int32_t *pos_dev) {
     HA_REQUIRE(x && weights && codes, HA_ERR_NULL_POINTER, "x/weights/codes is NULL");
     HA_REQUIRE(B > 0 && x_heads > 0 && n_heads > 0 && T > 0, HA_ERR_BAD_SHAPE, "B, x_heads, n_heads, T must be positive");
     HA_REQUIRE(n_heads <= 65535, HA_ERR_BAD_SHAPE, "n_heads is limited to 65535");
@@ -308,6 +309,13 @@ int validate_encode(const void *x, int B, int x_heads, int n_heads, int T, const
     HA_REQUIRE(final_dim == 32 || final_dim == 64, HA_ERR_BAD_SHAPE, "final_dim=%d, must be 32 or 64", final_dim);
     HA_REQUIRE(pos0 >= 0, HA_ERR_BAD_SHAPE, "pos0 must be non-negative");
     HA_REQUIRE(c_sh >= 0 && c_sb >= 0, HA_ERR_BAD_SHAPE, "negative code stride");
+    {
+        // positions given by the host are checked against the tokens a (sequence, head) row of the code buffer spans (from
+        // its strides, as launch_encode derives pos_cap); only positions read from device memory are left to the kernel
+        const int64_t span = n_heads > 1 ? c_sh : (B > 1 ? c_sb : 0), cap = span > 0 ? span / (final_dim / 32) : 0;
+        HA_REQUIRE(pos_dev || cap == 0 || (int64_t)pos0 + T <= cap, HA_ERR_BAD_SHAPE,
+                   "positions %d..%lld lie beyond the %lld tokens a code row spans", pos0, (long long)pos0 + T - 1, (long long)cap);
+    }
     HA_REQUIRE(ha_aligned(codes, 4) && ha_aligned(weights, 16), HA_ERR_MISALIGNED, "codes must be 4-byte, weights 16-byte aligned");
     return HA_OK;
 }
@@ -371,7 +379,7 @@ int ha_encode_pack(const void *x, int x_dtype, int64_t x_stride_b, int64_t x_str
                    uint32_t *codes, int64_t c_stride_b, int64_t c_stride_h, int pos0, const int32_t *pos_dev, float *logits,
                    void *stream) {
     int st = validate_encode(x, B, x_heads, n_heads, T, weights, n_layers, head_dim, int_dim, final_dim, codes, c_stride_b,
-                             c_stride_h, pos0);
+                             c_stride_h, pos0, pos_dev);
     if (st) return st;
     HA_REQUIRE(x_dtype == HA_F32 || x_dtype == HA_BF16 || x_dtype == HA_F16, HA_ERR_BAD_DTYPE, "x_dtype %d", x_dtype);
     HA_REQUIRE(arith == HA_ARITH_F32 || arith == HA_ARITH_BF16, HA_ERR_BAD_DTYPE, "arith %d", arith);
@@ -392,7 +400,7 @@ int ha_encode_step(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, in
                    const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim, int arith, uint32_t *kcodes,
                    int64_t kc_stride_b, int64_t kc_stride_h, int pos0, const int32_t *pos_dev, uint32_t *qcodes, void *stream) {
     int st = validate_encode(k_new, B, Hkv, Hc, T_new, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b,
-                             kc_stride_h, pos0);
+                             kc_stride_h, pos0, pos_dev);
     if (st) return st;
     HA_REQUIRE(q && weights_q && qcodes, HA_ERR_NULL_POINTER, "q/weights_q/qcodes is NULL");
     HA_REQUIRE(H > 0 && H + Hc <= 65535, HA_ERR_BAD_SHAPE, "H must be positive and H + Hc <= 65535");
@@ -417,7 +425,7 @@ int ha_encode_step_cached(const void *k_cache, int64_t k_stride_b, int64_t k_str
                           int int_dim, int final_dim, int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h,
                           uint32_t *qcodes, void *stream) {
     int st = validate_encode(k_cache, B, Hkv, Hc, 1, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b,
-                             kc_stride_h, 0);
+                             kc_stride_h, 0, seq_lens);
     if (st) return st;
     HA_REQUIRE(q && weights_q && qcodes && seq_lens, HA_ERR_NULL_POINTER, "q/weights_q/qcodes/seq_lens is NULL");
     HA_REQUIRE(H > 0 && H + Hc <= 65535, HA_ERR_BAD_SHAPE, "H must be positive and H + Hc <= 65535");
@@ -445,7 +453,7 @@ int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int 
     HA_REQUIRE(qkv && inv_freq && q_out && k_cache && v_cache, HA_ERR_NULL_POINTER, "qkv/inv_freq/q_out/k_cache/v_cache is NULL");
     HA_REQUIRE(H > 0 && Hkv > 0 && Hc > 0, HA_ERR_BAD_SHAPE, "H, Hkv, Hc must be positive");
     int st = validate_encode(qkv, B, Hkv, Hc, 1, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b, kc_stride_h,
-                             pos_dev ? 0 : pos);
+                             pos_dev ? 0 : pos, pos_dev);
     if (st) return st;
     HA_REQUIRE(weights_q && qcodes, HA_ERR_NULL_POINTER, "weights_q/qcodes is NULL");
     HA_REQUIRE(head_dim == HA_HEAD_DIM, HA_ERR_BAD_SHAPE, "the rotary front end needs 128-wide heads");

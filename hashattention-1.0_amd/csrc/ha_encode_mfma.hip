@@ -257,6 +257,13 @@ extern "C" int ha_encode_pack_prefill(const void *x, int64_t x_stride_b, int64_t
     HA_REQUIRE(ha_aligned(x, 16) && x_stride_b % 8 == 0 && x_stride_h % 8 == 0 && x_stride_t % 8 == 0 && x_stride_t >= kDim,
                HA_ERR_MISALIGNED, "x rows must be 16-byte aligned bf16 rows of 128");
     HA_REQUIRE(ha_aligned(weights_bf16, 8) && ha_aligned(codes, 4), HA_ERR_MISALIGNED, "weights/codes misaligned");
+    {
+        // tokens a (sequence, head) row of the code buffer spans, from its strides (a row nobody follows: unbounded)
+        const int W = final_dim / 32;
+        const int64_t c_cap = c_stride_h > 0 ? c_stride_h / W : (c_stride_b > 0 ? c_stride_b / W : INT64_MAX);
+        HA_REQUIRE(pos_dev || (int64_t)pos0 + T <= c_cap, HA_ERR_BAD_SHAPE, "pos0 + T = %lld exceeds the %lld tokens of a code row",
+                   (long long)pos0 + T, (long long)c_cap);
+    }
     int st = ha_require_device();
     if (st) return st;
 

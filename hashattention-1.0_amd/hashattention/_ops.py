@@ -113,6 +113,12 @@ def load_library() -> C.CDLL:
     lib.ha_sparse_decode_masked.restype = i32
     lib.ha_sparse_decode_masked.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, i64, vp, f32,
                                             vp, i64, i32, i32, vp, vp, sz, vp]
+    lib.ha_sparse_decode_paged.restype = i32
+    lib.ha_sparse_decode_paged.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, f32,
+                                           vp, i64, i32, i32, vp, i64, i64, vp, vp, sz, vp]
+    lib.ha_sparse_decode_fused_paged.restype = i32
+    lib.ha_sparse_decode_fused_paged.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32,
+                                                 vp, i32, i32, f64, vp, sz, i32, vp, vp, i64, i64, f32, vp, vp, sz, vp]
     lib.ha_window_partial_bytes.restype = sz
     lib.ha_window_partial_bytes.argtypes = [i32, i32]
     lib.ha_window_partial.restype = i32
@@ -195,6 +201,7 @@ def encode_pack(x: torch.Tensor, weights: torch.Tensor, n_layers: int, int_dim: 
     B, xh, T, d = x.shape
     n_heads = weights.shape[0]
     assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3]
+    assert codes.shape[0] >= B and codes.shape[1] == n_heads, "codes must be [>= B, n_heads, ., W] for x [B, ., T, d]"
     assert codes.dtype == torch.int32 and weights.dtype == torch.float32 and weights.is_contiguous()
     assert weights.shape[1] == lib.ha_usa_packed_floats(n_layers, d, int_dim, final_dim)
     if pos_dev is None:
@@ -252,6 +259,7 @@ def encode_pack_prefill(x: torch.Tensor, weights_bf16: torch.Tensor, n_layers: i
     n_heads = weights_bf16.shape[0]
     assert x.dtype == torch.bfloat16 and weights_bf16.dtype == torch.bfloat16 and weights_bf16.is_contiguous()
     assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3] and codes.dtype == torch.int32
+    assert codes.shape[0] >= B and codes.shape[1] == n_heads, "codes must be [>= B, n_heads, ., W] for x [B, ., T, d]"
     if pos_dev is None:
         assert pos0 + T <= codes.shape[2]
     _check(lib.ha_encode_pack_prefill(_ptr(x), x.stride(0), x.stride(1), x.stride(2), B, xh, n_heads, T,
@@ -270,6 +278,7 @@ def encode_pack_prefill_f32(x: torch.Tensor, weights: torch.Tensor, n_layers: in
     assert weights.dtype == torch.float32 and weights.is_contiguous()
     assert weights.shape[1] == lib.ha_usa_packed_floats(n_layers, d, int_dim, final_dim)
     assert x.stride(3) == 1 and codes.stride(3) == 1 and codes.stride(2) == codes.shape[3] and codes.dtype == torch.int32
+    assert codes.shape[0] >= B and codes.shape[1] == n_heads, "codes must be [>= B, n_heads, ., W] for x [B, ., T, d]"
     if pos_dev is None:
         assert pos0 + T <= codes.shape[2]
     _check(lib.ha_encode_pack_prefill_f32(_ptr(x), _DTYPE[x.dtype], x.stride(0), x.stride(1), x.stride(2), B, xh, n_heads, T,
@@ -407,17 +416,34 @@ def sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len) -> int:
     return load_library().ha_sparse_decode_fused_workspace_bytes(B, H, Hc, max_seq_len)
 
 
+def _slot_args(slots: torch.Tensor, n_seq: int, n_slots: int):
+    """slots int32 [n_seq, >= S] (or [1, .] expanded: row stride 0): the K/V row of token j of sequence b is row slots[b, j]."""
+    assert slots.dtype == torch.int32 and slots.dim() == 2 and slots.shape[0] == n_seq and slots.stride(1) == 1
+    return (_ptr(slots), slots.stride(0), int(n_slots))
+
+
 def sparse_decode_fused(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kcodes: torch.Tensor, qcodes: torch.Tensor,
                         max_seq_len: int, seq_lens: Optional[torch.Tensor], init_budget: int, recent_budget: int,
                         heavy_budget: float, ws_select: torch.Tensor, sm_scale: float, out: torch.Tensor, ws: torch.Tensor,
-                        thresholds_ready: bool = True, out_counts: Optional[torch.Tensor] = None) -> None:
+                        thresholds_ready: bool = True, out_counts: Optional[torch.Tensor] = None,
+                        slots: Optional[torch.Tensor] = None) -> None:
     """Attention over the selection prepared by select_prepare (same codes, budgets and seq_lens); out [B,H,128] in place.
-    thresholds_ready=False: the workspace was filled by select_histogram only; counts (optional, [B,H] int32) are written here."""
-    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws, out_counts)
+    thresholds_ready=False: the workspace was filled by select_histogram only; counts (optional, [B,H] int32) are written here.
+    slots: optional token -> slot table int32 [B, >= max_seq_len] of a paged cache; k, v are then [B or 1 (expanded), Hkv,
+    n_slots, 128] views of the row pool (`ha_sparse_decode_fused_paged`)."""
+    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws, out_counts, slots)
     lib = load_library()
     B, H, _ = q.shape
     Hc, W = kcodes.shape[1], kcodes.shape[3]
     assert out.is_contiguous() and out.dtype == q.dtype and kcodes.stride(3) == 1 and kcodes.stride(2) == W and qcodes.is_contiguous()
+    if slots is not None:
+        assert slots.shape[1] >= max_seq_len
+        _check(lib.ha_sparse_decode_fused_paged(*_kv_args(q, k, v), _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H,
+                                                k.shape[1], Hc, W, max_seq_len, _ptr(seq_lens), init_budget, recent_budget,
+                                                float(heavy_budget), _ptr(ws_select), ws_select.numel(), 1 if thresholds_ready else 0,
+                                                _ptr(out_counts), *_slot_args(slots, B, k.shape[2]), float(sm_scale), _ptr(out), _ptr(ws),
+                                                ws.numel(), _stream(q)), "ha_sparse_decode_fused_paged")
+        return
     _check(lib.ha_sparse_decode_fused(*_kv_args(q, k, v), _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H,
                                       k.shape[1], Hc, W, max_seq_len, _ptr(seq_lens), init_budget, recent_budget, float(heavy_budget),
                                       _ptr(ws_select), ws_select.numel(), 1 if thresholds_ready else 0, _ptr(out_counts),
@@ -438,14 +464,27 @@ def _kv_args(q, k, v):
 
 def sparse_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor,
                   sm_scale: float, out: torch.Tensor, ws: torch.Tensor, mask: Optional[torch.Tensor] = None,
-                  mask_by_slot: bool = False) -> None:
+                  mask_by_slot: bool = False, slots: Optional[torch.Tensor] = None, rows_per_sequence: int = 1) -> None:
     """q [B,H,128]; k,v [B,Hkv,S_cap,128]; idx [B,H,idx_cap] int32; counts [B,H] int32; out [B,H,128] (in place).
     mask: optional fp32 [B, n] (or [1, n] expanded: row stride 0) added to the scaled scores, indexed by token position,
-    or by the place in the list when mask_by_slot."""
-    _require_cuda(q, k, v, idx, counts, out, ws, mask)
+    or by the place in the list when mask_by_slot.
+    slots: optional token -> slot table int32 [n_seq, >= S] of a paged cache (`ha_sparse_decode_paged`): k, v are then
+    [n_seq or 1 (expanded), Hkv, n_slots, 128] views of the row pool; n_seq = B // rows_per_sequence."""
+    _require_cuda(q, k, v, idx, counts, out, ws, mask, slots)
     lib = load_library()
     B, H, _ = q.shape
     assert out.is_contiguous() and out.dtype == q.dtype and idx.is_contiguous() and counts.is_contiguous()
+    if slots is not None:
+        assert B % rows_per_sequence == 0
+        if mask is not None:
+            assert mask.dtype == torch.float32 and mask.dim() == 2 and mask.shape[0] == B and mask.stride(1) == 1
+        _check(lib.ha_sparse_decode_paged(*_kv_args(q, k, v), B, rows_per_sequence, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),
+                                          float(sm_scale), _ptr(mask), mask.stride(0) if mask is not None else 0,
+                                          mask.shape[1] if mask is not None else 0, 1 if mask_by_slot else 0,
+                                          *_slot_args(slots, B // rows_per_sequence, k.shape[2]), _ptr(out), _ptr(ws), ws.numel(),
+                                          _stream(q)), "ha_sparse_decode_paged")
+        return
+    assert rows_per_sequence == 1, "chunks of rows without a slot table go through sparse_decode_rows"
     if mask is not None:
         assert mask.dtype == torch.float32 and mask.dim() == 2 and mask.shape[0] == B and mask.stride(1) == 1
         _check(lib.ha_sparse_decode_masked(*_kv_args(q, k, v), B, H, k.shape[1], _ptr(idx), idx.shape[2], _ptr(counts),

@@ -213,6 +213,20 @@ class USA(nn.Module):
                                   arith=self.arith, want_logits=True)
         return torch.sign(logits), codes
 
+    def invalidate_packed(self) -> None:
+        """Forget the packed copies of the weights.  They are rebuilt whenever a parameter's version counter or storage
+        changes; an update that bypasses the counter (`p.data.add_(...)`, an EMA or optimizer writing through `.data`) must
+        be followed by this call.  Loading a state dict, `train()` / `eval()` and `train_step` call it themselves."""
+        self.__dict__.pop("_packed", None)
+
+    def train(self, mode: bool = True):
+        self.invalidate_packed()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_packed()
+        return super()._load_from_state_dict(*args, **kwargs)
+
     def _packed_weights(self, side: str, device) -> torch.Tensor:
         """The side's weights in the kernels' blob form, repacked only when a parameter changed (tensor versions) or moved."""
         params = [t for head in self.layers(side) for wb in head for t in wb]
@@ -253,7 +267,10 @@ class USA(nn.Module):
         _, qcodes = self._embed(Qh.contiguous(), "q", True, prepared=True)
         D = self.lth_final_dim
         # the t query tokens of a head are t "query heads" of its code head: one scoring launch for all of them
-        ham = _ops.hamming_score(kcodes, qcodes.reshape(b, a * t, qcodes.shape[-1]), s).view(b, a, t, s)
+        # (the launch takes up to 65535 of them: longer chunks go in slices of tokens)
+        t_slice = max(1, 65535 // a)
+        ham = torch.cat([_ops.hamming_score(kcodes, qcodes[:, :, t0:t0 + t_slice].reshape(b, -1, qcodes.shape[-1]), s)
+                         .view(b, a, -1, s) for t0 in range(0, t, t_slice)], dim=2)
         span = (D - 2 * ham.to(torch.int32)).to(K.dtype)
         span = torch.where(causal, span, torch.full([], torch.finfo(span.dtype).min, dtype=span.dtype, device=K.device))
         return span, ksign.to(K.dtype)
@@ -543,6 +560,7 @@ class HeavyHitterMixin:
         self.last_train_loss = loss.detach()
         if self._hash_layer is not None:       # the packed weights and the cached codes belong to the old parameters
             self._hash_layer = None
+        self.usa_module.invalidate_packed()
         if self.layer_idx == 5:
             print(self.layer_idx, K.shape[2], "Train Loss:", loss.item(), flush=True)
 

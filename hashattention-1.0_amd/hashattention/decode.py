@@ -92,6 +92,7 @@ class HashDecodeLayer:
         self.win = torch.empty(B, self.H, 130, dtype=torch.float32, device=dev)
         self.side_stream = torch.cuda.Stream(device=dev)
         self.n_cached = 0
+        self._chunk = None          # the chunk buffers are shaped by the batch
 
     def reset(self) -> None:
         """Forget the cached codes (a new prompt starts); buffers are kept."""
@@ -216,7 +217,7 @@ class HashDecodeLayer:
     def _chunk_buffers(self, n_rows: int, cap: int, s_max: int, dtype: torch.dtype):
         """Lists, counts, query codes, output rows and workspaces of `chunk_step`, kept between calls and grown when a
         chunk needs more."""
-        key = (n_rows, dtype)
+        key = (self.B, n_rows, dtype)      # the query codes [B, H, T, W] and the row lengths depend on B and T separately
         cb = getattr(self, "_chunk", None)
         if cb is None or cb["key"] != key or cb["cap"] < cap or cb["s_max"] < s_max:
             dev = self.device

@@ -234,7 +234,14 @@ int ha_select_static(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
  * (efficiency/kernels/flash_fwd_sparse.py:396-554, 775-815; sparse.py:12-187) and the masked dense
  * softmax of hashattention_llama.py:585-615.
  *   q   [B, H, 128] kv_dtype, strides q_stride_{b,h}
- *   k,v [B, Hkv, ., 128] kv_dtype, strides kv_stride_{b,h,s}; rows 16-byte aligned
+ *   k,v [B, Hkv, ., 128] kv_dtype, strides kv_stride_{b,h,s}; rows 16-byte aligned.  Any layout the three strides
+ *       describe is read in place: [B, Hkv, S, 128] (the Hugging Face cache) as well as the prototype's token-major
+ *       [B * S, H, 128] (torchatt.py:148-151, sparse.py:224-226: kv_stride_b = S * H * 128, kv_stride_h = 128,
+ *       kv_stride_s = H * 128)
+ *   idx The ORDER of a list is free: ascending (what ha_select writes, best for DRAM locality), torch.topk's score order
+ *       (torchatt.py:66-67) or a random permutation (sparse.py:231-233) give the same output up to the order of the fp32
+ *       additions.  An index that occurs twice counts twice, as in the reference's kernels.  Entries must lie inside the
+ *       cache: they are not range-checked.
  *   out [B, H, 128] kv_dtype contiguous
  *   workspace  ha_sparse_decode_workspace_bytes(...) bytes, 256-byte aligned; calls that share a
  *              workspace must not overlap
@@ -327,6 +334,41 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
                            const void *select_workspace, size_t select_workspace_bytes,
                            int thresholds_ready, int32_t *out_counts,
                            float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The same two attention launches over a cache addressed through a token -> slot table: the row of token j of sequence b
+ * is row slot_of_token[b * slot_stride_b + j] of k and v, i.e. it lies at k + b * kv_stride_b + (h / G) * kv_stride_h +
+ * slot * kv_stride_s.  This is the `Req_to_tokens [B, S]` table of the reference's sparse flash-decode
+ * (efficiency/kernels/flash_fwd_sparse.py:396-470; built at efficiency/kernels/torchatt.py:165), whose K and V are one pool
+ * [n_slots, Hkv, 128] shared by all sequences: pass kv_stride_b = 0, kv_stride_h = 128, kv_stride_s = Hkv * 128 for that
+ * layout.  Index lists, counts, masks by token position, seq_lens, codes and budgets keep speaking of token POSITIONS; only
+ * the K/V row addresses go through the table.  slot_of_token is int32 (the reference: int64), n_slots the number of rows
+ * k and v hold per (sequence, KV head) view - slots must lie in [0, n_slots); the fused launch clamps list entries to it.
+ *
+ * ha_sparse_decode_paged covers ha_sparse_decode, _masked and _rows: mask may be NULL, rows_per_sequence is 1 for one query
+ * per sequence (with more, kv_stride_b and slot_stride_b are strides between SEQUENCES, as for ha_sparse_decode_rows).
+ * ha_sparse_decode_fused_paged is ha_sparse_decode_fused with the table: the fused launch translates a token when it is
+ * placed in the row's LDS list (memory -> LDS requests that overwrite the entry, no register involved) and gathers one
+ * scan round behind the selection.  Outputs equal those of the unpaged entry points on the cache the table describes.
+ */
+int ha_sparse_decode_paged(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                           const void *k, const void *v, int kv_dtype,
+                           int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                           int B, int rows_per_sequence, int H, int Hkv,
+                           const int32_t *idx, int64_t idx_cap, const int32_t *counts, float sm_scale,
+                           const float *mask, int64_t mask_stride_b, int mask_len, int mask_by_slot,
+                           const int32_t *slot_of_token, int64_t slot_stride_b, int64_t n_slots,
+                           void *out, void *workspace, size_t workspace_bytes, void *stream);
+int ha_sparse_decode_fused_paged(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                                 const void *k, const void *v, int kv_dtype,
+                                 int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                                 const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                                 int B, int H, int Hkv, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                                 int init_budget, int recent_budget, double heavy_budget,
+                                 const void *select_workspace, size_t select_workspace_bytes,
+                                 int thresholds_ready, int32_t *out_counts,
+                                 const int32_t *slot_of_token, int64_t slot_stride_b, int64_t n_slots,
+                                 float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Dense flash-decode over all seq_len[b] keys (the baseline the sparse path is compared with).

@@ -307,6 +307,16 @@ def sparse_attend(q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, idx: Sequen
     return p @ v
 
 
+def rows_through_slot_table(pool: torch.Tensor, req_to_tokens: torch.Tensor) -> torch.Tensor:
+    """The cache a token -> slot table describes: pool [n_slots, Hkv, d] (K or V as the sparse flash-decode holds it), table
+    [B, S] -> [B, Hkv, S, d] with out[b, h, j] = pool[table[b, j], h].
+
+    reference: `k_loc = Req_to_tokens[cur_batch, topk_token_indices]; off_k = k_loc * stride_kbs + cur_kv_head * stride_kh`,
+    efficiency/kernels/flash_fwd_sparse.py:466-474 (the table built at efficiency/kernels/torchatt.py:165).
+    """
+    return pool[req_to_tokens.long()].permute(0, 2, 1, 3)
+
+
 def merge_splits(part_o: torch.Tensor, part_lse: torch.Tensor) -> torch.Tensor:
     """Merge per-split normalised outputs [n, d] with their log-sum-exp [n] into one output [d].
 

@@ -122,6 +122,16 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert masked(mask=odd) == HA_ERR_ALIGN
     assert masked(Hkv=3) == HA_ERR_SHAPE and masked(wsb=8) == HA_ERR_WS      # the checks of ha_sparse_decode apply
     assert masked() == HA_ERR_NODEV and masked(slot=1) == HA_ERR_NODEV
+
+    def paged(**kw):        # the list-fed attention through a token -> slot table
+        a = dict(tab=p, tsb=1000, n=5000, mask=null, rps=1, B=2, Hkv=2)
+        a.update(kw)
+        return lib.ha_sparse_decode_paged(p, 512, 128, p, p, _ops.HA_BF16, 0, 128, 256, a["B"], a["rps"], 4, a["Hkv"], p, 300, p,
+                                          C.c_float(0.088), a["mask"], 400, 400, 0, a["tab"], a["tsb"], a["n"], p, p, 1 << 16, null)
+
+    assert paged(tab=null) == HA_ERR_NULL and paged(tsb=-1) == HA_ERR_SHAPE and paged(n=0) == HA_ERR_SHAPE
+    assert paged(tab=odd) == HA_ERR_ALIGN and paged(rps=3) == HA_ERR_SHAPE and paged(Hkv=3) == HA_ERR_SHAPE
+    assert paged() == HA_ERR_NODEV and paged(mask=p) == HA_ERR_NODEV and paged(B=4, rps=2) == HA_ERR_NODEV
     assert lib.ha_dense_decode(p, 512, 128, p, p, _ops.HA_F32, 128000, 128000, 128, 1, 4, 2, 0, null, C.c_float(0.1), p, p, 1 << 16,
                                null) == HA_ERR_SHAPE           # max_seq_len must be positive
 
@@ -146,6 +156,12 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert enc_cached() == HA_ERR_NODEV
     assert enc(fd=48) == HA_ERR_SHAPE and enc(nl=4) == HA_ERR_SHAPE and enc(nh=3) == HA_ERR_SHAPE and enc(hd=300) == HA_ERR_SHAPE
     assert enc(dt=5) == HA_ERR_DTYPE and enc(ar=2) == HA_ERR_DTYPE
+    # positions given by the host must lie inside the row of the code buffer (16 tokens between heads here); positions
+    # read from device memory are the kernel's to skip
+    assert enc(pos0=7) == HA_ERR_SHAPE and b"code row" in lib.ha_last_error_string()
+    assert enc(pos0=6) == HA_ERR_NODEV and enc(pos0=7, pd=p) == HA_ERR_NODEV
+    assert lib.ha_encode_pack_prefill(p, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 128, 32, p, 64, 16, 7, null, null) == HA_ERR_SHAPE
+    assert lib.ha_encode_pack_prefill(p, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 128, 32, p, 64, 16, 6, null, null) == HA_ERR_NODEV
     assert lib.ha_encode_pack_prefill(p, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 64, 32, p, 64, 16, 0, null, null) == HA_ERR_SHAPE
     assert lib.ha_encode_pack_prefill(odd, 1280, 1280, 128, 1, 2, 4, 10, p, 3, 128, 128, 32, p, 64, 16, 0, null, null) == HA_ERR_ALIGN
     assert lib.ha_hamming_score(p, 1024, 1024, p, 1, 4, 2, 1, 1000, null, null, null) == HA_ERR_NULL
@@ -177,6 +193,16 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert fused(kc=null) == HA_ERR_NULL and fused(sws=null) == HA_ERR_NULL and fused(dt=9) == HA_ERR_DTYPE
     assert fused(Hc=3) == HA_ERR_SHAPE and fused(csh=999) == HA_ERR_SHAPE and fused(hb=C.c_double(0.9), S=60000, csb=60000, csh=60000) == HA_ERR_SHAPE
     assert fused(swsb=16) == HA_ERR_WS and fused(wsb=16) == HA_ERR_WS and fused(k=odd) == HA_ERR_ALIGN
+
+    def fused_paged(**kw):
+        a = dict(tab=p, tsb=1000, n=5000, Hc=2)
+        a.update(kw)
+        return lib.ha_sparse_decode_fused_paged(p, 512, 128, p, p, _ops.HA_BF16, 0, 128, 256, p, 1024, 1024, p, 1, 4, 2, a["Hc"], 1, 1000, null,
+                                                4, 4, C.c_double(0.25), p, 1 << 20, 1, null, a["tab"], a["tsb"], a["n"], C.c_float(0.088), p,
+                                                p, 1 << 20, null)
+
+    assert fused_paged(tab=null) == HA_ERR_NULL and fused_paged(n=1 << 40) == HA_ERR_SHAPE and fused_paged(tab=odd) == HA_ERR_ALIGN
+    assert fused_paged(Hc=3) == HA_ERR_SHAPE and fused_paged() == HA_ERR_NODEV
 
     # decoder plumbing
     def rope(**kw):

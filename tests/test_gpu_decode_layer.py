@@ -157,3 +157,30 @@ def test_chunk_of_tokens_in_one_selection_and_one_attention_launch(batch, T, mas
                     assert np.array_equal(got, (mask[b, h, i] & causal[i]).numpy()), (b, i, h)
         err = (out.cpu() - ref).abs().max().item()
         assert err < 2e-5, err
+
+
+def test_chunk_buffers_follow_the_batch_shape_at_constant_row_count():
+    # (B, T) = (2, 4) then (4, 2): the same number of rows, but the query codes [B, H, T, W] and the row lengths are shaped by
+    # B and T separately - buffers kept from the first shape must not serve the second
+    print("\n[case] chunk step (B, T) = (2, 4) then (4, 2)", flush=True)
+    S = 600
+    w4 = small_workload(batch=4, seq_lens=[S] * 4, dtype=torch.float32, seed=77)
+    p4 = make_problem(w4)
+    layer = _layer(w4, p4)
+    for (B, T) in ((2, 4), (4, 2), (2, 4)):
+        k, v = p4.k[:B].to(DEV), p4.v[:B].to(DEV)
+        layer.allocate(B, S)
+        layer.encode_keys(k)
+        layer.n_cached = S
+        q = torch.randn(B, w4.n_q_heads, T, w4.head_dim, generator=torch.Generator().manual_seed(B * 10 + T))
+        out = torch.empty(B, w4.n_q_heads, T, w4.head_dim, device=DEV)
+        heavy = layer.heavy_count(S)
+        layer.chunk_step(q.to(DEV), k, v, S, out, heavy + 0.5)
+        add = torch.zeros(B, 1, T, S)
+        rows = torch.arange(T).view(T, 1) + S - T
+        add.masked_fill_((torch.arange(S).view(1, S) > rows).view(1, 1, T, S), torch.finfo(torch.float32).min)
+        ref, _ = orc.reference_decode_attention(q, p4.k[:B], p4.v[:B], p4.usa.k, p4.usa.q, w4.init_budget, w4.recent_budget,
+                                                w4.heavy_budget, attention_mask=add)
+        assert layer._chunk["qc"].shape[:3] == (B, w4.n_q_heads, T)
+        err = (out.cpu() - ref).abs().max().item()
+        assert err < 2e-5, (B, T, err)

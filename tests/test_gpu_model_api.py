@@ -137,6 +137,35 @@ def test_usa_forward_and_mask_api():
     assert torch.equal(mask.cpu(), mask_ref)
 
 
+def test_usa_forward_with_more_query_rows_than_one_scoring_launch_takes():
+    # heads * query tokens beyond 65535 (the scoring launch's limit of query "heads"): USA.forward slices the tokens; also a
+    # parameter changed through .data (no version bump) followed by invalidate_packed() must reach the kernels
+    print("\n[case] USA.forward with 4 x 16500 query rows; invalidate_packed", flush=True)
+    torch.manual_seed(5)
+    cfg = _config(LlamaConfig)
+    usa = hl.load_usa(cfg, None)[0]
+    t, s = 16500, 16600
+    K = torch.randn(1, 4, s, 128, device=DEV)
+    Q = torch.randn(1, 4, t, 128, device=DEV)
+    span, _ = usa(K, Q, hard=True)
+    assert span.shape == (1, 4, t, s)
+    lo = 16384 - 3                                      # rows on both sides of the slice boundary (65535 // 4 = 16383)
+    small, _ = usa(K, Q[:, :, lo:lo + 6].contiguous(), hard=True)
+    rows = torch.arange(lo, lo + 6)
+    causal = torch.arange(s)[None, :] <= (rows[:, None] + s - t)
+    # the short call's causal edge sits at other columns: compare the columns both calls score
+    both = causal & (torch.arange(s)[None, :] <= (torch.arange(6)[:, None] + s - 6))
+    assert torch.equal(span[0, :, lo:lo + 6].cpu()[:, both], small[0].cpu()[:, both])
+    before = usa.k_embedding(K[:, :, :64].contiguous(), hard=True).clone()
+    with torch.no_grad():
+        for seq in usa.learning_to_hash_transformation_k:
+            seq[-1].weight.data.neg_()
+            seq[-1].bias.data.neg_()
+    usa.invalidate_packed()
+    after = usa.k_embedding(K[:, :, :64].contiguous(), hard=True)
+    assert torch.equal(after, -before)
+
+
 def test_recall_statistic_matches_the_oracle():
     # collect_stats=True: after a 1024-token prefill every layer holds the recall of its hash ranking (reference :319-398);
     # layer 0 is compared row by row with the oracle on the same queries and keys

@@ -283,6 +283,121 @@ def decoder_bench(args, torch):
     print(json.dumps(res))
 
 
+def hf_path_bench(args, torch):
+    """--config config3 --hf-path: the drop-in path itself.  A random-init `transformers` Llama of Llama-3.1-8B width with
+    `--layers` decoder layers goes through `load_usa(config, None)` + `convert_usa` (the reference's own call sequence,
+    README.md:37-55), its KV cache is filled directly with 131071 synthetic tokens per sequence (batch 4), and single-token
+    forward passes are timed - with `hashattention.cache.PreallocatedCache` (appends in place) and with the library's
+    `DynamicCache` (re-copies the layer's whole cache every step) - next to `LlamaShapedDecoder.from_hf` of the same model.
+    Per-layer figures are the slope between a model of `--layers` layers and one of half as many (embedding, final norm and
+    lm_head cancel)."""
+    from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
+    from hashattention import hashattention_llama as hl
+    from hashattention.cache import PreallocatedCache
+    from hashattention.decoder import LlamaShapedDecoder
+    from hashattention.synthetic import named_workload
+    w = named_workload("config3")
+    B, S = w.batch, w.max_seq_len
+    dev = "cuda:0"
+    steps, warm = max(8, min(args.steps, 64)), 3
+
+    def build(L):
+        cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=L, num_attention_heads=32, num_key_value_heads=8,
+                          head_dim=128, vocab_size=128256, max_position_embeddings=S + 4096, rope_theta=500000.0, rms_norm_eps=1e-5)
+        for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=w.init_budget,
+                         heavy_budget=w.heavy_budget, recent_budget=w.recent_budget, usa_retrieve_depth=0, usa_eval_mode="simple").items():
+            setattr(cfg, k, v)
+        torch.manual_seed(0)
+        with torch.device(dev):
+            model = LlamaForCausalLM(cfg).bfloat16()
+        usa = hl.load_usa(cfg, None)
+        return cfg, hl.convert_usa(model, cfg, usa, collect_stats=False, train_usa=False).eval(), usa
+
+    def fill(cache, L, n):
+        g = torch.Generator(device=dev).manual_seed(1)
+        for l in range(L):
+            k = torch.randn(B, 8, n, 128, generator=g, device=dev, dtype=torch.bfloat16)
+            v = torch.randn(B, 8, n, 128, generator=g, device=dev, dtype=torch.bfloat16)
+            cache.update(k, v, l)
+            del k, v
+
+    def time_tokens(model, cache, n_steps, n_warm):
+        ids = torch.randint(0, 128256, (B, 1), device=dev)
+        with torch.no_grad():
+            for _ in range(n_warm):                      # the first pass hashes the 131071 cached keys of every layer
+                model(ids, past_key_values=cache, use_cache=True)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            for _ in range(n_steps):
+                model(ids, past_key_values=cache, use_cache=True)
+            e1.record()
+            host_ms = (time.perf_counter() - t0) * 1e3 / n_steps     # time to issue a step from Python (no wait inside)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n_steps, host_ms
+
+    out = {}
+    L_full = max(2, args.layers if args.layers != 32 else 4)
+    for L in (L_full // 2, L_full):
+        cfg, model, usa = build(L)
+        cache = PreallocatedCache(capacity=S + 256, num_layers=L)
+        fill(cache, L, S - 1 - warm)
+        ms_pre, host_pre = time_tokens(model, cache, steps, warm)
+        # the attention module of one layer alone, at a fixed length: hidden states in, attention output out
+        layer = model.model.layers[0].self_attn
+        h = torch.randn(B, 1, 4096, device=dev, dtype=torch.bfloat16)
+        with torch.no_grad():
+            n_now = cache.get_seq_length()
+            pos = torch.full((B, 1), n_now, device=dev, dtype=torch.long)
+            pe = model.model.rotary_emb(h, pos)
+
+            def attn_only():
+                layer(hidden_states=h, position_embeddings=pe, attention_mask=None, past_key_values=cache)
+                cache.layers[0].crop(-1)
+            ms_attn = time_gpu(attn_only, steps, warm, torch)
+        del cache
+        hl.reset_usa(model)
+        dyn = DynamicCache()
+        fill(dyn, L, S - 1 - 2)
+        ms_dyn, _ = time_tokens(model, dyn, 4, 2)
+        del dyn
+        hl.reset_usa(model)
+        torch.cuda.empty_cache()
+        dec = LlamaShapedDecoder.from_hf(model, usa, batch=B, cache_len=S + 256)
+        dec.fill_cache_synthetic(S - 1)
+        tok = torch.randint(0, 128256, (B,), device=dev)
+        with torch.no_grad():
+            dec.generate(tok, 4)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            dec.generate(tok, steps)
+            e1.record()
+            torch.cuda.synchronize()
+        ms_dec = e0.elapsed_time(e1) / steps
+        out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre, patched_dynamic_cache_ms=ms_dyn,
+                      decoder_generate_ms=ms_dec, patched_attention_module_us=ms_attn * 1e3)
+        del dec, model, usa
+        torch.cuda.empty_cache()
+    lo, hi = out[L_full // 2], out[L_full]
+    dL = L_full - L_full // 2
+    per_layer = {k.replace("_ms", "_us_per_layer"): (hi[k] - lo[k]) / dL * 1e3 for k in hi if k.endswith("_ms")}
+    res = {
+        "metric": "decode_ms_per_token_patched_transformers_model", "value": hi["patched_preallocated_ms"], "unit": "ms/token-step",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": hi["patched_preallocated_ms"], "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config3 through the drop-in API: transformers Llama (hidden 4096, ffn 14336, 32/8 heads, vocab 128256), "
+                               f"{L_full} layers, load_usa(config, None) + convert_usa, B={B} context={S}, one key-side hash MLP per query "
+                               f"head (fp32 modules), init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g}"},
+        "layers": {str(k): v for k, v in out.items()},
+        "per_layer_slope": per_layer,
+        "how": "single-token forward passes of the patched model, eager launches from Python, HIP events around the timed passes; "
+               "per-layer = difference between the two layer counts; decoder = LlamaShapedDecoder.from_hf(...).generate (one HIP graph "
+               "replayed per token); patched_attention_module = self_attn.forward of one layer alone at a fixed length",
+    }
+    print(json.dumps(res))
+
+
 class InputSet:
     """One attention layer's worth of inputs and state: its own Q/K/V, hash weights, bit-cache, workspaces and output."""
 
@@ -446,6 +561,8 @@ def main():
     ap.add_argument("--overlap-windows", action="store_true", help="attend to sink|recent on a second stream (ha_window_partial)")
     ap.add_argument("--layers", type=int, default=32, help="decoder layers of the config3 whole-step workload")
     ap.add_argument("--layer-only", action="store_true", help="config3: time one attention layer-step instead of the whole decoder")
+    ap.add_argument("--hf-path", action="store_true", help="config3: time a transformers Llama patched with convert_usa (the drop-in path) "
+                    "next to LlamaShapedDecoder; --layers sets the layer count (default 4)")
     ap.add_argument("--traffic-probe", action="store_true", help="run the launches the HBM-traffic counters are read from, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -461,6 +578,9 @@ def main():
         print("bench.py needs a GPU: the HashAttention path has no CPU fallback", file=sys.stderr)
         sys.exit(2)
     _ops.load_library()
+    if args.config == "config3" and args.hf_path:
+        hf_path_bench(args, torch)
+        return
     if args.config == "config3" and not args.layer_only:
         decoder_bench(args, torch)
         return

@@ -46,7 +46,12 @@ struct EncSide {
 // QKV projection, rotate them (rotate-half RoPE at the sequence's position), write the rotated key and the value row
 // into the caches and the rotated query to q_out, and hash what they wrote.
 struct EncRope {
-    const float *inv_freq;  // [64]; nullptr: no front end, the sides read finished rows
+    const float *inv_freq;  // [64]; nullptr (and no cos_tab): no front end, the sides read finished rows
+    // the rotation given as tables instead: cos, sin [B, 128] of the element type (row stride cs_sb elements, 0 shares one
+    // row), as transformers hands them to its attention layers; the arithmetic then follows its apply_rotary_pos_emb,
+    // every product and the sum rounded to the element type
+    const void *cos_tab, *sin_tab;
+    int64_t cs_sb;
     const void *v_src;      // raw value rows [B, Hkv, 128], batch stride v_sb
     int64_t v_sb;
     void *q_out;            // [B, H, 128]
@@ -145,11 +150,11 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
                 int64_t at = t;
                 if (sd.x_at_pos) at = max(pos_dev ? pos_dev[b] + sd.pos_bias : pos0, 0);  // an empty sequence hashes row 0, written nowhere
                 xs[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + at * x_st + e, x_dtype);
-                if (rp.inv_freq) xpair[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + (e ^ 64), x_dtype);
+                if (rp.inv_freq || rp.cos_tab) xpair[it] = ha_load_elem(x, b * x_sb + in_head * x_sh + t * x_st + (e ^ 64), x_dtype);
             }
         }
     }
-    if (rp.inv_freq) {
+    if (rp.inv_freq || rp.cos_tab) {
         // rotate-half RoPE of the row this thread element belongs to (T = 1, d_in = 128): the angle in fp32, the table
         // rounded to the element type as transformers builds it, the result rounded as the cache stores it.  The first
         // code head of a KV head writes the key and copies the value row; every query head writes its query.
@@ -161,9 +166,16 @@ __global__ __launch_bounds__(kEncThreads) void encode_pack_kernel(const EncArgs 
             const int r = i / d_in, e = i % d_in, b = row0 + r;
             if (b >= n_rows) continue;
             const int p = rp.pos_dev ? rp.pos_dev[b] : rp.pos;
-            const float ang = (float)p * rp.inv_freq[e & 63];
-            const float c = ha_round_to(cosf(ang), x_dtype), sn = ha_round_to(sinf(ang), x_dtype);
-            const float y = ha_round_to(e < 64 ? xs[it] * c - xpair[it] * sn : xs[it] * c + xpair[it] * sn, x_dtype);
+            float y;
+            if (rp.cos_tab) {
+                const float c = ha_load_elem(rp.cos_tab, b * rp.cs_sb + e, x_dtype), sn = ha_load_elem(rp.sin_tab, b * rp.cs_sb + e, x_dtype);
+                const float direct = ha_round_to(__fmul_rn(xs[it], c), x_dtype), crossed = ha_round_to(__fmul_rn(xpair[it], sn), x_dtype);
+                y = ha_round_to(__fadd_rn(direct, e < 64 ? -crossed : crossed), x_dtype);
+            } else {
+                const float ang = (float)p * rp.inv_freq[e & 63];
+                const float c = ha_round_to(cosf(ang), x_dtype), sn = ha_round_to(sinf(ang), x_dtype);
+                y = ha_round_to(e < 64 ? xs[it] * c - xpair[it] * sn : xs[it] * c + xpair[it] * sn, x_dtype);
+            }
             xs[it] = y;
             if (second) {
                 ha_store_elem(rp.q_out, ((int64_t)b * n_heads + head) * HA_HEAD_DIM + e, y, x_dtype);
@@ -445,12 +457,15 @@ int ha_encode_step_cached(const void *k_cache, int64_t k_stride_b, int64_t k_str
     return launch_encode(a, B, Hc + H, (hipStream_t)stream);
 }
 
-int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
-                        const int32_t *pos_dev, const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
+static int rope_encode_step_impl(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                        const int32_t *pos_dev, const float *inv_freq, const void *cos_tab, const void *sin_tab, int64_t cs_sb,
+                        void *q_out, void *k_cache, void *v_cache,
                         int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, const float *weights_k,
                         const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim, int arith, uint32_t *kcodes,
                         int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream) {
-    HA_REQUIRE(qkv && inv_freq && q_out && k_cache && v_cache, HA_ERR_NULL_POINTER, "qkv/inv_freq/q_out/k_cache/v_cache is NULL");
+    HA_REQUIRE(qkv && (inv_freq || (cos_tab && sin_tab)) && q_out && k_cache && v_cache, HA_ERR_NULL_POINTER,
+               "qkv / rotation (inv_freq, or cos and sin) / q_out / k_cache / v_cache is NULL");
+    HA_REQUIRE(cs_sb >= 0 && (!cos_tab || (ha_aligned(cos_tab, 2) && ha_aligned(sin_tab, 2))), HA_ERR_BAD_SHAPE, "bad cos/sin table stride or alignment");
     HA_REQUIRE(H > 0 && Hkv > 0 && Hc > 0, HA_ERR_BAD_SHAPE, "H, Hkv, Hc must be positive");
     int st = validate_encode(qkv, B, Hkv, Hc, 1, weights_k, n_layers, head_dim, int_dim, final_dim, kcodes, kc_stride_b, kc_stride_h,
                              pos_dev ? 0 : pos, pos_dev);
@@ -475,9 +490,32 @@ int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int 
                         (int64_t)W, 0, nullptr, nullptr};
     a.B = B; a.T = 1; a.n_layers = n_layers; a.d_in = head_dim; a.d_int = int_dim; a.d_out = final_dim; a.arith = arith;
     a.per_head = ha_usa_packed_floats(n_layers, head_dim, int_dim, final_dim);
-    a.rope = EncRope{inv_freq, (const char *)qkv + (int64_t)(H + Hkv) * HA_HEAD_DIM * eb, qkv_stride_b, q_out, k_cache, v_cache, kv_stride_b,
-                     kv_stride_h, kv_stride_s, pos, pos_dev, cache_len};
+    a.rope = EncRope{inv_freq, cos_tab, sin_tab, cs_sb, (const char *)qkv + (int64_t)(H + Hkv) * HA_HEAD_DIM * eb, qkv_stride_b, q_out, k_cache,
+                     v_cache, kv_stride_b, kv_stride_h, kv_stride_s, pos, pos_dev, cache_len};
     return launch_encode(a, B, Hc + H, (hipStream_t)stream);
+}
+
+int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                        const int32_t *pos_dev, const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
+                        int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, const float *weights_k,
+                        const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim, int arith, uint32_t *kcodes,
+                        int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream) {
+    HA_REQUIRE(inv_freq, HA_ERR_NULL_POINTER, "inv_freq is NULL");
+    return rope_encode_step_impl(qkv, qkv_stride_b, x_dtype, B, H, Hkv, Hc, pos, pos_dev, inv_freq, nullptr, nullptr, 0, q_out, k_cache, v_cache,
+                                 kv_stride_b, kv_stride_h, kv_stride_s, cache_len, weights_k, weights_q, n_layers, head_dim, int_dim, final_dim,
+                                 arith, kcodes, kc_stride_b, kc_stride_h, qcodes, stream);
+}
+
+int ha_rope_encode_step_cos_sin(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                                const int32_t *pos_dev, const void *cos, const void *sin, int64_t cos_sin_stride_b, void *q_out,
+                                void *k_cache, void *v_cache, int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                                int64_t cache_len, const float *weights_k, const float *weights_q, int n_layers, int head_dim, int int_dim,
+                                int final_dim, int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes,
+                                void *stream) {
+    HA_REQUIRE(cos && sin, HA_ERR_NULL_POINTER, "cos/sin is NULL");
+    return rope_encode_step_impl(qkv, qkv_stride_b, x_dtype, B, H, Hkv, Hc, pos, pos_dev, nullptr, cos, sin, cos_sin_stride_b, q_out, k_cache,
+                                 v_cache, kv_stride_b, kv_stride_h, kv_stride_s, cache_len, weights_k, weights_q, n_layers, head_dim, int_dim,
+                                 final_dim, arith, kcodes, kc_stride_b, kc_stride_h, qcodes, stream);
 }
 
 }  // extern "C"

@@ -86,6 +86,9 @@ def load_library() -> C.CDLL:
     lib.ha_rope_encode_step.restype = i32
     lib.ha_rope_encode_step.argtypes = [vp, i64, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp, vp,
                                         i32, i32, i32, i32, i32, vp, i64, i64, vp, vp]
+    lib.ha_rope_encode_step_cos_sin.restype = i32
+    lib.ha_rope_encode_step_cos_sin.argtypes = [vp, i64, i32, i32, i32, i32, i32, i32, vp, vp, vp, i64, vp, vp, vp, i64, i64, i64, i64, vp, vp,
+                                                i32, i32, i32, i32, i32, vp, i64, i64, vp, vp]
     lib.ha_linear_skinny.restype = i32
     lib.ha_linear_skinny.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
     lib.ha_linear_skinny_fused.restype = i32
@@ -568,6 +571,29 @@ def rope_encode_step(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, pos: in
         _ptr(q_out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), k_cache.shape[2],
         _ptr(wk), _ptr(wq), n_layers, 128, int_dim, final_dim, arith, _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes),
         _stream(qkv)), "ha_rope_encode_step")
+
+
+def rope_encode_step_cos_sin(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, pos: int, cos: torch.Tensor, sin: torch.Tensor,
+                             q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, wk: torch.Tensor, wq: torch.Tensor,
+                             n_layers: int, int_dim: int, final_dim: int, kcodes: torch.Tensor, qcodes: torch.Tensor,
+                             arith: int = HA_ARITH_F32) -> None:
+    """`rope_encode_step` with the rotation given as the cos / sin rows a transformers layer receives: [B or 1, 128] of the
+    dtype of qkv (any leading singleton dimensions squeezed by the caller).  k_cache / v_cache [B, Hkv, capacity, 128]: the
+    new key and value go to token position `pos`."""
+    _require_cuda(qkv, cos, sin, q_out, k_cache, v_cache, wk, wq, kcodes, qcodes)
+    B = qkv.shape[0]
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and q_out.is_contiguous() and q_out.dtype == qkv.dtype == k_cache.dtype == v_cache.dtype
+    assert cos.dtype == sin.dtype == qkv.dtype and cos.dim() == 2 and cos.shape == sin.shape and cos.shape[1] == 128
+    assert cos.shape[0] in (1, B) and cos.stride(1) == 1 and sin.stride() == cos.stride()
+    assert k_cache.stride() == v_cache.stride() and k_cache.stride(3) == 1
+    assert kcodes.stride(3) == 1 and kcodes.stride(2) == kcodes.shape[3] and qcodes.is_contiguous()
+    assert kcodes.dtype == torch.int32 and qcodes.dtype == torch.int32 and qcodes.numel() == B * n_q_heads * (final_dim // 32)
+    assert 0 <= int(pos) < kcodes.shape[2] and int(pos) < k_cache.shape[2]
+    _check(load_library().ha_rope_encode_step_cos_sin(
+        _ptr(qkv), qkv.stride(0), _DTYPE[qkv.dtype], B, n_q_heads, n_kv_heads, wk.shape[0], int(pos), None, _ptr(cos), _ptr(sin),
+        0 if cos.shape[0] == 1 else cos.stride(0), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), k_cache.stride(1),
+        k_cache.stride(2), k_cache.shape[2], _ptr(wk), _ptr(wq), n_layers, 128, int_dim, final_dim, arith, _ptr(kcodes), kcodes.stride(0),
+        kcodes.stride(1), _ptr(qcodes), _stream(qkv)), "ha_rope_encode_step_cos_sin")
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:

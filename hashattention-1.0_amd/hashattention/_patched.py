@@ -29,6 +29,7 @@ import torch
 from torch import nn
 
 from . import _ops
+from .cache import PreallocatedLayer
 from .decode import HashDecodeLayer
 
 DECODE_MAX_Q_LEN = 128   # reference: `if q_len > 128 or self.train_usa` routes to the original forward (:529)
@@ -311,6 +312,9 @@ class HeavyHitterMixin:
         self._hash_layer: Optional[HashDecodeLayer] = None
         self._cache_ref = None       # weak reference to the KV cache object whose keys the bit-cache was made from
         self._cache_id = None
+        # single-token steps of a bf16 model on a cache that appends in place (cache.PreallocatedCache) take `_fast_decode`:
+        # five launches for the whole module instead of ~25 library calls; set False to keep every step on the general path
+        self.fast_decode = True
 
     def __repr__(self):
         return (f"{super().__repr__()}\nSparsification Setting(topk:{self.heavy_budget}  edge:{self.init_budget, self.recent_budget} "
@@ -475,10 +479,105 @@ class HeavyHitterMixin:
         return hl.chunk_step(query_states, key_states, value_states, S, out, heavy_abs,
                              q_hash=None if query_hash is query_states else query_hash, attn_mask=amask)
 
+    # ---- the single-token step as five launches
+    def _fused_qkv_weight(self) -> torch.Tensor:
+        """The q, k and v projection weights stacked as one [H d + 2 Hkv d, hidden] matrix (a copy, rebuilt when one of the
+        three parameters was replaced or updated in place through its version counter; after a write through `.data`
+        delete `self._qkv_fused`)."""
+        ws = (self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
+        key = tuple((w.data_ptr(), w._version, w.dtype, w.device) for w in ws)
+        hit = self.__dict__.get("_qkv_fused")
+        if hit is None or hit[0] != key:
+            hit = (key, torch.cat([w.detach() for w in ws], dim=0).contiguous())
+            self.__dict__["_qkv_fused"] = hit
+        return hit[1]
+
+    def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
+        """This layer's `PreallocatedLayer` of `cache` when the step can take `_fast_decode`, else None: one new token per
+        sequence, inference, bf16 hidden states and projections without biases, 128-wide heads, up to 16 sequences, a learned
+        hash whose codes can be cached, no KV offloading, an attention mask that changes nothing, and a cache whose layers
+        append in place."""
+        if not self.fast_decode or torch.is_grad_enabled() or self.train_usa or self.offloading_length is not None:
+            return None
+        b, q_len, hidden = hidden_states.shape
+        if q_len != 1 or b > 16 or hidden % 32 or self.head_dim != 128 or hidden_states.dtype != torch.bfloat16 \
+                or not hidden_states.is_contiguous() or position_embeddings is None:
+            return None
+        if self.q_proj.bias is not None or self.o_proj.bias is not None or self.q_proj.weight.dtype != torch.bfloat16:
+            return None
+        usa = self.usa_module
+        if usa is None or usa.rehash_every_step or getattr(cache, "offloading", False):
+            return None
+        layers = getattr(cache, "layers", None)
+        if layers is None:
+            return None
+        if len(layers) <= self.layer_idx:
+            make = getattr(cache, "layer_class_to_replicate", None)
+            if make is None or not (isinstance(make, type) and issubclass(make, PreallocatedLayer)):
+                return None
+            while len(layers) <= self.layer_idx:
+                layers.append(make())
+        slot = layers[self.layer_idx]
+        if not isinstance(slot, PreallocatedLayer):
+            return None
+        kb = slot._kbuf
+        if kb is not None and (kb.shape[0] != b or kb.shape[1] != self.num_key_value_heads or kb.shape[3] != 128
+                               or kb.dtype != torch.bfloat16 or kb.device != hidden_states.device or slot._vbuf is None
+                               or slot._vbuf.stride() != kb.stride()):
+            return None
+        cos, sin = position_embeddings
+        if cos.dtype != torch.bfloat16 or cos.shape[-1] != 128 or cos.shape[-2] != 1 or cos.shape[0] not in (1, b) or cos.dim() != 3 \
+                or cos.stride(-1) != 1 or sin.stride() != cos.stride():
+            return None
+        S = slot.get_seq_length() + 1
+        if self._additive_mask(attention_mask, b, 1, S) is not None:
+            return None
+        return slot
+
+    def _fast_decode(self, hidden_states, position_embeddings, slot):
+        """The decode branch (reference :551-625) for one new token per sequence in five launches: fused QKV projection
+        (ha_linear_skinny), rotary embedding + in-place cache append + both hashes (ha_rope_encode_step_cos_sin), distance
+        histograms, selection fused into the gather attention, output projection."""
+        b, _, hidden = hidden_states.shape
+        H, Hkv, d = self.num_heads, self.num_key_value_heads, self.head_dim
+        dev = hidden_states.device
+        sc = self.__dict__.get("_fast_scratch")
+        if sc is None or sc["qkv"].shape[0] != b or sc["qkv"].device != dev:
+            sc = dict(qkv=torch.empty(b, (H + 2 * Hkv) * d, dtype=torch.bfloat16, device=dev),
+                      q=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev),
+                      attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
+            self.__dict__["_fast_scratch"] = sc
+        _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
+        kbuf, vbuf, pos = slot.append_slots(hidden_states, b, Hkv, d, 1)
+        S = pos + 1
+        hl = self._ensure_hash_layer(b, S, dev)
+        if hl.n_cached > pos:
+            hl.reset()                       # the cache was rewound
+        if hl.n_cached < pos:                # keys cached by a prefill: hashed in bulk, once
+            hl.encode_keys_bulk(kbuf[:, :, hl.n_cached:pos], pos0=hl.n_cached)
+        cos, sin = position_embeddings
+        _ops.rope_encode_step_cos_sin(sc["qkv"], H, Hkv, pos, cos[:, 0, :], sin[:, 0, :], sc["q"], kbuf, vbuf, hl.wk, hl.wq, hl.num_layers,
+                                      hl.int_dim, hl.final_dim, hl.codes, hl.qcodes, arith=hl.arith)
+        hl.n_cached = S
+        heavy = hl.heavy_count(S)
+        saved = hl.heavy_budget
+        hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5
+        try:
+            hl._select_attend(sc["q"], kbuf, vbuf, S, sc["attn"], None)
+        finally:
+            hl.heavy_budget = saved
+        out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
+        _ops.linear_skinny(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden))
+        return out, None
+
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
         bsz, q_len, _ = hidden_states.shape
         self.ensure_gpu(cache, hidden_states.device)
         self._sync_bit_cache(cache)
+        if q_len == 1:
+            slot = self._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
+            if slot is not None:
+                return self._fast_decode(hidden_states, position_embeddings, slot)
         if q_len > DECODE_MAX_Q_LEN or self.train_usa:
             # prefill, and every step while the hash is being trained: the original dense forward (reference :529-550);
             # its keys are hashed lazily at the first decode step
@@ -498,6 +597,12 @@ class HeavyHitterMixin:
         query_states, key_states = self._apply_rope(query_states, key_states, cos, sin)
         if cache is not None:
             key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
+            # the tokens the cache holds, from the cache and not from the shape of what it returns: a cache that keeps capacity
+            # ahead of its length (`StaticCache`; `cache.PreallocatedCache` returns views of the right length already) hands out
+            # its whole buffer
+            S = self._cache_len(cache)
+            if 0 < S < key_states.shape[2]:
+                key_states, value_states = key_states[:, :, :S], value_states[:, :, :S]
         if key_states.stride(-1) != 1 or value_states.stride() != key_states.stride():
             key_states, value_states = key_states.contiguous(), value_states.contiguous()
         attn = self._sparse_attention(query_states.contiguous(), key_states, value_states, attention_mask)

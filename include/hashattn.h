@@ -414,6 +414,19 @@ int ha_rope_encode_step(const void *qkv, int64_t qkv_stride_b, int x_dtype, int 
                         const float *weights_k, const float *weights_q, int n_layers, int head_dim, int int_dim, int final_dim,
                         int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, uint32_t *qcodes, void *stream);
 /*
+ * ha_rope_encode_step with the rotation handed over as tables: cos, sin [B, 128] of x_dtype (row stride cos_sin_stride_b in
+ * elements; 0: one row for every sequence), the `position_embeddings` a transformers decoder layer passes to its attention
+ * module (what the patched layer receives: hashattention_llama.py:560-571).  The rotation follows transformers'
+ * apply_rotary_pos_emb to the rounding: q * cos and rotate_half(q) * sin each rounded to x_dtype, then their sum.  `pos`
+ * (or pos_dev[b]) is only the cache position the new key, value and key code are written to.
+ */
+int ha_rope_encode_step_cos_sin(const void *qkv, int64_t qkv_stride_b, int x_dtype, int B, int H, int Hkv, int Hc, int pos,
+                                const int32_t *pos_dev, const void *cos, const void *sin, int64_t cos_sin_stride_b, void *q_out,
+                                void *k_cache, void *v_cache, int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                                int64_t cache_len, const float *weights_k, const float *weights_q, int n_layers, int head_dim,
+                                int int_dim, int final_dim, int arith, uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h,
+                                uint32_t *qcodes, void *stream);
+/*
  * out[m, n] = sum_k x[m, k] * w[n, k] (+ residual[m, n]): a Linear layer (weight [N, K] as nn.Linear keeps it) applied to
  * M <= 16 rows, bf16 in and out, fp32 accumulation.  The decode step's projections (efficiency/model.py:236, 261,
  * 304-305: wqkv, wo, w1/w3, w2, and the lm_head of :158) are this shape: they stream every weight once per token, so

@@ -1,0 +1,143 @@
+"""`hashattention.cache.PreallocatedCache` - a DynamicCache whose layers append in place - and `StaticCache` under the patched
+layers: same logits and tokens as with the library's DynamicCache (whose update re-copies the whole cache every step)."""
+import pytest
+import torch
+from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM, StaticCache
+
+from hashattention import hashattention_llama as hl
+from hashattention.cache import PreallocatedCache, PreallocatedLayer
+from tests.test_gpu_model_api import _config
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _model(fast_decode=False):
+    torch.manual_seed(0)
+    cfg = _config(LlamaConfig)
+    model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
+    usa = hl.load_usa(cfg, None)
+    model = hl.convert_usa(model, cfg, usa, collect_stats=False, train_usa=False)
+    for layer in model.model.layers:        # the five-launch single-token path has a test of its own below
+        layer.self_attn.fast_decode = fast_decode
+    return cfg, model
+
+
+def _decode(model, ids, cache, steps):
+    outs = []
+    with torch.no_grad():
+        n0 = ids.shape[1] - sum(steps)
+        o = model(ids[:, :n0], past_key_values=cache, use_cache=True)
+        outs.append(o.logits[:, -1].float())
+        pos = n0
+        for n in steps:
+            o = model(ids[:, pos:pos + n], past_key_values=cache, use_cache=True)
+            outs.append(o.logits.float())
+            pos += n
+    return outs
+
+
+def test_preallocated_cache_gives_the_logits_of_dynamic_cache_and_never_recopies():
+    print("\n[case] PreallocatedCache vs DynamicCache", flush=True)
+    cfg, model = _model()
+    ids = torch.randint(0, cfg.vocab_size, (2, 300), generator=torch.Generator().manual_seed(1)).to(DEV)
+    steps = [1, 1, 7, 1, 1]
+    want = _decode(model, ids, DynamicCache(), steps)
+    hl.reset_usa(model)
+    cache = PreallocatedCache(capacity=512)
+    got = _decode(model, ids, cache, steps)
+    for g, w in zip(got, want):
+        assert torch.equal(g, w)
+    layer = cache.layers[0]
+    assert isinstance(layer, PreallocatedLayer) and layer.capacity == 512 and cache.get_seq_length() == 300
+    assert layer.keys.shape[2] == 300 and layer.keys.data_ptr() == layer._kbuf.data_ptr()
+    # the buffer never moved: appends were in place
+    ptr = layer._kbuf.data_ptr()
+    with torch.no_grad():
+        model(ids[:, :1], past_key_values=cache, use_cache=True)
+    assert layer._kbuf.data_ptr() == ptr and cache.get_seq_length() == 301
+    # outgrowing the capacity doubles it and keeps the content
+    small = PreallocatedCache(capacity=0)
+    hl.reset_usa(model)
+    got2 = _decode(model, ids, small, steps)
+    for g, w in zip(got2, want):
+        assert torch.equal(g, w)
+    assert small.layers[0].capacity >= 300
+    # cropping forgets tokens without touching the buffer; the bit-cache follows (same cache object, shorter)
+    cache.crop(-2)
+    assert cache.get_seq_length() == 299 and cache.layers[1].keys.shape[2] == 299
+
+
+def test_generate_with_a_preallocated_cache_gives_the_same_tokens():
+    print("\n[case] generate() with PreallocatedCache", flush=True)
+    cfg, model = _model()
+    ids = torch.randint(0, cfg.vocab_size, (2, 140), generator=torch.Generator().manual_seed(2)).to(DEV)
+    kw = dict(max_new_tokens=12, do_sample=False, pad_token_id=0)
+    want = model.generate(ids, past_key_values=DynamicCache(), **kw)
+    hl.reset_usa(model)
+    got = model.generate(ids, past_key_values=PreallocatedCache(capacity=160), **kw)
+    assert torch.equal(got, want)
+
+
+def test_static_cache_under_the_patched_layers():
+    # StaticCache.update returns its whole buffer: the layer must take the number of valid tokens from the cache
+    print("\n[case] StaticCache under the patched layers", flush=True)
+    cfg, model = _model()
+    ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(3)).to(DEV)
+    steps = [1, 1, 1]
+    want = _decode(model, ids, DynamicCache(), steps)
+    hl.reset_usa(model)
+    got = _decode(model, ids, StaticCache(config=cfg, max_cache_len=256), steps)
+    for g, w in zip(got[1:], want[1:]):             # decode steps (the prefill's dense attention sees a padded buffer either way)
+        assert (g - w).abs().max().item() < 2e-2, (g - w).abs().max().item()
+
+
+def test_single_token_steps_in_five_launches_match_the_general_path():
+    # on a PreallocatedCache a bf16 model's single-token steps run as fused QKV projection, rotary + in-place append + hashes,
+    # histograms, select-attend, output projection; the general path (library projections, torch rotary embedding,
+    # cache.update) must give the same logits up to bf16 rounding of different summation orders, and the same greedy tokens
+    print("\n[case] five-launch single-token path vs general path", flush=True)
+    cfg, model = _model(fast_decode=False)
+    ids = torch.randint(0, cfg.vocab_size, (3, 260), generator=torch.Generator().manual_seed(4)).to(DEV)
+    steps = [1, 1, 1, 6, 1, 1]                  # single tokens, a chunk (general path), single tokens again
+    want = _decode(model, ids, PreallocatedCache(capacity=300), steps)
+    hl.reset_usa(model)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = True
+        assert "_fast_scratch" not in layer.self_attn.__dict__
+    cache = PreallocatedCache(capacity=300)
+    got = _decode(model, ids, cache, steps)
+    assert all("_fast_scratch" in layer.self_attn.__dict__ for layer in model.model.layers), "the fast path was not taken"
+    assert cache.get_seq_length() == 260 and cache.layers[0].keys.shape[2] == 260
+    worst = max((g - w).abs().max().item() for g, w in zip(got, want))
+    scale = max(w.abs().max().item() for w in want)
+    print(f"max-abs logit difference {worst:.3e} (largest logit {scale:.2f})", flush=True)
+    assert worst <= 3e-2 * max(scale, 1.0)
+    # the keys the fused launch rotated and appended equal the ones torch rotated, bit for bit (same roundings)
+    ref_cache = PreallocatedCache(capacity=300)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = False
+    hl.reset_usa(model)
+    with torch.no_grad():
+        model(ids[:, :200], past_key_values=ref_cache, use_cache=True)
+        model(ids[:, 200:201], past_key_values=ref_cache, use_cache=True)
+    fast_cache = PreallocatedCache(capacity=300)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = True
+    hl.reset_usa(model)
+    with torch.no_grad():
+        model(ids[:, :200], past_key_values=fast_cache, use_cache=True)
+        model(ids[:, 200:201], past_key_values=fast_cache, use_cache=True)
+    k_ref, k_fast = ref_cache.layers[0].keys[:, :, 200], fast_cache.layers[0].keys[:, :, 200]
+    v_ref, v_fast = ref_cache.layers[0].values[:, :, 200], fast_cache.layers[0].values[:, :, 200]
+    # layer 0 sees the same hidden states on both paths; its projections differ by summation order only
+    assert (k_ref.float() - k_fast.float()).abs().max().item() <= 2e-2 and (v_ref.float() - v_fast.float()).abs().max().item() <= 2e-2
+    # greedy generation: same tokens
+    kw = dict(max_new_tokens=10, do_sample=False, pad_token_id=0)
+    hl.reset_usa(model)
+    fast_tokens = model.generate(ids[:, :150], past_key_values=PreallocatedCache(capacity=200), **kw)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = False
+    hl.reset_usa(model)
+    slow_tokens = model.generate(ids[:, :150], past_key_values=PreallocatedCache(capacity=200), **kw)
+    assert torch.equal(fast_tokens, slow_tokens)

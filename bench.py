@@ -280,7 +280,7 @@ def decoder_bench(args, torch):
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "algorithmic_bytes": ab["gather"], "us": ms_attend * 1e3},
     }
-    print(json.dumps(res))
+    return res
 
 
 def hf_path_bench(args, torch):
@@ -395,7 +395,7 @@ def hf_path_bench(args, torch):
                "per-layer = difference between the two layer counts; decoder = LlamaShapedDecoder.from_hf(...).generate (one HIP graph "
                "replayed per token); patched_attention_module = self_attn.forward of one layer alone at a fixed length",
     }
-    print(json.dumps(res))
+    return res
 
 
 class InputSet:
@@ -522,6 +522,55 @@ def first_step_probe(s, args, torch):
     return out
 
 
+def brief_layer_bench(name, args, torch, dev, n_sets=2):
+    """One of the other named configurations, timed like the headline one but without its side legs: the step over a rotation
+    of `n_sets` input sets (eager launches and a graph replay), its attention launch alone, its scoring launch alone, and the
+    dense flash-decode on the same inputs."""
+    from hashattention import _ops
+    from hashattention.synthetic import named_workload
+    w = named_workload(name)
+    sets = [InputSet(w, args, dev, torch, 101 * i) for i in range(n_sets)]
+    s0, layer = sets[0], sets[0].layer
+    B, H, S = w.batch, w.n_q_heads, w.max_seq_len
+    fused = layer.use_fused and layer.fused_ok and not layer.overlap_windows
+    steps, warmup = max(20, args.steps // 2), max(3, args.warmup // 2)
+    rot = lambda n: [getattr(s, n) for s in sets]
+    ms_eager, ms_graph, graph_ok = time_step(sets, steps, warmup, torch)
+    ms_step = min(ms_eager, ms_graph)
+    ms_prepare = time_rotating(rot("select_prepare"), steps, warmup, torch) if fused else None
+    for s in sets:
+        s.step()
+        if not fused:
+            s.select()
+    ms_attend = time_rotating(rot("attend_fused" if fused else "attend_lists"), steps, warmup, torch)
+    out_dense = torch.empty_like(s0.out)
+    ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), dev)
+    dense = [(lambda s=s: _ops.dense_decode(s.q3, s.p.k, s.p.v, S, s.seq_lens, layer.sm_scale, out_dense, ws_dense)) for s in sets]
+    ms_dense = time_rotating(dense, max(6, steps // 4), 2, torch)
+    s0.step()
+    if fused:
+        s0.select()
+    n_sel_rows = int(layer.counts.sum().item())
+    ab = algorithmic_bytes(w, n_sel_rows)
+    step_bytes = ab["score"] + ab["gather"] + (0 if fused else ab["select"])
+    res = {"workload": f"{w.name}: B={B} S={'ragged ' + str(min(w.seq_lens)) + '..' + str(S) if s0.ragged else S} code_heads={w.n_code_heads} "
+                       f"code_bits={w.lth_final_dim} heavy={w.heavy_budget:g} n_sel={n_sel_rows // (B * H)}",
+           "us_per_layer": ms_step * 1e3, "hip_graph_replay_us": ms_graph * 1e3, "eager_launches_from_python_us": ms_eager * 1e3,
+           "graph_replay_matches_eager": graph_ok, "input_sets": n_sets, "steps": steps,
+           "hbm_frac_step": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+           "speedup_vs_dense": ms_dense / ms_step, "dense_flash_decode_us": ms_dense * 1e3,
+           "dense_hbm_frac": ab["dense"] / (ms_dense * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+           "roofline": {"kernel": "sparse_attend_kernel (selection fused)" if fused else "sparse_attend_kernel", "bound": "hbm",
+                        "frac": ab["gather"] / (ms_attend * 1e-3) / 1e9 / HBM_PEAK_GBPS, "us": ms_attend * 1e3, "algorithmic_bytes": ab["gather"]}}
+    if fused:
+        res["score_roofline"] = {"kernel": "select_hist_kernel" + ("" if layer.local_thresholds else " + select_threshold_kernel"),
+                                 "frac": ab["score"] / (ms_prepare * 1e-3) / 1e9 / HBM_PEAK_GBPS, "us": ms_prepare * 1e3,
+                                 "algorithmic_bytes": ab["score"]}
+    del sets, dense
+    torch.cuda.empty_cache()
+    return res
+
+
 def time_step(sets, steps, warmup, torch):
     """The whole step over a rotation of input sets: eager launches and one HIP graph holding one pass over all sets,
     replayed.  Returns (ms eager, ms graph, graph replay reproduces the eager outputs)."""
@@ -553,6 +602,8 @@ def main():
                     "so that consecutive launches never touch the same rows (as consecutive layers of a model)")
     ap.add_argument("--no-code-heads-32", action="store_true", help="skip the extra timing of the one-code-per-query-head layout")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="config2 only: skip config1 / config3 / config4, the decoder step and "
+                    "the patched transformers model that the default run appends to its line")
     ap.add_argument("--no-first-step", action="store_true", help="skip timing the first decode step after a prefill (bulk hash of all cached keys)")
     ap.add_argument("--exact-encode", action="store_true", help="fill the bit-cache with the fp32 kernel instead of MFMA")
     ap.add_argument("--select-algo", type=int, default=0, help="0 auto, 1 histogram, 2 sampled (ha_select algo)")
@@ -579,10 +630,10 @@ def main():
         sys.exit(2)
     _ops.load_library()
     if args.config == "config3" and args.hf_path:
-        hf_path_bench(args, torch)
+        print(json.dumps(hf_path_bench(args, torch)))
         return
     if args.config == "config3" and not args.layer_only:
-        decoder_bench(args, torch)
+        print(json.dumps(decoder_bench(args, torch)))
         return
     dev = "cuda:0"
     w = named_workload(args.config)
@@ -740,6 +791,28 @@ def main():
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)
         res["cpu_sparse_port"] = cpu_sparse_stages(w, torch)
+    # the other named configurations, the 32-layer decoder step and the patched transformers model, in the same run
+    if args.config == "config2" and args.batch is None and args.code_heads is None and not args.two_launch and not args.no_other_configs:
+        del sets, s0, layer, dense
+        torch.cuda.empty_cache()
+        t0 = time.perf_counter()
+        res["other_configs"] = {name: brief_layer_bench(name, args, torch, dev) for name in ("config1", "config3", "config4")}
+        sub = argparse.Namespace(**{**vars(args), "steps": max(10, args.steps // 10), "warmup": 2})
+        d = decoder_bench(sub, torch)
+        res["decoder_config3"] = {"tokens_per_s": d["value"], "ms_per_step": d["ms_per_step"],
+                                  "generation_loop_ms": d["generation_loop"]["ms_per_token_step"],
+                                  "hip_graph_replay_ms": d["step_launch"]["hip_graph_replay_ms"],
+                                  "eager_launches_from_python_ms": d["step_launch"]["eager_launches_from_python_ms"],
+                                  "dense_attention_step_ms": d["dense_attention_step_ms"], "speedup_vs_dense_attention": d["speedup_vs_dense_attention"],
+                                  "attention_step_us_per_layer": d["attention_step_us_per_layer"], "hbm_frac_step": d["hbm_frac_step"],
+                                  "prefill_encode_ms_per_layer": d["prefill_encode_ms_per_layer"], "prefill_encode_tflops": d["prefill_encode_tflops"],
+                                  "graph_replay_matches_eager": d["graph_replay_matches_eager"], "workload": d["config"]["workload"],
+                                  "steps": sub.steps}
+        torch.cuda.empty_cache()
+        h = hf_path_bench(argparse.Namespace(**{**vars(args), "steps": 16, "layers": 4}), torch)
+        res["patched_transformers_model_config3"] = {"workload": h["config"]["workload"], "ms_per_token_step": h["value"], "layers": h["layers"],
+                                                     "per_layer_slope": h["per_layer_slope"], "how": h["how"]}
+        res["other_legs_seconds"] = time.perf_counter() - t0
     print(json.dumps(res))
 
 

@@ -410,9 +410,19 @@ __device__ __forceinline__ void request_4_bytes_to_lds(const int32_t *src, const
                  : "v"(src), "s"(lds_byte_address)
                  : "memory");
 }
+// What vmcnt(8) relies on, both stated where they are established: (a) at least eight vector-memory LOADS of the wave are
+// younger than the requests waited for (a gather step or the loop's priming: the static_assert in sparse_attend_kernel),
+// and (b) no global STORE of the wave is outstanding between those requests and this wait (loads and stores retire out of
+// order with respect to each other; the kernel stores only behind its loops).  -DHASHATTN_STAGE_WAIT_ALL builds the
+// conservative form, which must give the same bits.
 __device__ __forceinline__ void staged_codes_arrived(bool eight_younger_requests) {
+#ifdef HASHATTN_STAGE_WAIT_ALL
+    (void)eight_younger_requests;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#else
     if (eight_younger_requests) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
 }
 // Requests the codes of this wave's group of scan round `round` (geometry as in fused_round).  Lanes past the end of the
 // candidate range ask for the chunk's first codes instead (the range is not empty, so they exist); fused_round masks them.

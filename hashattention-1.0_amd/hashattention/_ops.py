@@ -42,7 +42,20 @@ def load_library() -> C.CDLL:
     if not os.path.exists(path):
         raise ImportError(f"{path} is missing: build it with `python hashattention-1.0_amd/build.py` "
                           "(hipcc --offload-arch=gfx950); there is no CPU fallback")
-    lib = C.CDLL(path)
+    _lib = _declare(C.CDLL(path))
+    return _lib
+
+
+def load_wait_all_variant() -> C.CDLL:
+    """The library's twin built with -DHASHATTN_STAGE_WAIT_ALL (tests compare the two builds bit for bit); not cached."""
+    path = os.path.join(os.path.dirname(lib_path()), "libhashattn_waitall.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: `python hashattention-1.0_amd/build.py` builds it next to the library")
+    return _declare(C.CDLL(path))
+
+
+def _declare(lib: C.CDLL) -> C.CDLL:
+    """Argument and result types of every entry point of include/hashattn.h on a loaded library."""
     vp, i32, i64, f32, f64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_double, C.c_size_t
     lib.ha_version.restype = i32
     lib.ha_status_string.restype = C.c_char_p
@@ -134,7 +147,6 @@ def load_library() -> C.CDLL:
     lib.ha_dense_decode.restype = i32
     lib.ha_dense_decode.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, f32,
                                     vp, vp, sz, vp]
-    _lib = lib
     return lib
 
 

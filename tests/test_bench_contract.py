@@ -35,3 +35,15 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > d["value"] and "sample" in cb
     assert d["graph_replay_matches_eager"] is True
+    # the other named configurations, the decoder step and the patched transformers model ride on the same line
+    assert set(d["other_configs"]) == {"config1", "config3", "config4"}
+    for name, o in d["other_configs"].items():
+        for key in ("us_per_layer", "hbm_frac_step", "speedup_vs_dense", "roofline", "graph_replay_matches_eager"):
+            assert key in o, (name, key)
+        assert 0.05 < o["roofline"]["frac"] < 1.0 and 0.0 < o["hbm_frac_step"] < 1.0 and o["graph_replay_matches_eager"] is True
+    dec = d["decoder_config3"]
+    for key in ("tokens_per_s", "ms_per_step", "generation_loop_ms"):
+        assert dec[key] > 0
+    hf = d["patched_transformers_model_config3"]
+    assert hf["ms_per_token_step"] > 0 and "patched_preallocated_us_per_layer" in hf["per_layer_slope"]
+    assert d["paged_cache_identity_table"]["same_bits_as_unpaged"] is True

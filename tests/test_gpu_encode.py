@@ -52,8 +52,10 @@ def test_bf16_arith_and_mfma_agree(layers, final):
     d_ref = _bits_differing(c_scalar, want_i32) / total
     d_mfma = _bits_differing(c_mfma, c_scalar) / total
     print(f"  bits differing: scalar-bf16 vs torch-bf16 {d_ref:.2e}, mfma vs scalar-bf16 {d_mfma:.2e}", flush=True)
-    assert d_ref < 5e-3
-    assert d_mfma < 5e-3
+    # observed over the six shapes: at most 1.2e-3 against torch's bf16 arithmetic (another summation order inside every
+    # Linear), at most one bit of 384 000 between the two kernels; bounds at three times that
+    assert d_ref < 3.5e-3
+    assert d_mfma < 1e-5
 
 
 def test_mfma_tail_and_offsets():

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from hashattention import _ops
+from oracle import c_oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -26,7 +27,7 @@ def _case(B, H, Hc, W, lens, init, recent, heavy, mode, depth, seed):
     return kc, qc, S, seq, cap
 
 
-def _both(B, H, Hc, W, lens, init=16, recent=16, heavy=0.125, mode=_ops.HA_SELECT_SIMPLE, depth=0, seed=0):
+def _both(B, H, Hc, W, lens, init=16, recent=16, heavy=0.125, mode=_ops.HA_SELECT_SIMPLE, depth=0, seed=0, check_oracle=True):
     kc, qc, S, seq, cap = _case(B, H, Hc, W, lens, init, recent, heavy, mode, depth, seed)
     idx_a = torch.full((B, H, cap), -1, dtype=torch.int32, device=DEV)
     idx_b = torch.full((B, H, cap), -1, dtype=torch.int32, device=DEV)
@@ -42,6 +43,10 @@ def _both(B, H, Hc, W, lens, init=16, recent=16, heavy=0.125, mode=_ops.HA_SELEC
     assert torch.equal(cnt_a, cnt_b), (cnt_a, cnt_b)
     assert torch.equal(idx_a, idx_b)
     assert int(cnt_a.max()) > 0
+    if check_oracle:        # and against the oracle directly, not only through ha_select
+        ref_idx, ref_cnt = c_oracle.select(kc.cpu().numpy(), qc.cpu().numpy(), np.array(lens, dtype=np.int32), init, recent, heavy, cap,
+                                           mode=0 if mode == _ops.HA_SELECT_SIMPLE else 1, depth=depth)
+        assert np.array_equal(cnt_b.cpu().numpy(), ref_cnt) and np.array_equal(idx_b.cpu().numpy(), ref_idx)
     return before, after
 
 
@@ -56,7 +61,7 @@ def test_select_static_matches_select_on_calls_in_a_row():
     _both(3, 8, 4, 2, [9000, 2000, 30000], heavy=1.0 / 16, seed=4)              # larger again, 64-bit codes
     _both(2, 8, 2, 1, [5000, 2500], mode=_ops.HA_SELECT_THRESHOLD, depth=2, seed=5)
     _both(2, 8, 2, 1, [100, 20], seed=6)                                        # rows that are all window
-    _both(16, 32, 8, 1, [65536] * 16, init=128, recent=128, heavy=1.0 / 32, seed=7)   # the headline shape: 1.2 MB of scratch
+    _both(16, 32, 8, 1, [65536] * 16, init=128, recent=128, heavy=1.0 / 32, seed=7, check_oracle=False)   # the headline shape: 1.2 MB of scratch
 
 
 def test_select_static_refuses_what_does_not_fit():

@@ -622,7 +622,9 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // NT threads = NT/16 row streams; U rows per stream per step.
 // MK: an additive term per list entry (AttnMask), natural-log units, added to the scaled score before the softmax; list-fed
 // launches only.
-template <typename E, int NT, int U, int FW, bool MK = false>
+// SL: the K/V rows are addressed through a token -> slot table (SlotMap); an instantiation of its own, so that launches
+// without a table carry none of it (as a run-time switch it cost the plain launches 0.7 - 1.3 us at 64K tokens x 16).
+template <typename E, int NT, int U, int FW, bool MK = false, bool SL = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
@@ -743,8 +745,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             hist_tile.request(fsel, row);
             if (tid < 32 * FW + 1) s_h[fsel.nchunk * (32 * FW + 1) + tid] = 0;  // the level totals (local_thresholds)
         }
-        fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr, smap.slots ? smap.slots + b * smap.stride_b : nullptr);
-        j_max = smap.slots ? smap.max_slot : max(S - 1, 0);
+        fused_windows<NT>(fsel, S, sp, cps, row_pieces, s_list, fr, SL ? smap.slots + b * smap.stride_b : nullptr);
+        j_max = SL ? smap.max_slot : max(S - 1, 0);
         r0 = 0;
         r1 = fr.nwin;  // until the thresholds are known the list is its windows
     } else {
@@ -780,7 +782,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const int64_t row_bytes = kv_ss * EL::bytes;
     constexpr int STEP = NS * U;  // rows of the list consumed per step by the workgroup
     // this sequence's token -> slot map (nullptr: rows lie at their token positions)
-    const int32_t *slot_row = smap.slots ? smap.slots + b_kv * smap.stride_b : nullptr;
+    const int32_t *slot_row = nullptr;
+    if constexpr (SL) slot_row = smap.slots + b_kv * smap.stride_b;
 
     // the query slice as it lies in memory: the score is dot8(q, k) * scale, two elements per instruction for 16-bit rows
     const Raw8<E> qraw = EL::load8((const char *)q + (b * q_sb + h * q_sh) * EL::bytes, sub);
@@ -820,8 +823,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
             for (int u = 0; u < U; ++u) mk[u] = mask_term(base, u, j0[u]);
         }
-        if constexpr (FW == 0) {
-            if (slot_row) {
+        if constexpr (FW == 0 && SL) {
+            {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     t_after[u] = list_index(base + 2 * STEP, u);
@@ -846,10 +849,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
         for (int u = 0; u < U; ++u) vn[u] = EL::load8s(vb + j_next[u] * row_bytes, sub);
         [[maybe_unused]] int32_t tok_after[U];
-        bool translated = false;
-        if constexpr (FW == 0) {
-            if (slot_row) {  // uniform: tokens of step + 2 arrived a step ago -> their slots; tokens of step + 3 requested
-                translated = true;
+        constexpr bool translated = FW == 0 && SL;
+        if constexpr (translated) {
+            {  // tokens of step + 2 arrived a step ago -> their slots; tokens of step + 3 requested
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int32_t t = t_after[u];
@@ -859,13 +861,16 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 }
             }
         }
-        if (!translated) {
+        if constexpr (!translated) {
 #pragma unroll
             for (int u = 0; u < U; ++u) j_after[u] = list_index(base + 2 * STEP, u);
         }
         if constexpr (MK) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) mk_next[u] = mask_term(base + STEP, u, translated ? tok_next[u] : j_next[u]);
+            for (int u = 0; u < U; ++u) {
+                if constexpr (translated) mk_next[u] = mask_term(base + STEP, u, tok_next[u]);
+                else mk_next[u] = mask_term(base + STEP, u, j_next[u]);
+            }
         }
 
         // ---- reduce the current step
@@ -901,7 +906,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             j_next[u] = j_after[u];
             if constexpr (MK) {
                 mk[u] = mk_next[u];
-                if (translated) tok_next[u] = tok_after[u];
+                if constexpr (translated) tok_next[u] = tok_after[u];
             }
         }
         base += STEP;
@@ -965,7 +970,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         int usable = fr.nwin, placed = fr.nwin;
         for (int k = 0; k < rounds; ++k) {
             int ready = fused_round<FW, GS, NW>(fsel, fr, b, h, qcode, k, n_groups, s_cnt, &s_cstar, s_list, s_raw, covered, slot_row);
-            if (slot_row) {
+            if constexpr (SL) {
                 usable = placed;
                 placed = min(ready, r1);
                 ready = usable;
@@ -989,7 +994,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 covered = true;
             }
         }
-        if (slot_row && rounds > 0) {
+        if (SL && rounds > 0) {
             // the last round's entries: run what the earlier rounds allow, then every wave waits for its own translations
             // and the waves meet
             if (!primed && usable >= min(2 * STEP, r1)) {
@@ -1288,9 +1293,9 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
     const dim3 grid(plan.nsplit_max, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-#define HA_SPARSE_LAUNCH(E_, NT_, U_, MK_)                                                                                           \
+#define HA_SPARSE_LAUNCH(E_, NT_, U_, MK_, SL_)                                                                                      \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0, MK_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v,   \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, NT_, U_, 0, MK_, SL_>), grid, dim3(NT_), 0, s, q, q_stride_b, q_stride_h, k, v, \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, idx, idx_cap, counts, sl2, plan.split_rows,               \
                            plan.nsplit_max, part_acc, part_ml, out, win_part, win_init, win_recent, seq_lens, max_seq_len,        \
                            FusedSel{}, amask, rows_per_seq, smap);                                                                \
@@ -1301,18 +1306,31 @@ static int sparse_decode_impl(const void *q, int64_t q_stride_b, int64_t q_strid
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
         }                                                                                                                         \
     } while (0)
-#define HA_SPARSE_DISPATCH(E_, U_)                                            \
-    do {                                                                      \
-        if (amask.values) {                                                   \
-            if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_, true);     \
-            else HA_SPARSE_LAUNCH(E_, 256, U_, true);                         \
-        } else if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_, false); \
-        else HA_SPARSE_LAUNCH(E_, 256, U_, false);                            \
+    // (256-thread workgroups exist as a tuning override only; a table takes the 512-thread form)
+#ifdef HASHATTN_TUNING_ENV
+#define HA_SPARSE_NT(E_, U_, MK_)                                                         \
+    do {                                                                                  \
+        if (smap.slots) HA_SPARSE_LAUNCH(E_, 512, U_, MK_, true);                         \
+        else if (plan.threads == 512) HA_SPARSE_LAUNCH(E_, 512, U_, MK_, false);          \
+        else HA_SPARSE_LAUNCH(E_, 256, U_, MK_, false);                                   \
+    } while (0)
+#else
+#define HA_SPARSE_NT(E_, U_, MK_)                                                         \
+    do {                                                                                  \
+        if (smap.slots) HA_SPARSE_LAUNCH(E_, 512, U_, MK_, true);                         \
+        else HA_SPARSE_LAUNCH(E_, 512, U_, MK_, false);                                   \
+    } while (0)
+#endif
+#define HA_SPARSE_DISPATCH(E_, U_)                 \
+    do {                                           \
+        if (amask.values) HA_SPARSE_NT(E_, U_, true); \
+        else HA_SPARSE_NT(E_, U_, false);          \
     } while (0)
     if (kv_dtype == HA_BF16) HA_SPARSE_DISPATCH(ElemBF16, 4);
     else if (kv_dtype == HA_F16) HA_SPARSE_DISPATCH(ElemF16, 4);
     else HA_SPARSE_DISPATCH(ElemF32, 2);
 #undef HA_SPARSE_DISPATCH
+#undef HA_SPARSE_NT
 #undef HA_SPARSE_LAUNCH
     return HA_OK;
 }
@@ -1453,9 +1471,9 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
     const dim3 grid(nsplit, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-#define HA_FUSED_LAUNCH(E_, U_, FW_)                                                                                              \
+#define HA_FUSED_LAUNCH_SL(E_, U_, FW_, SL_)                                                                                      \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v,      \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_, false, SL_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v, \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
                            part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1, smap);                 \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
@@ -1464,6 +1482,11 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
                                (int64_t)nsplit, H, 1, nsplit, out, nullptr, 0, 0, nullptr, 0);                                    \
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
         }                                                                                                                         \
+    } while (0)
+#define HA_FUSED_LAUNCH(E_, U_, FW_)                            \
+    do {                                                        \
+        if (smap.slots) HA_FUSED_LAUNCH_SL(E_, U_, FW_, true);  \
+        else HA_FUSED_LAUNCH_SL(E_, U_, FW_, false);            \
     } while (0)
     if (W == 1) {
         if (kv_dtype == HA_BF16) HA_FUSED_LAUNCH(ElemBF16, 4, 1);
@@ -1475,6 +1498,7 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
         else HA_FUSED_LAUNCH(ElemF32, 2, 2);
     }
 #undef HA_FUSED_LAUNCH
+#undef HA_FUSED_LAUNCH_SL
     return HA_OK;
 }
 

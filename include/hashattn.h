@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define HA_VERSION 100 /* 0.1.0 */
+#define HA_VERSION 200 /* 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
 
 typedef enum ha_status {
     HA_OK = 0,

@@ -286,3 +286,24 @@ def test_additive_masks_of_the_oracle():
             shifted = orc.sparse_attend(Q[bi, h, 0], K[bi, h], V[bi, h], idx.numpy(), 1 / d ** 0.5, slot_mask=torch.full((len(idx),), 1.5))
             assert (plain - shifted).abs().max().item() < 1e-6
             assert (plain - got).abs().max().item() > 1e-3          # and the random mask does change the result
+
+
+def test_rows_through_slot_table_against_loops_and_the_prototypes_identity_table():
+    # `K[Req_to_tokens[b, idx] * stride_kbs + kv_head * stride_kh]` (flash_fwd_sparse.py:466-474) written as explicit loops, and
+    # the table the prototype builds (torchatt.py:165, arange(B * N).reshape(B, N)), under which the pool IS the token-major
+    # cache that torch_fwd_sparse views as K.view(B, -1, H, D) (sparse.py:196-203): the two reference files must agree
+    g = torch.Generator().manual_seed(12)
+    B, N, H, D, spare = 3, 17, 2, 4, 5
+    pool = torch.randn(B * N + spare, H, D, generator=g)
+    table = torch.randperm(B * N + spare, generator=g)[:B * N].view(B, N)
+    got = orc.rows_through_slot_table(pool, table)
+    assert got.shape == (B, H, N, D)
+    for b in range(B):
+        for h in range(H):
+            for j in range(N):
+                assert torch.equal(got[b, h, j], pool[int(table[b, j]), h])
+    flat = pool[:B * N]
+    identity = torch.arange(B * N).reshape(B, N)
+    assert torch.equal(orc.rows_through_slot_table(flat, identity), flat.view(B, N, H, D).permute(0, 2, 1, 3))
+    # a transposed table (a plausible mistake: [S, B]) does not reproduce the loops
+    assert not torch.equal(orc.rows_through_slot_table(pool, table.t().contiguous().view(B, N)), got)

@@ -1,0 +1,78 @@
+"""Host logic of `hashattention.cache` on CPU tensors (no kernel involved): a PreallocatedLayer must behave as the DynamicLayer
+it replaces - same keys / values after every update, crop, batch selection and reordering - while appending in place."""
+import torch
+from transformers import DynamicCache
+
+from hashattention.cache import PreallocatedCache, PreallocatedLayer
+
+
+def _states(g, b, h, t, d=8):
+    return torch.randn(b, h, t, d, generator=g), torch.randn(b, h, t, d, generator=g)
+
+
+def test_updates_match_dynamic_cache_and_append_in_place():
+    g = torch.Generator().manual_seed(0)
+    ref, got = DynamicCache(), PreallocatedCache(capacity=16)
+    ptr = None
+    for step, t in enumerate([5, 1, 1, 3, 1]):                    # 11 tokens: inside the reserved 16
+        for layer in range(2):
+            k, v = _states(g, 2, 3, t)
+            rk, rv = ref.update(k, v, layer)
+            gk, gv = got.update(k, v, layer)
+            assert torch.equal(gk, rk) and torch.equal(gv, rv)
+            assert gk.shape == rk.shape and gk.stride(-1) == 1
+        if ptr is None:
+            ptr = got.layers[0]._kbuf.data_ptr()
+        assert got.layers[0]._kbuf.data_ptr() == ptr              # never reallocated
+        assert got.get_seq_length() == ref.get_seq_length() and got.get_seq_length(1) == ref.get_seq_length(1)
+    layer = got.layers[0]
+    assert isinstance(layer, PreallocatedLayer) and layer.capacity == 16 and layer.keys.shape[2] == 11
+    assert layer.get_mask_sizes(1) == ref.layers[0].get_mask_sizes(1)
+    # outgrowing the reservation doubles the buffer and keeps the content
+    k, v = _states(g, 2, 3, 9)
+    rk, _ = ref.update(k, v, 0)
+    gk, _ = got.update(k, v, 0)
+    assert torch.equal(gk, rk) and layer.capacity == 32 and layer._kbuf.data_ptr() != ptr
+
+
+def test_crop_selection_reordering_and_adoption():
+    g = torch.Generator().manual_seed(1)
+    ref, got = DynamicCache(), PreallocatedCache()
+    for layer in range(2):
+        k, v = _states(g, 4, 2, 7)
+        ref.update(k, v, layer)
+        got.update(k, v, layer)
+    ref.crop(-2)
+    got.crop(-2)
+    assert got.get_seq_length() == 5 and torch.equal(got.layers[1].keys, ref.layers[1].keys)
+    k, v = _states(g, 4, 2, 1)                                     # appending after a crop overwrites the cropped slots
+    assert torch.equal(got.update(k, v, 0)[0], ref.update(k, v, 0)[0])
+    idx = torch.tensor([2, 0])
+    ref.batch_select_indices(idx)
+    got.batch_select_indices(idx)
+    assert torch.equal(got.layers[0].keys, ref.layers[0].keys) and torch.equal(got.layers[0].values, ref.layers[0].values)
+    ref.batch_repeat_interleave(2)
+    got.batch_repeat_interleave(2)
+    assert torch.equal(got.layers[0].keys, ref.layers[0].keys) and got.layers[0].keys.shape[0] == 4
+    beam = torch.tensor([1, 1, 3, 0])
+    ref.reorder_cache(beam)
+    got.reorder_cache(beam)
+    assert torch.equal(got.layers[0].values, ref.layers[0].values)
+    k, v = _states(g, 4, 2, 2)                                     # and the adopted tensors keep growing
+    assert torch.equal(got.update(k, v, 0)[0], ref.update(k, v, 0)[0])
+    got.layers[0].reset()
+    assert got.layers[0].get_seq_length() == 0 and got.get_seq_length(1) == 5
+
+
+def test_append_slots_reserves_room_a_kernel_fills():
+    layer = PreallocatedLayer(capacity=4)
+    like = torch.zeros(1, dtype=torch.float32)
+    kb, vb, pos = layer.append_slots(like, batch=2, heads=3, head_dim=8)
+    assert pos == 0 and kb.shape == (2, 3, 4, 8) and layer.get_seq_length() == 1 and layer.keys.shape[2] == 1
+    kb[:, :, 0] = 1.0
+    vb[:, :, 0] = 2.0
+    for want in (1, 2, 3):
+        assert layer.append_slots(like, 2, 3, 8)[2] == want
+    kb2, _, pos = layer.append_slots(like, 2, 3, 8)                # the fifth token does not fit four slots
+    assert pos == 4 and layer.capacity == 8 and kb2.data_ptr() != kb.data_ptr()
+    assert (layer.keys[:, :, 0] == 1.0).all() and (layer.values[:, :, 0] == 2.0).all()

@@ -141,3 +141,68 @@ def test_single_token_steps_in_five_launches_match_the_general_path():
     hl.reset_usa(model)
     slow_tokens = model.generate(ids[:, :150], past_key_values=PreallocatedCache(capacity=200), **kw)
     assert torch.equal(fast_tokens, slow_tokens)
+
+
+def test_rope_encode_step_with_cos_sin_tables_matches_torch_bit_for_bit():
+    # ha_rope_encode_step_cos_sin against transformers' apply_rotary_pos_emb on the same bf16 rows (products and sum rounded
+    # alike), the in-place cache append, and the two hashes against ha_encode_step on the rotated rows
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    from hashattention import _ops
+    from hashattention.synthetic import make_usa_weights
+    from tests.parity_util import small_workload
+    print("\n[case] ha_rope_encode_step_cos_sin", flush=True)
+    B, H, Hkv, cap, pos = 3, 8, 2, 40, 17
+    g = torch.Generator().manual_seed(8)
+    w = small_workload(batch=B, seq_lens=[cap] * B, n_q_heads=H, n_kv_heads=Hkv, n_code_heads=Hkv, seed=5)
+    usa = make_usa_weights(w)
+    wk, wq = _ops.pack_usa_weights(usa.k, DEV), _ops.pack_usa_weights(usa.q, DEV)
+    qkv = torch.randn(B, (H + 2 * Hkv) * 128, generator=g).bfloat16().to(DEV)
+    ang = torch.rand(B, 64, generator=g) * 6.28
+    cos = torch.cat([ang.cos(), ang.cos()], -1).bfloat16().to(DEV)          # [B, 128], as rotary_emb builds them
+    sin = torch.cat([ang.sin(), ang.sin()], -1).bfloat16().to(DEV)
+    kc = torch.full((B, Hkv, cap, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((B, Hkv, cap, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+    q_out = torch.empty(B, H, 128, dtype=torch.bfloat16, device=DEV)
+    kcodes = torch.zeros(B, Hkv, cap, 1, dtype=torch.int32, device=DEV)
+    qcodes = torch.zeros(B, H, 1, 1, dtype=torch.int32, device=DEV)
+    _ops.rope_encode_step_cos_sin(qkv, H, Hkv, pos, cos, sin, q_out, kc, vc, wk, wq, 3, 128, 32, kcodes, qcodes)
+    q = qkv[:, :H * 128].view(B, 1, H, 128).transpose(1, 2)
+    k = qkv[:, H * 128:(H + Hkv) * 128].view(B, 1, Hkv, 128).transpose(1, 2)
+    v = qkv[:, (H + Hkv) * 128:].view(B, Hkv, 128)
+    q_ref, k_ref = apply_rotary_pos_emb(q, k, cos[:, None, :], sin[:, None, :])
+    assert torch.equal(q_out, q_ref[:, :, 0]) and torch.equal(kc[:, :, pos], k_ref[:, :, 0]) and torch.equal(vc[:, :, pos], v)
+    untouched = torch.ones(cap, dtype=torch.bool)
+    untouched[pos] = False
+    assert (kc[:, :, untouched] == 7.0).all() and (vc[:, :, untouched] == 7.0).all()
+    kcodes2 = torch.zeros_like(kcodes)
+    qcodes2 = torch.zeros_like(qcodes)
+    _ops.encode_step(k_ref.contiguous(), q_ref[:, :, 0].contiguous(), wk, wq, 3, 128, 32, kcodes2, qcodes2, pos0=pos)
+    assert torch.equal(kcodes, kcodes2) and torch.equal(qcodes, qcodes2)
+    # one table row shared by the batch (stride 0)
+    q_out2 = torch.empty_like(q_out)
+    _ops.rope_encode_step_cos_sin(qkv, H, Hkv, pos + 1, cos[:1], sin[:1], q_out2, kc, vc, wk, wq, 3, 128, 32, kcodes, qcodes)
+    q_ref2, _ = apply_rotary_pos_emb(q, k, cos[:1, None, :], sin[:1, None, :])
+    assert torch.equal(q_out2, q_ref2[:, :, 0])
+
+
+def test_mistral_takes_the_five_launch_step_too():
+    from transformers import MistralConfig, MistralForCausalLM
+    from hashattention import hashattention_mistral as hm
+    print("\n[case] five-launch single-token path, Mistral", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(MistralConfig, sliding_window=None)
+    model = MistralForCausalLM(cfg).bfloat16().to(DEV)
+    model = hm.convert_usa(model, cfg, hm.load_usa(cfg, None), collect_stats=False, train_usa=False)
+    ids = torch.randint(0, cfg.vocab_size, (2, 220), generator=torch.Generator().manual_seed(6)).to(DEV)
+    steps = [1, 1, 1]
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = False
+    want = _decode(model, ids, PreallocatedCache(capacity=256), steps)
+    hm.reset_usa(model)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = True
+    got = _decode(model, ids, PreallocatedCache(capacity=256), steps)
+    assert all("_fast_scratch" in layer.self_attn.__dict__ for layer in model.model.layers)
+    worst = max((g - w).abs().max().item() for g, w in zip(got, want))
+    scale = max(w.abs().max().item() for w in want)
+    assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)

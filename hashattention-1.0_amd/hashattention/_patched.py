@@ -338,7 +338,10 @@ class HeavyHitterMixin:
     def ensure_gpu(self, cache, device):
         layer = self._cache_layer(cache)
         if layer is not None and not layer.keys.is_cuda:
+            known = self._holds_known_keys(cache)
             layer.keys, layer.values = layer.keys.to(device), layer.values.to(device)
+            if known:
+                self._note_key_storage(cache)       # moved by this layer itself: the same contents
 
     def offload_if_necessary_cpu(self, cache):
         layer = self._cache_layer(cache)
@@ -362,11 +365,38 @@ class HeavyHitterMixin:
         layer = self._cache_layer(cache)
         return 0 if layer is None else int(layer.keys.shape[-2])
 
+    def _key_storage(self, cache):
+        """What identifies the contents this layer's cache holds between two forward passes: the tensor object its layer
+        keeps the keys in (`DynamicLayer` and `StaticLayer` replace that object whenever they reorder, select or repeat batch
+        entries), or, for a `PreallocatedLayer`, the layer and its count of outside assignments (its buffer is also replaced
+        when it grows, with the same contents)."""
+        if cache is None or not hasattr(cache, "layers") or len(cache.layers) <= self.layer_idx:
+            return None
+        layer = cache.layers[self.layer_idx]
+        if isinstance(layer, PreallocatedLayer):
+            return ("preallocated", id(layer), layer.epoch)
+        keys = getattr(layer, "keys", None)
+        return keys if isinstance(keys, torch.Tensor) else None
+
+    def _note_key_storage(self, cache) -> None:
+        """Remember the key storage as this forward pass leaves it (`_holds_known_keys` at the next pass)."""
+        held = self._key_storage(cache)
+        self.__dict__["_keys_seen"] = weakref.ref(held) if isinstance(held, torch.Tensor) else held
+
+    def _holds_known_keys(self, cache) -> bool:
+        seen = self.__dict__.get("_keys_seen")
+        if seen is None:
+            return False
+        now = self._key_storage(cache)
+        return now is not None and ((seen() is now) if isinstance(seen, weakref.ref) else seen == now)
+
     def _sync_bit_cache(self, cache) -> None:
         """Keep the bit-cache in step with the KV cache before a forward pass appends to it.  The reference is stateless
         here (`past_key_signatures` stays None, :407-408, every key is re-hashed every step), so a caller may start a new
         prompt without `reset_usa`: codes are kept only while the SAME cache object still holds at least the tokens they
-        were made from.  Another cache object drops them all; a cache that was rewound keeps the codes of its prefix."""
+        were made from, in the storage this layer last saw.  Another cache object drops them all, and so does a cache whose
+        batch entries were reordered, selected or repeated between two passes (beam search); a cache that was rewound
+        keeps the codes of its prefix."""
         if cache is None:
             same = False
         elif self._cache_ref is not None:
@@ -382,6 +412,8 @@ class HeavyHitterMixin:
         hl = self._hash_layer
         if hl is None:
             return
+        if same and hl.n_cached > 0 and not self._holds_known_keys(cache):
+            same = False        # same cache object, other contents: beam search reordered it, or rows were selected or repeated
         if not same:
             hl.reset()
         else:
@@ -577,7 +609,9 @@ class HeavyHitterMixin:
         if q_len == 1:
             slot = self._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
             if slot is not None:
-                return self._fast_decode(hidden_states, position_embeddings, slot)
+                ret = self._fast_decode(hidden_states, position_embeddings, slot)
+                self._note_key_storage(cache)
+                return ret
         if q_len > DECODE_MAX_Q_LEN or self.train_usa:
             # prefill, and every step while the hash is being trained: the original dense forward (reference :529-550);
             # its keys are hashed lazily at the first decode step
@@ -586,6 +620,7 @@ class HeavyHitterMixin:
             if self.collect_stats or self.train_usa:
                 self.usa_local_compute(hidden_states, attention_mask, None, cache, position_embeddings)
             self.offload_if_necessary_cpu(cache)
+            self._note_key_storage(cache)
             return ret
         hidden_shape = (bsz, q_len, -1, self.head_dim)
         query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
@@ -609,6 +644,7 @@ class HeavyHitterMixin:
         attn = attn.transpose(1, 2).reshape(bsz, q_len, -1).contiguous()
         out = self.o_proj(attn)
         self.offload_if_necessary_cpu(cache)
+        self._note_key_storage(cache)
         return out, None
 
     # ---- reference API kept for callers; outside the accelerated path

@@ -33,7 +33,9 @@ class PreallocatedLayer(DynamicLayer):
     def __init__(self, capacity: Optional[int] = None, **kwargs):
         self._kbuf = self._vbuf = None
         self._len = 0
+        self.epoch = 0
         super().__init__()
+        self.epoch = 0      # counts assignments to `keys` from here on: contents replaced from outside (beam reordering, batch selection)
         self.capacity_hint = int(self.default_capacity if capacity is None else capacity)
 
     # -- keys / values as views of the buffers
@@ -43,6 +45,7 @@ class PreallocatedLayer(DynamicLayer):
 
     @keys.setter
     def keys(self, t):
+        self.epoch += 1
         self._kbuf = t
         self._len = 0 if t is None or t.dim() < 3 else int(t.shape[-2])
         if t is not None and t.dim() < 3:

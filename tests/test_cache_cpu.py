@@ -76,3 +76,20 @@ def test_append_slots_reserves_room_a_kernel_fills():
     kb2, _, pos = layer.append_slots(like, 2, 3, 8)                # the fifth token does not fit four slots
     assert pos == 4 and layer.capacity == 8 and kb2.data_ptr() != kb.data_ptr()
     assert (layer.keys[:, :, 0] == 1.0).all() and (layer.values[:, :, 0] == 2.0).all()
+
+
+def test_epoch_counts_outside_assignments_only():
+    # the patched layers keep their codes while `epoch` stands still: growth and appends leave it, reordering bumps it
+    cache = PreallocatedCache(capacity=2)
+    g = torch.Generator().manual_seed(3)
+    for _ in range(5):                                             # outgrows the capacity twice
+        cache.update(*_states(g, 2, 2, 1), 0)
+    layer = cache.layers[0]
+    assert layer.epoch == 0 and layer.capacity >= 5
+    layer.append_slots(torch.zeros(1), 2, 2, 8)
+    layer.crop(-1)
+    assert layer.epoch == 0
+    cache.reorder_cache(torch.tensor([1, 0]))
+    assert layer.epoch == 1
+    cache.batch_repeat_interleave(2)
+    assert layer.epoch == 2 and layer.keys.shape[0] == 4

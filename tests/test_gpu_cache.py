@@ -206,3 +206,30 @@ def test_mistral_takes_the_five_launch_step_too():
     worst = max((g - w).abs().max().item() for g, w in zip(got, want))
     scale = max(w.abs().max().item() for w in want)
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
+
+
+@pytest.mark.parametrize("kind", ["dynamic", "preallocated", "preallocated_fast"])
+def test_reordering_the_cache_between_steps_drops_the_stale_codes(kind):
+    # beam search permutes, selects and repeats batch entries of the cache between two steps (`Cache.reorder_cache`): the codes
+    # the layers keep for the cached keys then belong to other rows.  The reference re-hashes every key at every step; here the
+    # layers notice that the cache's key storage is no longer the one they left and hash the cache afresh.
+    print(f"\n[case] cache reordered between steps, {kind}", flush=True)
+    cfg, model = _model(fast_decode=kind.endswith("fast"))
+    make = (lambda: DynamicCache()) if kind == "dynamic" else (lambda: PreallocatedCache(capacity=400))
+    ids = torch.randint(0, cfg.vocab_size, (3, 264), generator=torch.Generator().manual_seed(5)).to(DEV)
+    perm = torch.tensor([2, 0, 0], device=DEV)          # a permutation with a repeat, as beams do
+    with torch.no_grad():
+        # the run to compare with: the reordered batch from the start
+        want_cache = make()
+        model(ids[perm, :260], past_key_values=want_cache, use_cache=True)
+        want = [model(ids[perm, 260 + i:261 + i], past_key_values=want_cache, use_cache=True).logits.float() for i in range(4)]
+        hl.reset_usa(model)
+        cache = make()
+        model(ids[:, :260], past_key_values=cache, use_cache=True)
+        for i in range(2):                              # two steps in the original order fill the bit-cache
+            model(ids[:, 260 + i:261 + i], past_key_values=cache, use_cache=True)
+        cache.crop(-2)
+        cache.reorder_cache(perm)
+        got = [model(ids[perm, 260 + i:261 + i], past_key_values=cache, use_cache=True).logits.float() for i in range(4)]
+    for g, w in zip(got, want):
+        assert torch.equal(g, w), (g - w).abs().max().item()

@@ -233,3 +233,25 @@ def test_reordering_the_cache_between_steps_drops_the_stale_codes(kind):
         got = [model(ids[perm, 260 + i:261 + i], past_key_values=cache, use_cache=True).logits.float() for i in range(4)]
     for g, w in zip(got, want):
         assert torch.equal(g, w), (g - w).abs().max().item()
+
+
+@pytest.mark.parametrize("kind", ["dynamic", "preallocated_fast"])
+def test_beam_search_gives_the_tokens_of_a_run_that_rehashes_every_step(kind):
+    # generate() with beams reorders the cache at every step.  The run to compare with forgets its codes before every forward
+    # pass (`reset_usa`), which is what the reference does by construction (it hashes every cached key at every step).
+    print(f"\n[case] beam search, {kind}", flush=True)
+    cfg, model = _model(fast_decode=kind.endswith("fast"))
+    make = (lambda: DynamicCache()) if kind == "dynamic" else (lambda: PreallocatedCache(capacity=256))
+    ids = torch.randint(0, cfg.vocab_size, (2, 150), generator=torch.Generator().manual_seed(6)).to(DEV)
+    kw = dict(max_new_tokens=10, do_sample=False, num_beams=3, pad_token_id=0)
+    def forget(module, args):
+        hl.reset_usa(module)            # (a pre-hook's return value would replace the arguments)
+
+    hook = model.register_forward_pre_hook(forget)
+    try:
+        want = model.generate(ids, past_key_values=make(), **kw)
+    finally:
+        hook.remove()
+    hl.reset_usa(model)
+    got = model.generate(ids, past_key_values=make(), **kw)
+    assert torch.equal(got, want)

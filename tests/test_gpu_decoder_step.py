@@ -3,9 +3,10 @@ SwiGLU, lm_head) against a `transformers` Llama of the same weights whose attent
 `convert_usa`: both run the HIP attention, so this checks the plumbing around it.  fp32, tight tolerance."""
 import pytest
 import torch
-from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
+from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM, MistralConfig, MistralForCausalLM
 
 from hashattention import hashattention_llama as hl
+from hashattention import hashattention_mistral as hm
 from hashattention.decoder import LlamaShapedDecoder
 from hashattention.synthetic import UsaWeights
 
@@ -297,13 +298,19 @@ def test_generate_replays_one_graph_for_successive_tokens(n_heads, batch):
         decs[1].generate(first, 2000)
 
 
-def test_decoder_from_hf_prefill_and_generate_match_the_patched_model():
-    # the serving path end to end: a transformers Llama + hash modules -> LlamaShapedDecoder.from_hf, prefill by the model
-    # itself, greedy generation by graph replay; against `generate` of the same model patched with convert_usa
-    print("\n[case] decoder from_hf + prefill_from_hf + generate vs patched model.generate", flush=True)
+@pytest.mark.parametrize("family", ["llama", "mistral"])
+def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
+    # the serving path end to end: a transformers Llama (or Mistral: the same decoder shape) + hash modules ->
+    # LlamaShapedDecoder.from_hf, prefill by the model itself, greedy generation by graph replay; against `generate` of the
+    # same model patched with convert_usa
+    print(f"\n[case] decoder from_hf + prefill_from_hf + generate vs patched model.generate, {family}", flush=True)
     torch.manual_seed(2)
-    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
-                      head_dim=128, vocab_size=512, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5)
+    shape = dict(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                 head_dim=128, vocab_size=512, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5)
+    if family == "llama":
+        cfg, LlamaForCausalLM, hl = LlamaConfig(**shape), globals()["LlamaForCausalLM"], globals()["hl"]
+    else:
+        cfg, LlamaForCausalLM, hl = MistralConfig(sliding_window=None, **shape), MistralForCausalLM, hm
     for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
                      recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
         setattr(cfg, k, v)

@@ -795,12 +795,21 @@ class HeavyHitterMixin:
 
 # ------------------------------------------------------------------------------------------ module-patch helpers
 
+def _head_dim_of(config) -> int:
+    """Width of an attention head; the kernels are built for 128 (Llama-3.x 8B / 70B, Mistral-7B: the models the reference's
+    checkpoints are for) and say so before anything is patched rather than at the first decode step."""
+    head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+    if head_dim != 128:
+        raise NotImplementedError(f"the HIP attention kernels of this build are written for 128-wide heads; this model has head_dim={head_dim}")
+    return head_dim
+
+
 def build_usa_modules(config, path, force_num_layers=None) -> nn.ModuleList:
     """Body of `load_usa` (reference :633-646): one USA per decoder layer, optionally loaded from a state dict.
     `force_num_layers`: the depth of the hash MLP when the family's reference ignores `config.lth_num_layers` (Mistral)."""
     cfg = {"lth_int_dim": config.lth_init_dim, "lth_final_dim": config.lth_final_dim, "lth_thold": config.lth_thold,
            "lth_num_layers": force_num_layers if force_num_layers is not None else config.lth_num_layers}
-    head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+    head_dim = _head_dim_of(config)
     mods = nn.ModuleList([USA(config.num_attention_heads, head_dim, cfg) for _ in range(config.num_hidden_layers)])
     if path is not None:
         # checkpoints are plain state dicts of tensors: load them without executing anything from the file
@@ -814,6 +823,7 @@ def build_usa_modules(config, path, force_num_layers=None) -> nn.ModuleList:
 
 def convert_modules(model, config, usa_modules, collect_stats, train_usa, original_cls, patched_cls):
     """Body of `convert_usa` (reference :650-667): replace every `original_cls` by `patched_cls` in place."""
+    _head_dim_of(config)
     for name, module in reversed(model._modules.items()):
         if len(list(module.children())) > 0:
             model._modules[name] = convert_modules(module, config, usa_modules, collect_stats, train_usa,

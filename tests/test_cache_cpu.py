@@ -93,3 +93,22 @@ def test_epoch_counts_outside_assignments_only():
     assert layer.epoch == 1
     cache.batch_repeat_interleave(2)
     assert layer.epoch == 2 and layer.keys.shape[0] == 4
+
+
+def test_models_with_other_head_widths_are_refused_before_anything_is_patched():
+    # the kernels are built for 128-wide heads: say so at load_usa / convert_usa, not at the first decode step
+    import pytest
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from hashattention import hashattention_llama as hl
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=2,
+                      head_dim=64, vocab_size=64)
+    for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
+                     recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
+        setattr(cfg, k, v)
+    with pytest.raises(NotImplementedError, match="128-wide heads"):
+        hl.load_usa(cfg, None)
+    model = LlamaForCausalLM(cfg)
+    before = type(model.model.layers[0].self_attn)
+    with pytest.raises(NotImplementedError, match="128-wide heads"):
+        hl.convert_usa(model, cfg, [None], collect_stats=False, train_usa=False)
+    assert type(model.model.layers[0].self_attn) is before

@@ -396,7 +396,8 @@ class HeavyHitterMixin:
         prompt without `reset_usa`: codes are kept only while the SAME cache object still holds at least the tokens they
         were made from, in the storage this layer last saw.  Another cache object drops them all, and so does a cache whose
         batch entries were reordered, selected or repeated between two passes (beam search); a cache that was rewound
-        keeps the codes of its prefix."""
+        keeps the codes of its prefix when its storage is still the same (`PreallocatedCache.crop`; the library's
+        `DynamicCache.crop` leaves a new tensor behind and is hashed afresh)."""
         if cache is None:
             same = False
         elif self._cache_ref is not None:
@@ -606,7 +607,7 @@ class HeavyHitterMixin:
         bsz, q_len, _ = hidden_states.shape
         self.ensure_gpu(cache, hidden_states.device)
         self._sync_bit_cache(cache)
-        if q_len == 1:
+        if q_len == 1 and not kwargs.get("output_attentions"):
             slot = self._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
             if slot is not None:
                 ret = self._fast_decode(hidden_states, position_embeddings, slot)
@@ -622,6 +623,9 @@ class HeavyHitterMixin:
             self.offload_if_necessary_cpu(cache)
             self._note_key_storage(cache)
             return ret
+        if kwargs.get("output_attentions"):
+            # the reference returns the weights of its dense product (:615-631); the gather attention never forms them
+            raise NotImplementedError("output_attentions=True: the sparse decode branch does not materialise attention weights")
         hidden_shape = (bsz, q_len, -1, self.head_dim)
         query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
         key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)

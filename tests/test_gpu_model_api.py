@@ -255,3 +255,21 @@ def test_a_new_prompt_needs_no_reset_usa():
     ref = _greedy(model, torch.cat([prompts[1][:, :400], tail], dim=1), 5)
     assert torch.equal(got[0], ref[0])
     assert (got[1] - ref[1]).abs().max().item() < 2e-2      # the prefill was chunked differently (500 | 150 against 550 at once)
+
+
+def test_attention_weights_are_refused_on_the_decode_branch():
+    # the reference returns the weights of its dense product when asked (hashattention_llama.py:615-631); the gather attention
+    # never forms them, and says so instead of returning None
+    print("\n[case] output_attentions on the decode branch", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(LlamaConfig)
+    model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
+    model = hl.convert_usa(model, cfg, hl.load_usa(cfg, None), collect_stats=False, train_usa=False)
+    attn = model.model.layers[0].self_attn
+    hidden = torch.randn(1, 1, cfg.hidden_size, device=DEV, dtype=torch.bfloat16)
+    cos = torch.ones(1, 1, 128, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        out, weights = attn(hidden, position_embeddings=(cos, torch.zeros_like(cos)), past_key_values=DynamicCache())
+        assert out.shape == hidden.shape and weights is None
+        with pytest.raises(NotImplementedError, match="attention weights"):
+            attn(hidden, position_embeddings=(cos, torch.zeros_like(cos)), past_key_values=DynamicCache(), output_attentions=True)

@@ -522,6 +522,37 @@ def first_step_probe(s, args, torch):
     return out
 
 
+def chunk_steps_probe(s, args, torch):
+    """Chunked decode (1 < q_len <= 128 new tokens per sequence, the reference's `compute_mask_multi` branch with one causal
+    window per query row, hashattention_llama.py:423-428): the chunk's rows become batch entries of ONE selection and ONE attention
+    launch.  Microseconds per chunk and layer for 8 and 64 rows per sequence, and the gather's share of the HBM roofline
+    (516 bytes per selected (row, head, token))."""
+    from hashattention.decode import HashDecodeLayer
+    from hashattention.synthetic import make_usa_weights
+    w, S = s.w, s.S
+    usa = make_usa_weights(w)
+    layer = HashDecodeLayer(usa.k, usa.q, w.n_q_heads, w.n_kv_heads, w.head_dim, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim,
+                            w.init_budget, w.recent_budget, w.heavy_budget, device=s.dev)
+    layer.allocate(w.batch, S)
+    layer.encode_keys_bulk(s.p.k[:, :, :S])
+    layer.n_cached = S
+    heavy = layer.heavy_count(S)
+    out = {"sequences": w.batch, "cached_tokens": S}
+    for T in (8, 64):
+        q = torch.randn(w.batch, w.n_q_heads, T, w.head_dim, device=s.dev).to(s.p.k.dtype)
+        o = torch.empty_like(q)
+        run = lambda: layer.chunk_step(q, s.p.k, s.p.v, S, o, heavy + 0.5)
+        ms = time_gpu(run, 3, 1, torch)
+        n_sel = int(layer._chunk["cnt"].sum().item())
+        out[f"rows_{T}"] = {"us_per_chunk": ms * 1e3, "us_per_row": ms * 1e3 / T, "selected_row_head_tokens": n_sel,
+                            "gather_hbm_frac_of_whole_chunk_step": n_sel * 516 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        layer._chunk = None
+        del q, o
+    del layer
+    torch.cuda.empty_cache()
+    return out
+
+
 def brief_layer_bench(name, args, torch, dev, n_sets=2):
     """One of the other named configurations, timed like the headline one but without its side legs: the step over a rotation
     of `n_sets` input sets (eager launches and a graph replay), its attention launch alone, its scoring launch alone, and the
@@ -790,6 +821,7 @@ def main():
             "roofline": roofline_obj("sparse_attend_kernel (selection fused)" if t_fused else "sparse_attend_kernel", ab2["gather"], t_attend)}
         if not args.no_first_step:
             res["first_step_after_prefill"] = first_step_probe(twins[0], args, torch)
+            res["chunked_decode"] = chunk_steps_probe(sets[0], args, torch)
         del twins
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(w, torch)

@@ -212,9 +212,11 @@ class LlamaShapedDecoder:
         return F.linear(x, self.lm_head)
 
     # ------------------------------------------------------------------ greedy generation, one graph for all tokens
-    def generate(self, tokens: torch.Tensor, n_new: int, use_graph: bool = True) -> torch.Tensor:
+    def generate(self, tokens: torch.Tensor, n_new: int, use_graph: bool = True, sampler=None) -> torch.Tensor:
         """Greedy decoding: `tokens` [B] are fed at position `seq_len`, then each step's arg-max, `n_new` steps in all;
-        returns the [B, n_new] tokens produced.  The protocol of the reference's harness (efficiency/generate.py:68-96,
+        returns the [B, n_new] tokens produced.  `sampler`: a function logits [B, vocab] -> tokens [B] (int64, on the device,
+        without a host synchronisation if the loop is to stay free of them) in place of the arg-max, which is what the
+        reference's `sample` takes (efficiency/generate.py:44-49).  The protocol of the reference's harness (efficiency/generate.py:68-96,
         `decode_n_tokens`, its step compiled at :340-348): the step is captured ONCE as a HIP graph whose kernels read the position
         from device memory, and replayed per token; between replays only the arg-max and the position increment are
         launched, and nothing waits for the host."""
@@ -250,7 +252,10 @@ class LlamaShapedDecoder:
                 self._gen_logits = step()
         for i in range(n_new):
             run()
-            torch.argmax(self._gen_logits, dim=-1, out=self.tok_dev)
+            if sampler is None:
+                torch.argmax(self._gen_logits, dim=-1, out=self.tok_dev)
+            else:
+                self.tok_dev.copy_(sampler(self._gen_logits).reshape(B))
             out[:, i].copy_(self.tok_dev)
             self.pos_dev.add_(1)
             self.len_dev.add_(1)

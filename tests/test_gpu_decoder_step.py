@@ -296,6 +296,20 @@ def test_generate_replays_one_graph_for_successive_tokens(n_heads, batch):
     assert torch.equal(decs[0].k_cache[0][:, :, :ctx + 1], decs[1].k_cache[0][:, :, :ctx + 1])
     with pytest.raises(ValueError):
         decs[1].generate(first, 2000)
+    # a sampler in place of the arg-max: the reference's `sample` (arg-max of the probabilities) gives the greedy tokens again;
+    # a top-k sampler with its own generator runs through the same captured graph
+    more = decs[1].generate(graph[:, -1], 4)
+    with torch.no_grad():
+        again = decs[2].generate(eager[:, -1], 4, use_graph=False, sampler=lambda lg: torch.softmax(lg.float(), -1).argmax(-1))
+    assert torch.equal(more, again)
+    g = torch.Generator(device=DEV).manual_seed(0)
+
+    def top_k(lg, k=5):
+        v, i = torch.topk(lg.float(), k, dim=-1)
+        return i.gather(-1, torch.multinomial(torch.softmax(v, -1), 1, generator=g))[:, 0]
+
+    sampled = decs[1].generate(more[:, -1], 6, sampler=top_k)
+    assert sampled.shape == (batch, 6) and int(sampled.min()) >= 0 and int(sampled.max()) < 512
 
 
 @pytest.mark.parametrize("family", ["llama", "mistral"])

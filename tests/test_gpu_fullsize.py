@@ -10,17 +10,24 @@ import torch
 
 from hashattention import _ops
 from hashattention.decode import HashDecodeLayer
-from hashattention.synthetic import make_problem_on_device, named_workload
+from hashattention.synthetic import Workload, make_problem_on_device, named_workload
 from oracle import c_oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("name", ["config1", "config2", "config3", "config4"])
+def _long_rows(name):
+    # rows of more than 262144 tokens: more chunks than the attention launch derives thresholds for by itself, so the step is
+    # encode, ha_select_prepare, ha_sparse_decode_fused on ready thresholds; an absolute heavy budget keeps a row's list in LDS
+    lens = [300_000, 300_000] if name == "long_uniform" else [300_000, 277_123]
+    return Workload(name, batch=2, seq_lens=lens, n_q_heads=16, n_kv_heads=4, n_code_heads=4, heavy_budget=4000.0)
+
+
+@pytest.mark.parametrize("name", ["config1", "config2", "config3", "config4", "long_uniform", "long_ragged"])
 def test_full_size_configuration(name):
     print(f"\n[case] full size {name}", flush=True)
-    w = named_workload(name)
+    w = _long_rows(name) if name.startswith("long") else named_workload(name)
     p = make_problem_on_device(w, DEV)
     B, H, Hkv, S, W = w.batch, w.n_q_heads, w.n_kv_heads, w.max_seq_len, w.code_words
     layer = HashDecodeLayer(p.usa.k, p.usa.q, H, Hkv, 128, w.lth_num_layers, w.lth_int_dim, w.lth_final_dim, w.init_budget,
@@ -29,6 +36,8 @@ def test_full_size_configuration(name):
     layer.encode_keys(p.k, use_mfma=True)
     ragged = len(set(w.seq_lens)) > 1
     seq = p.seq_lens if ragged else None
+    if name.startswith("long"):
+        assert layer.use_fused and layer.fused_ok and not layer.local_thresholds
     out = torch.empty(B, H, 128, dtype=w.dtype, device=DEV)
     if ragged:
         layer.step(p.q, p.k, p.v, S, out, seq_lens=seq)

@@ -20,11 +20,13 @@ DEV = "cuda:0"
 def _long_rows(name):
     # rows of more than 262144 tokens: more chunks than the attention launch derives thresholds for by itself, so the step is
     # encode, ha_select_prepare, ha_sparse_decode_fused on ready thresholds; an absolute heavy budget keeps a row's list in LDS
+    if name == "long_million":      # one sequence of a million tokens, the 8B head layout
+        return Workload(name, batch=1, seq_lens=[1_000_000], heavy_budget=4000.0)
     lens = [300_000, 300_000] if name == "long_uniform" else [300_000, 277_123]
     return Workload(name, batch=2, seq_lens=lens, n_q_heads=16, n_kv_heads=4, n_code_heads=4, heavy_budget=4000.0)
 
 
-@pytest.mark.parametrize("name", ["config1", "config2", "config3", "config4", "long_uniform", "long_ragged"])
+@pytest.mark.parametrize("name", ["config1", "config2", "config3", "config4", "long_uniform", "long_ragged", "long_million"])
 def test_full_size_configuration(name):
     print(f"\n[case] full size {name}", flush=True)
     w = _long_rows(name) if name.startswith("long") else named_workload(name)

@@ -344,6 +344,13 @@ def hf_path_bench(args, torch):
         cache = PreallocatedCache(capacity=S + 256, num_layers=L)
         fill(cache, L, S - 1 - warm)
         ms_pre, host_pre = time_tokens(model, cache, steps, warm)
+        # the same with only the attention module in few launches (the decoder layer around it through the library's own forward)
+        for lyr in model.model.layers:
+            lyr.self_attn.fast_layer = False
+        cache.crop(-(steps + warm))
+        ms_attn_fast, _ = time_tokens(model, cache, steps, warm)
+        for lyr in model.model.layers:
+            lyr.self_attn.fast_layer = True
         # the attention module of one layer alone, at a fixed length: hidden states in, attention output out
         layer = model.model.layers[0].self_attn
         h = torch.randn(B, 1, 4096, device=dev, dtype=torch.bfloat16)
@@ -375,7 +382,8 @@ def hf_path_bench(args, torch):
             e1.record()
             torch.cuda.synchronize()
         ms_dec = e0.elapsed_time(e1) / steps
-        out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre, patched_dynamic_cache_ms=ms_dyn,
+        out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre,
+                      patched_preallocated_attention_module_only_ms=ms_attn_fast, patched_dynamic_cache_ms=ms_dyn,
                       decoder_generate_ms=ms_dec, patched_attention_module_us=ms_attn * 1e3)
         del dec, model, usa
         torch.cuda.empty_cache()
@@ -391,7 +399,9 @@ def hf_path_bench(args, torch):
                                f"head (fp32 modules), init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g}"},
         "layers": {str(k): v for k, v in out.items()},
         "per_layer_slope": per_layer,
-        "how": "single-token forward passes of the patched model, eager launches from Python, HIP events around the timed passes; "
+        "how": "single-token forward passes of the patched model, eager launches from Python, HIP events around the timed passes "
+               "(patched_preallocated: whole decoder layers in seven launches each; ..._attention_module_only: the attention module in five "
+               "launches inside the library's own decoder layer); "
                "per-layer = difference between the two layer counts; decoder = LlamaShapedDecoder.from_hf(...).generate (one HIP graph "
                "replayed per token); patched_attention_module = self_attn.forward of one layer alone at a fixed length",
     }

@@ -315,6 +315,7 @@ class HeavyHitterMixin:
         # single-token steps of a bf16 model on a cache that appends in place (cache.PreallocatedCache) take `_fast_decode`:
         # five launches for the whole module instead of ~25 library calls; set False to keep every step on the general path
         self.fast_decode = True
+        self.fast_layer = True      # ... and the decoder layer around this module as well (`fast_decoder_layer_forward`)
 
     def __repr__(self):
         return (f"{super().__repr__()}\nSparsification Setting(topk:{self.heavy_budget}  edge:{self.init_budget, self.recent_budget} "
@@ -567,10 +568,12 @@ class HeavyHitterMixin:
             return None
         return slot
 
-    def _fast_decode(self, hidden_states, position_embeddings, slot):
+    def _fast_decode(self, hidden_states, position_embeddings, slot, norm=None, residual=None):
         """The decode branch (reference :551-625) for one new token per sequence in five launches: fused QKV projection
         (ha_linear_skinny), rotary embedding + in-place cache append + both hashes (ha_rope_encode_step_cos_sin), distance
-        histograms, selection fused into the gather attention, output projection."""
+        histograms, selection fused into the gather attention, output projection.  For the decoder layer around it
+        (`fast_decoder_layer_forward`): `norm` = (weight, eps) of an RMSNorm applied to hidden_states inside the QKV projection,
+        `residual` [b, hidden] added inside the output projection."""
         b, _, hidden = hidden_states.shape
         H, Hkv, d = self.num_heads, self.num_key_value_heads, self.head_dim
         dev = hidden_states.device
@@ -580,7 +583,10 @@ class HeavyHitterMixin:
                       q=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev),
                       attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
             self.__dict__["_fast_scratch"] = sc
-        _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
+        if norm is None:
+            _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
+        else:
+            _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"], norm_weight=norm[0], eps=norm[1])
         kbuf, vbuf, pos = slot.append_slots(hidden_states, b, Hkv, d, 1)
         S = pos + 1
         hl = self._ensure_hash_layer(b, S, dev)
@@ -600,7 +606,7 @@ class HeavyHitterMixin:
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
-        _ops.linear_skinny(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden))
+        _ops.linear_skinny(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
 
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
@@ -795,6 +801,86 @@ class HeavyHitterMixin:
         st[3] = st[0] / st[2]
         st[4] = math.sqrt(max(st[1] / st[2] - st[3] ** 2, 0.0))
         self.last_overlap_ratio = r.permute(0, 2, 1)                                             # [b, H, q_len], for tests
+
+
+# ------------------------------------------------------------------------------------------ the decoder layer around it
+
+def _stacked_gate_up(attn, mlp) -> torch.Tensor:
+    """gate_proj and up_proj weights as one [2 F, hidden] matrix (gate rows, then up rows: what the projection kernel's
+    SwiGLU form reads); a copy, kept on the attention module and rebuilt when a parameter was replaced or updated in place
+    through its version counter."""
+    ws = (mlp.gate_proj.weight, mlp.up_proj.weight)
+    key = tuple((w.data_ptr(), w._version, w.dtype, w.device) for w in ws)
+    hit = attn.__dict__.get("_gate_up_fused")
+    if hit is None or hit[0] != key:
+        hit = (key, torch.cat([w.detach() for w in ws], dim=0).contiguous())
+        attn.__dict__["_gate_up_fused"] = hit
+    return hit[1]
+
+
+def _layer_takes_fast_path(layer, hidden_states) -> bool:
+    """A single-token step of up to 8 sequences through a decoder layer of the Llama shape in bf16: RMSNorm, attention,
+    residual, RMSNorm, SiLU-gated MLP without biases, residual; rows of at most 16384 elements (the projection kernel's
+    fused forms)."""
+    mlp, n1, n2 = getattr(layer, "mlp", None), getattr(layer, "input_layernorm", None), getattr(layer, "post_attention_layernorm", None)
+    if mlp is None or n1 is None or n2 is None or hidden_states.shape[0] > 8 or hidden_states.shape[1] != 1:
+        return False
+    lin = [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+    if any(not isinstance(m, nn.Linear) or m.bias is not None or m.weight.dtype != torch.bfloat16 for m in lin):
+        return False
+    act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
+    if not (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") or lin[0].out_features > 16384 or lin[0].in_features > 16384:
+        return False
+    for n in (n1, n2):
+        w = getattr(n, "weight", None)
+        if w is None or w.dtype != torch.bfloat16 or not hasattr(n, "variance_epsilon") or type(n).__name__.find("RMSNorm") < 0:
+            return False
+    return True
+
+
+def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
+                               position_embeddings=None, **kwargs):
+    """`forward` of a transformers decoder layer whose attention module was converted.  A single-token step that the attention
+    module takes in five launches (`_fast_decode_slot`) runs the WHOLE layer in seven: input RMSNorm inside the QKV
+    projection, the attention step, residual inside the output projection, post-attention RMSNorm in front of and SwiGLU
+    behind the stacked gate/up projection, residual inside the down projection (the launches of `LlamaShapedDecoder`) -
+    instead of the ~25 library calls of the layer's own forward, which at these sizes are bound by the host.  Everything
+    else goes to the layer's own forward.  Outputs differ from it by bf16 roundings (one rounding per RMSNorm instead of
+    two, other summation orders)."""
+    attn = layer.self_attn
+    cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
+    if getattr(attn, "fast_layer", False) and not kwargs.get("output_attentions") and _layer_takes_fast_path(layer, hidden_states):
+        attn.ensure_gpu(cache, hidden_states.device)
+        attn._sync_bit_cache(cache)
+        slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
+        if slot is not None:
+            b, _, hidden = hidden_states.shape
+            n1, n2, mlp = layer.input_layernorm, layer.post_attention_layernorm, layer.mlp
+            x1, _ = attn._fast_decode(hidden_states, position_embeddings, slot, norm=(n1.weight, float(n1.variance_epsilon)),
+                                      residual=hidden_states[:, 0, :])
+            attn._note_key_storage(cache)
+            act = attn.__dict__.get("_fast_act")
+            if act is None or act.shape != (b, mlp.gate_proj.out_features) or act.device != hidden_states.device:
+                act = torch.empty(b, mlp.gate_proj.out_features, dtype=torch.bfloat16, device=hidden_states.device)
+                attn.__dict__["_fast_act"] = act
+            _ops.linear_skinny(x1[:, 0, :], _stacked_gate_up(attn, mlp), act, norm_weight=n2.weight, eps=float(n2.variance_epsilon),
+                               swiglu=True)
+            out = torch.empty_like(x1)
+            _ops.linear_skinny(act, mlp.down_proj.weight, out[:, 0, :], residual=x1[:, 0, :])
+            return out
+    return layer._hf_forward(hidden_states, attention_mask=attention_mask, position_ids=position_ids, past_key_values=past_key_values,
+                             use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+
+
+def install_fast_layers(model):
+    """Route the decoder layers that hold a converted attention module through `fast_decoder_layer_forward`."""
+    import types
+    for layer in model.modules():
+        attn = getattr(layer, "self_attn", None)
+        if isinstance(attn, HeavyHitterMixin) and "_hf_forward" not in layer.__dict__ and hasattr(layer, "mlp"):
+            layer.__dict__["_hf_forward"] = layer.forward
+            layer.forward = types.MethodType(fast_decoder_layer_forward, layer)
+    return model
 
 
 # ------------------------------------------------------------------------------------------ module-patch helpers

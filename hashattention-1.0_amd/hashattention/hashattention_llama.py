@@ -15,7 +15,7 @@ import torch
 from torch import nn
 from transformers.models.llama.modeling_llama import LlamaAttention, apply_rotary_pos_emb
 
-from ._patched import (DEFAULT_USA_CFG, USA, HeavyHitterMixin, SignSTE, build_usa_modules, convert_modules,
+from ._patched import (DEFAULT_USA_CFG, USA, HeavyHitterMixin, SignSTE, build_usa_modules, convert_modules, install_fast_layers,
                        memory_efficient_softmax, ste_sign, walk)
 
 __all__ = ["USA", "LlamaAttention_heavy_hitter", "load_usa", "convert_usa", "reset_usa", "set_train_usa_mode",
@@ -57,7 +57,8 @@ def load_usa(config, path):
 
 def convert_usa(model, config, usa_modules, collect_stats, train_usa):
     """Replace every `LlamaAttention` of `model` in place by a `LlamaAttention_heavy_hitter` sharing its weights."""
-    return convert_modules(model, config, usa_modules, collect_stats, train_usa, LlamaAttention, LlamaAttention_heavy_hitter)
+    return install_fast_layers(convert_modules(model, config, usa_modules, collect_stats, train_usa, LlamaAttention,
+                                              LlamaAttention_heavy_hitter))
 
 
 def reset_usa(model):

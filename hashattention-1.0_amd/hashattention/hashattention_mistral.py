@@ -9,7 +9,7 @@ import torch
 from torch import nn
 from transformers.models.mistral.modeling_mistral import MistralAttention, apply_rotary_pos_emb
 
-from ._patched import (DEFAULT_USA_CFG, USA, HeavyHitterMixin, SignSTE, build_usa_modules, convert_modules,
+from ._patched import (DEFAULT_USA_CFG, USA, HeavyHitterMixin, SignSTE, build_usa_modules, convert_modules, install_fast_layers,
                        memory_efficient_softmax, ste_sign, walk)
 
 __all__ = ["USA", "MistralAttention_heavy_hitter", "load_usa", "convert_usa", "reset_usa", "set_train_usa_mode",
@@ -48,7 +48,8 @@ def load_usa(config, path):
 
 
 def convert_usa(model, config, usa_modules, collect_stats, train_usa):
-    return convert_modules(model, config, usa_modules, collect_stats, train_usa, MistralAttention, MistralAttention_heavy_hitter)
+    return install_fast_layers(convert_modules(model, config, usa_modules, collect_stats, train_usa, MistralAttention,
+                                              MistralAttention_heavy_hitter))
 
 
 def reset_usa(model):

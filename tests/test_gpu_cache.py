@@ -12,9 +12,11 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _model(fast_decode=False):
+def _model(fast_decode=False, **usa_cfg):
     torch.manual_seed(0)
     cfg = _config(LlamaConfig)
+    for k, v in usa_cfg.items():
+        setattr(cfg, k, v)
     model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
     usa = hl.load_usa(cfg, None)
     model = hl.convert_usa(model, cfg, usa, collect_stats=False, train_usa=False)
@@ -92,12 +94,20 @@ def test_static_cache_under_the_patched_layers():
         assert (g - w).abs().max().item() < 2e-2, (g - w).abs().max().item()
 
 
-def test_single_token_steps_in_five_launches_match_the_general_path():
+@pytest.mark.parametrize("whole_layer", [False, True])
+def test_single_token_steps_in_five_launches_match_the_general_path(whole_layer):
     # on a PreallocatedCache a bf16 model's single-token steps run as fused QKV projection, rotary + in-place append + hashes,
     # histograms, select-attend, output projection; the general path (library projections, torch rotary embedding,
-    # cache.update) must give the same logits up to bf16 rounding of different summation orders, and the same greedy tokens
-    print("\n[case] five-launch single-token path vs general path", flush=True)
-    cfg, model = _model(fast_decode=False)
+    # cache.update) must give the same logits up to bf16 rounding of different summation orders, and the same greedy tokens.
+    # whole_layer: the decoder layer around the attention module in the same style (norms and residuals inside the
+    # projections, stacked gate/up projection with SwiGLU behind it): seven launches per layer
+    print(f"\n[case] five-launch single-token path vs general path, whole layer: {whole_layer}", flush=True)
+    # the whole-layer path rounds its norms once where the library rounds twice: queries and keys differ in their last bf16
+    # digit, a few hash bits flip and with them a few selected tokens - so its logits and greedy tokens are compared with
+    # every candidate selected (heavy budget = all), where only the arithmetic differs
+    cfg, model = _model(fast_decode=False, **(dict(heavy_budget=0.999) if whole_layer else {}))
+    for layer in model.model.layers:
+        layer.self_attn.fast_layer = whole_layer
     ids = torch.randint(0, cfg.vocab_size, (3, 260), generator=torch.Generator().manual_seed(4)).to(DEV)
     steps = [1, 1, 1, 6, 1, 1]                  # single tokens, a chunk (general path), single tokens again
     want = _decode(model, ids, PreallocatedCache(capacity=300), steps)
@@ -108,6 +118,7 @@ def test_single_token_steps_in_five_launches_match_the_general_path():
     cache = PreallocatedCache(capacity=300)
     got = _decode(model, ids, cache, steps)
     assert all("_fast_scratch" in layer.self_attn.__dict__ for layer in model.model.layers), "the fast path was not taken"
+    assert all(("_fast_act" in layer.self_attn.__dict__) == whole_layer for layer in model.model.layers)
     assert cache.get_seq_length() == 260 and cache.layers[0].keys.shape[2] == 260
     worst = max((g - w).abs().max().item() for g, w in zip(got, want))
     scale = max(w.abs().max().item() for w in want)
@@ -188,9 +199,10 @@ def test_rope_encode_step_with_cos_sin_tables_matches_torch_bit_for_bit():
 def test_mistral_takes_the_five_launch_step_too():
     from transformers import MistralConfig, MistralForCausalLM
     from hashattention import hashattention_mistral as hm
-    print("\n[case] five-launch single-token path, Mistral", flush=True)
+    print("\n[case] five-launch single-token path and whole-layer path, Mistral", flush=True)
     torch.manual_seed(0)
     cfg = _config(MistralConfig, sliding_window=None)
+    cfg.heavy_budget = 0.999           # every candidate selected: the paths differ by arithmetic only (see the Llama test above)
     model = MistralForCausalLM(cfg).bfloat16().to(DEV)
     model = hm.convert_usa(model, cfg, hm.load_usa(cfg, None), collect_stats=False, train_usa=False)
     ids = torch.randint(0, cfg.vocab_size, (2, 220), generator=torch.Generator().manual_seed(6)).to(DEV)
@@ -202,7 +214,7 @@ def test_mistral_takes_the_five_launch_step_too():
     for layer in model.model.layers:
         layer.self_attn.fast_decode = True
     got = _decode(model, ids, PreallocatedCache(capacity=256), steps)
-    assert all("_fast_scratch" in layer.self_attn.__dict__ for layer in model.model.layers)
+    assert all("_fast_scratch" in layer.self_attn.__dict__ and "_fast_act" in layer.self_attn.__dict__ for layer in model.model.layers)
     worst = max((g - w).abs().max().item() for g, w in zip(got, want))
     scale = max(w.abs().max().item() for w in want)
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)

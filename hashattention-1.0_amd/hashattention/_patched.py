@@ -828,6 +828,10 @@ def _layer_takes_fast_path(layer, hidden_states) -> bool:
     lin = [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
     if any(not isinstance(m, nn.Linear) or m.bias is not None or m.weight.dtype != torch.bfloat16 for m in lin):
         return False
+    # hooks on the modules this path does not call (activation capture, adapters that wrap a forward) keep the library's layer
+    for m in (layer.self_attn, mlp, n1, n2, *lin):
+        if m._forward_hooks or m._forward_pre_hooks:
+            return False
     act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
     if not (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") or lin[0].out_features > 16384 or lin[0].in_features > 16384:
         return False

@@ -267,3 +267,22 @@ def test_beam_search_gives_the_tokens_of_a_run_that_rehashes_every_step(kind):
     hl.reset_usa(model)
     got = model.generate(ids, past_key_values=make(), **kw)
     assert torch.equal(got, want)
+
+
+def test_hooks_on_the_layers_modules_keep_the_librarys_decoder_layer():
+    # the whole-layer path calls neither `mlp.forward` nor the norms: a forward hook on one of them must keep firing
+    print("\n[case] forward hook on the MLP of a converted layer", flush=True)
+    cfg, model = _model(fast_decode=True)
+    ids = torch.randint(0, cfg.vocab_size, (2, 150), generator=torch.Generator().manual_seed(7)).to(DEV)
+    cache = PreallocatedCache(capacity=200)
+    seen = []
+    hook = model.model.layers[1].mlp.register_forward_hook(lambda m, a, o: seen.append(o.shape))
+    with torch.no_grad():
+        model(ids[:, :140], past_key_values=cache, use_cache=True)
+        model(ids[:, 140:141], past_key_values=cache, use_cache=True)
+    assert len(seen) == 2 and seen[1] == (2, 1, cfg.hidden_size)
+    assert "_fast_act" in model.model.layers[0].self_attn.__dict__ and "_fast_act" not in model.model.layers[1].self_attn.__dict__
+    hook.remove()
+    with torch.no_grad():
+        model(ids[:, 141:142], past_key_values=cache, use_cache=True)
+    assert len(seen) == 2 and "_fast_act" in model.model.layers[1].self_attn.__dict__

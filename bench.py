@@ -296,7 +296,8 @@ def hf_path_bench(args, torch):
     from hashattention.cache import PreallocatedCache
     from hashattention.decoder import LlamaShapedDecoder
     from hashattention.synthetic import named_workload
-    w = named_workload("config3")
+    shape = args.config if args.config in ("config2", "config3") else "config3"     # config2: 16 sequences of 65536 tokens
+    w = named_workload(shape)
     B, S = w.batch, w.max_seq_len
     dev = "cuda:0"
     steps, warm = max(8, min(args.steps, 64)), 3
@@ -394,7 +395,7 @@ def hf_path_bench(args, torch):
         "metric": "decode_ms_per_token_patched_transformers_model", "value": hi["patched_preallocated_ms"], "unit": "ms/token-step",
         "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": hi["patched_preallocated_ms"], "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"config3 through the drop-in API: transformers Llama (hidden 4096, ffn 14336, 32/8 heads, vocab 128256), "
+        "config": {"workload": f"{shape} through the drop-in API: transformers Llama (hidden 4096, ffn 14336, 32/8 heads, vocab 128256), "
                                f"{L_full} layers, load_usa(config, None) + convert_usa, B={B} context={S}, one key-side hash MLP per query "
                                f"head (fp32 modules), init={w.init_budget} recent={w.recent_budget} heavy={w.heavy_budget:g}"},
         "layers": {str(k): v for k, v in out.items()},
@@ -670,7 +671,7 @@ def main():
         print("bench.py needs a GPU: the HashAttention path has no CPU fallback", file=sys.stderr)
         sys.exit(2)
     _ops.load_library()
-    if args.config == "config3" and args.hf_path:
+    if args.config in ("config2", "config3") and args.hf_path:
         print(json.dumps(hf_path_bench(args, torch)))
         return
     if args.config == "config3" and not args.layer_only:

@@ -539,6 +539,8 @@ class HeavyHitterMixin:
             return None
         if self.q_proj.bias is not None or self.o_proj.bias is not None or self.q_proj.weight.dtype != torch.bfloat16:
             return None
+        if self.q_proj.weight.device != hidden_states.device:       # a model spread over devices: its own hooks move the inputs
+            return None
         usa = self.usa_module
         if usa is None or usa.rehash_every_step or getattr(cache, "offloading", False):
             return None

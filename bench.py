@@ -298,7 +298,7 @@ def hf_path_bench(args, torch):
     from hashattention.synthetic import named_workload
     shape = args.config if args.config in ("config2", "config3") else "config3"     # config2: 16 sequences of 65536 tokens
     w = named_workload(shape)
-    B, S = w.batch, w.max_seq_len
+    B, S = (args.batch or w.batch), w.max_seq_len
     dev = "cuda:0"
     steps, warm = max(8, min(args.steps, 64)), 3
 

@@ -155,7 +155,15 @@ def _check(status: int, where: str):
         raise HashAttnError(status, where, load_library().ha_last_error_string().decode())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor):
+    """The current stream of t's device as the hipStream_t the library takes.  Through torch's raw-handle accessor where
+    there is one: building a `torch.cuda.Stream` object per launch costs ~5 us, a fifth of what a decode layer's launches
+    cost the host."""
+    if _raw_stream is not None:
+        return C.c_void_p(_raw_stream(t.device.index))
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 

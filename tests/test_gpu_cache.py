@@ -286,3 +286,14 @@ def test_hooks_on_the_layers_modules_keep_the_librarys_decoder_layer():
     with torch.no_grad():
         model(ids[:, 141:142], past_key_values=cache, use_cache=True)
     assert len(seen) == 2 and "_fast_act" in model.model.layers[1].self_attn.__dict__
+
+
+def test_ops_launch_on_torchs_current_stream():
+    # the binding takes the current stream's raw handle from torch without building a Stream object per launch
+    from hashattention import _ops
+    t = torch.zeros(1, device=DEV)
+    assert (_ops._stream(t).value or 0) == torch.cuda.current_stream(DEV).cuda_stream
+    side = torch.cuda.Stream(device=DEV)
+    with torch.cuda.stream(side):
+        assert _ops._stream(t).value == side.cuda_stream
+    assert (_ops._stream(t).value or 0) == torch.cuda.current_stream(DEV).cuda_stream

@@ -10,7 +10,8 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// y[m, n] = sum_k x[m, k] W[n, k] (+ res[m, n]), bf16 in, fp32 accumulate, bf16 out, M <= 16.  HBM-bound on W
+// y[m, n] = sum_k x[m, k] W[n, k] (+ res[m, n]), bf16 in, fp32 accumulate, bf16 out, M <= 16 (with a residual the product is
+// rounded to bf16 before the addition, as a Linear followed by `x + h` rounds it: efficiency/model.py:190-191).  HBM-bound on W
 // (2 N K bytes, read once).  One workgroup owns 16 consecutive output columns n; its NWAVE waves split K.  A wave
 // feeds v_mfma_f32_16x16x32_bf16 with A = the 16 rows of W (lane: row l % 16, 8 consecutive k at 8 (l / 16)) and
 // B = x^T padded to 16 columns, so a wave load brings 64 contiguous bytes of each of the 16 rows and two consecutive
@@ -53,8 +54,9 @@ template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
-// FUSE bit 0: RMSNorm of x in front (x <- bf16(x * rsqrt(mean x^2 + eps) * norm_w), the rounding of a separate norm
-// launch): every workgroup holds all of x, so it norms it itself.  FUSE bit 1: SwiGLU behind (W = [gate rows; up rows],
+// FUSE bit 0: RMSNorm of x in front, x <- bf16(bf16(x * rsqrt(mean x^2 + eps)) * norm_w): the two roundings of the RMSNorm
+// modules this replaces (transformers' LlamaRMSNorm, and efficiency/model.py:314-319 of the reference's harness: the
+// normalised row is cast to the input type before it meets the weight).  Every workgroup holds all of x, so it norms it itself.  FUSE bit 1: SwiGLU behind (W = [gate rows; up rows],
 // N = 2 F): a workgroup owns RB / 2 gate rows and the RB / 2 up rows of the same columns and writes
 // bf16(bf16(silu(bf16 gate)) * bf16 up) to out [M, F], the roundings of a separate activation launch.
 template <int NWAVE, int XCH, int R, int MM, int FUSE>
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
                 uint32_t *p = reinterpret_cast<uint32_t *>(&xr[c][m]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float lo = __uint_as_float(p[i] << 16) * rstd[m] * __uint_as_float(g[i] << 16);
-                    const float hi = __uint_as_float(p[i] & 0xffff0000u) * rstd[m] * __uint_as_float(g[i] & 0xffff0000u);
+                    const float lo = ha_round_bf16(__uint_as_float(p[i] << 16) * rstd[m]) * __uint_as_float(g[i] << 16);
+                    const float hi = ha_round_bf16(__uint_as_float(p[i] & 0xffff0000u) * rstd[m]) * __uint_as_float(g[i] & 0xffff0000u);
                     p[i] = ha_f32_to_bf16_bits(lo) | (ha_f32_to_bf16_bits(hi) << 16);
                 }
             }
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
             for (int o = tid; o < nrows * M; o += NWAVE * 64) {
                 const int m = o / nrows, r = o % nrows;  // consecutive threads write consecutive columns of y
                 float y = total(r, m);
-                if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + r] << 16);
+                if (res) y = ha_round_bf16(y) + __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + r] << 16);  // the Linear's rounding, then the addition's
                 out[(int64_t)m * out_sm + n0 + r] = (uint16_t)ha_f32_to_bf16_bits(y);
             }
         }
@@ -286,7 +288,7 @@ __global__ __launch_bounds__(NWAVE * 64) void skinny_linear_kernel(const uint16_
         float y = 0.f;
 #pragma unroll
         for (int wv = 0; wv < NWAVE; ++wv) y += s_c[wv][nl][m];
-        if (res) y += __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + nl] << 16);
+        if (res) y = ha_round_bf16(y) + __uint_as_float((uint32_t)res[(int64_t)m * res_sm + n0 + nl] << 16);  // the Linear's rounding, then the addition's
         out[(int64_t)m * out_sm + n0 + nl] = (uint16_t)ha_f32_to_bf16_bits(y);
     }
 }

@@ -428,7 +428,8 @@ int ha_rope_encode_step_cos_sin(const void *qkv, int64_t qkv_stride_b, int x_dty
                                 uint32_t *qcodes, void *stream);
 /*
  * out[m, n] = sum_k x[m, k] * w[n, k] (+ residual[m, n]): a Linear layer (weight [N, K] as nn.Linear keeps it) applied to
- * M <= 16 rows, bf16 in and out, fp32 accumulation.  The decode step's projections (efficiency/model.py:236, 261,
+ * M <= 16 rows, bf16 in and out, fp32 accumulation; with a residual the product is rounded to bf16 before the addition
+ * and the sum rounded again, as `x + linear(h)` rounds (efficiency/model.py:190-191).  The decode step's projections (efficiency/model.py:236, 261,
  * 304-305: wqkv, wo, w1/w3, w2, and the lm_head of :158) are this shape: they stream every weight once per token, so
  * the kernel is bound by HBM.  K must be a multiple of 32, rows 16-byte aligned; strides in elements.
  */
@@ -436,9 +437,10 @@ int ha_linear_skinny(const void *x, int64_t x_stride_m, const void *w, int64_t w
                      const void *residual, int64_t residual_stride_m, void *out, int64_t out_stride_m,
                      int M, int N, int K, void *stream);
 /*
- * The same product with the neighbouring elementwise steps of the decoder layer folded in (efficiency/model.py:88-96
+ * The same product with the neighbouring elementwise steps of the decoder layer folded in (efficiency/model.py:308-319
  * RMSNorm, :261 feed-forward `w2(silu(w1 x) * w3 x)`):
- *   norm_weight != NULL  x is RMS-normalised first: x <- bf16(x * rsqrt(mean_k x^2 + eps) * norm_weight[k]);
+ *   norm_weight != NULL  x is RMS-normalised first: x <- bf16(bf16(x * rsqrt(mean_k x^2 + eps)) * norm_weight[k]), the two
+ *                        roundings of the module it replaces (efficiency/model.py:314-319; transformers' LlamaRMSNorm);
  *   act == HA_ACT_SWIGLU w holds F gate rows followed by F up rows (N = 2 F); out [M, F] = silu(gate) * up with the
  *                        roundings of ha_swiglu on a bf16 gate/up buffer; no residual.
  * Both need M <= 8 and K <= 16384 (the row-streaming kernel).  With norm_weight == NULL and act == HA_ACT_NONE this is

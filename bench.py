@@ -366,6 +366,16 @@ def hf_path_bench(args, torch):
             ms_attn = time_gpu(attn_only, steps, warm, torch)
         del cache
         hl.reset_usa(model)
+        # a cache that the caller (or `generate`) created as the library's DynamicCache: taken over in place at the first decode
+        # step (the default), and left to the library (one torch.cat of every layer's whole cache per token)
+        dyn = DynamicCache()
+        fill(dyn, L, S - 1 - warm)
+        ms_adopted, _ = time_tokens(model, dyn, steps, warm)
+        del dyn
+        hl.reset_usa(model)
+        torch.cuda.empty_cache()
+        for lyr in model.model.layers:
+            lyr.self_attn.adopt_cache = False
         dyn = DynamicCache()
         fill(dyn, L, S - 1 - 2)
         ms_dyn, _ = time_tokens(model, dyn, 4, 2)
@@ -384,7 +394,8 @@ def hf_path_bench(args, torch):
             torch.cuda.synchronize()
         ms_dec = e0.elapsed_time(e1) / steps
         out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre,
-                      patched_preallocated_attention_module_only_ms=ms_attn_fast, patched_dynamic_cache_ms=ms_dyn,
+                      patched_preallocated_attention_module_only_ms=ms_attn_fast, patched_dynamic_cache_adopted_ms=ms_adopted,
+                      patched_dynamic_cache_ms=ms_dyn,
                       decoder_generate_ms=ms_dec, patched_attention_module_us=ms_attn * 1e3)
         del dec, model, usa
         torch.cuda.empty_cache()
@@ -402,7 +413,9 @@ def hf_path_bench(args, torch):
         "per_layer_slope": per_layer,
         "how": "single-token forward passes of the patched model, eager launches from Python, HIP events around the timed passes "
                "(patched_preallocated: whole decoder layers in seven launches each; ..._attention_module_only: the attention module in five "
-               "launches inside the library's own decoder layer); "
+               "launches inside the library's own decoder layer; patched_dynamic_cache_adopted: the caller hands over a plain DynamicCache, "
+               "whose layers the attention modules turn into in-place ones at the first decode step; patched_dynamic_cache: the same "
+               "with that switched off, torch.cat per layer and token); "
                "per-layer = difference between the two layer counts; decoder = LlamaShapedDecoder.from_hf(...).generate (one HIP graph "
                "replayed per token); patched_attention_module = self_attn.forward of one layer alone at a fixed length",
     }

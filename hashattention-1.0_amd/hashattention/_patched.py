@@ -29,7 +29,7 @@ import torch
 from torch import nn
 
 from . import _ops
-from .cache import PreallocatedLayer
+from .cache import PreallocatedLayer, adopt_dynamic_layer
 from .decode import HashDecodeLayer
 
 DECODE_MAX_Q_LEN = 128   # reference: `if q_len > 128 or self.train_usa` routes to the original forward (:529)
@@ -314,6 +314,7 @@ class HeavyHitterMixin:
         self._cache_id = None
         # single-token steps of a bf16 model on a cache that appends in place (cache.PreallocatedCache) take `_fast_decode`:
         # five launches for the whole module instead of ~25 library calls; set False to keep every step on the general path
+        self.adopt_cache = True     # a plain DynamicLayer of the caller's cache is turned into one that appends in place
         self.fast_decode = True
         self.fast_layer = True      # ... and the decoder layer around this module as well (`fast_decoder_layer_forward`)
 
@@ -611,9 +612,24 @@ class HeavyHitterMixin:
         _ops.linear_skinny(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
 
+    def _adopt_cache_layer(self, cache) -> None:
+        """Before a decode step: this layer's part of a cache that `generate` (or the caller) created as a plain `DynamicCache`
+        becomes a `PreallocatedLayer` in place (`cache.adopt_dynamic_layer`), so that neither this step nor any later one
+        re-copies the layer's cache - and single-token steps can take the few-launch paths.  Not for offloaded caches, whose
+        owner moves the tensors around."""
+        if not self.adopt_cache or cache is None or getattr(cache, "offloading", False) or self.offloading_length is not None:
+            return
+        layers = getattr(cache, "layers", None)
+        if layers is not None and len(layers) > self.layer_idx and not isinstance(layers[self.layer_idx], PreallocatedLayer):
+            known = self._holds_known_keys(cache)
+            if adopt_dynamic_layer(layers[self.layer_idx]) and known:
+                self._note_key_storage(cache)       # the same contents under their new description
+
     def _heavy_hitter_forward(self, hidden_states, position_embeddings, attention_mask, cache, **kwargs):
         bsz, q_len, _ = hidden_states.shape
         self.ensure_gpu(cache, hidden_states.device)
+        if q_len <= DECODE_MAX_Q_LEN and not self.train_usa:
+            self._adopt_cache_layer(cache)
         self._sync_bit_cache(cache)
         if q_len == 1 and not kwargs.get("output_attentions"):
             slot = self._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
@@ -857,6 +873,8 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
     cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
     if getattr(attn, "fast_layer", False) and not kwargs.get("output_attentions") and _layer_takes_fast_path(layer, hidden_states):
         attn.ensure_gpu(cache, hidden_states.device)
+        if not attn.train_usa:
+            attn._adopt_cache_layer(cache)
         attn._sync_bit_cache(cache)
         slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
         if slot is not None:

@@ -29,6 +29,7 @@ class PreallocatedLayer(DynamicLayer):
 
     default_capacity = 0
     growth = 2.0
+    min_growth = 0
 
     def __init__(self, capacity: Optional[int] = None, **kwargs):
         self._kbuf = self._vbuf = None
@@ -67,7 +68,7 @@ class PreallocatedLayer(DynamicLayer):
         have = 0 if self._kbuf is None else self._kbuf.shape[-2]
         if self._kbuf is not None and self._vbuf is not None and need <= have and self._kbuf.device == key_states.device:
             return
-        cap = max(need, self.capacity_hint, int(have * self.growth))
+        cap = max(need, self.capacity_hint, int(have * self.growth), have + self.min_growth if have else 0)
         b, h, _, dk = key_states.shape
         kbuf = torch.empty(b, h, cap, dk, dtype=key_states.dtype, device=key_states.device)
         vbuf = torch.empty(b, h, cap, value_states.shape[-1], dtype=value_states.dtype, device=value_states.device)
@@ -119,6 +120,29 @@ class PreallocatedLayer(DynamicLayer):
     @property
     def capacity(self) -> int:
         return 0 if self._kbuf is None else int(self._kbuf.shape[-2])
+
+
+def adopt_dynamic_layer(layer) -> bool:
+    """Turn a plain `DynamicLayer` that already holds tokens into a `PreallocatedLayer` IN PLACE: same object, same tensors
+    (they become its buffers, full to the brim, so the next append allocates the usual doubled capacity once), same behaviour
+    towards the cache that owns it - but later appends copy only the new tokens.  This is how a cache that `generate` created
+    on its own (`DynamicCache`, one `torch.cat` of the layer's whole cache per token) is taken over by the converted attention
+    modules.  Only the exact class is taken: sliding-window, quantized or static layers keep their own logic.  Returns
+    whether the layer is a `PreallocatedLayer` afterwards."""
+    if isinstance(layer, PreallocatedLayer):
+        return True
+    if type(layer) is not DynamicLayer or not getattr(layer, "is_initialized", False):
+        return False
+    k, v = layer.__dict__.get("keys"), layer.__dict__.get("values")
+    if not isinstance(k, torch.Tensor) or not isinstance(v, torch.Tensor) or k.dim() != 4 or v.dim() != 4 or k.shape[-2] == 0:
+        return False
+    del layer.__dict__["keys"], layer.__dict__["values"]       # the names are properties of the new class
+    layer.__class__ = PreallocatedLayer
+    layer._kbuf, layer._vbuf, layer._len = k, v, int(k.shape[-2])
+    layer.capacity_hint = 0
+    layer.growth, layer.min_growth = 1.25, 256      # nobody said how long this cache will get: a quarter more room at a time
+    layer.epoch = 0
+    return True
 
 
 class PreallocatedCache(DynamicCache):

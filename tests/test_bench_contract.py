@@ -47,6 +47,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     hf = d["patched_transformers_model_config3"]
     assert hf["ms_per_token_step"] > 0 and "patched_preallocated_us_per_layer" in hf["per_layer_slope"]
     assert "patched_preallocated_attention_module_only_us_per_layer" in hf["per_layer_slope"]
+    assert hf["per_layer_slope"]["patched_dynamic_cache_adopted_us_per_layer"] < 0.5 * hf["per_layer_slope"]["patched_dynamic_cache_us_per_layer"]
     assert d["paged_cache_identity_table"]["same_bits_as_unpaged"] is True
     for rows in ("rows_8", "rows_64"):
         assert 0.2 < d["chunked_decode"][rows]["gather_hbm_frac_of_whole_chunk_step"] < 1.0

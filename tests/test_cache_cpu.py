@@ -3,7 +3,7 @@ it replaces - same keys / values after every update, crop, batch selection and r
 import torch
 from transformers import DynamicCache
 
-from hashattention.cache import PreallocatedCache, PreallocatedLayer
+from hashattention.cache import PreallocatedCache, PreallocatedLayer, adopt_dynamic_layer
 
 
 def _states(g, b, h, t, d=8):
@@ -112,3 +112,29 @@ def test_models_with_other_head_widths_are_refused_before_anything_is_patched():
     with pytest.raises(NotImplementedError, match="128-wide heads"):
         hl.convert_usa(model, cfg, [None], collect_stats=False, train_usa=False)
     assert type(model.model.layers[0].self_attn) is before
+
+
+def test_a_dynamic_layer_is_adopted_in_place():
+    from transformers.cache_utils import DynamicLayer, DynamicSlidingWindowLayer
+    g = torch.Generator().manual_seed(4)
+    ref, got = DynamicCache(), DynamicCache()
+    for t in (6, 1):
+        k, v = _states(g, 2, 2, t)
+        ref.update(k, v, 0)
+        got.update(k, v, 0)
+    layer = got.layers[0]
+    assert type(layer) is DynamicLayer and adopt_dynamic_layer(layer) and got.layers[0] is layer
+    assert isinstance(layer, PreallocatedLayer) and layer.get_seq_length() == 7 and layer.capacity == 7 and layer.epoch == 0
+    assert "keys" not in layer.__dict__ and torch.equal(layer.keys, ref.layers[0].keys)
+    for t in (1, 1, 3):                                            # grows by a quarter (at least 256 tokens), then appends in place
+        k, v = _states(g, 2, 2, t)
+        a, b = got.update(k, v, 0)
+        c, d = ref.update(k, v, 0)
+        assert torch.equal(a, c) and torch.equal(b, d)
+    assert layer.capacity == 7 + 256 and got.get_seq_length() == 12
+    ptr = layer._kbuf.data_ptr()
+    got.update(*_states(g, 2, 2, 1), 0)
+    assert layer._kbuf.data_ptr() == ptr
+    # other layer kinds, and layers that hold nothing yet, are left alone
+    assert not adopt_dynamic_layer(DynamicLayer()) and not adopt_dynamic_layer(DynamicSlidingWindowLayer(sliding_window=4))
+    assert adopt_dynamic_layer(layer)                              # already one

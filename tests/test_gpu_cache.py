@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _model(fast_decode=False, **usa_cfg):
+def _model(fast_decode=False, adopt_cache=False, **usa_cfg):
     torch.manual_seed(0)
     cfg = _config(LlamaConfig)
     for k, v in usa_cfg.items():
@@ -22,6 +22,7 @@ def _model(fast_decode=False, **usa_cfg):
     model = hl.convert_usa(model, cfg, usa, collect_stats=False, train_usa=False)
     for layer in model.model.layers:        # the five-launch single-token path has a test of its own below
         layer.self_attn.fast_decode = fast_decode
+        layer.self_attn.adopt_cache = adopt_cache       # off: a DynamicCache stays what the library made it
     return cfg, model
 
 
@@ -295,3 +296,50 @@ def test_ops_launch_on_torchs_current_stream():
     with torch.cuda.stream(side):
         assert _ops._stream(t).value == side.cuda_stream
     assert (_ops._stream(t).value or 0) == torch.cuda.current_stream(DEV).cuda_stream
+
+
+@pytest.mark.parametrize("fast", [False, True])
+def test_a_cache_that_generate_made_itself_is_taken_over_in_place(fast):
+    # nothing but `model.generate(ids)`, as the reference's README runs it: transformers creates a DynamicCache, whose layers
+    # re-copy their whole cache per token; at the first decode step every converted attention module turns its layer of that
+    # cache into one that appends in place (same object, same tensors).  Same tokens as with the library's own layers.
+    print(f"\n[case] DynamicCache adopted in place, few-launch steps: {fast}", flush=True)
+    cfg, model = _model(fast_decode=fast, adopt_cache=False)
+    ids = torch.randint(0, cfg.vocab_size, (2, 150), generator=torch.Generator().manual_seed(8)).to(DEV)
+    kw = dict(max_new_tokens=12, do_sample=False, pad_token_id=0, return_dict_in_generate=True)
+    want = model.generate(ids, **kw)
+    from transformers.cache_utils import DynamicLayer
+    assert all(type(l) is DynamicLayer for l in want.past_key_values.layers)
+    for layer in model.model.layers:
+        layer.self_attn.adopt_cache = True
+    hl.reset_usa(model)
+    got = model.generate(ids, **kw)
+    assert torch.equal(got.sequences, want.sequences)
+    cache = got.past_key_values
+    assert type(cache) is DynamicCache and all(isinstance(l, PreallocatedLayer) for l in cache.layers)
+    assert cache.get_seq_length() == 150 + 12 - 1 and cache.layers[0].capacity > cache.get_seq_length()
+    # (the few-launch steps differ from the general path by bf16 roundings of other summation orders)
+    close = (lambda x, y: torch.equal(x, y)) if not fast else (lambda x, y: (x.float() - y.float()).abs().max().item() <= 3e-2)
+    assert close(cache.layers[1].keys, want.past_key_values.layers[1].keys)
+    # the caller's own DynamicCache, continued over two calls, cropped and reordered in between
+    own = DynamicCache()
+    with torch.no_grad():
+        model(ids[:, :140], past_key_values=own, use_cache=True)
+        a = model(ids[:, 140:141], past_key_values=own, use_cache=True).logits
+        assert isinstance(own.layers[0], PreallocatedLayer)
+        ptr = own.layers[0]._kbuf.data_ptr()
+        model(ids[:, 141:142], past_key_values=own, use_cache=True)
+        assert own.layers[0]._kbuf.data_ptr() == ptr            # appended in place
+        own.crop(-1)
+        own.reorder_cache(torch.tensor([1, 0], device=DEV))
+        b = model(ids[[1, 0], 141:142], past_key_values=own, use_cache=True).logits
+    ref = DynamicCache()
+    for layer in model.model.layers:
+        layer.self_attn.adopt_cache = False
+    hl.reset_usa(model)
+    with torch.no_grad():
+        model(ids[:, :140], past_key_values=ref, use_cache=True)
+        a_ref = model(ids[:, 140:141], past_key_values=ref, use_cache=True).logits
+        ref.reorder_cache(torch.tensor([1, 0], device=DEV))
+        b_ref = model(ids[[1, 0], 141:142], past_key_values=ref, use_cache=True).logits
+    assert close(a, a_ref) and close(b, b_ref)

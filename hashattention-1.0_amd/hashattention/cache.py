@@ -11,6 +11,9 @@ Everything else (`get_seq_length`, mask sizes, `crop`, beam reordering, offloadi
     cache = PreallocatedCache(capacity=prompt_len + max_new_tokens)
     out = model.generate(**inputs, past_key_values=cache, max_new_tokens=...)
 
+A caller who passes a plain `DynamicCache` (or none, so that `generate` makes one) needs to do nothing: the converted
+attention modules turn their layer of it into a `PreallocatedLayer` in place at the first decode step (`adopt_dynamic_layer`).
+
 `StaticCache` works with the patched layers as well (they take the number of valid tokens from the cache, not from the
 shape of the returned tensors), at the price of one device-to-host read of its length per layer and step.
 """

@@ -528,10 +528,10 @@ class HeavyHitterMixin:
         return hit[1]
 
     def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
-        """This layer's `PreallocatedLayer` of `cache` when the step can take `_fast_decode`, else None: one new token per
-        sequence, inference, bf16 hidden states and projections without biases, 128-wide heads, up to 16 sequences, a learned
-        hash whose codes can be cached, no KV offloading, an attention mask that changes nothing, and a cache whose layers
-        append in place."""
+        """(This layer's `PreallocatedLayer` of `cache`, the additive mask as fp32 [b, 1, S] or None when it changes nothing)
+        when the step can take `_fast_decode`, else None: one new token per sequence, inference, bf16 hidden states and
+        projections without biases, 128-wide heads, up to 16 sequences, a learned hash whose codes can be cached, no KV
+        offloading, and a cache whose layers append in place."""
         if not self.fast_decode or torch.is_grad_enabled() or self.train_usa or self.offloading_length is not None:
             return None
         b, q_len, hidden = hidden_states.shape
@@ -567,11 +567,9 @@ class HeavyHitterMixin:
                 or cos.stride(-1) != 1 or sin.stride() != cos.stride():
             return None
         S = slot.get_seq_length() + 1
-        if self._additive_mask(attention_mask, b, 1, S) is not None:
-            return None
-        return slot
+        return slot, self._additive_mask(attention_mask, b, 1, S)
 
-    def _fast_decode(self, hidden_states, position_embeddings, slot, norm=None, residual=None):
+    def _fast_decode(self, hidden_states, position_embeddings, slot, norm=None, residual=None, amask=None):
         """The decode branch (reference :551-625) for one new token per sequence in five launches: fused QKV projection
         (ha_linear_skinny), rotary embedding + in-place cache append + both hashes (ha_rope_encode_step_cos_sin), distance
         histograms, selection fused into the gather attention, output projection.  For the decoder layer around it
@@ -605,7 +603,8 @@ class HeavyHitterMixin:
         saved = hl.heavy_budget
         hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5
         try:
-            hl._select_attend(sc["q"], kbuf, vbuf, S, sc["attn"], None)
+            # a mask that matters (a padded batch): selection into memory, then the masked gather (reference :593-598)
+            hl._select_attend(sc["q"], kbuf, vbuf, S, sc["attn"], None, attn_mask=None if amask is None else amask[:, 0])
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
@@ -634,7 +633,7 @@ class HeavyHitterMixin:
         if q_len == 1 and not kwargs.get("output_attentions"):
             slot = self._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
             if slot is not None:
-                ret = self._fast_decode(hidden_states, position_embeddings, slot)
+                ret = self._fast_decode(hidden_states, position_embeddings, slot[0], amask=slot[1])
                 self._note_key_storage(cache)
                 return ret
         if q_len > DECODE_MAX_Q_LEN or self.train_usa:
@@ -880,8 +879,8 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
         if slot is not None:
             b, _, hidden = hidden_states.shape
             n1, n2, mlp = layer.input_layernorm, layer.post_attention_layernorm, layer.mlp
-            x1, _ = attn._fast_decode(hidden_states, position_embeddings, slot, norm=(n1.weight, float(n1.variance_epsilon)),
-                                      residual=hidden_states[:, 0, :])
+            x1, _ = attn._fast_decode(hidden_states, position_embeddings, slot[0], norm=(n1.weight, float(n1.variance_epsilon)),
+                                      residual=hidden_states[:, 0, :], amask=slot[1])
             attn._note_key_storage(cache)
             act = attn.__dict__.get("_fast_act")
             if act is None or act.shape != (b, mlp.gate_proj.out_features) or act.device != hidden_states.device:

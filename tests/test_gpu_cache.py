@@ -343,3 +343,33 @@ def test_a_cache_that_generate_made_itself_is_taken_over_in_place(fast):
         ref.reorder_cache(torch.tensor([1, 0], device=DEV))
         b_ref = model(ids[[1, 0], 141:142], past_key_values=ref, use_cache=True).logits
     assert close(a, a_ref) and close(b, b_ref)
+
+
+def test_a_left_padded_batch_takes_the_few_launch_steps_too():
+    # batched generation pads prompts on the left: the attention mask then matters (reference :593-598 adds it before the
+    # softmax), the step keeps its few launches and attends through the masked gather; against the general path
+    print("\n[case] left-padded batch through the few-launch steps", flush=True)
+    cfg, model = _model(fast_decode=False)
+    g = torch.Generator().manual_seed(9)
+    ids = torch.randint(1, cfg.vocab_size, (3, 200), generator=g).to(DEV)
+    am = torch.ones(3, 200, dtype=torch.long, device=DEV)
+    am[1, :37] = 0
+    am[2, :150] = 0
+    kw = dict(max_new_tokens=10, do_sample=False, pad_token_id=0, attention_mask=am)
+    want = model.generate(ids, past_key_values=PreallocatedCache(capacity=256), **kw)
+    hl.reset_usa(model)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = True
+    got = model.generate(ids, past_key_values=PreallocatedCache(capacity=256), **kw)
+    assert all("_fast_act" in layer.self_attn.__dict__ for layer in model.model.layers), "the few-launch step was not taken"
+    assert torch.equal(got, want)
+    with torch.no_grad():                       # one step's logits
+        outs = []
+        for fast in (False, True):
+            hl.reset_usa(model)
+            for layer in model.model.layers:
+                layer.self_attn.fast_decode = fast
+            cache = PreallocatedCache(capacity=256)
+            model(ids[:, :199], attention_mask=am[:, :199], past_key_values=cache, use_cache=True)
+            outs.append(model(ids[:, 199:], attention_mask=am, past_key_values=cache, use_cache=True).logits.float())
+    assert (outs[0] - outs[1]).abs().max().item() <= 3e-2 * max(1.0, outs[0].abs().max().item())

@@ -398,7 +398,41 @@ static int linear_skinny_impl(const void *x, int64_t x_stride_m, const void *w, 
         // norm of x, so fewer, larger workgroups win (whole decoder step 6.3 ms against 6.8 ms with 8 rows everywhere).
         const int chunks = (K + 511) / 512;
         const int fuse = (norm_weight ? 1 : 0) | (act == HA_ACT_SWIGLU ? 2 : 0);
-        const int RB = (fuse & 1) ? ((int64_t)N >= 64 * 1024 ? 64 : (int64_t)N >= 32 * 512 ? 32 : 16) : (chunks <= 8 && (int64_t)N < 64 * 1024) ? 8 : 16;
+        int RB = (fuse & 1) ? ((int64_t)N >= 64 * 1024 ? 64 : (int64_t)N >= 32 * 512 ? 32 : 16) : (chunks <= 8 && (int64_t)N < 64 * 1024) ? 8 : 16;
+        {
+            // A grid of a few blocks per CU is quantised: workgroups go round the 256 CUs, the launch lasts as long as the CU
+            // with the most rows, and a CU holds two of these workgroups (one of the 1024-thread ones).  When the usual row
+            // count gives more blocks than are resident at once but not many more (a second, partly filled round), take the row
+            // count (a multiple of 8) that leaves the busiest CU the fewest rows, and among equals the one that gives a CU its
+            // two workgroups (one), then the fewest.  Gate/up 28672 x 4096 at M = 4: 32 rows make 896 blocks, 4 on some CUs =
+            // 128 rows; 56 rows make 512, 2 x 56 everywhere: 49.1 -> 44.2 us launched alone (47.4 with 112 rows, 54.3 with
+            // 48), 45.3 -> 43.7 us inside the decoder step (whose 5.6 ms do not show the 50 us: 713 / 713 against 715 / 703 tokens/s on one box).  Grids that fit one round keep the usual count: QKV 6144 x 4096
+            // (384 blocks of 16 rows) was 1.5 us faster alone with 24 rows (one block per CU) and 0.9 us slower inside the step.
+            constexpr int kCUs = 256;
+            const int64_t units = act == HA_ACT_SWIGLU ? N / 2 : N;     // rows that a block's RB (RB / 2 gate rows) stand for
+            const int per_block = act == HA_ACT_SWIGLU ? RB / 2 : RB;
+            const int64_t usual = (units + per_block - 1) / per_block;
+            if (usual > 2 * kCUs && usual <= 4 * kCUs) {
+                const int MMx = M <= 4 ? 4 : 8, NWx = chunks <= 8 ? 8 : 16;
+                const int rb_max = min(128, 4096 / (MMx * NWx));           // the partial sums of a block fit 64 KB of LDS
+                const int want = NWx == 8 ? 2 : 1;
+                int64_t best_rows = -1;
+                int best_rank = 0;
+                for (int rb = 8; rb <= rb_max; rb += 8) {
+                    const int pb = act == HA_ACT_SWIGLU ? rb / 2 : rb;
+                    const int64_t blocks = (units + pb - 1) / pb, per_cu = (blocks + kCUs - 1) / kCUs, rows = per_cu * rb;
+                    const int rank = per_cu == want ? 0 : per_cu == 3 - want ? 1 : (int)per_cu;
+                    if (best_rows < 0 || rows < best_rows || (rows == best_rows && rank < best_rank)) {
+                        best_rows = rows;
+                        best_rank = rank;
+                        RB = rb;
+                    }
+                }
+            }
+        }
+#ifdef HASHATTN_TUNING_ENV
+        if (const char *e = getenv("HA_GEMV_RB")) RB = atoi(e);
+#endif
         const int nblk = act == HA_ACT_SWIGLU ? (N / 2 + RB / 2 - 1) / (RB / 2) : (N + RB - 1) / RB;
         // one workgroup per row block: the kernel can walk several blocks per workgroup, but a grid cut down to the
         // resident workgroups measured no better (gate/up 43.3 - 48.1 us against 42.2; whole decoder step unchanged)

@@ -170,7 +170,8 @@ def test_decoder_step_on_the_fused_attention_path_matches_the_two_launch_path():
     assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
 
 
-@pytest.mark.parametrize("M,N,K", [(4, 6144, 4096), (1, 512, 1024), (8, 1000, 4096), (3, 96, 8192), (4, 200, 16384), (5, 64, 64)])
+@pytest.mark.parametrize("M,N,K", [(4, 6144, 4096), (1, 512, 1024), (8, 1000, 4096), (3, 96, 8192), (4, 200, 16384), (5, 64, 64),
+                                   (4, 10240, 8192), (2, 9000, 4096)])      # the last two: row counts chosen for whole rounds
 def test_linear_skinny_with_rmsnorm_in_front(M, N, K):
     # against the RMSNorm module of transformers (and of the reference's harness, efficiency/model.py:314-319: the normalised
     # row is rounded to the input type, then multiplied by the weight and rounded again), followed by the fp32 product

@@ -50,6 +50,11 @@ __device__ __forceinline__ uint4 stream16_or_zero(const void *p, bool ok) {
     if (ok) v = ha_load16_stream(reinterpret_cast<const uint4 *>(p));
     return v;
 }
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// two floats rounded to bf16 (nearest even, v_cvt_pk_bf16_f32) in one word: `lo` in the low half
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
@@ -152,9 +157,11 @@ __global__ __launch_bounds__(NWAVE * 64) void gemv_rows_kernel(const uint16_t *_
                 uint32_t *p = reinterpret_cast<uint32_t *>(&xr[c][m]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float lo = ha_round_bf16(__uint_as_float(p[i] << 16) * rstd[m]) * __uint_as_float(g[i] << 16);
-                    const float hi = ha_round_bf16(__uint_as_float(p[i] & 0xffff0000u) * rstd[m]) * __uint_as_float(g[i] & 0xffff0000u);
-                    p[i] = ha_f32_to_bf16_bits(lo) | (ha_f32_to_bf16_bits(hi) << 16);
+                    // both roundings with the packed hardware conversion (round to nearest even): every instruction here is
+                    // on the path of every workgroup before its first product
+                    const uint32_t n = pack_bf16x2(__uint_as_float(p[i] << 16) * rstd[m], __uint_as_float(p[i] & 0xffff0000u) * rstd[m]);
+                    p[i] = pack_bf16x2(__uint_as_float(n << 16) * __uint_as_float(g[i] << 16),
+                                       __uint_as_float(n & 0xffff0000u) * __uint_as_float(g[i] & 0xffff0000u));
                 }
             }
         }

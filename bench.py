@@ -880,7 +880,7 @@ def main():
                                   "steps": sub.steps}
 
         def hf_leg():
-            h = hf_path_bench(argparse.Namespace(**{**vars(args), "steps": 16, "layers": 4}), torch)
+            h = hf_path_bench(argparse.Namespace(**{**vars(args), "steps": 16, "layers": 4, "config": "config3"}), torch)
             return {"workload": h["config"]["workload"], "ms_per_token_step": h["value"], "layers": h["layers"],
                     "per_layer_slope": h["per_layer_slope"], "how": h["how"]}
 

@@ -46,6 +46,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
         assert dec[key] > 0
     hf = d["patched_transformers_model_config3"]
     assert hf["ms_per_token_step"] > 0 and "patched_preallocated_us_per_layer" in hf["per_layer_slope"]
+    assert hf["workload"].startswith("config3 ") and "B=4 " in hf["workload"]
     assert "patched_preallocated_attention_module_only_us_per_layer" in hf["per_layer_slope"]
     assert hf["per_layer_slope"]["patched_dynamic_cache_adopted_us_per_layer"] < 0.5 * hf["per_layer_slope"]["patched_dynamic_cache_us_per_layer"]
     assert d["paged_cache_identity_table"]["same_bits_as_unpaged"] is True

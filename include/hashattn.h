@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define HA_VERSION 200 /* 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
+#define HA_VERSION 201 /* 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
 
 typedef enum ha_status {
     HA_OK = 0,

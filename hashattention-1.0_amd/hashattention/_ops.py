@@ -163,12 +163,12 @@ def _stream(t: torch.Tensor):
     there is one: building a `torch.cuda.Stream` object per launch costs ~5 us, a fifth of what a decode layer's launches
     cost the host."""
     if _raw_stream is not None:
-        return C.c_void_p(_raw_stream(t.device.index))
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+        return _raw_stream(t.device.index)          # a plain integer: ctypes turns it into the void * the signature asks for
+    return torch.cuda.current_stream(t.device).cuda_stream
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else C.c_void_p(t.data_ptr())
+    return None if t is None else t.data_ptr()
 
 
 def _require_cuda(*tensors):

@@ -291,11 +291,11 @@ def test_ops_launch_on_torchs_current_stream():
     # the binding takes the current stream's raw handle from torch without building a Stream object per launch
     from hashattention import _ops
     t = torch.zeros(1, device=DEV)
-    assert (_ops._stream(t).value or 0) == torch.cuda.current_stream(DEV).cuda_stream
+    assert (_ops._stream(t) or 0) == torch.cuda.current_stream(DEV).cuda_stream
     side = torch.cuda.Stream(device=DEV)
     with torch.cuda.stream(side):
-        assert _ops._stream(t).value == side.cuda_stream
-    assert (_ops._stream(t).value or 0) == torch.cuda.current_stream(DEV).cuda_stream
+        assert _ops._stream(t) == side.cuda_stream
+    assert (_ops._stream(t) or 0) == torch.cuda.current_stream(DEV).cuda_stream
 
 
 @pytest.mark.parametrize("fast", [False, True])

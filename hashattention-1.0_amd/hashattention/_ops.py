@@ -627,6 +627,25 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
 HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1
 
 
+def _linear_skinny_unchecked(x, w, out, residual=None, norm_weight=None, eps=0.0, swiglu=False):
+    """`linear_skinny` for callers that made these tensors themselves (2-D bf16 on one GPU, rows contiguous): no checks on
+    the Python side - a decode layer's seven launches should not cost the host more than they cost the GPU.  The library
+    still validates sizes, strides and alignment."""
+    lib = _lib or load_library()
+    M, K = x.shape
+    N = w.shape[0]
+    if norm_weight is None and not swiglu:
+        st = lib.ha_linear_skinny(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None if residual is None else residual.data_ptr(),
+                                  0 if residual is None else residual.stride(0), out.data_ptr(), out.stride(0), M, N, K, _stream(x))
+    else:
+        st = lib.ha_linear_skinny_fused(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None if residual is None else residual.data_ptr(),
+                                        0 if residual is None else residual.stride(0), None if norm_weight is None else norm_weight.data_ptr(),
+                                        eps, HA_ACT_SWIGLU if swiglu else HA_ACT_NONE, out.data_ptr(), out.stride(0), M, N, K, _stream(x))
+    if st:
+        _check(st, "ha_linear_skinny")
+    return out
+
+
 def linear_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
                   norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5, swiglu: bool = False) -> torch.Tensor:
     """out [M, N] = x [M, K] @ w[N, K]^T (+ residual [M, N]); bf16, M <= 16.  Streams w once.

@@ -585,9 +585,9 @@ class HeavyHitterMixin:
                       attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
             self.__dict__["_fast_scratch"] = sc
         if norm is None:
-            _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
+            _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
         else:
-            _ops.linear_skinny(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"], norm_weight=norm[0], eps=norm[1])
+            _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"], norm_weight=norm[0], eps=norm[1])
         kbuf, vbuf, pos = slot.append_slots(hidden_states, b, Hkv, d, 1)
         S = pos + 1
         hl = self._ensure_hash_layer(b, S, dev)
@@ -608,7 +608,7 @@ class HeavyHitterMixin:
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
-        _ops.linear_skinny(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
+        _ops._linear_skinny_unchecked(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
 
     def _adopt_cache_layer(self, cache) -> None:
@@ -835,28 +835,44 @@ def _stacked_gate_up(attn, mlp) -> torch.Tensor:
     return hit[1]
 
 
-def _layer_takes_fast_path(layer, hidden_states) -> bool:
-    """A single-token step of up to 8 sequences through a decoder layer of the Llama shape in bf16: RMSNorm, attention,
-    residual, RMSNorm, SiLU-gated MLP without biases, residual; rows of at most 16384 elements (the projection kernel's
-    fused forms)."""
-    mlp, n1, n2 = getattr(layer, "mlp", None), getattr(layer, "input_layernorm", None), getattr(layer, "post_attention_layernorm", None)
-    if mlp is None or n1 is None or n2 is None or hidden_states.shape[0] > 8 or hidden_states.shape[1] != 1:
+def _layer_modules(layer):
+    """(mlp, input norm, post-attention norm, gate, up, down) of a decoder layer of the Llama shape - RMSNorm, attention,
+    residual, RMSNorm, SiLU-gated MLP without biases, residual - or False; looked up once per layer."""
+    found = layer.__dict__.get("_fast_modules")
+    if found is None:
+        mlp, n1, n2 = getattr(layer, "mlp", None), getattr(layer, "input_layernorm", None), getattr(layer, "post_attention_layernorm", None)
+        lin = [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")] if mlp is not None else [None]
+        act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
+        ok = n1 is not None and n2 is not None and all(isinstance(m, nn.Linear) and m.bias is None for m in lin) \
+            and (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") \
+            and all(getattr(n, "weight", None) is not None and hasattr(n, "variance_epsilon") and "RMSNorm" in type(n).__name__ for n in (n1, n2))
+        found = (mlp, n1, n2, *lin) if ok else False
+        layer.__dict__["_fast_modules"] = found
+    return found
+
+
+def _layer_takes_fast_path(layer, hidden_states):
+    """The layer's modules (`_layer_modules`) when a single-token step of up to 8 sequences can run as seven launches: bf16
+    weights, rows of at most 16384 elements (the projection kernel's fused forms), and no forward hook on a module that this
+    path would not call (activation capture, adapters that wrap a forward); else False."""
+    if hidden_states.shape[0] > 8 or hidden_states.shape[1] != 1:
         return False
-    lin = [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
-    if any(not isinstance(m, nn.Linear) or m.bias is not None or m.weight.dtype != torch.bfloat16 for m in lin):
+    mods = _layer_modules(layer)
+    if not mods:
         return False
-    # hooks on the modules this path does not call (activation capture, adapters that wrap a forward) keep the library's layer
-    for m in (layer.self_attn, mlp, n1, n2, *lin):
+    if layer.self_attn._forward_hooks or layer.self_attn._forward_pre_hooks:
+        return False
+    for m in mods:
         if m._forward_hooks or m._forward_pre_hooks:
             return False
-    act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
-    if not (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") or lin[0].out_features > 16384 or lin[0].in_features > 16384:
+    gate, down = mods[3], mods[5]
+    if gate.out_features > 16384 or gate.in_features > 16384:
         return False
-    for n in (n1, n2):
-        w = getattr(n, "weight", None)
-        if w is None or w.dtype != torch.bfloat16 or not hasattr(n, "variance_epsilon") or type(n).__name__.find("RMSNorm") < 0:
-            return False
-    return True
+    bf16 = torch.bfloat16
+    if gate.weight.dtype != bf16 or mods[4].weight.dtype != bf16 or down.weight.dtype != bf16 or mods[1].weight.dtype != bf16 \
+            or mods[2].weight.dtype != bf16:
+        return False
+    return mods
 
 
 def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
@@ -866,30 +882,32 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
     projection, the attention step, residual inside the output projection, post-attention RMSNorm in front of and SwiGLU
     behind the stacked gate/up projection, residual inside the down projection (the launches of `LlamaShapedDecoder`) -
     instead of the ~25 library calls of the layer's own forward, which at these sizes are bound by the host.  Everything
-    else goes to the layer's own forward.  Outputs differ from it by bf16 roundings (one rounding per RMSNorm instead of
-    two, other summation orders)."""
+    else goes to the layer's own forward.  The fused forms round where the modules they replace round, so outputs differ
+    from the layer's own by the bf16 rounding of other summation orders only."""
     attn = layer.self_attn
     cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
-    if getattr(attn, "fast_layer", False) and not kwargs.get("output_attentions") and _layer_takes_fast_path(layer, hidden_states):
+    mods = getattr(attn, "fast_layer", False) and not kwargs.get("output_attentions") and _layer_takes_fast_path(layer, hidden_states)
+    if mods:
         attn.ensure_gpu(cache, hidden_states.device)
         if not attn.train_usa:
             attn._adopt_cache_layer(cache)
         attn._sync_bit_cache(cache)
         slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
         if slot is not None:
-            b, _, hidden = hidden_states.shape
-            n1, n2, mlp = layer.input_layernorm, layer.post_attention_layernorm, layer.mlp
+            b = hidden_states.shape[0]
+            mlp, n1, n2, gate, _, down = mods
             x1, _ = attn._fast_decode(hidden_states, position_embeddings, slot[0], norm=(n1.weight, float(n1.variance_epsilon)),
                                       residual=hidden_states[:, 0, :], amask=slot[1])
             attn._note_key_storage(cache)
             act = attn.__dict__.get("_fast_act")
-            if act is None or act.shape != (b, mlp.gate_proj.out_features) or act.device != hidden_states.device:
-                act = torch.empty(b, mlp.gate_proj.out_features, dtype=torch.bfloat16, device=hidden_states.device)
+            if act is None or act.shape[0] != b or act.shape[1] != gate.out_features or act.device != hidden_states.device:
+                act = torch.empty(b, gate.out_features, dtype=torch.bfloat16, device=hidden_states.device)
                 attn.__dict__["_fast_act"] = act
-            _ops.linear_skinny(x1[:, 0, :], _stacked_gate_up(attn, mlp), act, norm_weight=n2.weight, eps=float(n2.variance_epsilon),
-                               swiglu=True)
+            x1_rows = x1[:, 0, :]
+            _ops._linear_skinny_unchecked(x1_rows, _stacked_gate_up(attn, mlp), act, norm_weight=n2.weight, eps=float(n2.variance_epsilon),
+                                          swiglu=True)
             out = torch.empty_like(x1)
-            _ops.linear_skinny(act, mlp.down_proj.weight, out[:, 0, :], residual=x1[:, 0, :])
+            _ops._linear_skinny_unchecked(act, down.weight, out[:, 0, :], residual=x1_rows)
             return out
     return layer._hf_forward(hidden_states, attention_mask=attention_mask, position_ids=position_ids, past_key_values=past_key_values,
                              use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)

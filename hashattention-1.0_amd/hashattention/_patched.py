@@ -853,7 +853,7 @@ def _layer_modules(layer):
 
 def _layer_takes_fast_path(layer, hidden_states):
     """The layer's modules (`_layer_modules`) when a single-token step of up to 8 sequences can run as seven launches: bf16
-    weights, rows of at most 16384 elements (the projection kernel's fused forms), and no forward hook on a module that this
+    weights, hidden states of at most 16384 elements (the projection kernel's fused forms), and no forward hook on a module that this
     path would not call (activation capture, adapters that wrap a forward); else False."""
     if hidden_states.shape[0] > 8 or hidden_states.shape[1] != 1:
         return False
@@ -866,7 +866,7 @@ def _layer_takes_fast_path(layer, hidden_states):
         if m._forward_hooks or m._forward_pre_hooks:
             return False
     gate, down = mods[3], mods[5]
-    if gate.out_features > 16384 or gate.in_features > 16384:
+    if gate.in_features > 16384:        # the norm-in-front form keeps a row of hidden states in registers
         return False
     bf16 = torch.bfloat16
     if gate.weight.dtype != bf16 or mods[4].weight.dtype != bf16 or down.weight.dtype != bf16 or mods[1].weight.dtype != bf16 \

@@ -373,3 +373,25 @@ def test_a_left_padded_batch_takes_the_few_launch_steps_too():
             model(ids[:, :199], attention_mask=am[:, :199], past_key_values=cache, use_cache=True)
             outs.append(model(ids[:, 199:], attention_mask=am, past_key_values=cache, use_cache=True).logits.float())
     assert (outs[0] - outs[1]).abs().max().item() <= 3e-2 * max(1.0, outs[0].abs().max().item())
+
+
+def test_whole_layer_step_with_an_mlp_wider_than_the_row_streaming_kernel_takes():
+    # intermediate size above 16384 (Llama-3.1-70B has 28672): the down projection's rows are too long for the row-streaming
+    # form of the projection kernel and take its matrix-core form; the layer still runs in seven launches
+    print("\n[case] whole-layer step, intermediate size 16512", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(LlamaConfig)
+    cfg.intermediate_size = 16512
+    model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
+    model = hl.convert_usa(model, cfg, hl.load_usa(cfg, None), collect_stats=False, train_usa=False)
+    ids = torch.randint(0, cfg.vocab_size, (2, 203), generator=torch.Generator().manual_seed(11)).to(DEV)
+    outs = []
+    for fast in (False, True):
+        hl.reset_usa(model)
+        for layer in model.model.layers:
+            layer.self_attn.fast_decode = fast
+        outs.append(_decode(model, ids, PreallocatedCache(capacity=256), [1, 1, 1]))
+    assert all("_fast_act" in layer.self_attn.__dict__ for layer in model.model.layers)
+    worst = max((g - w).abs().max().item() for g, w in zip(outs[1], outs[0]))
+    scale = max(w.abs().max().item() for w in outs[0])
+    assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)

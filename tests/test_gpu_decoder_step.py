@@ -100,7 +100,8 @@ def test_rope_append_and_swiglu_against_torch(dtype):
 
 
 @pytest.mark.parametrize("M,N,K", [(4, 4096, 4096), (1, 1000, 512), (16, 6144, 4096), (4, 4096, 14336), (3, 20, 64), (4, 128256, 1024),
-                                   (8, 4100, 4096), (5, 333, 8192), (7, 50, 14336), (2, 4096, 16416), (12, 77, 96)])
+                                   (8, 4100, 4096), (5, 333, 8192), (7, 50, 14336), (2, 4096, 16416), (12, 77, 96),
+                                   (4, 8192, 28672)])       # the last one: the down projection of a 70B model (rows too long for the row-streaming form)
 def test_linear_skinny_against_fp32_matmul(M, N, K):
     # bf16 inputs, fp32 accumulation: against the fp32 product of the same bf16 values, one bf16 rounding of the result apart
     print(f"\n[case] linear_skinny {M}x{N}x{K}", flush=True)
@@ -205,7 +206,7 @@ def test_linear_skinny_with_rmsnorm_in_front(M, N, K):
         assert (hn != h).float().mean().item() <= 1e-3, (hn != h).float().mean().item()
 
 
-@pytest.mark.parametrize("M,F,K", [(4, 14336, 4096), (1, 100, 512), (8, 777, 4096), (2, 48, 8192), (4, 40, 64)])
+@pytest.mark.parametrize("M,F,K", [(4, 14336, 4096), (1, 100, 512), (8, 777, 4096), (2, 48, 8192), (4, 40, 64), (4, 28672, 8192)])
 def test_linear_skinny_with_swiglu_behind(M, F, K):
     # against the unfused pair: ha_linear_skinny into a bf16 gate/up buffer, then ha_swiglu - same roundings, same sums
     print(f"\n[case] linear_skinny + SwiGLU {M}x{F}x{K}", flush=True)

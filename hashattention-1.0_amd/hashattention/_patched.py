@@ -538,6 +538,9 @@ class HeavyHitterMixin:
         if q_len != 1 or b > 16 or hidden % 32 or self.head_dim != 128 or hidden_states.dtype != torch.bfloat16 \
                 or not hidden_states.is_contiguous() or position_embeddings is None:
             return None
+        own = self._modules     # plain nn.Linear projections only: a wrapper around one (an adapter) has a forward of its own
+        if any(type(own.get(n)) is not nn.Linear for n in ("q_proj", "k_proj", "v_proj", "o_proj")):
+            return None
         if self.q_proj.bias is not None or self.o_proj.bias is not None or self.q_proj.weight.dtype != torch.bfloat16:
             return None
         if self.q_proj.weight.device != hidden_states.device:       # a model spread over devices: its own hooks move the inputs
@@ -837,18 +840,23 @@ def _stacked_gate_up(attn, mlp) -> torch.Tensor:
 
 def _layer_modules(layer):
     """(mlp, input norm, post-attention norm, gate, up, down) of a decoder layer of the Llama shape - RMSNorm, attention,
-    residual, RMSNorm, SiLU-gated MLP without biases, residual - or False; looked up once per layer."""
-    found = layer.__dict__.get("_fast_modules")
-    if found is None:
-        mlp, n1, n2 = getattr(layer, "mlp", None), getattr(layer, "input_layernorm", None), getattr(layer, "post_attention_layernorm", None)
-        lin = [getattr(mlp, n, None) for n in ("gate_proj", "up_proj", "down_proj")] if mlp is not None else [None]
-        act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
-        ok = n1 is not None and n2 is not None and all(isinstance(m, nn.Linear) and m.bias is None for m in lin) \
-            and (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") \
-            and all(getattr(n, "weight", None) is not None and hasattr(n, "variance_epsilon") and "RMSNorm" in type(n).__name__ for n in (n1, n2))
-        found = (mlp, n1, n2, *lin) if ok else False
-        layer.__dict__["_fast_modules"] = found
-    return found
+    residual, RMSNorm, SiLU-gated MLP of plain nn.Linear projections without biases, residual - or False.  Looked up once
+    and again whenever one of these modules is no longer the object that was looked at (an adapter library replaces
+    projections by wrappers with a forward of their own; such a layer keeps the library's path)."""
+    seen = layer.__dict__.get("_fast_seen")
+    own = layer._modules
+    mlp = own.get("mlp")
+    sub = mlp._modules if mlp is not None else {}
+    now = (mlp, own.get("input_layernorm"), own.get("post_attention_layernorm"), sub.get("gate_proj"), sub.get("up_proj"), sub.get("down_proj"))
+    if seen is not None and all(a is b for a, b in zip(seen[0], now)):
+        return seen[1]
+    n1, n2, lin = now[1], now[2], now[3:]
+    act = getattr(mlp, "act_fn", None)      # nn.SiLU, or the class transformers keeps under "silu"
+    ok = mlp is not None and n1 is not None and n2 is not None and all(type(m) is nn.Linear and m.bias is None for m in lin) \
+        and (isinstance(act, nn.SiLU) or type(act).__name__ == "SiLUActivation") \
+        and all(getattr(n, "weight", None) is not None and hasattr(n, "variance_epsilon") and "RMSNorm" in type(n).__name__ for n in (n1, n2))
+    layer.__dict__["_fast_seen"] = (now, now if ok else False)
+    return now if ok else False
 
 
 def _layer_takes_fast_path(layer, hidden_states):

@@ -395,3 +395,48 @@ def test_whole_layer_step_with_an_mlp_wider_than_the_row_streaming_kernel_takes(
     worst = max((g - w).abs().max().item() for g, w in zip(outs[1], outs[0]))
     scale = max(w.abs().max().item() for w in outs[0])
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
+
+
+def test_a_wrapper_around_a_projection_keeps_its_say():
+    # adapter libraries replace nn.Linear projections by wrappers with a forward of their own: the few-launch steps read
+    # weights directly, so they step aside for such a module (its output must show in the logits) and come back when it is gone
+    print("\n[case] projections wrapped after convert_usa", flush=True)
+
+    class Shifted(torch.nn.Module):
+        def __init__(self, base):
+            super().__init__()
+            self.base_layer = base
+            self.weight, self.bias = base.weight, base.bias       # as adapter wrappers expose them
+
+        def forward(self, x):
+            return self.base_layer(x) + 0.5
+
+    cfg, model = _model(fast_decode=True)
+    ids = torch.randint(0, cfg.vocab_size, (2, 180), generator=torch.Generator().manual_seed(12)).to(DEV)
+
+    def step_logits():
+        hl.reset_usa(model)
+        cache = PreallocatedCache(capacity=256)
+        with torch.no_grad():
+            model(ids[:, :179], past_key_values=cache, use_cache=True)
+            return model(ids[:, 179:], past_key_values=cache, use_cache=True).logits.float()
+
+    plain = step_logits()
+    for where, name in ((model.model.layers[0].mlp, "down_proj"), (model.model.layers[1].self_attn, "q_proj")):
+        base = getattr(where, name)
+        setattr(where, name, Shifted(base))
+        for layer in model.model.layers:
+            layer.self_attn.fast_decode = True
+        got = step_logits()
+        for layer in model.model.layers:
+            layer.self_attn.fast_decode = False
+        want = step_logits()
+        assert (got - want).abs().max().item() <= 3e-2 * max(1.0, want.abs().max().item()), name
+        assert (got - plain).abs().max().item() > 10 * (got - want).abs().max().item(), name      # the wrapper was heard
+        setattr(where, name, base)
+    for layer in model.model.layers:
+        layer.self_attn.fast_decode = True
+        layer.self_attn.__dict__.pop("_fast_act", None)
+    again = step_logits()
+    assert all("_fast_act" in layer.self_attn.__dict__ for layer in model.model.layers)
+    assert (again - plain).abs().max().item() <= 3e-2 * max(1.0, plain.abs().max().item())

@@ -49,15 +49,20 @@ def _oracle_forward(layer, usa, cfg, apply_rope, **variant):
         cos, sin = position_embeddings
         q, k = apply_rope(q, k, cos, sin)
         k, v = past_key_values.update(k, v, self.layer_idx)
+        add = attention_mask            # added to the scores (reference :593-598); the library may hand it over as booleans
+        if add is not None:
+            add = add[..., :k.shape[2]]
+            if add.dtype == torch.bool:
+                add = torch.zeros(add.shape, dtype=q.dtype).masked_fill_(~add, float("-inf"))
         out, _ = orc.reference_decode_attention(q, k, v, k_heads, q_heads, cfg.init_budget, cfg.recent_budget, cfg.heavy_budget,
-                                                **variant)
+                                                attention_mask=add, **variant)
         return self.o_proj(out.transpose(1, 2).reshape(b, q_len, -1)), None
 
     layer.forward = types.MethodType(forward, layer)
 
 
-def _run(model, ids, steps):
-    cache = DynamicCache()
+def _run(model, ids, steps, make_cache=DynamicCache):
+    cache = make_cache()
     outs = []
     with torch.no_grad():
         o = model(ids[:, :-sum(steps)], past_key_values=cache, use_cache=True)
@@ -107,6 +112,41 @@ def test_patched_model_matches_reference_semantics(family):
     got2 = _run(model, ids.to(DEV), steps)
     for g, g2 in zip(got, got2):
         assert torch.equal(g, g2)
+
+
+def test_mistral_sliding_window_cache():
+    # A Mistral configuration with a sliding window: the library's cache (what `generate` builds from the configuration) keeps
+    # the last window - 1 tokens only, so every decode step sees a window whose first token moved.  The reference's patched
+    # forward attends to whatever the cache returns (hashattention_mistral.py has no sliding-window logic of its own); so does
+    # this one, re-hashing the window each step.
+    print("\n[case] model api mistral, sliding-window cache", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(MistralConfig, sliding_window=48)
+    model = MistralForCausalLM(cfg).bfloat16().float()
+    ref = copy.deepcopy(model)
+    usa = hm.load_usa(cfg, None)
+    model = hm.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False).float()
+    rope = __import__("transformers.models.mistral.modeling_mistral", fromlist=["apply_rotary_pos_emb"]).apply_rotary_pos_emb
+    for li, layer in enumerate(ref.model.layers):
+        _oracle_forward(layer.self_attn, usa[li], cfg, rope)
+    ids = torch.randint(0, cfg.vocab_size, (2, 150 + 1 + 1 + 3 + 1 + 1), generator=torch.Generator().manual_seed(4))
+    steps = [1, 1, 3, 1, 1]
+    seen = []
+
+    def make():
+        seen.append(DynamicCache(config=cfg))
+        return seen[-1]
+    got = _run(model, ids.to(DEV), steps, make)
+    assert type(seen[0].layers[0]).__name__ == "DynamicSlidingWindowLayer" and seen[0].layers[0].keys.shape[2] == 47
+    want = _run(ref, ids, steps, make)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        err = (g - w).abs().max().item()
+        print(f"  step rows {tuple(g.shape)}: max err {err:.2e}", flush=True)
+        assert err < 2e-3, err
+    # the same through generate, which builds that cache itself
+    out = model.generate(ids[:, :150].to(DEV), max_new_tokens=6, do_sample=False, pad_token_id=0)
+    assert out.shape == (2, 156)
 
 
 def test_usa_forward_and_mask_api():

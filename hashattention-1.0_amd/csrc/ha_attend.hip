@@ -1094,24 +1094,30 @@ __global__ __launch_bounds__(HA_HEAD_DIM) void merge_splits_kernel(const float *
 }
 
 // ------------------------------------------------------------------------------------------------
-// Dense flash-decode.  grid (nsplit_max, Hkv, B).  A workgroup streams `chunk` consecutive keys of one
-// KV head once and scores them against the G query heads of the group.
+// Dense flash-decode.  grid (nsplit_max, Hkv * passes, B).  A workgroup streams `chunk` consecutive keys of one
+// KV head once and scores them against G query heads of its group of `group` heads: passes = ceil(group / G), and a
+// group that is not 1, 2, 4 or 8 heads wide leaves the last slots of its last pass idle (24 query heads on 8 KV heads:
+// G = 4, one pass, three slots used).
 // WIN: the same over the sink and recent windows only (win_init, win_recent; grid (1, Hkv, B)): the result is
 // left as an unnormalised partial (acc, m, l) per row for the sparse kernel to merge, so this small launch can
 // run on another stream while the selection is still being computed.
 template <typename E, int G, bool WIN>
 __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                                    const void *__restrict__ k, const void *__restrict__ v,
-                                                                   int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int max_S,
-                                                                   const int32_t *__restrict__ seq_lens, float scale_log2e, int chunk,
-                                                                   int nsplit_max, float *__restrict__ part_acc,
+                                                                   int64_t kv_sb, int64_t kv_sh, int64_t kv_ss, int H, int group,
+                                                                   int max_S, const int32_t *__restrict__ seq_lens, float scale_log2e,
+                                                                   int chunk, int nsplit_max, float *__restrict__ part_acc,
                                                                    float *__restrict__ part_ml, void *__restrict__ out, int win_init,
                                                                    int win_recent) {
     using EL = Elem<E>;
     __shared__ float s_m[kStreams], s_l[kStreams];
     __shared__ float s_acc[kStreams * HA_HEAD_DIM];
 
-    const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int sp = blockIdx.x, b = blockIdx.z;
+    const int passes = (group + G - 1) / G;
+    const int hk = blockIdx.y / passes;
+    const int h0 = hk * group + (blockIdx.y % passes) * G;  // query head of slot 0
+    const int n_slots = min(G, (hk + 1) * group - h0);      // slots of this workgroup that hold a query head
     const int tid = threadIdx.x, sub = tid & 15, stream = tid >> 4;
     int S = seq_lens ? seq_lens[b] : max_S;
     if (S > max_S) S = max_S;
@@ -1123,7 +1129,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
     if (sp >= nsplit) return;
     if (!WIN && S == 0) {
         if (tid < HA_HEAD_DIM)
-            for (int g = 0; g < G; ++g) EL::store1((char *)out + ((int64_t)b * H + hk * G + g) * HA_HEAD_DIM * EL::bytes, tid, 0.f);
+            for (int g = 0; g < n_slots; ++g) EL::store1((char *)out + ((int64_t)b * H + h0 + g) * HA_HEAD_DIM * EL::bytes, tid, 0.f);
         return;
     }
     const int r0 = WIN ? 0 : sp * chunk, r1 = WIN ? n_rows : min(r0 + chunk, S);
@@ -1136,7 +1142,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         float t[8];
-        EL::unpack(EL::load8((const char *)q + (b * q_sb + (hk * G + g) * q_sh) * EL::bytes, sub), t);
+        EL::unpack(EL::load8((const char *)q + (b * q_sb + (h0 + min(g, n_slots - 1)) * q_sh) * EL::bytes, sub), t);  // idle slots repeat the last head
 #pragma unroll
         for (int i = 0; i < 8; ++i) qf[g][i] = t[i] * scale_log2e;
     }
@@ -1214,10 +1220,10 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
 #pragma unroll
         for (int i = 0; i < 8; ++i) s_acc[stream * HA_HEAD_DIM + sub * 8 + i] = acc[g][i];
         __syncthreads();
-        if (tid < HA_HEAD_DIM) {
+        if (tid < HA_HEAD_DIM && g < n_slots) {
             float M, L, A;
             merge_streams<kStreams>(s_m, s_l, s_acc, tid, M, L, A);
-            const int64_t row = (int64_t)b * H + hk * G + g;
+            const int64_t row = (int64_t)b * H + h0 + g;
             if (WIN) {  // one record per row: acc[128], m, l
                 part_acc[row * (HA_HEAD_DIM + 2) + tid] = A;
                 if (tid == 0) {
@@ -1237,6 +1243,9 @@ __global__ __launch_bounds__(kAttThreads) void dense_attend_kernel(const void *_
         }
     }
 }
+
+// query-head slots per workgroup of the dense kernel for a group of `group` query heads per KV head
+inline int dense_slots(int group) { return group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : 8; }
 
 int validate_qkv(const void *q, int64_t q_sb, int64_t q_sh, const void *k, const void *v, int kv_dtype, int64_t kv_sb, int64_t kv_sh,
                  int64_t kv_ss, int B, int H, int Hkv, const void *out) {
@@ -1570,16 +1579,17 @@ int ha_window_partial(const void *q, int64_t q_stride_b, int64_t q_stride_h, con
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, window_partial);
     if (st) return st;
     HA_REQUIRE(init_budget >= 0 && recent_budget >= 0 && max_seq_len > 0, HA_ERR_BAD_SHAPE, "bad window budgets or max_seq_len");
-    const int G = H / Hkv;
-    HA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, HA_ERR_BAD_SHAPE, "H/Hkv=%d, must be 1, 2, 4 or 8", G);
+    const int group = H / Hkv;
+    const int G = dense_slots(group);
+    HA_REQUIRE((int64_t)Hkv * ((group + G - 1) / G) <= 65535, HA_ERR_BAD_SHAPE, "too many heads");
     if ((st = ha_require_device())) return st;
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(1, Hkv, B);
+    const dim3 grid(1, Hkv * ((group + G - 1) / G), B);
     const float sl2 = sm_scale * kLog2e;
 #define HA_WIN_LAUNCH(E_, G_)                                                                                                      \
     do {                                                                                                                           \
         hipLaunchKernelGGL((dense_attend_kernel<E_, G_, true>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,    \
-                           kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, 0, 1, window_partial,             \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, group, max_seq_len, seq_lens, sl2, 0, 1, window_partial,      \
                            (float *)nullptr, (void *)nullptr, init_budget, recent_budget);                                         \
         HA_CHECK_LAUNCH("dense_attend_kernel<window>");                                                                            \
     } while (0)
@@ -1615,8 +1625,9 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(max_seq_len > 0, HA_ERR_BAD_SHAPE, "max_seq_len must be positive");
-    const int G = H / Hkv;
-    HA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, HA_ERR_BAD_SHAPE, "H/Hkv=%d, must be 1, 2, 4 or 8", G);
+    const int group = H / Hkv;
+    const int G = dense_slots(group), passes = (group + G - 1) / G;
+    HA_REQUIRE((int64_t)Hkv * passes <= 65535, HA_ERR_BAD_SHAPE, "too many heads");
     const DensePlan plan = dense_plan(B, Hkv, max_seq_len);
     const size_t need = part_bytes((int64_t)B * H, plan.nsplit_max);
     HA_REQUIRE(workspace && workspace_bytes >= need, HA_ERR_WORKSPACE, "dense decode workspace: need %zu bytes, got %zu", need,
@@ -1628,13 +1639,13 @@ int ha_dense_decode(const void *q, int64_t q_stride_b, int64_t q_stride_h, const
     float *part_acc = (float *)workspace;
     float *part_ml = part_acc + rows * plan.nsplit_max * HA_HEAD_DIM;
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(plan.nsplit_max, Hkv, B), mgrid(H, B);
+    const dim3 grid(plan.nsplit_max, Hkv * passes, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
 #define HA_DENSE_LAUNCH(E_, G_)                                                                                                    \
     do {                                                                                                                           \
         hipLaunchKernelGGL((dense_attend_kernel<E_, G_, false>), grid, dim3(kAttThreads), 0, s, q, q_stride_b, q_stride_h, k, v,   \
-                           kv_stride_b, kv_stride_h, kv_stride_s, H, max_seq_len, seq_lens, sl2, plan.chunk, plan.nsplit_max,      \
-                           part_acc, part_ml, out, 0, 0);                                                                          \
+                           kv_stride_b, kv_stride_h, kv_stride_s, H, group, max_seq_len, seq_lens, sl2, plan.chunk,                \
+                           plan.nsplit_max, part_acc, part_ml, out, 0, 0);                                                         \
         HA_CHECK_LAUNCH("dense_attend_kernel");                                                                                    \
         if (plan.nsplit_max > 1) {                                                                                                 \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, seq_lens, 1,            \

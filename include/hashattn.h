@@ -175,6 +175,9 @@ int ha_hamming_score(const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_str
  *   out_idx    int32 [B, H, idx_cap]: ascending token indices; nothing is written past idx_cap
  *   out_counts int32 [B, H]: number selected (the true count, even if it exceeds idx_cap)
  *   workspace  ha_select_workspace_bytes(...) bytes, 256-byte aligned
+ * H / Hc (query heads that share one code head) must be 1, 2, 4 or 8, else HA_ERR_BAD_SHAPE; the reference keeps one
+ * key-side hash per query head, Hc = H (hashattention_llama.py:642).  The attention entry points take any whole
+ * number of query heads per KV head.
  * kc_stride_b may be 0: every batch entry then reads the same codes, i.e. B queries (each with its own row of
  * qcodes and its own seq_lens[b]) against one sequence - the rows of a multi-token chunk
  * (hashattention_llama.py:423-428) or of the recall statistic (:319-398) in one call.

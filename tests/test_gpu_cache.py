@@ -397,6 +397,26 @@ def test_whole_layer_step_with_an_mlp_wider_than_the_row_streaming_kernel_takes(
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
 
 
+def test_few_launch_steps_with_three_query_heads_per_kv_head():
+    # 6 query heads on 2 KV heads (Llama-3.2-3B has 24 on 8): the seven-launch layer against the general path
+    print("\n[case] whole-layer step, three query heads per KV head", flush=True)
+    torch.manual_seed(0)
+    cfg = _config(LlamaConfig, hidden_size=768, num_attention_heads=6)
+    model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
+    model = hl.convert_usa(model, cfg, hl.load_usa(cfg, None), collect_stats=False, train_usa=False)
+    ids = torch.randint(0, cfg.vocab_size, (3, 230), generator=torch.Generator().manual_seed(12)).to(DEV)
+    outs = []
+    for fast in (False, True):
+        hl.reset_usa(model)
+        for layer in model.model.layers:
+            layer.self_attn.fast_decode = fast
+        outs.append(_decode(model, ids, PreallocatedCache(capacity=256), [1, 1, 4, 1]))
+    assert all("_fast_act" in layer.self_attn.__dict__ for layer in model.model.layers)
+    worst = max((g - w).abs().max().item() for g, w in zip(outs[1], outs[0]))
+    scale = max(w.abs().max().item() for w in outs[0])
+    assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
+
+
 def test_a_wrapper_around_a_projection_keeps_its_say():
     # adapter libraries replace nn.Linear projections by wrappers with a forward of their own: the few-launch steps read
     # weights directly, so they step aside for such a module (its output must show in the logits) and come back when it is gone

@@ -21,8 +21,10 @@ USA_CFG = dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3
 
 
 def _config(cls, **kw):
-    cfg = cls(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
-              head_dim=128, vocab_size=512, max_position_embeddings=4096, **kw)
+    shape = dict(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                 head_dim=128, vocab_size=512, max_position_embeddings=4096)
+    shape.update(kw)
+    cfg = cls(**shape)
     for k, v in USA_CFG.items():
         setattr(cfg, k, v)
     return cfg
@@ -75,12 +77,15 @@ def _run(model, ids, steps, make_cache=DynamicCache):
     return outs
 
 
-@pytest.mark.parametrize("family", ["llama", "mistral"])
+@pytest.mark.parametrize("family", ["llama", "mistral", "llama_3_per_kv"])
 def test_patched_model_matches_reference_semantics(family):
     print(f"\n[case] model api {family}", flush=True)
     torch.manual_seed(0)
     if family == "llama":
         cfg, model_cls, api = _config(LlamaConfig), LlamaForCausalLM, hl
+    elif family == "llama_3_per_kv":    # three query heads per KV head (Llama-3.2-3B: 24 on 8)
+        cfg, model_cls, api = _config(LlamaConfig, hidden_size=768, num_attention_heads=6), LlamaForCausalLM, hl
+        family = "llama"
     else:
         cfg, model_cls, api = _config(MistralConfig, sliding_window=None), MistralForCausalLM, hm
     model = model_cls(cfg).bfloat16().float()           # bf16-representable weights: convert_usa's bf16 cast is then lossless

@@ -36,6 +36,24 @@ def test_group_sizes(gq):
     run_decode_case(small_workload(n_q_heads=8, n_kv_heads=8 // gq, n_code_heads=8 // gq, seed=20 + gq), verbose=True)
 
 
+def test_three_query_heads_per_kv_head():
+    # 24 query heads on 8 KV heads (Llama-3.2-3B's ratio) in the reference's layout, one K hash MLP per query head: the gather
+    # reads K/V through a group of three.  A code head shared by three query heads is refused, not mis-read.
+    _announce("H/Hkv = 3, Hc == H")
+    run_decode_case(small_workload(n_q_heads=6, n_kv_heads=2, n_code_heads=6, seed=31), verbose=True)
+    run_decode_case(small_workload(batch=3, seq_lens=[9000, 4100, 77], n_q_heads=12, n_kv_heads=4, n_code_heads=12, seed=32))
+    # wider groups than the dense kernel's eight slots: two passes over the KV head (12 = 8 + 4; 16 = 8 + 8, Llama-3.1-405B's ratio)
+    run_decode_case(small_workload(n_q_heads=12, n_kv_heads=1, n_code_heads=12, seed=33))
+    run_decode_case(small_workload(batch=2, seq_lens=[3000, 0], n_q_heads=32, n_kv_heads=2, n_code_heads=32, seed=34))
+    dev = "cuda:0"
+    kc = torch.zeros(1, 2, 256, 1, dtype=torch.int32, device=dev)
+    qc = torch.zeros(1, 6, 1, 1, dtype=torch.int32, device=dev)
+    ws = _ops.workspace(1 << 20, dev)
+    with pytest.raises(_ops.HashAttnError, match="must be 1, 2, 4 or 8"):
+        _ops.select(kc, qc, 256, torch.tensor([256], dtype=torch.int32, device=dev), 4, 4, 0.125,
+                    torch.zeros(1, 6, 64, dtype=torch.int32, device=dev), torch.zeros(1, 6, dtype=torch.int32, device=dev), ws)
+
+
 def test_64bit_codes_ragged():
     # 2-layer MLP, 64-bit codes (two words), ragged batch: the configs[4] shape in small
     _announce("W=2 ragged")

@@ -541,7 +541,7 @@ class HeavyHitterMixin:
         own = self._modules     # plain nn.Linear projections only: a wrapper around one (an adapter) has a forward of its own
         if any(type(own.get(n)) is not nn.Linear for n in ("q_proj", "k_proj", "v_proj", "o_proj")):
             return None
-        if self.q_proj.bias is not None or self.o_proj.bias is not None or self.q_proj.weight.dtype != torch.bfloat16:
+        if any(own[n].bias is not None for n in ("q_proj", "k_proj", "v_proj", "o_proj")) or self.q_proj.weight.dtype != torch.bfloat16:
             return None
         if self.q_proj.weight.device != hidden_states.device:       # a model spread over devices: its own hooks move the inputs
             return None

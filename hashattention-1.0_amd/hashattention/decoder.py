@@ -276,6 +276,15 @@ class LlamaShapedDecoder:
         cfg, usa0 = model.config, usa_modules[0]
         if usa0.rehash_every_step:
             raise NotImplementedError("the LSH baseline and CENTER re-hash the whole cache every step: use the patched layer")
+        # what this decoder's launches do not express is refused here rather than dropped in silence
+        if getattr(cfg, "attention_bias", False) or getattr(cfg, "mlp_bias", False):
+            raise NotImplementedError("projections with biases: use the patched model (convert_usa), which calls the modules")
+        rot = model.model.rotary_emb
+        if float(getattr(rot, "attention_scaling", 1.0)) != 1.0 or getattr(rot, "rope_type", "default") in ("dynamic", "longrope"):
+            raise NotImplementedError(f"rotary embedding of type {getattr(rot, 'rope_type', '?')!r} (scaled cos/sin, or frequencies that "
+                                      "change with the length): use the patched model, which takes the model's own cos/sin")
+        if getattr(cfg, "hidden_act", "silu") != "silu":
+            raise NotImplementedError(f"hidden_act={cfg.hidden_act!r}: the gate/up launch applies SiLU")
         head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
         dec = cls(n_layers=cfg.num_hidden_layers, hidden=cfg.hidden_size, ffn=cfg.intermediate_size, n_heads=cfg.num_attention_heads,
                   n_kv_heads=cfg.num_key_value_heads, head_dim=head_dim, vocab=cfg.vocab_size, rms_eps=cfg.rms_norm_eps,

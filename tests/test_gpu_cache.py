@@ -397,11 +397,17 @@ def test_whole_layer_step_with_an_mlp_wider_than_the_row_streaming_kernel_takes(
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
 
 
-def test_few_launch_steps_with_three_query_heads_per_kv_head():
-    # 6 query heads on 2 KV heads (Llama-3.2-3B has 24 on 8): the seven-launch layer against the general path
-    print("\n[case] whole-layer step, three query heads per KV head", flush=True)
+@pytest.mark.parametrize("shape", ["three_per_kv", "yarn"])
+def test_few_launch_steps_on_other_model_shapes(shape):
+    # 6 query heads on 2 KV heads (Llama-3.2-3B has 24 on 8); a rotary embedding that scales its cos/sin (yarn: the step takes
+    # the tables the model hands over): the seven-launch layer against the general path
+    print(f"\n[case] whole-layer step, {shape}", flush=True)
     torch.manual_seed(0)
-    cfg = _config(LlamaConfig, hidden_size=768, num_attention_heads=6)
+    if shape == "three_per_kv":
+        cfg = _config(LlamaConfig, hidden_size=768, num_attention_heads=6)
+    else:
+        cfg = _config(LlamaConfig, rope_parameters=dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=1024,
+                                                        rope_theta=10000.0))
     model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
     model = hl.convert_usa(model, cfg, hl.load_usa(cfg, None), collect_stats=False, train_usa=False)
     ids = torch.randint(0, cfg.vocab_size, (3, 230), generator=torch.Generator().manual_seed(12)).to(DEV)

@@ -322,7 +322,7 @@ def test_generate_replays_one_graph_for_successive_tokens(n_heads, batch):
     assert sampled.shape == (batch, 6) and int(sampled.min()) >= 0 and int(sampled.max()) < 512
 
 
-@pytest.mark.parametrize("family", ["llama", "mistral"])
+@pytest.mark.parametrize("family", ["llama", "mistral", "llama3_rope"])
 def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
     # the serving path end to end: a transformers Llama (or Mistral: the same decoder shape) + hash modules ->
     # LlamaShapedDecoder.from_hf, prefill by the model itself, greedy generation by graph replay; against `generate` of the
@@ -333,12 +333,19 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
                  head_dim=128, vocab_size=512, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5)
     if family == "llama":
         cfg, LlamaForCausalLM, hl = LlamaConfig(**shape), globals()["LlamaForCausalLM"], globals()["hl"]
+    elif family == "llama3_rope":   # Llama-3.1's frequency scaling: the decoder takes the model's own (scaled) frequencies
+        del shape["rope_theta"]
+        cfg = LlamaConfig(rope_parameters=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                               original_max_position_embeddings=64, rope_theta=500000.0), **shape)
+        LlamaForCausalLM, hl = globals()["LlamaForCausalLM"], globals()["hl"]
     else:
         cfg, LlamaForCausalLM, hl = MistralConfig(sliding_window=None, **shape), MistralForCausalLM, hm
     for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
                      recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
         setattr(cfg, k, v)
     model = LlamaForCausalLM(cfg).bfloat16().float()
+    if family == "llama3_rope":
+        assert model.model.rotary_emb.rope_type == "llama3"
     usa = hl.load_usa(cfg, None)
     model = hl.convert_usa(model.to(DEV), cfg, usa, collect_stats=False, train_usa=False).float()
     B, S0, n_new = 2, 200, 8
@@ -355,6 +362,31 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
     print("  tokens:", got.tolist(), flush=True)
     assert torch.equal(got, want)
     assert dec.seq_len == S0 + n_new - 1
+
+
+@pytest.mark.parametrize("what", ["attention_bias", "mlp_bias", "yarn", "dynamic"])
+def test_decoder_from_hf_refuses_what_its_launches_do_not_express(what):
+    print(f"\n[case] decoder from_hf refuses {what}", flush=True)
+    shape = dict(hidden_size=512, intermediate_size=1024, num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=2,
+                 head_dim=128, vocab_size=512, max_position_embeddings=4096)
+    if what == "yarn":
+        shape["rope_parameters"] = dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=1024, rope_theta=10000.0)
+    elif what == "dynamic":
+        shape["rope_parameters"] = dict(rope_type="dynamic", factor=2.0, rope_theta=10000.0)
+    else:
+        shape[what] = True
+    cfg = LlamaConfig(**shape)
+    for k, v in dict(lth_init_dim=128, lth_final_dim=32, lth_thold=0, lth_num_layers=3, init_budget=8, heavy_budget=0.125,
+                     recent_budget=8, usa_retrieve_depth=6, usa_eval_mode="simple").items():
+        setattr(cfg, k, v)
+    model = LlamaForCausalLM(cfg).bfloat16().to(DEV)
+    with pytest.raises(NotImplementedError):
+        LlamaShapedDecoder.from_hf(model, hl.load_usa(cfg, None), batch=1, cache_len=64, dtype=torch.float32, device=DEV)
+    # the patched model takes all of these: biases through the modules, the rotary embedding through the model's own cos/sin
+    model = hl.convert_usa(model, cfg, hl.load_usa(cfg, None), collect_stats=False, train_usa=False)
+    ids = torch.randint(1, 512, (2, 150), generator=torch.Generator().manual_seed(6)).to(DEV)
+    out = model.generate(ids, max_new_tokens=4, do_sample=False, pad_token_id=0)
+    assert out.shape == (2, 154)
 
 
 def test_ragged_prompts_through_the_decoder_generation_loop():

@@ -77,7 +77,7 @@ def _run(model, ids, steps, make_cache=DynamicCache):
     return outs
 
 
-@pytest.mark.parametrize("family", ["llama", "mistral", "llama_3_per_kv"])
+@pytest.mark.parametrize("family", ["llama", "mistral", "llama_3_per_kv", "llama_bias_yarn"])
 def test_patched_model_matches_reference_semantics(family):
     print(f"\n[case] model api {family}", flush=True)
     torch.manual_seed(0)
@@ -86,6 +86,10 @@ def test_patched_model_matches_reference_semantics(family):
     elif family == "llama_3_per_kv":    # three query heads per KV head (Llama-3.2-3B: 24 on 8)
         cfg, model_cls, api = _config(LlamaConfig, hidden_size=768, num_attention_heads=6), LlamaForCausalLM, hl
         family = "llama"
+    elif family == "llama_bias_yarn":   # projections with biases, cos/sin scaled by the rotary embedding (yarn's attention factor)
+        cfg = _config(LlamaConfig, attention_bias=True, mlp_bias=True,
+                      rope_parameters=dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=1024, rope_theta=10000.0))
+        model_cls, api, family = LlamaForCausalLM, hl, "llama"
     else:
         cfg, model_cls, api = _config(MistralConfig, sliding_window=None), MistralForCausalLM, hm
     model = model_cls(cfg).bfloat16().float()           # bf16-representable weights: convert_usa's bf16 cast is then lossless

@@ -397,7 +397,7 @@ def test_whole_layer_step_with_an_mlp_wider_than_the_row_streaming_kernel_takes(
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
 
 
-@pytest.mark.parametrize("shape", ["three_per_kv", "yarn"])
+@pytest.mark.parametrize("shape", ["three_per_kv", "yarn", "heads_narrower_than_hidden"])
 def test_few_launch_steps_on_other_model_shapes(shape):
     # 6 query heads on 2 KV heads (Llama-3.2-3B has 24 on 8); a rotary embedding that scales its cos/sin (yarn: the step takes
     # the tables the model hands over): the seven-launch layer against the general path
@@ -405,6 +405,8 @@ def test_few_launch_steps_on_other_model_shapes(shape):
     torch.manual_seed(0)
     if shape == "three_per_kv":
         cfg = _config(LlamaConfig, hidden_size=768, num_attention_heads=6)
+    elif shape == "heads_narrower_than_hidden":     # Mistral-Nemo: 32 heads of 128 on a hidden size of 5120
+        cfg = _config(LlamaConfig, hidden_size=640)
     else:
         cfg = _config(LlamaConfig, rope_parameters=dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=1024,
                                                         rope_theta=10000.0))

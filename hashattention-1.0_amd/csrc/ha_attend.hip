@@ -131,6 +131,9 @@ struct AttnMask {
     const float *values;
     int64_t stride_b;
     int len, by_slot;
+    // fused launch only (kernel parameter LP): tokens [0, masked_prefix[b]) of sequence b score -inf - the additive mask of
+    // a left-padded batch in the one form it takes there
+    const int32_t *masked_prefix;
 };
 // Token -> slot map of a paged cache (the `Req_to_tokens` table of efficiency/kernels/flash_fwd_sparse.py:396-470): the K/V
 // row of token j of sequence b is row slots[b * stride_b + j] of the cache.  slots == nullptr: the identity.
@@ -624,7 +627,10 @@ __device__ __forceinline__ int fused_round(const FusedSel &f, const FusedRow &fr
 // launches only.
 // SL: the K/V rows are addressed through a token -> slot table (SlotMap); an instantiation of its own, so that launches
 // without a table carry none of it (as a run-time switch it cost the plain launches 0.7 - 1.3 us at 64K tokens x 16).
-template <typename E, int NT, int U, int FW, bool MK = false, bool SL = false>
+// LP: fused launches of a left-padded batch: a list entry below amask.masked_prefix[b] scores -inf (it stays in the list and
+// in the counts: the selection does not see the mask, hashattention_llama.py:593-598).  The token of a row being reduced is
+// read back from the LDS list, so the gather loop carries no extra register.
+template <typename E, int NT, int U, int FW, bool MK = false, bool SL = false, bool LP = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sparse_attend_kernel(const void *__restrict__ q, int64_t q_sb, int64_t q_sh,
                                                            const void *__restrict__ k, const void *__restrict__ v, int64_t kv_sb,
                                                            int64_t kv_sh, int64_t kv_ss, int H, int G,
@@ -637,6 +643,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                                                            const AttnMask amask, int rows_per_seq, const SlotMap smap) {
     using EL = Elem<E>;
     static_assert(!MK || FW == 0, "the additive mask exists for list-fed launches only");
+    static_assert(!LP || (FW > 0 && !SL), "the masked prefix exists for fused launches without a slot table");
     // staged_codes_arrived(true) waits with vmcnt(8): a gather step (and the loop's priming) must put at least eight
     // vector-memory loads per wave behind the staged codes' requests - U key rows and U value rows of 8 elements, one
     // 128-bit load per 16 bytes
@@ -726,9 +733,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     FusedRow fr = {};
     [[maybe_unused]] HistTileRegs<(FW > 0 ? FW : 1), NT> hist_tile;
     int j_max = 0;  // fused: last token of the sequence (list entries are clamped to it: a wrong entry must not become a wild address)
+    [[maybe_unused]] int masked_below = 0;
     if constexpr (FW > 0) {
         int S = seq_lens ? seq_lens[b] : max_S;
         if (S > max_S) S = max_S;
+        if constexpr (LP) masked_below = amask.masked_prefix[b];
         nsplit = nsplit_max;  // every workgroup of the grid owns chunks; an empty one leaves an empty partial
         if (sp >= row_pieces) {  // nothing of this row here (uniform over the workgroup): an empty partial
             if (tid < HA_HEAD_DIM) {
@@ -879,7 +888,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int u = 0; u < U; ++u) {
             float d = row16_sum(EL::dot8(qraw, kr[u])) * scale_log2e;
             if constexpr (MK) d += mk[u];
-            sc[u] = (base + stream + u * NS < r1) ? d : -INFINITY;
+            bool live = base + stream + u * NS < r1;
+            if constexpr (LP) live = live && s_list[min(base + stream + u * NS, kFusedListCap - 1)] >= masked_below;
+            sc[u] = live ? d : -INFINITY;
             mloc = fmaxf(mloc, sc[u]);
         }
         if (mloc > -INFINITY) {  // at least one live row in this stream's step
@@ -1429,7 +1440,8 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
                            int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc, int W, int max_seq_len,
                            const int32_t *seq_lens, int init_budget, int recent_budget, double heavy_budget,
                            const void *select_workspace, size_t select_workspace_bytes, int thresholds_ready, int32_t *out_counts,
-                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream, const SlotMap smap) {
+                           float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream, const SlotMap smap,
+                           const int32_t *masked_prefix = nullptr) {
     int st = validate_qkv(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, B, H, Hkv, out);
     if (st) return st;
     HA_REQUIRE(kcodes && qcodes && select_workspace, HA_ERR_NULL_POINTER, "kcodes/qcodes/select_workspace is NULL");
@@ -1480,11 +1492,13 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
     const dim3 grid(nsplit, H, B), mgrid(H, B);
     const float sl2 = sm_scale * kLog2e;
     const int G = H / Hkv;
-#define HA_FUSED_LAUNCH_SL(E_, U_, FW_, SL_)                                                                                      \
+    HA_REQUIRE(!(masked_prefix && smap.slots), HA_ERR_BAD_SHAPE, "a masked prefix and a slot table cannot be combined");
+    const AttnMask amask{nullptr, 0, 0, 0, masked_prefix};
+#define HA_FUSED_LAUNCH_SL(E_, U_, FW_, SL_, LP_)                                                                                 \
     do {                                                                                                                          \
-        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_, false, SL_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v, \
+        hipLaunchKernelGGL((sparse_attend_kernel<E_, 512, U_, FW_, false, SL_, LP_>), grid, dim3(512), 0, s, q, q_stride_b, q_stride_h, k, v, \
                            kv_stride_b, kv_stride_h, kv_stride_s, H, G, nullptr, (int64_t)kFusedListCap, nullptr, sl2, 0, nsplit, \
-                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, AttnMask{}, 1, smap);                 \
+                           part_acc, part_ml, out, nullptr, 0, 0, seq_lens, max_seq_len, f, amask, 1, smap);                      \
         HA_CHECK_LAUNCH("sparse_attend_kernel (fused selection)");                                                                \
         if (nsplit > 1) {                                                                                                         \
             hipLaunchKernelGGL(merge_splits_kernel<E_>, mgrid, dim3(HA_HEAD_DIM), 0, s, part_acc, part_ml, nullptr, 0,            \
@@ -1492,10 +1506,11 @@ static int sparse_decode_fused_impl(const void *q, int64_t q_stride_b, int64_t q
             HA_CHECK_LAUNCH("merge_splits_kernel");                                                                               \
         }                                                                                                                         \
     } while (0)
-#define HA_FUSED_LAUNCH(E_, U_, FW_)                            \
-    do {                                                        \
-        if (smap.slots) HA_FUSED_LAUNCH_SL(E_, U_, FW_, true);  \
-        else HA_FUSED_LAUNCH_SL(E_, U_, FW_, false);            \
+#define HA_FUSED_LAUNCH(E_, U_, FW_)                                          \
+    do {                                                                      \
+        if (smap.slots) HA_FUSED_LAUNCH_SL(E_, U_, FW_, true, false);         \
+        else if (masked_prefix) HA_FUSED_LAUNCH_SL(E_, U_, FW_, false, true); \
+        else HA_FUSED_LAUNCH_SL(E_, U_, FW_, false, false);                   \
     } while (0)
     if (W == 1) {
         if (kv_dtype == HA_BF16) HA_FUSED_LAUNCH(ElemBF16, 4, 1);
@@ -1521,6 +1536,21 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
                                     kc_stride_h, qcodes, B, H, Hkv, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget, heavy_budget,
                                     select_workspace, select_workspace_bytes, thresholds_ready, out_counts, sm_scale, out, workspace,
                                     workspace_bytes, stream, SlotMap{});
+}
+
+int ha_sparse_decode_fused_prefix_masked(const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *k, const void *v, int kv_dtype,
+                                         int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, const uint32_t *kcodes,
+                                         int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes, int B, int H, int Hkv, int Hc,
+                                         int W, int max_seq_len, const int32_t *seq_lens, int init_budget, int recent_budget,
+                                         double heavy_budget, const void *select_workspace, size_t select_workspace_bytes,
+                                         int thresholds_ready, int32_t *out_counts, const int32_t *masked_prefix, float sm_scale,
+                                         void *out, void *workspace, size_t workspace_bytes, void *stream) {
+    HA_REQUIRE(masked_prefix, HA_ERR_NULL_POINTER, "masked_prefix is NULL");
+    HA_REQUIRE(ha_aligned(masked_prefix, 4), HA_ERR_MISALIGNED, "masked_prefix misaligned");
+    return sparse_decode_fused_impl(q, q_stride_b, q_stride_h, k, v, kv_dtype, kv_stride_b, kv_stride_h, kv_stride_s, kcodes, kc_stride_b,
+                                    kc_stride_h, qcodes, B, H, Hkv, Hc, W, max_seq_len, seq_lens, init_budget, recent_budget, heavy_budget,
+                                    select_workspace, select_workspace_bytes, thresholds_ready, out_counts, sm_scale, out, workspace,
+                                    workspace_bytes, stream, SlotMap{}, masked_prefix);
 }
 
 static int validate_slot_map(const int32_t *slot_of_token, int64_t slot_stride_b, int64_t n_slots) {

@@ -135,6 +135,9 @@ def _declare(lib: C.CDLL) -> C.CDLL:
     lib.ha_sparse_decode_fused_paged.restype = i32
     lib.ha_sparse_decode_fused_paged.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32,
                                                  vp, i32, i32, f64, vp, sz, i32, vp, vp, i64, i64, f32, vp, vp, sz, vp]
+    lib.ha_sparse_decode_fused_prefix_masked.restype = i32
+    lib.ha_sparse_decode_fused_prefix_masked.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32,
+                                                         i32, i32, vp, i32, i32, f64, vp, sz, i32, vp, vp, f32, vp, vp, sz, vp]
     lib.ha_window_partial_bytes.restype = sz
     lib.ha_window_partial_bytes.argtypes = [i32, i32]
     lib.ha_window_partial.restype = i32
@@ -449,16 +452,27 @@ def sparse_decode_fused(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kcode
                         max_seq_len: int, seq_lens: Optional[torch.Tensor], init_budget: int, recent_budget: int,
                         heavy_budget: float, ws_select: torch.Tensor, sm_scale: float, out: torch.Tensor, ws: torch.Tensor,
                         thresholds_ready: bool = True, out_counts: Optional[torch.Tensor] = None,
-                        slots: Optional[torch.Tensor] = None) -> None:
+                        slots: Optional[torch.Tensor] = None, masked_prefix: Optional[torch.Tensor] = None) -> None:
     """Attention over the selection prepared by select_prepare (same codes, budgets and seq_lens); out [B,H,128] in place.
     thresholds_ready=False: the workspace was filled by select_histogram only; counts (optional, [B,H] int32) are written here.
     slots: optional token -> slot table int32 [B, >= max_seq_len] of a paged cache; k, v are then [B or 1 (expanded), Hkv,
-    n_slots, 128] views of the row pool (`ha_sparse_decode_fused_paged`)."""
-    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws, out_counts, slots)
+    n_slots, 128] views of the row pool (`ha_sparse_decode_fused_paged`).
+    masked_prefix: optional int32 [B]: tokens below masked_prefix[b] score -inf, the mask of a left-padded batch
+    (`ha_sparse_decode_fused_prefix_masked`)."""
+    _require_cuda(q, k, v, kcodes, qcodes, seq_lens, ws_select, out, ws, out_counts, slots, masked_prefix)
     lib = load_library()
     B, H, _ = q.shape
     Hc, W = kcodes.shape[1], kcodes.shape[3]
     assert out.is_contiguous() and out.dtype == q.dtype and kcodes.stride(3) == 1 and kcodes.stride(2) == W and qcodes.is_contiguous()
+    if masked_prefix is not None:
+        assert slots is None and masked_prefix.dtype == torch.int32 and masked_prefix.is_contiguous() and masked_prefix.numel() == B
+        _check(lib.ha_sparse_decode_fused_prefix_masked(*_kv_args(q, k, v), _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes),
+                                                        B, H, k.shape[1], Hc, W, max_seq_len, _ptr(seq_lens), init_budget, recent_budget,
+                                                        float(heavy_budget), _ptr(ws_select), ws_select.numel(),
+                                                        1 if thresholds_ready else 0, _ptr(out_counts), _ptr(masked_prefix),
+                                                        float(sm_scale), _ptr(out), _ptr(ws), ws.numel(), _stream(q)),
+               "ha_sparse_decode_fused_prefix_masked")
+        return
     if slots is not None:
         assert slots.shape[1] >= max_seq_len
         _check(lib.ha_sparse_decode_fused_paged(*_kv_args(q, k, v), _ptr(kcodes), kcodes.stride(0), kcodes.stride(1), _ptr(qcodes), B, H,

@@ -61,7 +61,31 @@ def ste_sign(x: torch.Tensor) -> torch.Tensor:
     return SignSTE.apply(x)
 
 
-_MASK_PROBE = [None, None, False]   # last attention mask examined: weak reference, (version, length), "changes something"
+# last attention mask examined: weak reference, (version, length, batch, rows), the `_StepMask` it became (None: changes nothing)
+_MASK_PROBE = [None, None, None]
+
+
+class _StepMask:
+    """The additive attention mask of one forward pass in the forms the kernels take; one object serves all layers of the
+    pass.  `prefix`: int32 [b] on the device when the mask of a single-token step blocks exactly the first prefix[b] tokens of
+    every sequence and nothing else (a left-padded batch) - the fused launch takes that; else None.  `rows()`: fp32
+    [b, q, S]; `table()`: fp32 [b, S] of a single-token step."""
+    __slots__ = ("_m", "b", "q_len", "S", "prefix", "_rows")
+
+    def __init__(self, m, b, q_len, S, prefix):
+        self._m, self.b, self.q_len, self.S, self.prefix, self._rows = m, b, q_len, S, prefix, None
+
+    def rows(self) -> torch.Tensor:
+        if self._rows is None:
+            m = self._m
+            if m.dtype == torch.bool:
+                m = torch.zeros(m.shape, dtype=torch.float32, device=m.device).masked_fill_(torch.logical_not(m), float("-inf"))
+            self._rows = m.float().expand(self.b, self.q_len, self.S).contiguous()
+            self._m = None
+        return self._rows
+
+    def table(self) -> torch.Tensor:
+        return self.rows()[:, 0]
 
 LSH_PAD = 3     # zero coordinates after the lifted one: the encode kernels take input widths that are multiples of 4
 
@@ -453,29 +477,40 @@ class HeavyHitterMixin:
 
     def _additive_mask(self, attention_mask, b: int, q_len: int, S: int):
         """The reference adds `attention_mask` [b, 1, q, S] to the scores before the keep-mask and the softmax (:593-598).
-        Returns it as fp32 [b, q, S], or None when it changes nothing for any row's causal part (the kernels apply the
+        Returns it as a `_StepMask`, or None when it changes nothing for any row's causal part (the kernels apply the
         causal structure themselves), which is the case for every unpadded batch.  A boolean mask (True = attend) is
-        accepted as well.  Deciding costs one device-to-host read per forward pass, not per layer: the layers of a model
-        are handed the same tensor object."""
+        accepted as well.  Deciding costs one device-to-host read per forward pass, not per layer, and the fp32 form is
+        made once per pass: the layers of a model are handed the same tensor object."""
         if attention_mask is None:
             return None
         if attention_mask.dim() != 4 or attention_mask.shape[1] != 1 or attention_mask.shape[2] != q_len \
                 or attention_mask.shape[3] < S or attention_mask.shape[0] not in (1, b):
             raise ValueError(f"Attention mask should be of size {(b, 1, q_len, S)}, but is {tuple(attention_mask.size())}")
         probe = _MASK_PROBE
-        hit = probe[0] is not None and probe[0]() is attention_mask and probe[1] == (attention_mask._version, S)
-        if not hit:
-            m = attention_mask[:, 0, :, :S]
-            causal = torch.tril(torch.ones(q_len, S, dtype=torch.bool, device=m.device), diagonal=S - q_len)
-            blocked = torch.logical_not(m) if m.dtype == torch.bool else m != 0
-            probe[0], probe[1], probe[2] = weakref.ref(attention_mask), (attention_mask._version, S), \
-                bool((blocked & causal).any().item())
-        if not probe[2]:
-            return None
+        key = (attention_mask._version, S, b, q_len)
+        if probe[0] is not None and probe[0]() is attention_mask and probe[1] == key:
+            return probe[2]
         m = attention_mask[:, 0, :, :S]
+        if m.dtype != torch.bool and not m.is_floating_point():
+            m = m.float()
         if m.dtype == torch.bool:
-            m = torch.zeros(m.shape, dtype=torch.float32, device=m.device).masked_fill_(torch.logical_not(m), float("-inf"))
-        return m.float().expand(b, q_len, S).contiguous()
+            blocked = torch.logical_not(m)
+            hard = blocked
+        else:
+            blocked = m != 0
+            hard = (m == torch.finfo(m.dtype).min) | (m == float("-inf"))      # what the library writes for "do not attend"
+        if q_len == 1:
+            # a left-padded batch: per sequence a prefix is blocked for good, nothing else
+            row = blocked[:, 0]
+            n = row.sum(-1)
+            is_prefix = (row == (torch.arange(S, device=m.device)[None, :] < n[:, None])).all() & (hard[:, 0] == row).all()
+            matters, is_prefix = torch.stack([row.any(), is_prefix]).tolist()
+            prefix = n.to(torch.int32).expand(b).contiguous() if (matters and is_prefix) else None
+        else:
+            causal = torch.tril(torch.ones(q_len, S, dtype=torch.bool, device=m.device), diagonal=S - q_len)
+            matters, prefix = bool((blocked & causal).any().item()), None
+        probe[0], probe[1], probe[2] = weakref.ref(attention_mask), key, (_StepMask(m, b, q_len, S, prefix) if matters else None)
+        return probe[2]
 
     def _sparse_attention(self, query_states, key_states, value_states, attention_mask=None):
         """query [b, H, q, d] (q <= 128), key/value [b, Hkv, S, d] holding the whole cache including the new tokens.
@@ -502,7 +537,7 @@ class HeavyHitterMixin:
             try:
                 hl.step(query_states, key_states, value_states, S, out[:, :, 0],
                         hash_inputs=None if key_hash is key_states else (key_hash, query_hash),
-                        attn_mask=None if amask is None else amask[:, 0])
+                        attn_mask=amask)
             finally:
                 hl.heavy_budget = saved
             return out
@@ -512,7 +547,8 @@ class HeavyHitterMixin:
         hl.encode_keys(key_hash[:, :, S - q_len:S], pos0=S - q_len)
         hl.n_cached = S
         return hl.chunk_step(query_states, key_states, value_states, S, out, heavy_abs,
-                             q_hash=None if query_hash is query_states else query_hash, attn_mask=amask)
+                             q_hash=None if query_hash is query_states else query_hash,
+                             attn_mask=None if amask is None else amask.rows())
 
     # ---- the single-token step as five launches
     def _fused_qkv_weight(self) -> torch.Tensor:
@@ -528,7 +564,7 @@ class HeavyHitterMixin:
         return hit[1]
 
     def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
-        """(This layer's `PreallocatedLayer` of `cache`, the additive mask as fp32 [b, 1, S] or None when it changes nothing)
+        """(This layer's `PreallocatedLayer` of `cache`, the additive mask as a `_StepMask` or None when it changes nothing)
         when the step can take `_fast_decode`, else None: one new token per sequence, inference, bf16 hidden states and
         projections without biases, 128-wide heads, up to 16 sequences, a learned hash whose codes can be cached, no KV
         offloading, and a cache whose layers append in place."""
@@ -606,8 +642,9 @@ class HeavyHitterMixin:
         saved = hl.heavy_budget
         hl.heavy_budget = 0.0 if heavy == 0 else heavy + 0.5
         try:
-            # a mask that matters (a padded batch): selection into memory, then the masked gather (reference :593-598)
-            hl._select_attend(sc["q"], kbuf, vbuf, S, sc["attn"], None, attn_mask=None if amask is None else amask[:, 0])
+            # a mask that matters (reference :593-598): the prefix of a left-padded batch goes into the fused launch; any other
+            # takes the selection into memory and the masked gather
+            hl._select_attend(sc["q"], kbuf, vbuf, S, sc["attn"], None, attn_mask=amask)
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)

@@ -141,10 +141,11 @@ class HashDecodeLayer:
                             self.recent_budget, self.heavy_budget, self.counts, self.ws_select, self.mode, self.depth)
 
     def attend_fused(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, max_seq_len: int,
-                     seq_lens: Optional[torch.Tensor]) -> None:
+                     seq_lens: Optional[torch.Tensor], masked_prefix: Optional[torch.Tensor] = None) -> None:
         _ops.sparse_decode_fused(q3, k, v, self.codes, self.qcodes.view(self.B, self.H, self.W), max_seq_len, seq_lens,
                                  self.init_budget, self.recent_budget, self.heavy_budget, self.ws_select, self.sm_scale, out,
-                                 self.ws_fused, thresholds_ready=not self.local_thresholds, out_counts=self.counts)
+                                 self.ws_fused, thresholds_ready=not self.local_thresholds, out_counts=self.counts,
+                                 masked_prefix=masked_prefix)
 
     def attend(self, q3: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
                attn_mask: Optional[torch.Tensor] = None) -> None:
@@ -192,6 +193,15 @@ class HashDecodeLayer:
         return self._select_attend(q3, k_cache, v_cache, seq_len, out, seq_lens, main, attn_mask)
 
     def _select_attend(self, q3, k_cache, v_cache, seq_len, out, seq_lens, main=None, attn_mask=None):
+        """attn_mask: fp32 [B, >= seq_len] added to the scores, or an object that describes the mask of a left-padded batch -
+        `.prefix` int32 [B] (tokens below it are blocked) and `.table()` for the fp32 form: the fused launch takes the
+        prefix, every other path the table."""
+        if attn_mask is not None and not torch.is_tensor(attn_mask):
+            if attn_mask.prefix is not None and self.use_fused and self.fused_ok and not self.overlap_windows:
+                self.select_prepare(seq_len, seq_lens)
+                self.attend_fused(q3, k_cache, v_cache, out, seq_len, seq_lens, masked_prefix=attn_mask.prefix)
+                return out
+            attn_mask = attn_mask.table()
         if attn_mask is not None:
             if self.overlap_windows:
                 raise RuntimeError("an attention mask is not supported together with the second-stream window partial")

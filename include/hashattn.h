@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define HA_VERSION 201 /* 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
+#define HA_VERSION 202 /* 0.2.2: + ha_sparse_decode_fused_prefix_masked; the dense baseline and the window partial take any number of query heads per KV head; 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
 
 typedef enum ha_status {
     HA_OK = 0,
@@ -337,6 +337,25 @@ int ha_sparse_decode_fused(const void *q, int64_t q_stride_b, int64_t q_stride_h
                            const void *select_workspace, size_t select_workspace_bytes,
                            int thresholds_ready, int32_t *out_counts,
                            float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * ha_sparse_decode_fused for a LEFT-PADDED batch: the additive attention mask the reference adds to the scores
+ * (hashattention_llama.py:593-598) blocks, for one new token per sequence, exactly the padding in front of each prompt, so
+ * it is handed over as one number per sequence: tokens [0, masked_prefix[b]) of sequence b score -inf.  As in the
+ * reference the selection does not see the mask: such tokens are counted and listed like any other (out_counts as
+ * ha_sparse_decode_fused), they only add nothing to the softmax.  Output equals ha_select + ha_sparse_decode_masked with the
+ * mask {-inf below masked_prefix[b], 0 from there on} up to the order of the fp32 additions.  masked_prefix int32 [B] in
+ * device memory; every other argument as ha_sparse_decode_fused.  A row whose every listed token is masked gives zeros.
+ */
+int ha_sparse_decode_fused_prefix_masked(const void *q, int64_t q_stride_b, int64_t q_stride_h,
+                                         const void *k, const void *v, int kv_dtype,
+                                         int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                                         const uint32_t *kcodes, int64_t kc_stride_b, int64_t kc_stride_h, const uint32_t *qcodes,
+                                         int B, int H, int Hkv, int Hc, int W, int max_seq_len, const int32_t *seq_lens,
+                                         int init_budget, int recent_budget, double heavy_budget,
+                                         const void *select_workspace, size_t select_workspace_bytes,
+                                         int thresholds_ready, int32_t *out_counts, const int32_t *masked_prefix,
+                                         float sm_scale, void *out, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * The same two attention launches over a cache addressed through a token -> slot table: the row of token j of sequence b

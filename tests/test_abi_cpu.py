@@ -35,7 +35,7 @@ def test_every_declared_symbol_is_exported(lib):
             "ha_device_count"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.ha_version() == 201
+    assert lib.ha_version() == 202
     assert lib.ha_status_string(0) == b"ok" and lib.ha_status_string(HA_ERR_WS) == b"workspace missing or too small"
 
 

@@ -120,8 +120,25 @@ def _run(model, ids, am, steps):
     return outs
 
 
-def test_left_padded_batch_through_the_patched_model():
-    print("\n[case] patched model, left-padded batch", flush=True)
+@pytest.mark.parametrize("fused", [False, True])
+def test_left_padded_batch_through_the_patched_model(fused, monkeypatch):
+    # fused: batches of 32 and more (sequence, head) rows take the fused select-attend launch, which is handed the padding as one
+    # number per sequence; here the threshold is lowered so that the tiny model takes it (and the call is counted)
+    print(f"\n[case] patched model, left-padded batch, fused launch: {fused}", flush=True)
+    from hashattention import decode
+    seen = []
+    if fused:
+        allocate, launch = decode.HashDecodeLayer.allocate, _ops.sparse_decode_fused
+
+        def allocate_low(self, *a, **kw):
+            self.fused_min_rows = 1
+            return allocate(self, *a, **kw)
+
+        def launch_counted(*a, **kw):
+            seen.append(kw.get("masked_prefix"))
+            return launch(*a, **kw)
+        monkeypatch.setattr(decode.HashDecodeLayer, "allocate", allocate_low)
+        monkeypatch.setattr(_ops, "sparse_decode_fused", launch_counted)
     torch.manual_seed(7)
     cfg = _config(LlamaConfig)
     model = LlamaForCausalLM(cfg).bfloat16().float()
@@ -142,6 +159,8 @@ def test_left_padded_batch_through_the_patched_model():
         err = (a - b).abs().max().item()
         print(f"  max |logit difference| {err:.2e}", flush=True)
         assert a.shape == b.shape and err < 2e-3, err
+    if fused:       # three single-token steps of two layers went through the fused launch with the prefix [0, 45]
+        assert len(seen) == 6 and all(p is not None and p.tolist() == [0, 45] for p in seen), seen
     # the mask matters: without it the padded sequence's logits differ, the unpadded one's do not
     hl.reset_usa(model)
     plain = _run(model, ids.to(DEV), torch.ones_like(am).to(DEV), steps)
@@ -174,3 +193,92 @@ def test_generate_with_a_left_padded_batch():
     print("  new tokens:", got[:, 150:].tolist(), flush=True)
     assert got.shape == (2, 156) and torch.equal(got, want)
     assert model.model.layers[0].self_attn._hash_layer.n_cached == 155      # the last token is sampled, not fed back
+
+
+@pytest.mark.parametrize("case", ["ragged", "uniform_split_rows", "wide_codes"])
+def test_fused_launch_with_a_masked_prefix_matches_the_oracle(case):
+    # the mask of a left-padded batch inside the fused select-attend launch (ha_sparse_decode_fused_prefix_masked): the tokens in
+    # front of masked_prefix[b] stay selected and counted - the selection does not see the mask, hashattention_llama.py:593-598 -
+    # and add nothing to the softmax.  Against the oracle's gather attention with -inf on those entries, and against
+    # ha_select + ha_sparse_decode_masked with the same mask as a table.
+    from oracle import c_oracle
+    from hashattention.synthetic import make_problem
+    from tests.parity_util import ATOL, oracle_codes, small_workload, to_i32
+    print(f"\n[case] fused launch, masked prefix: {case}", flush=True)
+    if case == "ragged":         # prefixes: none, inside the sink window, into the candidates, all but the last token, everything
+        w = small_workload(batch=5, seq_lens=[1500, 1111, 3000, 700, 900], heavy_budget=0.125, seed=41)
+        prefix, ragged = [0, 9, 1200, 699, 900], True
+    elif case == "uniform_split_rows":   # long equal rows (cut into pieces), lengths given on the host
+        w = small_workload(batch=2, seq_lens=[20000, 20000], n_q_heads=4, n_kv_heads=2, n_code_heads=4, heavy_budget=1 / 16, seed=42,
+                           dtype=torch.float16)
+        prefix, ragged = [4097, 15], False
+    else:                        # 64-bit codes
+        w = small_workload(batch=3, seq_lens=[5000, 2500, 4000], lth_num_layers=2, lth_final_dim=64, heavy_budget=0.25, seed=43,
+                           dtype=torch.float32)
+        prefix, ragged = [100, 0, 3990], True
+    p = make_problem(w)
+    B, H, Hc, S, W = w.batch, w.n_q_heads, w.n_code_heads, w.max_seq_len, w.code_words
+    _, _, kc64, qc64 = oracle_codes(p)
+    kc_np, qc_np, seq_np = to_i32(kc64), to_i32(qc64), p.seq_lens.numpy()
+    kcodes, qcodes = torch.from_numpy(kc_np).to(DEV), torch.from_numpy(qc_np).to(DEV)
+    q3, k, v = p.q[:, :, 0, :].contiguous().to(DEV), p.k.to(DEV), p.v.to(DEV)
+    seq = p.seq_lens.to(DEV) if ragged else None
+    assert _ops.fused_applies(B, H, Hc, W, S, w.init_budget, w.recent_budget, w.heavy_budget)
+    cap = max(w.n_selected(s) for s in w.seq_lens)
+    idx_ref, counts_ref = c_oracle.select(kc_np, qc_np, seq_np, w.init_budget, w.recent_budget, w.heavy_budget, cap, mode=0, depth=0)
+    pre = torch.tensor(prefix, dtype=torch.int32, device=DEV)
+    sm = 1 / 128 ** 0.5
+    ws = _ops.workspace(_ops.select_workspace_bytes(B, H, Hc, W, S), DEV)
+    ws4 = _ops.workspace(_ops.sparse_decode_fused_workspace_bytes(B, H, Hc, S), DEV)
+    outs = []
+    for ready in (True, False):
+        if not ready and not _ops.fused_local_thresholds(B, Hc, S):
+            continue
+        counts = torch.full((B, H), -5, dtype=torch.int32, device=DEV)
+        out = torch.empty(B, H, 128, dtype=w.dtype, device=DEV)
+        if ready:
+            _ops.select_prepare(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, counts, ws)
+        else:
+            _ops.select_histogram(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, ws)
+        _ops.sparse_decode_fused(q3, k, v, kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws, sm, out, ws4,
+                                 thresholds_ready=ready, out_counts=counts, masked_prefix=pre)
+        torch.cuda.synchronize()
+        assert np.array_equal(counts.cpu().numpy(), counts_ref), "the mask must not change what is selected"
+        outs.append(out)
+    if len(outs) == 2:
+        assert torch.equal(outs[0], outs[1])
+    got = outs[0].float().cpu()
+    worst = 0.0
+    G = H // w.n_kv_heads
+    for b in range(B):
+        for h in range(H):
+            n = int(counts_ref[b, h])
+            ii = torch.from_numpy(idx_ref[b, h, :n].astype(np.int64))
+            terms = torch.where(ii < prefix[b], torch.tensor(float("-inf")), torch.tensor(0.0))
+            if n == 0 or not torch.isfinite(terms).any():
+                assert (got[b, h] == 0).all(), (b, h)
+                continue
+            want = orc.sparse_attend(p.q[b, h, 0], p.k[b, h // G], p.v[b, h // G], ii.numpy(), sm, slot_mask=terms)
+            worst = max(worst, (got[b, h] - want).abs().max().item())
+    print(f"  max abs error {worst:.2e}", flush=True)
+    assert worst <= ATOL[w.dtype]
+    # the same mask as a table through the two-launch path
+    idx = torch.full((B, H, cap), -1, dtype=torch.int32, device=DEV)
+    counts = torch.zeros(B, H, dtype=torch.int32, device=DEV)
+    _ops.select(kcodes, qcodes, S, p.seq_lens.to(DEV), w.init_budget, w.recent_budget, w.heavy_budget, idx, counts, ws)
+    table = torch.zeros(B, S, device=DEV)
+    for b in range(B):
+        table[b, :prefix[b]] = float("-inf")
+    out2 = torch.empty_like(outs[0])
+    _ops.sparse_decode(q3, k, v, idx, counts, sm, out2, _ops.workspace(_ops.sparse_decode_workspace_bytes(B, H, cap), DEV), mask=table)
+    torch.cuda.synchronize()
+    same = (out2.float() - outs[0].float()).abs().max().item()
+    assert same <= (1e-5 if w.dtype == torch.float32 else 1e-2), same
+    # a prefix of zero everywhere is the plain fused launch, bit for bit
+    out3, out4 = torch.empty_like(out2), torch.empty_like(out2)
+    _ops.select_prepare(kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, counts, ws)
+    _ops.sparse_decode_fused(q3, k, v, kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws, sm, out3, ws4)
+    _ops.sparse_decode_fused(q3, k, v, kcodes, qcodes, S, seq, w.init_budget, w.recent_budget, w.heavy_budget, ws, sm, out4, ws4,
+                             masked_prefix=torch.zeros(B, dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(out3, out4)

@@ -322,17 +322,24 @@ def hf_path_bench(args, torch):
             cache.update(k, v, l)
             del k, v
 
-    def time_tokens(model, cache, n_steps, n_warm):
+    def time_tokens(model, cache, n_steps, n_warm, padded=False):
         ids = torch.randint(0, 128256, (B, 1), device=dev)
+
+        def one():
+            am = None
+            if padded:      # a left-padded batch, as batched generation makes them: five padding tokens in front of sequence 0
+                am = torch.ones(B, cache.get_seq_length() + 1, dtype=torch.long, device=dev)
+                am[0, :5] = 0
+            model(ids, attention_mask=am, past_key_values=cache, use_cache=True)
         with torch.no_grad():
             for _ in range(n_warm):                      # the first pass hashes the 131071 cached keys of every layer
-                model(ids, past_key_values=cache, use_cache=True)
+                one()
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
             e0.record()
             for _ in range(n_steps):
-                model(ids, past_key_values=cache, use_cache=True)
+                one()
             e1.record()
             host_ms = (time.perf_counter() - t0) * 1e3 / n_steps     # time to issue a step from Python (no wait inside)
             torch.cuda.synchronize()
@@ -345,6 +352,9 @@ def hf_path_bench(args, torch):
         cache = PreallocatedCache(capacity=S + 256, num_layers=L)
         fill(cache, L, S - 1 - warm)
         ms_pre, host_pre = time_tokens(model, cache, steps, warm)
+        # the same steps on a left-padded batch (the padding mask inside the fused launch)
+        cache.crop(-(steps + warm))
+        ms_padded, _ = time_tokens(model, cache, steps, warm, padded=True)
         # the same with only the attention module in few launches (the decoder layer around it through the library's own forward)
         for lyr in model.model.layers:
             lyr.self_attn.fast_layer = False
@@ -393,7 +403,7 @@ def hf_path_bench(args, torch):
             e1.record()
             torch.cuda.synchronize()
         ms_dec = e0.elapsed_time(e1) / steps
-        out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre,
+        out[L] = dict(patched_preallocated_ms=ms_pre, patched_preallocated_host_issue_ms=host_pre, patched_left_padded_batch_ms=ms_padded,
                       patched_preallocated_attention_module_only_ms=ms_attn_fast, patched_dynamic_cache_adopted_ms=ms_adopted,
                       patched_dynamic_cache_ms=ms_dyn,
                       decoder_generate_ms=ms_dec, patched_attention_module_us=ms_attn * 1e3)
@@ -413,7 +423,8 @@ def hf_path_bench(args, torch):
         "per_layer_slope": per_layer,
         "how": "single-token forward passes of the patched model, eager launches from Python, HIP events around the timed passes "
                "(patched_preallocated: whole decoder layers in seven launches each; ..._attention_module_only: the attention module in five "
-               "launches inside the library's own decoder layer; patched_dynamic_cache_adopted: the caller hands over a plain DynamicCache, "
+               "launches inside the library's own decoder layer; patched_left_padded_batch: the seven-launch steps with an attention mask that "
+               "blocks five padding tokens in front of sequence 0, handed to the fused launch as one number per sequence; patched_dynamic_cache_adopted: the caller hands over a plain DynamicCache, "
                "whose layers the attention modules turn into in-place ones at the first decode step; patched_dynamic_cache: the same "
                "with that switched off, torch.cat per layer and token); "
                "per-layer = difference between the two layer counts; decoder = LlamaShapedDecoder.from_hf(...).generate (one HIP graph "

@@ -61,8 +61,9 @@ def ste_sign(x: torch.Tensor) -> torch.Tensor:
     return SignSTE.apply(x)
 
 
-# last attention mask examined: weak reference, (version, length, batch, rows), the `_StepMask` it became (None: changes nothing)
-_MASK_PROBE = [None, None, None]
+# last attention mask examined, as ONE tuple so that a reader never sees parts of two examinations: (weak reference,
+# (version, length, batch, rows), the `_StepMask` it became or None when it changes nothing)
+_MASK_PROBE = [(None, None, None)]
 
 
 class _StepMask:
@@ -486,10 +487,10 @@ class HeavyHitterMixin:
         if attention_mask.dim() != 4 or attention_mask.shape[1] != 1 or attention_mask.shape[2] != q_len \
                 or attention_mask.shape[3] < S or attention_mask.shape[0] not in (1, b):
             raise ValueError(f"Attention mask should be of size {(b, 1, q_len, S)}, but is {tuple(attention_mask.size())}")
-        probe = _MASK_PROBE
         key = (attention_mask._version, S, b, q_len)
-        if probe[0] is not None and probe[0]() is attention_mask and probe[1] == key:
-            return probe[2]
+        last = _MASK_PROBE[0]
+        if last[0] is not None and last[0]() is attention_mask and last[1] == key:
+            return last[2]
         m = attention_mask[:, 0, :, :S]
         if m.dtype != torch.bool and not m.is_floating_point():
             m = m.float()
@@ -509,8 +510,9 @@ class HeavyHitterMixin:
         else:
             causal = torch.tril(torch.ones(q_len, S, dtype=torch.bool, device=m.device), diagonal=S - q_len)
             matters, prefix = bool((blocked & causal).any().item()), None
-        probe[0], probe[1], probe[2] = weakref.ref(attention_mask), key, (_StepMask(m, b, q_len, S, prefix) if matters else None)
-        return probe[2]
+        step_mask = _StepMask(m, b, q_len, S, prefix) if matters else None
+        _MASK_PROBE[0] = (weakref.ref(attention_mask), key, step_mask)
+        return step_mask
 
     def _sparse_attention(self, query_states, key_states, value_states, attention_mask=None):
         """query [b, H, q, d] (q <= 128), key/value [b, Hkv, S, d] holding the whole cache including the new tokens.

@@ -641,6 +641,9 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
 HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1
 
 
+LINEAR_SKINNY_MAX_ROWS = 16     # rows of x that ha_linear_skinny takes
+
+
 def _linear_skinny_unchecked(x, w, out, residual=None, norm_weight=None, eps=0.0, swiglu=False):
     """`linear_skinny` for callers that made these tensors themselves (2-D bf16 on one GPU, rows contiguous): no checks on
     the Python side - a decode layer's seven launches should not cost the host more than they cost the GPU.  The library

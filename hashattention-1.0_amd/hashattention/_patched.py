@@ -568,12 +568,12 @@ class HeavyHitterMixin:
     def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
         """(This layer's `PreallocatedLayer` of `cache`, the additive mask as a `_StepMask` or None when it changes nothing)
         when the step can take `_fast_decode`, else None: one new token per sequence, inference, bf16 hidden states and
-        projections without biases, 128-wide heads, up to 16 sequences, a learned hash whose codes can be cached, no KV
-        offloading, and a cache whose layers append in place."""
+        projections without biases, 128-wide heads, a learned hash whose codes can be cached, no KV offloading, and a cache
+        whose layers append in place."""
         if not self.fast_decode or torch.is_grad_enabled() or self.train_usa or self.offloading_length is not None:
             return None
         b, q_len, hidden = hidden_states.shape
-        if q_len != 1 or b > 16 or hidden % 32 or self.head_dim != 128 or hidden_states.dtype != torch.bfloat16 \
+        if q_len != 1 or hidden % 32 or self.head_dim != 128 or hidden_states.dtype != torch.bfloat16 \
                 or not hidden_states.is_contiguous() or position_embeddings is None:
             return None
         own = self._modules     # plain nn.Linear projections only: a wrapper around one (an adapter) has a forward of its own
@@ -612,7 +612,7 @@ class HeavyHitterMixin:
 
     def _fast_decode(self, hidden_states, position_embeddings, slot, norm=None, residual=None, amask=None):
         """The decode branch (reference :551-625) for one new token per sequence in five launches: fused QKV projection
-        (ha_linear_skinny), rotary embedding + in-place cache append + both hashes (ha_rope_encode_step_cos_sin), distance
+        (ha_linear_skinny; the library's GEMM on the stacked weight for more than 16 sequences), rotary embedding + in-place cache append + both hashes (ha_rope_encode_step_cos_sin), distance
         histograms, selection fused into the gather attention, output projection.  For the decoder layer around it
         (`fast_decoder_layer_forward`): `norm` = (weight, eps) of an RMSNorm applied to hidden_states inside the QKV projection,
         `residual` [b, hidden] added inside the output projection."""
@@ -625,7 +625,9 @@ class HeavyHitterMixin:
                       q=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev),
                       attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
             self.__dict__["_fast_scratch"] = sc
-        if norm is None:
+        if b > _ops.LINEAR_SKINNY_MAX_ROWS:     # more sequences than the projection kernel takes: the library's GEMM, still one call
+            torch.mm(hidden_states[:, 0, :], self._fused_qkv_weight().t(), out=sc["qkv"])
+        elif norm is None:
             _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
         else:
             _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"], norm_weight=norm[0], eps=norm[1])
@@ -650,7 +652,10 @@ class HeavyHitterMixin:
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
-        _ops._linear_skinny_unchecked(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
+        if b > _ops.LINEAR_SKINNY_MAX_ROWS:
+            torch.mm(sc["attn"].view(b, H * d), self.o_proj.weight.t(), out=out.view(b, hidden))
+        else:
+            _ops._linear_skinny_unchecked(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
 
     def _adopt_cache_layer(self, cache) -> None:

@@ -341,9 +341,86 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const void *__restrict__ ga
     ha_store_elem(out, (int64_t)b * F + i, ha_round_to(g / (1.0f + __expf(-g)), dtype) * u, dtype);
 }
 
+// One workgroup per row: y = round(round(x * rsqrt(mean x^2 + eps)) * w), both roundings to the element type - the RMSNorm
+// modules of transformers (LlamaRMSNorm: the normalised row is cast back to the input type before it meets the weight) and of
+// the reference's harness (efficiency/model.py:314-319).  VEC: 16-bit elements, rows of whole 16-byte pieces.
+template <bool VEC>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const void *__restrict__ x, int64_t x_sm, const void *__restrict__ w, int dtype,
+                                                      int K, float eps, void *__restrict__ y, int64_t y_sm) {
+    __shared__ float s_sum[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const char *xr = (const char *)x + (int64_t)m * x_sm * (dtype == HA_F32 ? 4 : 2);
+    char *yr = (char *)y + (int64_t)m * y_sm * (dtype == HA_F32 ? 4 : 2);
+    auto widen = [&](uint32_t bits16) {
+        return dtype == HA_BF16 ? __uint_as_float(bits16 << 16) : __half2float(__ushort_as_half((unsigned short)bits16));
+    };
+    float a = 0.f;
+    if constexpr (VEC) {
+        for (int k = tid * 8; k < K; k += 256 * 8) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(xr + k * 2);
+            const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float lo = widen(p[i] & 0xffffu), hi = widen(p[i] >> 16);
+                a = fmaf(lo, lo, fmaf(hi, hi, a));
+            }
+        }
+    } else {
+        for (int k = tid; k < K; k += 256) {
+            const float v = ha_load_elem(xr, k, dtype);
+            a = fmaf(v, v, a);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) a += __shfl_xor(a, o);
+    if ((tid & 63) == 0) s_sum[tid >> 6] = a;
+    __syncthreads();
+    const float rstd = rsqrtf((s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3]) / (float)K + eps);
+    auto narrow = [&](float f) {
+        return dtype == HA_BF16 ? ha_f32_to_bf16_bits(f) : (uint32_t)__half_as_ushort(__float2half(f));
+    };
+    if constexpr (VEC) {
+        for (int k = tid * 8; k < K; k += 256 * 8) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(xr + k * 2);
+            const uint4 g = *reinterpret_cast<const uint4 *>((const char *)w + k * 2);
+            const uint32_t p[4] = {v.x, v.y, v.z, v.w}, q[4] = {g.x, g.y, g.z, g.w};
+            uint32_t r[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float lo = ha_round_to(widen(p[i] & 0xffffu) * rstd, dtype) * widen(q[i] & 0xffffu);
+                const float hi = ha_round_to(widen(p[i] >> 16) * rstd, dtype) * widen(q[i] >> 16);
+                r[i] = narrow(lo) | (narrow(hi) << 16);
+            }
+            *reinterpret_cast<uint4 *>(yr + k * 2) = make_uint4(r[0], r[1], r[2], r[3]);
+        }
+    } else {
+        for (int k = tid; k < K; k += 256)
+            ha_store_elem(yr, k, ha_round_to(ha_load_elem(xr, k, dtype) * rstd, dtype) * ha_load_elem(w, k, dtype), dtype);
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int ha_rmsnorm(const void *x, int64_t x_stride_m, const void *weight, int dtype, int M, int K, float eps, void *out, int64_t out_stride_m,
+               void *stream) {
+    HA_REQUIRE(x && weight && out, HA_ERR_NULL_POINTER, "x/weight/out is NULL");
+    HA_REQUIRE(dtype == HA_F32 || dtype == HA_BF16 || dtype == HA_F16, HA_ERR_BAD_DTYPE, "unknown dtype %d", dtype);
+    HA_REQUIRE(M > 0 && K > 0 && x_stride_m >= K && out_stride_m >= K && eps >= 0.f, HA_ERR_BAD_SHAPE, "bad rmsnorm shape");
+    int st = ha_require_device();
+    if (st) return st;
+    const bool vec = dtype != HA_F32 && K % 8 == 0 && x_stride_m % 8 == 0 && out_stride_m % 8 == 0 && ha_aligned(x, 16) &&
+                     ha_aligned(weight, 16) && ha_aligned(out, 16);
+    if (vec)
+        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(M), dim3(256), 0, (hipStream_t)stream, x, x_stride_m, weight, dtype, K, eps, out,
+                           out_stride_m);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(M), dim3(256), 0, (hipStream_t)stream, x, x_stride_m, weight, dtype, K, eps, out,
+                           out_stride_m);
+    HA_CHECK_LAUNCH("rmsnorm_kernel");
+    return HA_OK;
+}
 
 int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int H, int Hkv, int pos, const int32_t *pos_dev,
                    const float *inv_freq, void *q_out, void *k_cache, void *v_cache, int64_t kv_stride_b, int64_t kv_stride_h,

@@ -138,6 +138,8 @@ def _declare(lib: C.CDLL) -> C.CDLL:
     lib.ha_sparse_decode_fused_prefix_masked.restype = i32
     lib.ha_sparse_decode_fused_prefix_masked.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32,
                                                          i32, i32, vp, i32, i32, f64, vp, sz, i32, vp, vp, f32, vp, vp, sz, vp]
+    lib.ha_rmsnorm.restype = i32
+    lib.ha_rmsnorm.argtypes = [vp, i64, vp, i32, i32, i32, f32, vp, i64, vp]
     lib.ha_window_partial_bytes.restype = sz
     lib.ha_window_partial_bytes.argtypes = [i32, i32]
     lib.ha_window_partial.restype = i32
@@ -636,6 +638,15 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and out.is_contiguous() and out.dtype == gate_up.dtype
     B, F = out.shape
     _check(load_library().ha_swiglu(_ptr(gate_up), gate_up.stride(0), _DTYPE[gate_up.dtype], B, F, _ptr(out), _stream(gate_up)), "ha_swiglu")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """x [M, K] -> out [M, K] = round(round(x * rsqrt(mean x^2 + eps)) * weight): the two roundings of LlamaRMSNorm."""
+    _require_cuda(x, weight, out)
+    assert x.dim() == 2 and out.shape == x.shape and x.stride(1) == 1 and out.stride(1) == 1 and weight.is_contiguous()
+    assert weight.dtype == x.dtype == out.dtype and weight.numel() == x.shape[1]
+    _check(load_library().ha_rmsnorm(_ptr(x), x.stride(0), _ptr(weight), _DTYPE[x.dtype], x.shape[0], x.shape[1], float(eps), _ptr(out),
+                                     out.stride(0), _stream(x)), "ha_rmsnorm")
 
 
 HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1

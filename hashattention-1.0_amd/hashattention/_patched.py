@@ -903,11 +903,15 @@ def _layer_modules(layer):
     return now if ok else False
 
 
+FUSED_LAYER_MAX_ROWS = 8     # sequences for which the projection kernel takes the norm in front and SwiGLU behind
+
+
 def _layer_takes_fast_path(layer, hidden_states):
-    """The layer's modules (`_layer_modules`) when a single-token step of up to 8 sequences can run as seven launches: bf16
-    weights, hidden states of at most 16384 elements (the projection kernel's fused forms), and no forward hook on a module that this
-    path would not call (activation capture, adapters that wrap a forward); else False."""
-    if hidden_states.shape[0] > 8 or hidden_states.shape[1] != 1:
+    """The layer's modules (`_layer_modules`) when a single-token step can run as a handful of launches - seven for up to 8
+    sequences, twelve calls above: bf16 weights, for the seven-launch form hidden states of at most 16384 elements (the
+    projection kernel's fused forms), and no forward hook on a module that this path would not call (activation capture,
+    adapters that wrap a forward); else False."""
+    if hidden_states.shape[1] != 1:
         return False
     mods = _layer_modules(layer)
     if not mods:
@@ -918,7 +922,7 @@ def _layer_takes_fast_path(layer, hidden_states):
         if m._forward_hooks or m._forward_pre_hooks:
             return False
     gate, down = mods[3], mods[5]
-    if gate.in_features > 16384:        # the norm-in-front form keeps a row of hidden states in registers
+    if gate.in_features > 16384 and hidden_states.shape[0] <= FUSED_LAYER_MAX_ROWS:    # the norm-in-front form keeps a row of hidden states in registers
         return False
     bf16 = torch.bfloat16
     if gate.weight.dtype != bf16 or mods[4].weight.dtype != bf16 or down.weight.dtype != bf16 or mods[1].weight.dtype != bf16 \
@@ -930,7 +934,7 @@ def _layer_takes_fast_path(layer, hidden_states):
 def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
                                position_embeddings=None, **kwargs):
     """`forward` of a transformers decoder layer whose attention module was converted.  A single-token step that the attention
-    module takes in five launches (`_fast_decode_slot`) runs the WHOLE layer in seven: input RMSNorm inside the QKV
+    module takes in five launches (`_fast_decode_slot`) runs the WHOLE layer in seven for up to 8 sequences (twelve calls above): input RMSNorm inside the QKV
     projection, the attention step, residual inside the output projection, post-attention RMSNorm in front of and SwiGLU
     behind the stacked gate/up projection, residual inside the down projection (the launches of `LlamaShapedDecoder`) -
     instead of the ~25 library calls of the layer's own forward, which at these sizes are bound by the host.  Everything
@@ -945,6 +949,25 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
             attn._adopt_cache_layer(cache)
         attn._sync_bit_cache(cache)
         slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
+        if slot is not None and hidden_states.shape[0] > FUSED_LAYER_MAX_ROWS:
+            # more sequences than the fused forms take: the same layer in twelve calls - each RMSNorm one launch with the module's
+            # two roundings, the attention step, the library's GEMM on the stacked gate/up weight and on the down projection,
+            # SwiGLU one launch, the two residual additions - instead of the library layer's ~26
+            b, _, hidden = hidden_states.shape
+            mlp, n1, n2, gate, _, down = mods
+            h = torch.empty_like(hidden_states)
+            _ops.rmsnorm(hidden_states[:, 0, :], n1.weight, float(n1.variance_epsilon), h[:, 0, :])
+            y, _ = attn._fast_decode(h, position_embeddings, slot[0], amask=slot[1])
+            attn._note_key_storage(cache)
+            x1 = hidden_states + y
+            _ops.rmsnorm(x1[:, 0, :], n2.weight, float(n2.variance_epsilon), h[:, 0, :])
+            gate_up = torch.mm(h[:, 0, :], _stacked_gate_up(attn, mlp).t())
+            act = attn.__dict__.get("_fast_act")
+            if act is None or act.shape[0] != b or act.shape[1] != gate.out_features or act.device != hidden_states.device:
+                act = torch.empty(b, gate.out_features, dtype=torch.bfloat16, device=hidden_states.device)
+                attn.__dict__["_fast_act"] = act
+            _ops.swiglu(gate_up, act)
+            return x1 + torch.mm(act, down.weight.t()).view(b, 1, hidden)
         if slot is not None:
             b = hidden_states.shape[0]
             mlp, n1, n2, gate, _, down = mods

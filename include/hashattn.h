@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define HA_VERSION 202 /* 0.2.2: + ha_sparse_decode_fused_prefix_masked; the dense baseline and the window partial take any number of query heads per KV head; 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
+#define HA_VERSION 202 /* 0.2.2: + ha_sparse_decode_fused_prefix_masked, ha_rmsnorm; the dense baseline and the window partial take any number of query heads per KV head; 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
 
 typedef enum ha_status {
     HA_OK = 0,
@@ -422,6 +422,14 @@ int ha_rope_append(const void *qkv, int64_t qkv_stride_b, int dtype, int B, int 
                    const float *inv_freq, void *q_out, void *k_cache, void *v_cache,
                    int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s, int64_t cache_len, void *stream);
 int ha_swiglu(const void *gate_up, int64_t gate_up_stride_b, int dtype, int B, int F, void *out, void *stream);
+/*
+ * RMSNorm of M rows of K elements as one launch: out = round(round(x * rsqrt(mean_k x^2 + eps)) * weight), both roundings
+ * to `dtype` - the module of the reference's harness (efficiency/model.py:308-319: `self._norm(x.float()).type_as(x)` times
+ * the weight) and transformers' LlamaRMSNorm.  For batches too large for the norm-in-front form of ha_linear_skinny_fused.
+ * Strides in elements; `out` must not overlap `x`.
+ */
+int ha_rmsnorm(const void *x, int64_t x_stride_m, const void *weight, int dtype, int M, int K, float eps,
+               void *out, int64_t out_stride_m, void *stream);
 /*
  * ha_rope_append followed by ha_encode_step, in one launch: the workgroup that hashes a head also rotates it.  qkv as for
  * ha_rope_append; the rotated query goes to q_out, the rotated key and the value into the caches at position pos (or

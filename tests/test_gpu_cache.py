@@ -425,20 +425,26 @@ def test_few_launch_steps_on_other_model_shapes(shape):
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
 
 
-def test_five_launch_step_with_more_sequences_than_the_projection_kernel_takes():
+@pytest.mark.parametrize("batch,whole_layer", [(18, False), (18, True), (12, True)])
+def test_few_call_steps_with_more_sequences_than_the_fused_projections_take(batch, whole_layer):
     # 18 sequences: the attention module keeps its five-call step (the library's GEMM on the stacked QKV weight and on the
-    # output projection, the rotary/append/hash launch, histograms, select-attend); the decoder layer around it is the library's
-    print("\n[case] five-launch attention step, 18 sequences", flush=True)
+    # output projection, the rotary/append/hash launch, histograms, select-attend).  The decoder layer around it: the library's
+    # own, or (whole_layer, the default) twelve calls - one launch per RMSNorm with the module's roundings, one GEMM on the
+    # stacked gate/up weight, one SwiGLU launch.  12 sequences: the same with the projection kernel's matrix-core form inside
+    # the attention step.
+    print(f"\n[case] few-call steps, {batch} sequences, whole layer: {whole_layer}", flush=True)
     cfg, model = _model(fast_decode=False)
-    ids = torch.randint(0, cfg.vocab_size, (18, 140), generator=torch.Generator().manual_seed(13)).to(DEV)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 140), generator=torch.Generator().manual_seed(13)).to(DEV)
     outs = []
     for fast in (False, True):
         hl.reset_usa(model)
         for layer in model.model.layers:
             layer.self_attn.fast_decode = fast
+            layer.self_attn.fast_layer = whole_layer
             layer.self_attn.__dict__.pop("_fast_scratch", None)
         outs.append(_decode(model, ids, PreallocatedCache(capacity=160), [1, 1, 3, 1]))
-    assert all("_fast_scratch" in layer.self_attn.__dict__ and "_fast_act" not in layer.self_attn.__dict__ for layer in model.model.layers)
+    assert all("_fast_scratch" in layer.self_attn.__dict__ and ("_fast_act" in layer.self_attn.__dict__) == whole_layer
+               for layer in model.model.layers)
     worst = max((g - w).abs().max().item() for g, w in zip(outs[1], outs[0]))
     scale = max(w.abs().max().item() for w in outs[0])
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)

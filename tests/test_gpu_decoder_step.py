@@ -5,6 +5,7 @@ import pytest
 import torch
 from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM, MistralConfig, MistralForCausalLM
 
+from hashattention import _ops
 from hashattention import hashattention_llama as hl
 from hashattention import hashattention_mistral as hm
 from hashattention.decoder import LlamaShapedDecoder
@@ -362,6 +363,34 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
     print("  tokens:", got.tolist(), flush=True)
     assert torch.equal(got, want)
     assert dec.seq_len == S0 + n_new - 1
+
+
+@pytest.mark.parametrize("dtype,M,K", [(torch.bfloat16, 12, 4096), (torch.bfloat16, 3, 5120), (torch.float16, 5, 1024),
+                                       (torch.float32, 4, 768), (torch.bfloat16, 2, 100)])
+def test_rmsnorm_launch_rounds_as_the_module_it_replaces(dtype, M, K):
+    # ha_rmsnorm against transformers' LlamaRMSNorm in the same dtype: the normalised row rounded to the element type, then the
+    # product with the weight rounded again.  The sum of squares is added in another order, so a rounding may fall the other way
+    # for a few elements: one unit in the last place at most, in fewer than one element of a thousand.
+    from transformers.models.llama.modeling_llama import LlamaRMSNorm
+    print(f"\n[case] ha_rmsnorm {dtype} {M}x{K}", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(K + M)
+    x = (torch.randn(M, K, generator=g, device=DEV) * 3).to(dtype)
+    mod = LlamaRMSNorm(K, eps=1e-5).to(DEV, dtype)
+    mod.weight.data = (1 + 0.3 * torch.randn(K, generator=g, device=DEV)).to(dtype)
+    want = mod(x)
+    xs = torch.empty(M, K + 8, dtype=dtype, device=DEV)[:, :K]      # rows with a stride of their own
+    xs.copy_(x)
+    for src in (x, xs):
+        out = torch.full((M, K), 7.0, dtype=dtype, device=DEV)
+        _ops.rmsnorm(src, mod.weight, 1e-5, out)
+        torch.cuda.synchronize()
+        if dtype == torch.float32:
+            assert (out - want).abs().max().item() <= 1e-5 * want.abs().max().item()
+            continue
+        differ = out != want
+        assert differ.float().mean().item() <= 1e-3, differ.float().mean().item()
+        ulp = (out.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert int(ulp.max()) <= 1
 
 
 @pytest.mark.parametrize("what", ["attention_bias", "mlp_bias", "yarn", "dynamic"])

@@ -33,6 +33,7 @@ class PreallocatedLayer(DynamicLayer):
     default_capacity = 0
     growth = 2.0
     min_growth = 0
+    max_growth = None   # most tokens of room added at a time (None: no bound, the geometric growth alone)
 
     def __init__(self, capacity: Optional[int] = None, **kwargs):
         self._kbuf = self._vbuf = None
@@ -71,7 +72,10 @@ class PreallocatedLayer(DynamicLayer):
         have = 0 if self._kbuf is None else self._kbuf.shape[-2]
         if self._kbuf is not None and self._vbuf is not None and need <= have and self._kbuf.device == key_states.device:
             return
-        cap = max(need, self.capacity_hint, int(have * self.growth), have + self.min_growth if have else 0)
+        grown = int(have * self.growth)
+        if self.max_growth is not None:
+            grown = min(grown, have + self.max_growth)
+        cap = max(need, self.capacity_hint, grown, have + self.min_growth if have else 0)
         b, h, _, dk = key_states.shape
         kbuf = torch.empty(b, h, cap, dk, dtype=key_states.dtype, device=key_states.device)
         vbuf = torch.empty(b, h, cap, value_states.shape[-1], dtype=value_states.dtype, device=value_states.device)
@@ -127,7 +131,7 @@ class PreallocatedLayer(DynamicLayer):
 
 def adopt_dynamic_layer(layer) -> bool:
     """Turn a plain `DynamicLayer` that already holds tokens into a `PreallocatedLayer` IN PLACE: same object, same tensors
-    (they become its buffers, full to the brim, so the next append allocates the usual doubled capacity once), same behaviour
+    (they become its buffers, full to the brim, so the next append allocates a larger buffer once), same behaviour
     towards the cache that owns it - but later appends copy only the new tokens.  This is how a cache that `generate` created
     on its own (`DynamicCache`, one `torch.cat` of the layer's whole cache per token) is taken over by the converted attention
     modules.  Only the exact class is taken: sliding-window, quantized or static layers keep their own logic.  Returns
@@ -143,7 +147,10 @@ def adopt_dynamic_layer(layer) -> bool:
     layer.__class__ = PreallocatedLayer
     layer._kbuf, layer._vbuf, layer._len = k, v, int(k.shape[-2])
     layer.capacity_hint = 0
-    layer.growth, layer.min_growth = 1.25, 256      # nobody said how long this cache will get: a quarter more room at a time
+    # nobody said how long this cache will get: a quarter more room at a time, 256 to 8192 tokens - a prompt of 131072 tokens must
+    # not reserve 32768 more per layer for an answer of a few hundred, and copying the layer once per 8192 appended tokens costs
+    # nothing that shows
+    layer.growth, layer.min_growth, layer.max_growth = 1.25, 256, 8192
     layer.epoch = 0
     return True
 

@@ -135,6 +135,12 @@ def test_a_dynamic_layer_is_adopted_in_place():
     ptr = layer._kbuf.data_ptr()
     got.update(*_states(g, 2, 2, 1), 0)
     assert layer._kbuf.data_ptr() == ptr
+    # a long prompt: the room added at a time is bounded (8192 tokens), not a quarter of the prompt
+    long = DynamicCache()
+    long.update(torch.zeros(1, 1, 100000, 4), torch.zeros(1, 1, 100000, 4), 0)
+    assert adopt_dynamic_layer(long.layers[0])
+    long.update(torch.zeros(1, 1, 1, 4), torch.zeros(1, 1, 1, 4), 0)
+    assert long.layers[0].capacity == 100000 + 8192 and long.get_seq_length() == 100001
     # other layer kinds, and layers that hold nothing yet, are left alone
     assert not adopt_dynamic_layer(DynamicLayer()) and not adopt_dynamic_layer(DynamicSlidingWindowLayer(sliding_window=4))
     assert adopt_dynamic_layer(layer)                              # already one

@@ -1,0 +1,93 @@
+"""Host logic of the patched layer that needs no GPU: how the attention mask of a forward pass is examined - what the reference
+adds to the scores before its softmax (hashattention_llama.py:593-598) - and in which form it is handed to the kernels."""
+import torch
+
+from hashattention import _patched
+
+
+def _layer():
+    return _patched.HeavyHitterMixin.__new__(_patched.HeavyHitterMixin)
+
+
+def _additive(keep: torch.Tensor, dtype=torch.float32) -> torch.Tensor:
+    """The library's float form of a keep-mask: 0 where a token may be attended, the most negative value elsewhere."""
+    return torch.zeros(keep.shape, dtype=dtype).masked_fill_(~keep, torch.finfo(dtype).min)
+
+
+def test_a_mask_that_blocks_nothing_is_dropped():
+    layer, b, S = _layer(), 3, 40
+    assert layer._additive_mask(None, b, 1, S) is None
+    keep = torch.ones(b, 1, 1, S, dtype=torch.bool)
+    assert layer._additive_mask(keep, b, 1, S) is None
+    assert layer._additive_mask(_additive(keep, torch.bfloat16), b, 1, S) is None
+    # a chunk of rows: what the mask blocks beyond the causal edge changes nothing, the kernels apply that edge themselves
+    causal = torch.tril(torch.ones(5, S, dtype=torch.bool), diagonal=S - 5)[None, None].expand(b, 1, 5, S)
+    assert layer._additive_mask(causal, b, 5, S) is None
+    # longer than the cache (a buffer with room ahead): only the first S columns count
+    wide = torch.ones(b, 1, 1, S + 9, dtype=torch.bool)
+    wide[..., S:] = False
+    assert layer._additive_mask(wide, b, 1, S) is None
+
+
+def test_left_padding_is_recognised_as_one_number_per_sequence():
+    layer, b, S = _layer(), 3, 40
+    keep = torch.ones(b, 1, 1, S, dtype=torch.bool)
+    keep[1, ..., :7] = False
+    keep[2, ..., :39] = False
+    for mask in (keep, _additive(keep), _additive(keep, torch.bfloat16), _additive(keep, torch.float16),
+                 torch.zeros(b, 1, 1, S).masked_fill_(~keep, float("-inf"))):
+        sm = layer._additive_mask(mask, b, 1, S)
+        assert sm is not None and sm.prefix is not None and sm.prefix.dtype == torch.int32 and sm.prefix.tolist() == [0, 7, 39]
+        table = sm.table()
+        assert table.shape == (b, S) and table.dtype == torch.float32
+        assert torch.equal(table == 0, keep[:, 0, 0]) and bool((table[~keep[:, 0, 0]] <= -6e4).all())
+    # one mask row shared by the batch
+    one = torch.ones(1, 1, 1, S, dtype=torch.bool)
+    one[..., :4] = False
+    sm = layer._additive_mask(one, b, 1, S)
+    assert sm.prefix.tolist() == [4, 4, 4] and sm.table().shape == (b, S)
+
+
+def test_other_masks_keep_their_table():
+    layer, b, S = _layer(), 2, 40
+    hole = torch.ones(b, 1, 1, S, dtype=torch.bool)
+    hole[0, ..., 10:13] = False                                    # not a prefix
+    sm = layer._additive_mask(hole, b, 1, S)
+    assert sm is not None and sm.prefix is None and torch.equal(sm.table() == 0, hole[:, 0, 0])
+    bias = torch.zeros(b, 1, 1, S)
+    bias[1, ..., :5] = -2.5                                        # a prefix, but of finite terms: they are added, not dropped
+    sm = layer._additive_mask(bias, b, 1, S)
+    assert sm is not None and sm.prefix is None and torch.equal(sm.table(), bias[:, 0, 0])
+    mixed = _additive(torch.ones(b, 1, 1, S, dtype=torch.bool))
+    mixed[0, ..., :3] = torch.finfo(torch.float32).min
+    mixed[0, ..., 3] = -1.0
+    sm = layer._additive_mask(mixed, b, 1, S)
+    assert sm.prefix is None
+    # a chunk of rows with padding: the fp32 rows, no prefix form
+    keep = torch.tril(torch.ones(4, S, dtype=torch.bool), diagonal=S - 4)[None, None].repeat(b, 1, 1, 1)
+    keep[1, ..., :6] = False
+    sm = layer._additive_mask(keep, b, 4, S)
+    assert sm is not None and sm.prefix is None and sm.rows().shape == (b, 4, S) and bool((sm.rows()[1, :, :6] == float("-inf")).all())
+
+
+def test_one_examination_serves_every_layer_of_a_pass_and_a_changed_mask_is_examined_again():
+    a, c, b, S = _layer(), _layer(), 2, 30
+    keep = torch.ones(b, 1, 1, S, dtype=torch.bool)
+    keep[0, ..., :5] = False
+    first = a._additive_mask(keep, b, 1, S)
+    assert c._additive_mask(keep, b, 1, S) is first and first.rows() is first.rows()      # the fp32 form is made once
+    keep[0, ..., :9] = False                                       # written in place: the tensor's version moved
+    again = c._additive_mask(keep, b, 1, S)
+    assert again is not first and again.prefix.tolist() == [9, 0]
+    assert a._additive_mask(keep, b, 1, S - 1) is not again         # another length: examined again
+    other = keep.clone()
+    assert a._additive_mask(other, b, 1, S) is not again
+
+
+def test_a_mask_of_the_wrong_shape_is_refused():
+    import pytest
+    layer = _layer()
+    with pytest.raises(ValueError, match="Attention mask should be of size"):
+        layer._additive_mask(torch.ones(2, 1, 1, 10, dtype=torch.bool), 2, 1, 12)
+    with pytest.raises(ValueError):
+        layer._additive_mask(torch.ones(3, 1, 1, 12, dtype=torch.bool), 2, 1, 12)

@@ -1,5 +1,6 @@
 """Host logic of the patched layer that needs no GPU: how the attention mask of a forward pass is examined - what the reference
-adds to the scores before its softmax (hashattention_llama.py:593-598) - and in which form it is handed to the kernels."""
+adds to the scores before its softmax (hashattention_llama.py:593-598) - and in which form it is handed to the kernels; which
+decoder layers take the few-launch step."""
 import torch
 
 from hashattention import _patched
@@ -91,3 +92,47 @@ def test_a_mask_of_the_wrong_shape_is_refused():
         layer._additive_mask(torch.ones(2, 1, 1, 10, dtype=torch.bool), 2, 1, 12)
     with pytest.raises(ValueError):
         layer._additive_mask(torch.ones(3, 1, 1, 12, dtype=torch.bool), 2, 1, 12)
+
+
+def _decoder_layer(**kw):
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaDecoderLayer
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=1, num_attention_heads=2, num_key_value_heads=1,
+                      head_dim=128, vocab_size=64, **kw)
+    return LlamaDecoderLayer(cfg, 0).bfloat16()
+
+
+def test_which_decoder_layers_take_the_few_launch_step():
+    # the whole-layer step reads weights directly: it is for layers of the Llama shape made of plain modules, and steps aside for
+    # anything that wants a say (wrappers around a projection, hooks, biases, another activation)
+    layer = _decoder_layer()
+    x = torch.zeros(2, 1, 256, dtype=torch.bfloat16)
+    mods = _patched._layer_modules(layer)
+    assert mods and mods[0] is layer.mlp and mods[3] is layer.mlp.gate_proj and mods[5] is layer.mlp.down_proj
+    assert _patched._layer_takes_fast_path(layer, x) is mods
+    assert _patched._layer_takes_fast_path(layer, torch.zeros(2, 3, 256, dtype=torch.bfloat16)) is False      # a chunk of tokens
+    assert _patched._layer_takes_fast_path(layer, torch.zeros(40, 1, 256, dtype=torch.bfloat16)) is mods      # any number of sequences
+
+    class Wrapped(torch.nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, t):
+            return self.inner(t) + 1
+
+    plain = layer.mlp.up_proj
+    layer.mlp.up_proj = Wrapped(plain)
+    assert _patched._layer_modules(layer) is False and _patched._layer_takes_fast_path(layer, x) is False
+    layer.mlp.up_proj = plain                                       # the wrapper is gone: the step comes back
+    assert _patched._layer_takes_fast_path(layer, x)
+    handle = layer.mlp.down_proj.register_forward_hook(lambda m, a, o: None)
+    assert _patched._layer_takes_fast_path(layer, x) is False
+    handle.remove()
+    assert _patched._layer_takes_fast_path(layer, x)
+    handle = layer.self_attn.register_forward_pre_hook(lambda m, a: None)
+    assert _patched._layer_takes_fast_path(layer, x) is False
+    handle.remove()
+    assert _patched._layer_takes_fast_path(layer.float(), x) is False       # fp32 weights
+    assert _patched._layer_modules(_decoder_layer(mlp_bias=True)) is False
+    assert _patched._layer_modules(_decoder_layer(hidden_act="gelu")) is False

@@ -136,3 +136,57 @@ def test_which_decoder_layers_take_the_few_launch_step():
     assert _patched._layer_takes_fast_path(layer.float(), x) is False       # fp32 weights
     assert _patched._layer_modules(_decoder_layer(mlp_bias=True)) is False
     assert _patched._layer_modules(_decoder_layer(hidden_act="gelu")) is False
+
+
+class _Codes:
+    """Stands in for the hash layer: what `_sync_bit_cache` reads and writes."""
+
+    def __init__(self, n):
+        self.n_cached, self.resets = n, 0
+
+    def reset(self):
+        self.n_cached, self.resets = 0, self.resets + 1
+
+
+def _attn(n_cached):
+    layer = _layer()
+    layer.layer_idx, layer._cache_ref, layer._cache_id, layer._hash_layer = 0, None, None, _Codes(n_cached)
+    return layer
+
+
+def test_codes_follow_the_cache_they_were_made_from():
+    # the reference re-hashes every key at every step (hashattention_llama.py:407-408), so nothing a caller does to the cache
+    # between two passes may leave codes of other contents behind: another cache object, reordered or selected batch entries
+    # (beam search), a rewound cache
+    from transformers import DynamicCache
+    from hashattention.cache import PreallocatedCache
+    k = torch.zeros(3, 1, 6, 4)
+    for make in (DynamicCache, lambda: PreallocatedCache(capacity=16)):
+        cache = make()
+        cache.update(k, k, 0)
+        attn = _attn(0)
+        attn._sync_bit_cache(cache)                  # first sight of this cache
+        attn._hash_layer.n_cached = 6                # ... the pass hashes its keys and notes where they lie
+        attn._note_key_storage(cache)
+        attn._sync_bit_cache(cache)
+        assert attn._hash_layer.n_cached == 6 and attn._hash_layer.resets == 1      # untouched cache: codes kept
+        cache.update(k[:, :, :1], k[:, :, :1], 0)    # the cache's own append (a new tensor for DynamicCache): seen by the pass
+        attn._hash_layer.n_cached = 7
+        attn._note_key_storage(cache)
+        attn._sync_bit_cache(cache)
+        assert attn._hash_layer.n_cached == 7
+        cache.reorder_cache(torch.tensor([2, 0, 1]))     # beam search moved batch entries
+        attn._sync_bit_cache(cache)
+        assert attn._hash_layer.n_cached == 0 and attn._hash_layer.resets == 2
+        attn._hash_layer.n_cached = 7
+        attn._note_key_storage(cache)
+        cache.crop(4)                                # rewound: the in-place cache keeps the codes of its prefix, the library's
+        attn._sync_bit_cache(cache)                  # leaves a new tensor behind and is hashed afresh
+        assert attn._hash_layer.n_cached == (4 if isinstance(cache, PreallocatedCache) else 0)
+        other = make()
+        other.update(k, k, 0)
+        attn._hash_layer.n_cached = 4
+        attn._sync_bit_cache(other)                  # another cache object: nothing is kept
+        assert attn._hash_layer.n_cached == 0
+        attn._sync_bit_cache(None)
+        assert attn._hash_layer.n_cached == 0

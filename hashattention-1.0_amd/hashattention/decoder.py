@@ -158,8 +158,8 @@ class LlamaShapedDecoder:
 
         Per layer (bf16, up to 8 sequences): QKV projection with its RMSNorm folded in, ha_rope_append, the attention
         step, output projection with the residual folded in, gate/up projection with its RMSNorm and SwiGLU folded in,
-        down GEMM with the residual folded in (addmm).  Other dtypes and batches: the same steps as library calls plus
-        ha_swiglu."""
+        down projection with the residual folded in.  Other dtypes and batches: the same steps as library calls plus
+        ha_rmsnorm and ha_swiglu."""
         B, H, Hkv, d = self.B, self.H, self.Hkv, self.d
         if self.lengths is not None and not device_pos:
             raise RuntimeError("a ragged batch keeps its positions on the device: use generate()")
@@ -169,11 +169,21 @@ class LlamaShapedDecoder:
         # the row-streaming kernel against the library GEMM at B = 4: QKV 11.3 us (19.3), output projection 9.5 (19.1),
         # gate/up 40.9 (59.8), down projection 24.7 (25.1), lm_head 174.8 (184.7)
         skinny = self.use_skinny and self.dtype == torch.bfloat16 and B <= 8
+        # 16-bit models outside the fused forms keep their roundings: the norm's two (ha_rmsnorm), the projection's own before a
+        # residual is added (efficiency/model.py:314-319, :190-191); fp32 has none to keep
+        lowp = self.dtype != torch.float32
+
+        def norm(t, weight):
+            if not lowp:
+                return F.rms_norm(t, (self.hidden,), weight, self.eps)
+            out = torch.empty_like(t)
+            _ops.rmsnorm(t, weight, self.eps, out)
+            return out
         for l, p in enumerate(self.layers):
             if skinny:      # RMSNorm rides in the projection that consumes it
                 qkv = _ops.linear_skinny(x, p["wqkv"], self.qkv, norm_weight=p["attn_norm"], eps=self.eps)
             else:
-                qkv = F.linear(F.rms_norm(x, (self.hidden,), p["attn_norm"], self.eps), p["wqkv"])
+                qkv = F.linear(norm(x, p["attn_norm"]), p["wqkv"])
             hl = self.hash[l]
             if device_pos:
                 if dense or d != 128:
@@ -197,19 +207,22 @@ class LlamaShapedDecoder:
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             else:
-                x = x.addmm_(self.attn_out.view(B, H * d), p["wo"].t())
-                h = F.rms_norm(x, (self.hidden,), p["ffn_norm"], self.eps)
-                _ops.swiglu(F.linear(h, p["w13"]), self.ffn_act)
+                if lowp:
+                    x = x + F.linear(self.attn_out.view(B, H * d), p["wo"])
+                else:
+                    x = x.addmm_(self.attn_out.view(B, H * d), p["wo"].t())
+                _ops.swiglu(F.linear(norm(x, p["ffn_norm"]), p["w13"]), self.ffn_act)
             if skinny and self.skinny_all:
                 x = _ops.linear_skinny(self.ffn_act, p["w2"], self.x_attn[1], residual=x)
+            elif lowp and not skinny:
+                x = x + F.linear(self.ffn_act, p["w2"])
             else:
                 x = x.addmm_(self.ffn_act, p["w2"].t())      # in place: the out-of-place form first copies x into its result
         if advance and not device_pos:
             self.seq_len = S
         if skinny and self.skinny_all:
             return _ops.linear_skinny(x, self.lm_head, self.logits, norm_weight=self.final_norm, eps=self.eps)
-        x = F.rms_norm(x, (self.hidden,), self.final_norm, self.eps)
-        return F.linear(x, self.lm_head)
+        return F.linear(norm(x, self.final_norm), self.lm_head)
 
     # ------------------------------------------------------------------ greedy generation, one graph for all tokens
     def generate(self, tokens: torch.Tensor, n_new: int, use_graph: bool = True, sampler=None) -> torch.Tensor:

@@ -77,6 +77,28 @@ def test_full_size_configuration(name):
     err = np.abs(out.float().cpu().numpy() - ref).max()
     print(f"  n_selected {cnt.min()}..{cnt.max()}, sparse max-abs error {err:.2e}", flush=True)
     assert err <= 2e-2
+    if name in ("config2", "config3", "config4"):
+        # the fused launch with a masked prefix per sequence (the mask of a left-padded batch, hashattention_llama.py:593-598):
+        # sequences without one keep the plain launch's output bit for bit; for the others a list entry at -inf is a list
+        # without that entry, which the oracle attends to
+        prefix = [0 if b % 2 == 0 else 1000 + 37 * b for b in range(B)]
+        out_m = torch.empty_like(out)
+        layer.select_prepare(S, seq)
+        layer.attend_fused(p.q[:, :, 0], p.k, p.v, out_m, S, seq, masked_prefix=torch.tensor(prefix, dtype=torch.int32, device=DEV))
+        torch.cuda.synchronize()
+        assert torch.equal(out_m[0::2], out[0::2])
+        idx_m, cnt_m = np.zeros_like(ref_idx), ref_cnt.copy()
+        for b in range(B):
+            for h in range(H):
+                n = ref_cnt[b, h]
+                skip = int(np.searchsorted(ref_idx[b, h, :n], prefix[b]))
+                idx_m[b, h, :n - skip] = ref_idx[b, h, skip:n]
+                cnt_m[b, h] = n - skip
+        assert (cnt_m[1::2] < ref_cnt[1::2]).all()
+        ref_m = c_oracle.sparse_attend(p.q[:, :, 0].cpu(), p.k.cpu(), p.v.cpu(), idx_m, cnt_m, 1 / math.sqrt(128))
+        err_m = np.abs(out_m.float().cpu().numpy() - ref_m).max()
+        print(f"  masked prefix: sparse max-abs error {err_m:.2e}", flush=True)
+        assert err_m <= 2e-2
     if name != "config2":       # dense baseline against the oracle too (config2: 4 GB of K/V through a scalar loop is slow)
         outd = torch.empty_like(out)
         ws = _ops.workspace(_ops.dense_decode_workspace_bytes(B, H, S), DEV)

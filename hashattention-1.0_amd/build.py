@@ -9,7 +9,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SOURCES = ["ha_core.hip", "ha_encode.hip", "ha_encode_mfma.hip", "ha_encode_mfma_f32.hip", "ha_select.hip", "ha_select_sampled.hip", "ha_attend.hip", "ha_decoder.hip"]
+SOURCES = ["ha_core.hip", "ha_encode.hip", "ha_encode_mfma.hip", "ha_encode_mfma_f32.hip", "ha_select.hip", "ha_select_sampled.hip", "ha_attend.hip", "ha_decoder.hip", "ha_linear_tiled.hip"]
 LIB = os.path.join(HERE, "hashattention", "libhashattn.so")
 
 FLAGS = [

@@ -138,6 +138,12 @@ def _declare(lib: C.CDLL) -> C.CDLL:
     lib.ha_sparse_decode_fused_prefix_masked.restype = i32
     lib.ha_sparse_decode_fused_prefix_masked.argtypes = [vp, i64, i64, vp, vp, i32, i64, i64, i64, vp, i64, i64, vp, i32, i32, i32, i32,
                                                          i32, i32, vp, i32, i32, f64, vp, sz, i32, vp, vp, f32, vp, vp, sz, vp]
+    lib.ha_weight_tiles_elems.restype = i64
+    lib.ha_weight_tiles_elems.argtypes = [i32, i32, i32]
+    lib.ha_pack_weight_tiles.restype = i32
+    lib.ha_pack_weight_tiles.argtypes = [vp, i64, i32, i32, i32, vp, vp]
+    lib.ha_linear_tiled.restype = i32
+    lib.ha_linear_tiled.argtypes = [vp, i64, vp, vp, i64, i32, vp, i64, i32, i32, i32, vp]
     lib.ha_rmsnorm.restype = i32
     lib.ha_rmsnorm.argtypes = [vp, i64, vp, i32, i32, i32, f32, vp, i64, vp]
     lib.ha_window_partial_bytes.restype = sz
@@ -653,6 +659,42 @@ HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1
 
 
 LINEAR_SKINNY_MAX_ROWS = 16     # rows of x that ha_linear_skinny takes
+LINEAR_TILED_MAX_K = 8192       # inputs that ha_linear_tiled takes
+
+
+def pack_weight_tiles(w: torch.Tensor, glu: bool = False) -> torch.Tensor:
+    """The tiled copy of w [N, K] bf16 that `linear_tiled` reads (glu: w = [gate rows; up rows], tiles of 8 + 8)."""
+    _require_cuda(w)
+    assert w.dim() == 2 and w.dtype == torch.bfloat16 and w.stride(1) == 1
+    N, K = w.shape
+    n = load_library().ha_weight_tiles_elems(N, K, 1 if glu else 0)
+    if n <= 0:
+        raise ValueError(f"a [{N}, {K}] matrix cannot be tiled (K a multiple of 32, an even N for gate/up)")
+    tiles = torch.empty(n, dtype=torch.bfloat16, device=w.device)
+    _check(load_library().ha_pack_weight_tiles(_ptr(w), w.stride(0), N, K, 1 if glu else 0, _ptr(tiles), _stream(w)), "ha_pack_weight_tiles")
+    return tiles
+
+
+def linear_tiled(x: torch.Tensor, tiles: torch.Tensor, N: int, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                 swiglu: bool = False) -> torch.Tensor:
+    """out [M, N] (or [M, N / 2] with swiglu) = x [M, K] . W^T (+ residual) from the tiled copy of W [N, K].  M <= 16,
+    K <= 8192."""
+    _require_cuda(x, tiles, out, residual)
+    assert x.dim() == 2 and x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1
+    M, K = x.shape
+    assert tiles.dtype == torch.bfloat16 and tiles.is_contiguous()
+    assert tiles.numel() == load_library().ha_weight_tiles_elems(N, K, 1 if swiglu else 0), "tiles of another shape"
+    assert out.shape == (M, N // 2 if swiglu else N)
+    assert residual is None or (residual.shape == (M, N) and residual.dtype == torch.bfloat16 and residual.stride(1) == 1)
+    _linear_tiled_unchecked(x, tiles, N, out, residual, swiglu)
+    return out
+
+
+def _linear_tiled_unchecked(x, tiles, N, out, residual=None, swiglu=False):
+    _check(load_library().ha_linear_tiled(x.data_ptr(), x.stride(0), tiles.data_ptr(), _ptr(residual),
+                                          residual.stride(0) if residual is not None else 0,
+                                          HA_ACT_SWIGLU if swiglu else HA_ACT_NONE, out.data_ptr(), out.stride(0), x.shape[0], N,
+                                          x.shape[1], _stream(x)), "ha_linear_tiled")
 
 
 def _linear_skinny_unchecked(x, w, out, residual=None, norm_weight=None, eps=0.0, swiglu=False):

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define HA_VERSION 202 /* 0.2.2: + ha_sparse_decode_fused_prefix_masked, ha_rmsnorm; the dense baseline and the window partial take any number of query heads per KV head; 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
+#define HA_VERSION 202 /* 0.2.2: + ha_sparse_decode_fused_prefix_masked, ha_rmsnorm, ha_linear_tiled (+ ha_pack_weight_tiles); the dense baseline and the window partial take any number of query heads per KV head; 0.2.1: ha_linear_skinny[_fused] round as the modules they replace (two roundings per RMSNorm, the product's before a residual); 0.2.0: + ha_sparse_decode_paged, ha_sparse_decode_fused_paged, ha_rope_encode_step_cos_sin */
 
 typedef enum ha_status {
     HA_OK = 0,
@@ -480,6 +480,24 @@ enum { HA_ACT_NONE = 0, HA_ACT_SWIGLU = 1 };
 int ha_linear_skinny_fused(const void *x, int64_t x_stride_m, const void *w, int64_t w_stride_n, const void *residual,
                            int64_t residual_stride_m, const void *norm_weight, float eps, int act, void *out,
                            int64_t out_stride_m, int M, int N, int K, void *stream);
+
+/*
+ * The same products for 9 to 16 rows of x (and fewer) from a TILED copy of the weights: tiles of 16 rows x 32 inputs laid out
+ * as the operand of the bf16 matrix instruction, so that a wave load is one contiguous KiB (row-major weights give such a
+ * batch 64-byte pieces of 16 rows per load, 2.5 - 4 TB/s).  For callers that own a copy of the weights anyway (a decoding
+ * harness as efficiency/model.py:236-262, 304-305; the stacked QKV and gate/up matrices of a patched layer).
+ *   ha_weight_tiles_elems  bf16 elements of the tiled copy of a [N, K] matrix (rows padded to whole tiles), 0 for a bad shape
+ *   ha_pack_weight_tiles   w [N, K] bf16 row-major (row stride w_stride_n) -> tiles.  glu = 1: w is [F gate rows; F up rows]
+ *                          and every tile holds 8 gate rows followed by the 8 up rows of the same columns
+ *   ha_linear_tiled        out [M, N] = x [M, K] . W^T (+ residual), M <= 16, K <= 8192 a multiple of 32;
+ *                          act = HA_ACT_SWIGLU (tiles packed with glu = 1, N = 2 F): out [M, F] = silu(gate) * up.
+ *                          Roundings as ha_linear_skinny_fused: those of the modules replaced.  (An RMSNorm in front is
+ *                          ha_rmsnorm, a launch of its own, for batches of this size.)
+ */
+int64_t ha_weight_tiles_elems(int N, int K, int glu);
+int ha_pack_weight_tiles(const void *w, int64_t w_stride_n, int N, int K, int glu, void *tiles, void *stream);
+int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const void *residual, int64_t residual_stride_m,
+                    int act, void *out, int64_t out_stride_m, int M, int N, int K, void *stream);
 
 #ifdef __cplusplus
 }

@@ -365,6 +365,53 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
     assert dec.seq_len == S0 + n_new - 1
 
 
+@pytest.mark.parametrize("M,N,K,form", [(16, 6144, 4096, "plain"), (12, 4096, 4096, "residual"), (16, 2 * 14336, 4096, "glu"),
+                                        (9, 1000, 64, "plain"), (1, 40, 32, "residual"), (16, 2 * 100, 1536, "glu"),
+                                        (13, 4096, 8192, "residual"), (4, 520, 2080, "plain")])
+def test_linear_tiled_against_fp32_matmul(M, N, K, form):
+    # the matrix-core projection on a tiled copy of the weights (ha_pack_weight_tiles, ha_linear_tiled) against the product in fp32
+    # with the roundings of the modules it stands for: the projection's output rounded to bf16 before a residual is added;
+    # SwiGLU on rounded gate and up values.  Shapes: whole and ragged tile rows, one to sixteen rows of x, K from one k-step to
+    # the 8192 inputs a workgroup holds, a K that leaves waves without work
+    print(f"\n[case] ha_linear_tiled M={M} N={N} K={K} {form}", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(N + K + M)
+    x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device=DEV) * K ** -0.5).to(torch.bfloat16)
+    tiles = _ops.pack_weight_tiles(w, glu=form == "glu")
+    y = x.float() @ w.float().t()
+    if form == "glu":
+        gate, up = y[:, :N // 2].bfloat16().float(), y[:, N // 2:].bfloat16().float()
+        want = torch.nn.functional.silu(gate).bfloat16().float() * up
+        out = torch.full((M, N // 2), 7.0, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_tiled(x, tiles, N, out, swiglu=True)
+    elif form == "residual":
+        res = torch.randn(M, N, generator=g, device=DEV).to(torch.bfloat16)
+        want = y.bfloat16().float() + res.float()
+        out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_tiled(x, tiles, N, out, residual=res)
+    else:
+        want = y
+        out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        _ops.linear_tiled(x, tiles, N, out)
+    torch.cuda.synchronize()
+    # bf16 output: half a unit in the last place of the largest value, plus a rounding of gate / up / product that may fall the other way
+    tol = 2.0 ** -8 * max(1.0, want.abs().max().item()) * (3 if form != "plain" else 1)
+    err = (out.float() - want).abs().max().item()
+    assert err <= tol, (err, tol)
+    # the same rows with a stride of their own, written into a wider buffer
+    xs = torch.zeros(M, K + 64, dtype=torch.bfloat16, device=DEV)[:, :K]
+    xs.copy_(x)
+    wide = torch.full((M, out.shape[1] + 24), 7.0, dtype=torch.bfloat16, device=DEV)
+    if form == "glu":
+        _ops.linear_tiled(xs, tiles, N, wide[:, :out.shape[1]], swiglu=True)
+    elif form == "residual":
+        _ops.linear_tiled(xs, tiles, N, wide[:, :out.shape[1]], residual=res)
+    else:
+        _ops.linear_tiled(xs, tiles, N, wide[:, :out.shape[1]])
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:, :out.shape[1]], out) and bool((wide[:, out.shape[1]:] == 7.0).all())
+
+
 @pytest.mark.parametrize("dtype,M,K", [(torch.bfloat16, 12, 4096), (torch.bfloat16, 3, 5120), (torch.float16, 5, 1024),
                                        (torch.float32, 4, 768), (torch.bfloat16, 2, 100)])
 def test_rmsnorm_launch_rounds_as_the_module_it_replaces(dtype, M, K):

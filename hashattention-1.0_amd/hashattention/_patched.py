@@ -64,6 +64,7 @@ def ste_sign(x: torch.Tensor) -> torch.Tensor:
 # last attention mask examined, as ONE tuple so that a reader never sees parts of two examinations: (weak reference,
 # (version, length, batch, rows), the `_StepMask` it became or None when it changes nothing)
 _MASK_PROBE = [(None, None, None)]
+_FUSED_ROWS = 8
 
 
 class _StepMask:
@@ -565,6 +566,20 @@ class HeavyHitterMixin:
             self.__dict__["_qkv_fused"] = hit
         return hit[1]
 
+    def _weight_tiles(self, name: str, weights, glu: bool = False) -> torch.Tensor:
+        """The tiled copy (`ha_pack_weight_tiles`) of the given weights stacked row-wise, which `ha_linear_tiled` reads for
+        batches of 9 to 16 sequences; kept under `name`, rebuilt like `_fused_qkv_weight`."""
+        key = tuple((w.data_ptr(), w._version, w.dtype, w.device) for w in weights)
+        hit = self.__dict__.get(name)
+        if hit is None or hit[0] != key:
+            stacked = weights[0].detach() if len(weights) == 1 else torch.cat([w.detach() for w in weights], dim=0)
+            hit = (key, _ops.pack_weight_tiles(stacked, glu=glu))
+            self.__dict__[name] = hit
+        return hit[1]
+
+    def _takes_tiled_projections(self, b: int, hidden: int) -> bool:
+        return _FUSED_ROWS < b <= _ops.LINEAR_SKINNY_MAX_ROWS and max(hidden, self.num_heads * self.head_dim) <= _ops.LINEAR_TILED_MAX_K
+
     def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
         """(This layer's `PreallocatedLayer` of `cache`, the additive mask as a `_StepMask` or None when it changes nothing)
         when the step can take `_fast_decode`, else None: one new token per sequence, inference, bf16 hidden states and
@@ -625,8 +640,13 @@ class HeavyHitterMixin:
                       q=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev),
                       attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
             self.__dict__["_fast_scratch"] = sc
-        if b > _ops.LINEAR_SKINNY_MAX_ROWS:     # more sequences than the projection kernel takes: the library's GEMM, still one call
+        tiled = self._takes_tiled_projections(b, hidden)
+        if b > _ops.LINEAR_SKINNY_MAX_ROWS:     # more sequences than the projection kernels take: the library's GEMM, still one call
             torch.mm(hidden_states[:, 0, :], self._fused_qkv_weight().t(), out=sc["qkv"])
+        elif tiled:                             # 9 to 16 sequences: the matrix cores on a tiled copy of the stacked weight
+            _ops._linear_tiled_unchecked(hidden_states[:, 0, :], self._weight_tiles("_qkv_tiles", (self.q_proj.weight, self.k_proj.weight,
+                                                                                                 self.v_proj.weight)),
+                                         sc["qkv"].shape[1], sc["qkv"])
         elif norm is None:
             _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
         else:
@@ -654,6 +674,11 @@ class HeavyHitterMixin:
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
         if b > _ops.LINEAR_SKINNY_MAX_ROWS:
             torch.mm(sc["attn"].view(b, H * d), self.o_proj.weight.t(), out=out.view(b, hidden))
+            if residual is not None:
+                out.view(b, hidden).add_(residual)      # the projection's rounding, then the addition's
+        elif tiled:
+            _ops._linear_tiled_unchecked(sc["attn"].view(b, H * d), self._weight_tiles("_o_tiles", (self.o_proj.weight,)), hidden,
+                                         out.view(b, hidden), residual=residual)
         else:
             _ops._linear_skinny_unchecked(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
@@ -903,7 +928,7 @@ def _layer_modules(layer):
     return now if ok else False
 
 
-FUSED_LAYER_MAX_ROWS = 8     # sequences for which the projection kernel takes the norm in front and SwiGLU behind
+FUSED_LAYER_MAX_ROWS = _FUSED_ROWS     # sequences for which the projection kernel takes the norm in front and SwiGLU behind
 
 
 def _layer_takes_fast_path(layer, hidden_states):
@@ -950,23 +975,26 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
         attn._sync_bit_cache(cache)
         slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
         if slot is not None and hidden_states.shape[0] > FUSED_LAYER_MAX_ROWS:
-            # more sequences than the fused forms take: the same layer in twelve calls - each RMSNorm one launch with the module's
-            # two roundings, the attention step, the library's GEMM on the stacked gate/up weight and on the down projection,
-            # SwiGLU one launch, the two residual additions - instead of the library layer's ~26
+            # more sequences than the fused forms take: the same layer in ten to twelve calls - each RMSNorm one launch with the
+            # module's two roundings, the attention step (the first residual inside its output projection), gate/up with SwiGLU
+            # (9 to 16 sequences: one launch on a tiled copy of the stacked weight; above: the library's GEMM and ha_swiglu), the
+            # library's GEMM for the down projection, the second residual addition - instead of the library layer's ~26
             b, _, hidden = hidden_states.shape
             mlp, n1, n2, gate, _, down = mods
             h = torch.empty_like(hidden_states)
             _ops.rmsnorm(hidden_states[:, 0, :], n1.weight, float(n1.variance_epsilon), h[:, 0, :])
-            y, _ = attn._fast_decode(h, position_embeddings, slot[0], amask=slot[1])
+            x1, _ = attn._fast_decode(h, position_embeddings, slot[0], residual=hidden_states[:, 0, :], amask=slot[1])
             attn._note_key_storage(cache)
-            x1 = hidden_states + y
             _ops.rmsnorm(x1[:, 0, :], n2.weight, float(n2.variance_epsilon), h[:, 0, :])
-            gate_up = torch.mm(h[:, 0, :], _stacked_gate_up(attn, mlp).t())
             act = attn.__dict__.get("_fast_act")
             if act is None or act.shape[0] != b or act.shape[1] != gate.out_features or act.device != hidden_states.device:
                 act = torch.empty(b, gate.out_features, dtype=torch.bfloat16, device=hidden_states.device)
                 attn.__dict__["_fast_act"] = act
-            _ops.swiglu(gate_up, act)
+            if attn._takes_tiled_projections(b, hidden):    # 9 to 16 sequences: gate/up on the matrix cores, SwiGLU inside
+                _ops._linear_tiled_unchecked(h[:, 0, :], attn._weight_tiles("_gate_up_tiles", (mlp.gate_proj.weight, mlp.up_proj.weight),
+                                                                            glu=True), 2 * gate.out_features, act, swiglu=True)
+            else:
+                _ops.swiglu(torch.mm(h[:, 0, :], _stacked_gate_up(attn, mlp).t()), act)
             return x1 + torch.mm(act, down.weight.t()).view(b, 1, hidden)
         if slot is not None:
             b = hidden_states.shape[0]

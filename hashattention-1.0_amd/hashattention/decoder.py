@@ -105,6 +105,23 @@ class LlamaShapedDecoder:
         self.len_dev = torch.ones(B, dtype=torch.int32, device=self.device)
         self._gen_graph = self._gen_logits = None
         self.ws_dense = _ops.workspace(_ops.dense_decode_workspace_bytes(B, self.H, S_cap), self.device)
+        self._pack_tiles()
+
+    def _tiled(self) -> bool:
+        """9 to 16 sequences of a bf16 model: the projections whose inputs fit (QKV, output, gate/up) run on the matrix cores
+        from tiled copies of their weights (`ha_linear_tiled`)."""
+        return self.use_skinny and self.dtype == torch.bfloat16 and 8 < getattr(self, "B", 0) <= _ops.LINEAR_SKINNY_MAX_ROWS \
+            and max(self.hidden, self.H * self.d) <= _ops.LINEAR_TILED_MAX_K
+
+    def _pack_tiles(self) -> None:
+        """(Re)make the tiled copies for the batch this decoder was allocated for; dropped when they do not apply."""
+        for p in self.layers:
+            for name in ("wqkv_t", "wo_t", "w13_t"):
+                p.pop(name, None)
+            if self._tiled() and "wqkv" in p:
+                p["wqkv_t"] = _ops.pack_weight_tiles(p["wqkv"])
+                p["wo_t"] = _ops.pack_weight_tiles(p["wo"])
+                p["w13_t"] = _ops.pack_weight_tiles(p["w13"], glu=True)
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
         """Put `seq_len` synthetic tokens (N(0,1) keys/values) in every layer's cache and hash all keys with the MFMA
@@ -179,9 +196,12 @@ class LlamaShapedDecoder:
             out = torch.empty_like(t)
             _ops.rmsnorm(t, weight, self.eps, out)
             return out
+        tiled = self._tiled() and "wqkv_t" in self.layers[0]
         for l, p in enumerate(self.layers):
             if skinny:      # RMSNorm rides in the projection that consumes it
                 qkv = _ops.linear_skinny(x, p["wqkv"], self.qkv, norm_weight=p["attn_norm"], eps=self.eps)
+            elif tiled:
+                qkv = _ops.linear_tiled(norm(x, p["attn_norm"]), p["wqkv_t"], self.qkv.shape[1], self.qkv)
             else:
                 qkv = F.linear(norm(x, p["attn_norm"]), p["wqkv"])
             hl = self.hash[l]
@@ -206,6 +226,9 @@ class LlamaShapedDecoder:
                 x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn[0 if self.skinny_all else (l + 1) % 2], residual=x)
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
+            elif tiled:     # residual inside the output projection, SwiGLU inside the gate/up projection
+                x = _ops.linear_tiled(self.attn_out.view(B, H * d), p["wo_t"], self.hidden, self.x_attn[l % 2], residual=x)
+                _ops.linear_tiled(norm(x, p["ffn_norm"]), p["w13_t"], 2 * self.ffn, self.ffn_act, swiglu=True)
             else:
                 if lowp:
                     x = x + F.linear(self.attn_out.view(B, H * d), p["wo"])
@@ -357,3 +380,5 @@ class LlamaShapedDecoder:
             p["wo"] = cast(sd[pre + "self_attn.o_proj.weight"])
             p["w13"] = torch.cat([cast(sd[pre + "mlp.gate_proj.weight"]), cast(sd[pre + "mlp.up_proj.weight"])], dim=0)
             p["w2"] = cast(sd[pre + "mlp.down_proj.weight"])
+        if getattr(self, "B", 0):
+            self._pack_tiles()

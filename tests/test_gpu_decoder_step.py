@@ -149,6 +149,32 @@ def test_bf16_decoder_step_with_and_without_the_skinny_projections():
     assert (c - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
 
 
+def test_bf16_decoder_step_of_a_dozen_sequences_on_tiled_weights():
+    # 9 to 16 sequences: QKV, output and gate/up projections on the matrix cores from tiled copies of the weights (residual and
+    # SwiGLU inside), RMSNorm as one launch; against the same step through the library's GEMMs, and through graph replay
+    print("\n[case] bf16 decoder step, 12 sequences, tiled projections on/off", flush=True)
+    dec = LlamaShapedDecoder(n_layers=2, hidden=512, ffn=1024, n_heads=4, n_kv_heads=2, head_dim=128, vocab=512, n_code_heads=2,
+                             init_budget=8, recent_budget=8, heavy_budget=0.125, dtype=torch.bfloat16, device=DEV, seed=5)
+    dec.allocate(12, 400)
+    dec.fill_cache_synthetic(300)
+    assert dec._tiled() and "w13_t" in dec.layers[0]
+    tokens = torch.arange(12, device=DEV) * 7 + 3
+    with torch.no_grad():
+        a = dec.decode_step(tokens, advance=False).float()
+        dec.use_skinny = False
+        assert not dec._tiled()
+        b = dec.decode_step(tokens, advance=False).float()
+        dec.use_skinny = True
+        got = dec.generate(tokens, 5)
+        dec.seq_len -= 5
+        for hl in dec.hash:
+            hl.n_cached -= 5
+        want = dec.generate(tokens, 5, use_graph=False)
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 0.05 * max(1.0, b.abs().max().item())
+    assert torch.equal(got, want)
+
+
 def test_decoder_step_on_the_fused_attention_path_matches_the_two_launch_path():
     # 32 (sequence, head) rows: every layer takes ha_select_histogram + ha_sparse_decode_fused; the same step through
     # ha_select + ha_sparse_decode must agree to bf16 noise, and the index lists the fused path never writes stay usable

@@ -354,17 +354,35 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void *__restrict__ x
     auto widen = [&](uint32_t bits16) {
         return dtype == HA_BF16 ? __uint_as_float(bits16 << 16) : __half2float(__ushort_as_half((unsigned short)bits16));
     };
+    auto narrow = [&](float f) {
+        return dtype == HA_BF16 ? ha_f32_to_bf16_bits(f) : (uint32_t)__half_as_ushort(__float2half(f));
+    };
+    // VEC: the row and the weight are requested together and stay in registers between the two passes (rows of up to 8192
+    // elements: one memory round trip for the whole launch); what lies beyond is read again
+    constexpr int kHold = 4;
+    [[maybe_unused]] uint4 xv[kHold], gv[kHold];
     float a = 0.f;
     if constexpr (VEC) {
-        for (int k = tid * 8; k < K; k += 256 * 8) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(xr + k * 2);
+#pragma unroll
+        for (int i = 0; i < kHold; ++i) {
+            const int k = (tid + i * 256) * 8;
+            xv[i] = gv[i] = make_uint4(0u, 0u, 0u, 0u);
+            if (k < K) {
+                xv[i] = *reinterpret_cast<const uint4 *>(xr + k * 2);
+                gv[i] = *reinterpret_cast<const uint4 *>((const char *)w + k * 2);
+            }
+        }
+        auto squares = [&](const uint4 &v) {
             const uint32_t p[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float lo = widen(p[i] & 0xffffu), hi = widen(p[i] >> 16);
                 a = fmaf(lo, lo, fmaf(hi, hi, a));
             }
-        }
+        };
+#pragma unroll
+        for (int i = 0; i < kHold; ++i) squares(xv[i]);
+        for (int k = (tid + kHold * 256) * 8; k < K; k += 256 * 8) squares(*reinterpret_cast<const uint4 *>(xr + k * 2));
     } else {
         for (int k = tid; k < K; k += 256) {
             const float v = ha_load_elem(xr, k, dtype);
@@ -376,13 +394,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void *__restrict__ x
     if ((tid & 63) == 0) s_sum[tid >> 6] = a;
     __syncthreads();
     const float rstd = rsqrtf((s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3]) / (float)K + eps);
-    auto narrow = [&](float f) {
-        return dtype == HA_BF16 ? ha_f32_to_bf16_bits(f) : (uint32_t)__half_as_ushort(__float2half(f));
-    };
     if constexpr (VEC) {
-        for (int k = tid * 8; k < K; k += 256 * 8) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(xr + k * 2);
-            const uint4 g = *reinterpret_cast<const uint4 *>((const char *)w + k * 2);
+        auto scaled = [&](const uint4 &v, const uint4 &g) {
             const uint32_t p[4] = {v.x, v.y, v.z, v.w}, q[4] = {g.x, g.y, g.z, g.w};
             uint32_t r[4];
 #pragma unroll
@@ -391,8 +404,16 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void *__restrict__ x
                 const float hi = ha_round_to(widen(p[i] >> 16) * rstd, dtype) * widen(q[i] >> 16);
                 r[i] = narrow(lo) | (narrow(hi) << 16);
             }
-            *reinterpret_cast<uint4 *>(yr + k * 2) = make_uint4(r[0], r[1], r[2], r[3]);
+            return make_uint4(r[0], r[1], r[2], r[3]);
+        };
+#pragma unroll
+        for (int i = 0; i < kHold; ++i) {
+            const int k = (tid + i * 256) * 8;
+            if (k < K) *reinterpret_cast<uint4 *>(yr + k * 2) = scaled(xv[i], gv[i]);
         }
+        for (int k = (tid + kHold * 256) * 8; k < K; k += 256 * 8)
+            *reinterpret_cast<uint4 *>(yr + k * 2) =
+                scaled(*reinterpret_cast<const uint4 *>(xr + k * 2), *reinterpret_cast<const uint4 *>((const char *)w + k * 2));
     } else {
         for (int k = tid; k < K; k += 256)
             ha_store_elem(yr, k, ha_round_to(ha_load_elem(xr, k, dtype) * rstd, dtype) * ha_load_elem(w, k, dtype), dtype);

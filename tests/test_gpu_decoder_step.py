@@ -439,7 +439,7 @@ def test_linear_tiled_against_fp32_matmul(M, N, K, form):
 
 
 @pytest.mark.parametrize("dtype,M,K", [(torch.bfloat16, 12, 4096), (torch.bfloat16, 3, 5120), (torch.float16, 5, 1024),
-                                       (torch.float32, 4, 768), (torch.bfloat16, 2, 100)])
+                                       (torch.float32, 4, 768), (torch.bfloat16, 2, 100), (torch.bfloat16, 2, 14336)])
 def test_rmsnorm_launch_rounds_as_the_module_it_replaces(dtype, M, K):
     # ha_rmsnorm against transformers' LlamaRMSNorm in the same dtype: the normalised row rounded to the element type, then the
     # product with the weight rounded again.  The sum of squares is added in another order, so a rounding may fall the other way

@@ -48,7 +48,8 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint16_t *__restr
 // GLU: SwiGLU behind (tiles packed with `glu`): out [M, F] = bf16(bf16(silu(bf16 gate)) * bf16 up).
 // (An RMSNorm in front, as the row-streaming kernel has it, would keep a second copy of the slice alive while it is applied:
 // 241 registers at 16 k-steps per wave.  Batches of this size run ha_rmsnorm as a launch of its own.)
-template <int NWAVE, int XS, bool GLU>
+// MB: blocks of 16 rows of x (1 or 2): with 17 to 32 rows every weight operand is multiplied twice.
+template <int NWAVE, int XS, bool GLU, int MB>
 __global__ __launch_bounds__(NWAVE * 64) void tiled_linear_kernel(const uint16_t *__restrict__ x, int64_t x_sm,
                                                                   const uint16_t *__restrict__ tiles,
                                                                   const uint16_t *__restrict__ res, int64_t res_sm,
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(NWAVE * 64) void tiled_linear_kernel(const uint16_t
     constexpr int PF = 4;  // k-steps requested together
     constexpr bool kGlu = GLU;
     static_assert(XS % PF == 0, "a wave's slice is whole groups of k-steps");
-    __shared__ float s_c[NWAVE][16][17];
+    __shared__ float s_c[NWAVE][16][16 * MB + 1];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 15, g = lane >> 4;
     const int ksteps = K / kTileK;
     const int s_beg = wave * XS;  // this wave's k-steps [s_beg, s_beg + XS); those beyond ksteps are zero
@@ -75,31 +76,40 @@ __global__ __launch_bounds__(NWAVE * 64) void tiled_linear_kernel(const uint16_t
     int nt = blockIdx.x;
     fetch(nt, 0, wc);  // the first weights are on their way before x is set up
 
-    uint4 xr[XS];
+    uint4 xr[MB][XS];
 #pragma unroll
-    for (int j = 0; j < XS; ++j) {
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (m < M && s_beg + j < ksteps) v = *reinterpret_cast<const uint4 *>(x + (int64_t)m * x_sm + (s_beg + j) * kTileK + 8 * g);
-        xr[j] = v;
-    }
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int j = 0; j < XS; ++j) {
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (16 * mb + m < M && s_beg + j < ksteps)
+                v = *reinterpret_cast<const uint4 *>(x + (int64_t)(16 * mb + m) * x_sm + (s_beg + j) * kTileK + 8 * g);
+            xr[mb][j] = v;
+        }
 
     while (nt < n_tiles) {
         const int nt_next = nt + gridDim.x;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        f32x4 acc[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j0 = 0; j0 < XS; j0 += PF) {
             if (j0 + PF < XS) fetch(nt, j0 + PF, wn);
             else fetch(nt_next, 0, wn);  // nothing is requested past the last tile row
 #pragma unroll
             for (int i = 0; i < PF; ++i)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wc[i]), __builtin_bit_cast(bf16x8, xr[j0 + i]), acc,
-                                                              0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wc[i]),
+                                                                      __builtin_bit_cast(bf16x8, xr[mb][j0 + i]), acc[mb], 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < PF; ++i) wc[i] = wn[i];
         }
-        // acc[i] = sum for tile row 4 g + i and row m of x
+        // acc[mb][i] = sum for tile row 4 g + i and row 16 mb + m of x
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_c[wave][4 * g + i][m] = acc[i];
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_c[wave][4 * g + i][16 * mb + m] = acc[mb][i];
         __syncthreads();
         if constexpr (kGlu) {
             const int F = N / 2;
@@ -160,8 +170,9 @@ int ha_pack_weight_tiles(const void *w, int64_t w_stride_n, int N, int K, int gl
 int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const void *residual, int64_t residual_stride_m, int act,
                     void *out, int64_t out_stride_m, int M, int N, int K, void *stream) {
     HA_REQUIRE(x && tiles && out, HA_ERR_NULL_POINTER, "x/tiles/out is NULL");
-    HA_REQUIRE(M >= 1 && M <= 16 && N >= 1 && K >= 32 && K % kTileK == 0, HA_ERR_BAD_SHAPE, "need 1 <= M <= 16, N >= 1, K a multiple of 32");
-    HA_REQUIRE(K <= 8192, HA_ERR_BAD_SHAPE, "K=%d: a workgroup keeps x in registers, up to 8192 inputs", K);
+    HA_REQUIRE(M >= 1 && M <= 32 && N >= 1 && K >= 32 && K % kTileK == 0, HA_ERR_BAD_SHAPE, "need 1 <= M <= 32, N >= 1, K a multiple of 32");
+    HA_REQUIRE(K <= (M <= 16 ? 8192 : 4096), HA_ERR_BAD_SHAPE,
+               "K=%d: a workgroup keeps x in registers, up to 8192 inputs of 16 rows or 4096 of 32", K);
     HA_REQUIRE(act == 0 || act == 1, HA_ERR_BAD_SHAPE, "unknown activation %d", act);
     const int n_out = act ? N / 2 : N;
     HA_REQUIRE(!act || (N % 2 == 0 && !residual), HA_ERR_BAD_SHAPE, "SwiGLU needs an even number of weight rows and no residual");
@@ -174,23 +185,29 @@ int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const 
     const int ksteps = K / kTileK;
     const int n_tiles = act ? (N / 2 + 7) / 8 : (N + kTileRows - 1) / kTileRows;
     // two 512-thread workgroups (one 1024-thread workgroup) per CU are resident; more tile rows than that are walked
-    const bool wide = ksteps > 128;
+    const bool wide = ksteps > 128 || (M > 16 && ksteps > 64);
     const int grid = n_tiles < (wide ? 256 : 512) ? n_tiles : (wide ? 256 : 512);
     const uint16_t *xp = (const uint16_t *)x, *tp = (const uint16_t *)tiles, *rp = (const uint16_t *)residual;
     uint16_t *op = (uint16_t *)out;
     hipStream_t s = (hipStream_t)stream;
-#define HA_TILED_LAUNCH(NW_, XS_, G_)                                                                                         \
-    hipLaunchKernelGGL((tiled_linear_kernel<NW_, XS_, G_>), dim3(grid), dim3(NW_ * 64), 0, s, xp, x_stride_m, tp, rp,         \
+#define HA_TILED_LAUNCH(NW_, XS_, G_, MB_)                                                                                    \
+    hipLaunchKernelGGL((tiled_linear_kernel<NW_, XS_, G_, MB_>), dim3(grid), dim3(NW_ * 64), 0, s, xp, x_stride_m, tp, rp,    \
                        residual_stride_m, op, out_stride_m, M, N, K)
-#define HA_TILED_FUSE(NW_, XS_)                  \
-    do {                                         \
-        if (act) HA_TILED_LAUNCH(NW_, XS_, true); \
-        else HA_TILED_LAUNCH(NW_, XS_, false);   \
+#define HA_TILED_FUSE(NW_, XS_, MB_)                   \
+    do {                                               \
+        if (act) HA_TILED_LAUNCH(NW_, XS_, true, MB_); \
+        else HA_TILED_LAUNCH(NW_, XS_, false, MB_);    \
     } while (0)
-    if (ksteps <= 32) HA_TILED_FUSE(8, 4);
-    else if (ksteps <= 64) HA_TILED_FUSE(8, 8);
-    else if (ksteps <= 128) HA_TILED_FUSE(8, 16);
-    else HA_TILED_FUSE(16, 16);
+    if (M <= 16) {
+        if (ksteps <= 32) HA_TILED_FUSE(8, 4, 1);
+        else if (ksteps <= 64) HA_TILED_FUSE(8, 8, 1);
+        else if (ksteps <= 128) HA_TILED_FUSE(8, 16, 1);
+        else HA_TILED_FUSE(16, 16, 1);
+    } else {  // 17 to 32 rows: twice the registers per k-step
+        if (ksteps <= 32) HA_TILED_FUSE(8, 4, 2);
+        else if (ksteps <= 64) HA_TILED_FUSE(8, 8, 2);
+        else HA_TILED_FUSE(16, 8, 2);
+    }
 #undef HA_TILED_FUSE
 #undef HA_TILED_LAUNCH
     HA_CHECK_LAUNCH("tiled_linear_kernel");

@@ -659,7 +659,12 @@ HA_ACT_NONE, HA_ACT_SWIGLU = 0, 1
 
 
 LINEAR_SKINNY_MAX_ROWS = 16     # rows of x that ha_linear_skinny takes
-LINEAR_TILED_MAX_K = 8192       # inputs that ha_linear_tiled takes
+LINEAR_TILED_MAX_K = 8192       # inputs that ha_linear_tiled takes for up to 16 rows of x
+LINEAR_TILED_MAX_ROWS = 32      # rows of x that ha_linear_tiled takes (above 16: up to LINEAR_TILED_MAX_K / 2 inputs)
+
+
+def linear_tiled_applies(rows: int, k: int) -> bool:
+    return rows <= 16 and k <= LINEAR_TILED_MAX_K or rows <= LINEAR_TILED_MAX_ROWS and k <= LINEAR_TILED_MAX_K // 2
 
 
 def pack_weight_tiles(w: torch.Tensor, glu: bool = False) -> torch.Tensor:
@@ -677,8 +682,8 @@ def pack_weight_tiles(w: torch.Tensor, glu: bool = False) -> torch.Tensor:
 
 def linear_tiled(x: torch.Tensor, tiles: torch.Tensor, N: int, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
                  swiglu: bool = False) -> torch.Tensor:
-    """out [M, N] (or [M, N / 2] with swiglu) = x [M, K] . W^T (+ residual) from the tiled copy of W [N, K].  M <= 16,
-    K <= 8192."""
+    """out [M, N] (or [M, N / 2] with swiglu) = x [M, K] . W^T (+ residual) from the tiled copy of W [N, K].  M <= 16 with
+    K <= 8192, or M <= 32 with K <= 4096."""
     _require_cuda(x, tiles, out, residual)
     assert x.dim() == 2 and x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1
     M, K = x.shape

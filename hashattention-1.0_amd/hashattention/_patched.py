@@ -568,7 +568,7 @@ class HeavyHitterMixin:
 
     def _weight_tiles(self, name: str, weights, glu: bool = False) -> torch.Tensor:
         """The tiled copy (`ha_pack_weight_tiles`) of the given weights stacked row-wise, which `ha_linear_tiled` reads for
-        batches of 9 to 16 sequences; kept under `name`, rebuilt like `_fused_qkv_weight`."""
+        batches of 9 to 32 sequences; kept under `name`, rebuilt like `_fused_qkv_weight`."""
         key = tuple((w.data_ptr(), w._version, w.dtype, w.device) for w in weights)
         hit = self.__dict__.get(name)
         if hit is None or hit[0] != key:
@@ -578,7 +578,7 @@ class HeavyHitterMixin:
         return hit[1]
 
     def _takes_tiled_projections(self, b: int, hidden: int) -> bool:
-        return _FUSED_ROWS < b <= _ops.LINEAR_SKINNY_MAX_ROWS and max(hidden, self.num_heads * self.head_dim) <= _ops.LINEAR_TILED_MAX_K
+        return b > _FUSED_ROWS and _ops.linear_tiled_applies(b, max(hidden, self.num_heads * self.head_dim))
 
     def _fast_decode_slot(self, hidden_states, position_embeddings, attention_mask, cache):
         """(This layer's `PreallocatedLayer` of `cache`, the additive mask as a `_StepMask` or None when it changes nothing)
@@ -641,12 +641,12 @@ class HeavyHitterMixin:
                       attn=torch.empty(b, H, d, dtype=torch.bfloat16, device=dev))
             self.__dict__["_fast_scratch"] = sc
         tiled = self._takes_tiled_projections(b, hidden)
-        if b > _ops.LINEAR_SKINNY_MAX_ROWS:     # more sequences than the projection kernels take: the library's GEMM, still one call
-            torch.mm(hidden_states[:, 0, :], self._fused_qkv_weight().t(), out=sc["qkv"])
-        elif tiled:                             # 9 to 16 sequences: the matrix cores on a tiled copy of the stacked weight
+        if tiled:                               # 9 to 32 sequences: the matrix cores on a tiled copy of the stacked weight
             _ops._linear_tiled_unchecked(hidden_states[:, 0, :], self._weight_tiles("_qkv_tiles", (self.q_proj.weight, self.k_proj.weight,
                                                                                                  self.v_proj.weight)),
                                          sc["qkv"].shape[1], sc["qkv"])
+        elif b > _ops.LINEAR_SKINNY_MAX_ROWS:   # more sequences than the projection kernels take: the library's GEMM, still one call
+            torch.mm(hidden_states[:, 0, :], self._fused_qkv_weight().t(), out=sc["qkv"])
         elif norm is None:
             _ops._linear_skinny_unchecked(hidden_states[:, 0, :], self._fused_qkv_weight(), sc["qkv"])
         else:
@@ -672,13 +672,13 @@ class HeavyHitterMixin:
         finally:
             hl.heavy_budget = saved
         out = torch.empty(b, 1, hidden, dtype=torch.bfloat16, device=dev)
-        if b > _ops.LINEAR_SKINNY_MAX_ROWS:
+        if tiled:
+            _ops._linear_tiled_unchecked(sc["attn"].view(b, H * d), self._weight_tiles("_o_tiles", (self.o_proj.weight,)), hidden,
+                                         out.view(b, hidden), residual=residual)
+        elif b > _ops.LINEAR_SKINNY_MAX_ROWS:
             torch.mm(sc["attn"].view(b, H * d), self.o_proj.weight.t(), out=out.view(b, hidden))
             if residual is not None:
                 out.view(b, hidden).add_(residual)      # the projection's rounding, then the addition's
-        elif tiled:
-            _ops._linear_tiled_unchecked(sc["attn"].view(b, H * d), self._weight_tiles("_o_tiles", (self.o_proj.weight,)), hidden,
-                                         out.view(b, hidden), residual=residual)
         else:
             _ops._linear_skinny_unchecked(sc["attn"].view(b, H * d), self.o_proj.weight, out.view(b, hidden), residual=residual)
         return out, None
@@ -977,7 +977,7 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
         if slot is not None and hidden_states.shape[0] > FUSED_LAYER_MAX_ROWS:
             # more sequences than the fused forms take: the same layer in ten to twelve calls - each RMSNorm one launch with the
             # module's two roundings, the attention step (the first residual inside its output projection), gate/up with SwiGLU
-            # (9 to 16 sequences: one launch on a tiled copy of the stacked weight; above: the library's GEMM and ha_swiglu), the
+            # (9 to 32 sequences: one launch on a tiled copy of the stacked weight; above: the library's GEMM and ha_swiglu), the
             # library's GEMM for the down projection, the second residual addition - instead of the library layer's ~26
             b, _, hidden = hidden_states.shape
             mlp, n1, n2, gate, _, down = mods
@@ -990,7 +990,7 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
             if act is None or act.shape[0] != b or act.shape[1] != gate.out_features or act.device != hidden_states.device:
                 act = torch.empty(b, gate.out_features, dtype=torch.bfloat16, device=hidden_states.device)
                 attn.__dict__["_fast_act"] = act
-            if attn._takes_tiled_projections(b, hidden):    # 9 to 16 sequences: gate/up on the matrix cores, SwiGLU inside
+            if attn._takes_tiled_projections(b, hidden):    # 9 to 32 sequences: gate/up on the matrix cores, SwiGLU inside
                 _ops._linear_tiled_unchecked(h[:, 0, :], attn._weight_tiles("_gate_up_tiles", (mlp.gate_proj.weight, mlp.up_proj.weight),
                                                                             glu=True), 2 * gate.out_features, act, swiglu=True)
             else:

@@ -108,10 +108,10 @@ class LlamaShapedDecoder:
         self._pack_tiles()
 
     def _tiled(self) -> bool:
-        """9 to 16 sequences of a bf16 model: the projections whose inputs fit (QKV, output, gate/up) run on the matrix cores
+        """9 to 32 sequences of a bf16 model: the projections whose inputs fit (QKV, output, gate/up) run on the matrix cores
         from tiled copies of their weights (`ha_linear_tiled`)."""
-        return self.use_skinny and self.dtype == torch.bfloat16 and 8 < getattr(self, "B", 0) <= _ops.LINEAR_SKINNY_MAX_ROWS \
-            and max(self.hidden, self.H * self.d) <= _ops.LINEAR_TILED_MAX_K
+        B = getattr(self, "B", 0)
+        return self.use_skinny and self.dtype == torch.bfloat16 and B > 8 and _ops.linear_tiled_applies(B, max(self.hidden, self.H * self.d))
 
     def _pack_tiles(self) -> None:
         """(Re)make the tiled copies for the batch this decoder was allocated for; dropped when they do not apply."""

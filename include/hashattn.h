@@ -482,14 +482,15 @@ int ha_linear_skinny_fused(const void *x, int64_t x_stride_m, const void *w, int
                            int64_t out_stride_m, int M, int N, int K, void *stream);
 
 /*
- * The same products for 9 to 16 rows of x (and fewer) from a TILED copy of the weights: tiles of 16 rows x 32 inputs laid out
+ * The same products for 9 to 32 rows of x (and fewer) from a TILED copy of the weights: tiles of 16 rows x 32 inputs laid out
  * as the operand of the bf16 matrix instruction, so that a wave load is one contiguous KiB (row-major weights give such a
  * batch 64-byte pieces of 16 rows per load, 2.5 - 4 TB/s).  For callers that own a copy of the weights anyway (a decoding
  * harness as efficiency/model.py:236-262, 304-305; the stacked QKV and gate/up matrices of a patched layer).
  *   ha_weight_tiles_elems  bf16 elements of the tiled copy of a [N, K] matrix (rows padded to whole tiles), 0 for a bad shape
  *   ha_pack_weight_tiles   w [N, K] bf16 row-major (row stride w_stride_n) -> tiles.  glu = 1: w is [F gate rows; F up rows]
  *                          and every tile holds 8 gate rows followed by the 8 up rows of the same columns
- *   ha_linear_tiled        out [M, N] = x [M, K] . W^T (+ residual), M <= 16, K <= 8192 a multiple of 32;
+ *   ha_linear_tiled        out [M, N] = x [M, K] . W^T (+ residual), K a multiple of 32; M <= 16 with K <= 8192, or M <= 32
+ *                          with K <= 4096 (every weight operand is then multiplied with two blocks of 16 rows);
  *                          act = HA_ACT_SWIGLU (tiles packed with glu = 1, N = 2 F): out [M, F] = silu(gate) * up.
  *                          Roundings as ha_linear_skinny_fused: those of the modules replaced.  (An RMSNorm in front is
  *                          ha_rmsnorm, a launch of its own, for batches of this size.)

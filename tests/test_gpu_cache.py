@@ -425,7 +425,7 @@ def test_few_launch_steps_on_other_model_shapes(shape):
     assert worst <= 3e-2 * max(scale, 1.0), (worst, scale)
 
 
-@pytest.mark.parametrize("batch,whole_layer", [(18, False), (18, True), (12, True), (12, False), (9, True)])
+@pytest.mark.parametrize("batch,whole_layer", [(18, False), (18, True), (12, True), (12, False), (9, True), (40, True)])
 def test_few_call_steps_with_more_sequences_than_the_fused_projections_take(batch, whole_layer):
     # 18 sequences: the attention module keeps its five-call step (the library's GEMM on the stacked QKV weight and on the
     # output projection, the rotary/append/hash launch, histograms, select-attend).  The decoder layer around it: the library's

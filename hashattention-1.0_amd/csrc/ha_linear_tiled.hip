@@ -8,6 +8,7 @@
 // The projections of the reference's decoding harness (efficiency/model.py:236-262, 304-305) with the elementwise steps next
 // to them (:308-319 RMSNorm, :190-191 residuals), roundings as those modules round.
 #include "ha_common.h"
+#include <cstdlib>
 
 namespace {
 
@@ -184,9 +185,13 @@ int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const 
     if (st) return st;
     const int ksteps = K / kTileK;
     const int n_tiles = act ? (N / 2 + 7) / 8 : (N + kTileRows - 1) / kTileRows;
-    // two 512-thread workgroups (one 1024-thread workgroup) per CU are resident; more tile rows than that are walked
-    const bool wide = ksteps > 128 || (M > 16 && ksteps > 64);
-    const int grid = n_tiles < (wide ? 256 : 512) ? n_tiles : (wide ? 256 : 512);
+    // One workgroup per CU, walking the tile rows: with two 512-thread workgroups resident per CU, grids between 256 and 512
+    // leave some CUs twice the rows of others (QKV 6144 x 4096, 16 rows of x: 384 workgroups 15.4 us, 192 or 256 13.1 us;
+    // gate/up 28672 x 4096: 512 workgroups 41.3 us, 256 40.7 us, 1792 47.4 us)
+    int grid = n_tiles < 256 ? n_tiles : 256;
+#ifdef HASHATTN_TUNING_ENV
+    if (const char *e = getenv("HA_TILED_GRID")) grid = atoi(e) < n_tiles ? atoi(e) : n_tiles;
+#endif
     const uint16_t *xp = (const uint16_t *)x, *tp = (const uint16_t *)tiles, *rp = (const uint16_t *)residual;
     uint16_t *op = (uint16_t *)out;
     hipStream_t s = (hipStream_t)stream;

@@ -143,6 +143,70 @@ __global__ __launch_bounds__(NWAVE * 64) void tiled_linear_kernel(const uint16_t
     }
 }
 
+// The same product for rows of W too long for x to stay in registers (the down projection: 14336 inputs): every wave requests
+// its slices of x next to the weight tiles they meet.  x is then read once per tile row - from L2, it is a few hundred KiB - so
+// this form is for matrices of few tile rows per workgroup, where keeping x would not save anything either.  Up to 16 rows of x.
+template <int NWAVE>
+__global__ __launch_bounds__(NWAVE * 64) void tiled_linear_stream_kernel(const uint16_t *__restrict__ x, int64_t x_sm,
+                                                                         const uint16_t *__restrict__ tiles,
+                                                                         const uint16_t *__restrict__ res, int64_t res_sm,
+                                                                         uint16_t *__restrict__ out, int64_t out_sm, int M, int N, int K) {
+    constexpr int PF = 4;
+    __shared__ float s_c[NWAVE][16][17];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 15, g = lane >> 4;
+    const int ksteps = K / kTileK;
+    const int per = ((ksteps + NWAVE - 1) / NWAVE + PF - 1) / PF * PF;  // k-steps per wave, whole groups of PF
+    const int s_beg = wave * per, s_end = min(s_beg + per, ksteps);
+    const int n_tiles = (N + kTileRows - 1) / kTileRows;
+    const uint16_t *xrow = x + (int64_t)min(m, M - 1) * x_sm + 8 * g;
+    const bool x_ok = m < M;
+    auto fetch = [&](int nt, int s0, uint4 (&wv)[PF], uint4 (&xv)[PF]) {
+        const uint4 *tp = reinterpret_cast<const uint4 *>(tiles) + ((int64_t)nt * ksteps + s0) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            const bool ok = nt < n_tiles && s0 + i < s_end;
+            uint4 wq = make_uint4(0u, 0u, 0u, 0u), xq = make_uint4(0u, 0u, 0u, 0u);
+            if (ok) wq = ha_load16_stream(tp + (int64_t)i * 64);
+            if (ok && x_ok) xq = *reinterpret_cast<const uint4 *>(xrow + (int64_t)(s0 + i) * kTileK);
+            wv[i] = wq;
+            xv[i] = xq;
+        }
+    };
+    uint4 wc[PF], xc[PF], wn[PF], xn[PF];
+    int nt = blockIdx.x;
+    fetch(nt, s_beg, wc, xc);
+    while (nt < n_tiles) {
+        const int nt_next = nt + gridDim.x;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int s0 = s_beg; s0 < s_end; s0 += PF) {
+            if (s0 + PF < s_end) fetch(nt, s0 + PF, wn, xn);
+            else fetch(nt_next, s_beg, wn, xn);
+#pragma unroll
+            for (int i = 0; i < PF; ++i)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wc[i]), __builtin_bit_cast(bf16x8, xc[i]), acc, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < PF; ++i) {
+                wc[i] = wn[i];
+                xc[i] = xn[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_c[wave][4 * g + i][m] = acc[i];
+        __syncthreads();
+        for (int t = tid; t < 16 * M; t += NWAVE * 64) {
+            const int mm = t >> 4, r = t & 15, n = 16 * nt + r;
+            if (n >= N) continue;
+            float y = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NWAVE; ++wv) y += s_c[wv][r][mm];
+            if (res) y = ha_round_bf16(y) + ha_bf16_lo((uint32_t)res[(int64_t)mm * res_sm + n]);  // the projection's rounding, then the addition's
+            out[(int64_t)mm * out_sm + n] = (uint16_t)ha_f32_to_bf16_bits(y);
+        }
+        nt = nt_next;
+        if (nt < n_tiles) __syncthreads();
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -172,9 +236,11 @@ int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const 
                     void *out, int64_t out_stride_m, int M, int N, int K, void *stream) {
     HA_REQUIRE(x && tiles && out, HA_ERR_NULL_POINTER, "x/tiles/out is NULL");
     HA_REQUIRE(M >= 1 && M <= 32 && N >= 1 && K >= 32 && K % kTileK == 0, HA_ERR_BAD_SHAPE, "need 1 <= M <= 32, N >= 1, K a multiple of 32");
-    HA_REQUIRE(K <= (M <= 16 ? 8192 : 4096), HA_ERR_BAD_SHAPE,
-               "K=%d: a workgroup keeps x in registers, up to 8192 inputs of 16 rows or 4096 of 32", K);
     HA_REQUIRE(act == 0 || act == 1, HA_ERR_BAD_SHAPE, "unknown activation %d", act);
+    // longer rows than a workgroup keeps of x in registers: the form that requests x next to the tiles (16 rows, no activation)
+    const bool stream_x = K > (M <= 16 ? 8192 : 4096);
+    HA_REQUIRE(!stream_x || (M <= 16 && !act), HA_ERR_BAD_SHAPE,
+               "K=%d: x stays in registers up to 8192 inputs of 16 rows or 4096 of 32; longer rows take up to 16 rows of x and no activation", K);
     const int n_out = act ? N / 2 : N;
     HA_REQUIRE(!act || (N % 2 == 0 && !residual), HA_ERR_BAD_SHAPE, "SwiGLU needs an even number of weight rows and no residual");
     HA_REQUIRE(x_stride_m >= K && out_stride_m >= n_out && (!residual || residual_stride_m >= N), HA_ERR_BAD_SHAPE,
@@ -195,6 +261,12 @@ int ha_linear_tiled(const void *x, int64_t x_stride_m, const void *tiles, const 
     const uint16_t *xp = (const uint16_t *)x, *tp = (const uint16_t *)tiles, *rp = (const uint16_t *)residual;
     uint16_t *op = (uint16_t *)out;
     hipStream_t s = (hipStream_t)stream;
+    if (stream_x) {
+        hipLaunchKernelGGL(tiled_linear_stream_kernel<16>, dim3(grid), dim3(1024), 0, s, xp, x_stride_m, tp, rp, residual_stride_m, op,
+                           out_stride_m, M, N, K);
+        HA_CHECK_LAUNCH("tiled_linear_stream_kernel");
+        return HA_OK;
+    }
 #define HA_TILED_LAUNCH(NW_, XS_, G_, MB_)                                                                                    \
     hipLaunchKernelGGL((tiled_linear_kernel<NW_, XS_, G_, MB_>), dim3(grid), dim3(NW_ * 64), 0, s, xp, x_stride_m, tp, rp,    \
                        residual_stride_m, op, out_stride_m, M, N, K)

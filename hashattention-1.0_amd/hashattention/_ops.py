@@ -682,8 +682,8 @@ def pack_weight_tiles(w: torch.Tensor, glu: bool = False) -> torch.Tensor:
 
 def linear_tiled(x: torch.Tensor, tiles: torch.Tensor, N: int, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
                  swiglu: bool = False) -> torch.Tensor:
-    """out [M, N] (or [M, N / 2] with swiglu) = x [M, K] . W^T (+ residual) from the tiled copy of W [N, K].  M <= 16 with
-    K <= 8192, or M <= 32 with K <= 4096."""
+    """out [M, N] (or [M, N / 2] with swiglu) = x [M, K] . W^T (+ residual) from the tiled copy of W [N, K].  M <= 16 (no
+    activation when K > 8192), or M <= 32 with K <= 4096."""
     _require_cuda(x, tiles, out, residual)
     assert x.dim() == 2 and x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.stride(1) == 1 and out.stride(1) == 1
     M, K = x.shape

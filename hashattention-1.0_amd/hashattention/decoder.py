@@ -35,6 +35,7 @@ class LlamaShapedDecoder:
         self.Hc = n_code_heads
         self.use_skinny = True   # ha_linear_skinny for the projections (bf16, batch <= 8) ...
         self.skinny_all = True   # ... including the down projection and the lm_head (False: library GEMMs for these two)
+        self.tile_few_rows = True     # batches of up to 8: output and down projection from tiled copies of their weights
         self.fuse_rope = True    # ha_rope_encode_step instead of ha_rope_append + ha_encode_step
         self.usa_shape = (lth_num_layers, lth_int_dim, lth_final_dim)
         self.budgets = (init_budget, recent_budget, heavy_budget)
@@ -115,13 +116,22 @@ class LlamaShapedDecoder:
 
     def _pack_tiles(self) -> None:
         """(Re)make the tiled copies for the batch this decoder was allocated for; dropped when they do not apply."""
+        few = self.use_skinny and self.dtype == torch.bfloat16 and 0 < getattr(self, "B", 0) <= 8 and self.tile_few_rows
         for p in self.layers:
-            for name in ("wqkv_t", "wo_t", "w13_t"):
+            for name in ("wqkv_t", "wo_t", "w13_t", "w2_t"):
                 p.pop(name, None)
-            if self._tiled() and "wqkv" in p:
+            if "wqkv" not in p:
+                continue
+            if self._tiled():
                 p["wqkv_t"] = _ops.pack_weight_tiles(p["wqkv"])
                 p["wo_t"] = _ops.pack_weight_tiles(p["wo"])
                 p["w13_t"] = _ops.pack_weight_tiles(p["w13"], glu=True)
+            elif few:
+                # up to 8 sequences: the two projections that carry no norm run from tiled copies as well (4 sequences, launched
+                # alone: output projection 8.5 us against 9.3 for the row-streaming kernel, down projection 21.8 against 23.8)
+                if self.H * self.d <= _ops.LINEAR_TILED_MAX_K:
+                    p["wo_t"] = _ops.pack_weight_tiles(p["wo"])
+                p["w2_t"] = _ops.pack_weight_tiles(p["w2"])
 
     def fill_cache_synthetic(self, seq_len: int, seed: int = 0) -> float:
         """Put `seq_len` synthetic tokens (N(0,1) keys/values) in every layer's cache and hash all keys with the MFMA
@@ -223,7 +233,11 @@ class LlamaShapedDecoder:
                 hl.step(self.q_rot.unsqueeze(2), self.k_cache[l], self.v_cache[l], S, self.attn_out)
             if skinny:
                 # x lives in one of two buffers from here on (the down projection below adds in place)
-                x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], self.x_attn[0 if self.skinny_all else (l + 1) % 2], residual=x)
+                xo = self.x_attn[0 if self.skinny_all else (l + 1) % 2]
+                if "wo_t" in p:
+                    x = _ops.linear_tiled(self.attn_out.view(B, H * d), p["wo_t"], self.hidden, xo, residual=x)
+                else:
+                    x = _ops.linear_skinny(self.attn_out.view(B, H * d), p["wo"], xo, residual=x)
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             elif tiled:     # residual inside the output projection, SwiGLU inside the gate/up projection
@@ -235,7 +249,9 @@ class LlamaShapedDecoder:
                 else:
                     x = x.addmm_(self.attn_out.view(B, H * d), p["wo"].t())
                 _ops.swiglu(F.linear(norm(x, p["ffn_norm"]), p["w13"]), self.ffn_act)
-            if skinny and self.skinny_all:
+            if skinny and self.skinny_all and "w2_t" in p:
+                x = _ops.linear_tiled(self.ffn_act, p["w2_t"], self.hidden, self.x_attn[1], residual=x)
+            elif skinny and self.skinny_all:
                 x = _ops.linear_skinny(self.ffn_act, p["w2"], self.x_attn[1], residual=x)
             elif lowp and not skinny:
                 x = x + F.linear(self.ffn_act, p["w2"])

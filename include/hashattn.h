@@ -489,8 +489,9 @@ int ha_linear_skinny_fused(const void *x, int64_t x_stride_m, const void *w, int
  *   ha_weight_tiles_elems  bf16 elements of the tiled copy of a [N, K] matrix (rows padded to whole tiles), 0 for a bad shape
  *   ha_pack_weight_tiles   w [N, K] bf16 row-major (row stride w_stride_n) -> tiles.  glu = 1: w is [F gate rows; F up rows]
  *                          and every tile holds 8 gate rows followed by the 8 up rows of the same columns
- *   ha_linear_tiled        out [M, N] = x [M, K] . W^T (+ residual), K a multiple of 32; M <= 16 with K <= 8192, or M <= 32
- *                          with K <= 4096 (every weight operand is then multiplied with two blocks of 16 rows);
+ *   ha_linear_tiled        out [M, N] = x [M, K] . W^T (+ residual), K a multiple of 32; M <= 16, or M <= 32 with K <= 4096
+ *                          (every weight operand is then multiplied with two blocks of 16 rows); with K > 8192 (the down
+ *                          projection) x is requested next to the tiles instead of kept in registers: M <= 16, no activation;
  *                          act = HA_ACT_SWIGLU (tiles packed with glu = 1, N = 2 F): out [M, F] = silu(gate) * up.
  *                          Roundings as ha_linear_skinny_fused: those of the modules replaced.  (An RMSNorm in front is
  *                          ha_rmsnorm, a launch of its own, for batches of this size.)

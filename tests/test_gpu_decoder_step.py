@@ -395,12 +395,13 @@ def test_decoder_from_hf_prefill_and_generate_match_the_patched_model(family):
                                         (9, 1000, 64, "plain"), (1, 40, 32, "residual"), (16, 2 * 100, 1536, "glu"),
                                         (13, 4096, 8192, "residual"), (4, 520, 2080, "plain"),
                                         (32, 6144, 4096, "plain"), (17, 4096, 4096, "residual"), (24, 2 * 14336, 4096, "glu"),
-                                        (29, 300, 96, "residual"), (20, 2 * 72, 2048, "glu")])
+                                        (29, 300, 96, "residual"), (20, 2 * 72, 2048, "glu"),
+                                        (16, 4096, 14336, "residual"), (10, 100, 8224, "plain"), (3, 4096, 28672, "residual")])
 def test_linear_tiled_against_fp32_matmul(M, N, K, form):
     # the matrix-core projection on a tiled copy of the weights (ha_pack_weight_tiles, ha_linear_tiled) against the product in fp32
     # with the roundings of the modules it stands for: the projection's output rounded to bf16 before a residual is added;
     # SwiGLU on rounded gate and up values.  Shapes: whole and ragged tile rows, one to thirty-two rows of x, K from one k-step to
-    # the 8192 inputs a workgroup holds, a K that leaves waves without work
+    # the 8192 inputs a workgroup holds and beyond (x requested next to the tiles), a K that leaves waves without work
     print(f"\n[case] ha_linear_tiled M={M} N={N} K={K} {form}", flush=True)
     g = torch.Generator(device=DEV).manual_seed(N + K + M)
     x = torch.randn(M, K, generator=g, device=DEV).to(torch.bfloat16)

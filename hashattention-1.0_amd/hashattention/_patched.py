@@ -995,6 +995,11 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
                                                                             glu=True), 2 * gate.out_features, act, swiglu=True)
             else:
                 _ops.swiglu(torch.mm(h[:, 0, :], _stacked_gate_up(attn, mlp).t()), act)
+            if b <= _ops.LINEAR_SKINNY_MAX_ROWS and attn._takes_tiled_projections(b, hidden):
+                out = torch.empty_like(x1)      # the down projection with its residual inside, x requested next to the tiles
+                _ops._linear_tiled_unchecked(act, attn._weight_tiles("_down_tiles", (down.weight,)), hidden, out[:, 0, :],
+                                             residual=x1[:, 0, :])
+                return out
             return x1 + torch.mm(act, down.weight.t()).view(b, 1, hidden)
         if slot is not None:
             b = hidden_states.shape[0]

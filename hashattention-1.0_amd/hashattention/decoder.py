@@ -126,6 +126,8 @@ class LlamaShapedDecoder:
                 p["wqkv_t"] = _ops.pack_weight_tiles(p["wqkv"])
                 p["wo_t"] = _ops.pack_weight_tiles(p["wo"])
                 p["w13_t"] = _ops.pack_weight_tiles(p["w13"], glu=True)
+                if self.B <= 16:        # with its residual inside: ahead of the library's GEMM plus an addition up to 16 rows
+                    p["w2_t"] = _ops.pack_weight_tiles(p["w2"])
             elif few:
                 # up to 8 sequences: the two projections that carry no norm run from tiled copies as well (4 sequences, launched
                 # alone: output projection 8.5 us against 9.3 for the row-streaming kernel, down projection 21.8 against 23.8)
@@ -241,7 +243,7 @@ class LlamaShapedDecoder:
                 # RMSNorm in front, SwiGLU behind: the gate/up projection writes the activated [B, ffn] directly
                 _ops.linear_skinny(x, p["w13"], self.ffn_act, norm_weight=p["ffn_norm"], eps=self.eps, swiglu=True)
             elif tiled:     # residual inside the output projection, SwiGLU inside the gate/up projection
-                x = _ops.linear_tiled(self.attn_out.view(B, H * d), p["wo_t"], self.hidden, self.x_attn[l % 2], residual=x)
+                x = _ops.linear_tiled(self.attn_out.view(B, H * d), p["wo_t"], self.hidden, self.x_attn[0], residual=x)
                 _ops.linear_tiled(norm(x, p["ffn_norm"]), p["w13_t"], 2 * self.ffn, self.ffn_act, swiglu=True)
             else:
                 if lowp:
@@ -253,6 +255,8 @@ class LlamaShapedDecoder:
                 x = _ops.linear_tiled(self.ffn_act, p["w2_t"], self.hidden, self.x_attn[1], residual=x)
             elif skinny and self.skinny_all:
                 x = _ops.linear_skinny(self.ffn_act, p["w2"], self.x_attn[1], residual=x)
+            elif tiled and "w2_t" in p:
+                x = _ops.linear_tiled(self.ffn_act, p["w2_t"], self.hidden, self.x_attn[1], residual=x)
             elif lowp and not skinny:
                 x = x + F.linear(self.ffn_act, p["w2"])
             else:

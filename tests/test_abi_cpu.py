@@ -239,6 +239,30 @@ def test_arguments_are_validated_before_any_device_work(lib):
     assert linf(act=5) == HA_ERR_SHAPE and linf(N=4095) == HA_ERR_SHAPE and linf(r=p, rs=4096) == HA_ERR_SHAPE      # SwiGLU: even rows, no residual
     assert linf(M=9) == HA_ERR_SHAPE and linf(K=32768, xs=32768, ws=32768) == HA_ERR_SHAPE and linf(g=odd) == HA_ERR_ALIGN
     assert linf(os=1000) == HA_ERR_SHAPE and linf(eps=C.c_float(-1.0)) == HA_ERR_ALIGN
+    # tiled projections, the RMSNorm launch, the fused launch with a masked prefix
+    assert lib.ha_weight_tiles_elems(6144, 4096, 0) == 6144 * 4096 and lib.ha_weight_tiles_elems(100, 64, 0) == 112 * 64
+    assert lib.ha_weight_tiles_elems(2 * 100, 64, 1) == 13 * 16 * 64            # 100 columns: 13 tiles of 8 gate + 8 up rows
+    assert lib.ha_weight_tiles_elems(64, 100, 0) == 0 and lib.ha_weight_tiles_elems(7, 64, 1) == 0 and lib.ha_weight_tiles_elems(0, 64, 0) == 0
+    pack = lambda **kw: lib.ha_pack_weight_tiles(*[{**dict(w=p, ws=4096, N=64, K=4096, glu=0, t=p, st=null), **kw}[k]
+                                                   for k in ("w", "ws", "N", "K", "glu", "t", "st")])
+    assert pack(t=null) == HA_ERR_NULL and pack(K=100) == HA_ERR_SHAPE and pack(ws=64) == HA_ERR_SHAPE and pack(N=7, glu=1) == HA_ERR_SHAPE
+    assert pack(w=odd) == HA_ERR_ALIGN and pack(glu=2) == HA_ERR_SHAPE
+    lint = lambda **kw: lib.ha_linear_tiled(*[{**dict(x=p, xs=4096, t=p, r=null, rs=0, act=0, o=p, os=4096, M=16, N=4096, K=4096, st=null), **kw}[k]
+                                              for k in ("x", "xs", "t", "r", "rs", "act", "o", "os", "M", "N", "K", "st")])
+    assert lint(t=null) == HA_ERR_NULL and lint(M=33) == HA_ERR_SHAPE and lint(K=100) == HA_ERR_SHAPE and lint(x=odd) == HA_ERR_ALIGN
+    assert lint(M=17, K=8192, xs=8192) == HA_ERR_SHAPE          # more than 16 rows: up to 4096 inputs
+    assert lint(K=16384, xs=16384, act=1, N=4096) == HA_ERR_SHAPE    # rows too long for registers: no activation
+    assert lint(act=1, r=p, rs=4096) == HA_ERR_SHAPE and lint(act=1, N=4095) == HA_ERR_SHAPE and lint(os=100) == HA_ERR_SHAPE
+    assert lint(r=p, rs=10) == HA_ERR_SHAPE and lint(act=3) == HA_ERR_SHAPE
+    norm = lambda **kw: lib.ha_rmsnorm(*[{**dict(x=p, xs=4096, w=p, dt=_ops.HA_BF16, M=4, K=4096, eps=C.c_float(1e-5), o=p, os=4096, st=null), **kw}[k]
+                                         for k in ("x", "xs", "w", "dt", "M", "K", "eps", "o", "os", "st")])
+    assert norm(w=null) == HA_ERR_NULL and norm(dt=9) == HA_ERR_DTYPE and norm(xs=100) == HA_ERR_SHAPE and norm(M=0) == HA_ERR_SHAPE
+    assert norm(eps=C.c_float(-1.0)) == HA_ERR_SHAPE
+    lib.ha_sparse_decode_fused_prefix_masked.restype = _C.c_int
+    fpm = lambda pre: lib.ha_sparse_decode_fused_prefix_masked(p, i64(4096), i64(128), p, p, _ops.HA_BF16, i64(8 * 1000 * 128), i64(1000 * 128), i64(128),
+                                                               p, i64(8000), i64(1000), p, 1, 32, 8, 8, 1, 1000, null, 4, 4, C.c_double(0.25),
+                                                               p, C.c_size_t(1 << 16), 1, null, pre, C.c_float(0.1), p, p, C.c_size_t(1 << 16), null)
+    assert fpm(null) == HA_ERR_NULL and fpm(odd) == HA_ERR_ALIGN
     assert lib.ha_swiglu(null, 64, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_NULL
     assert lib.ha_swiglu(p, 63, _ops.HA_BF16, 1, 32, p, null) == HA_ERR_SHAPE and lib.ha_swiglu(p, 64, 9, 1, 32, p, null) == HA_ERR_DTYPE
 

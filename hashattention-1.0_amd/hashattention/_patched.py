@@ -959,12 +959,13 @@ def _layer_takes_fast_path(layer, hidden_states):
 def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
                                position_embeddings=None, **kwargs):
     """`forward` of a transformers decoder layer whose attention module was converted.  A single-token step that the attention
-    module takes in five launches (`_fast_decode_slot`) runs the WHOLE layer in seven for up to 8 sequences (twelve calls above): input RMSNorm inside the QKV
-    projection, the attention step, residual inside the output projection, post-attention RMSNorm in front of and SwiGLU
-    behind the stacked gate/up projection, residual inside the down projection (the launches of `LlamaShapedDecoder`) -
-    instead of the ~25 library calls of the layer's own forward, which at these sizes are bound by the host.  Everything
-    else goes to the layer's own forward.  The fused forms round where the modules they replace round, so outputs differ
-    from the layer's own by the bf16 rounding of other summation orders only."""
+    module takes in five launches (`_fast_decode_slot`) runs the WHOLE layer in seven for up to 8 sequences: input RMSNorm
+    inside the QKV projection, the attention step, residual inside the output projection, post-attention RMSNorm in front of
+    and SwiGLU behind the stacked gate/up projection, residual inside the down projection (the launches of
+    `LlamaShapedDecoder`) - instead of the ~25 library calls of the layer's own forward, which at these sizes are bound by
+    the host.  Larger batches take nine to twelve calls (below).  Everything else goes to the layer's own forward.  The fused
+    forms round where the modules they replace round, so outputs differ from the layer's own by the bf16 rounding of other
+    summation orders only."""
     attn = layer.self_attn
     cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
     mods = getattr(attn, "fast_layer", False) and not kwargs.get("output_attentions") and _layer_takes_fast_path(layer, hidden_states)
@@ -975,10 +976,11 @@ def fast_decoder_layer_forward(layer, hidden_states, attention_mask=None, positi
         attn._sync_bit_cache(cache)
         slot = attn._fast_decode_slot(hidden_states, position_embeddings, attention_mask, cache)
         if slot is not None and hidden_states.shape[0] > FUSED_LAYER_MAX_ROWS:
-            # more sequences than the fused forms take: the same layer in ten to twelve calls - each RMSNorm one launch with the
+            # more sequences than the fused forms take: the same layer in nine to twelve calls - each RMSNorm one launch with the
             # module's two roundings, the attention step (the first residual inside its output projection), gate/up with SwiGLU
             # (9 to 32 sequences: one launch on a tiled copy of the stacked weight; above: the library's GEMM and ha_swiglu), the
-            # library's GEMM for the down projection, the second residual addition - instead of the library layer's ~26
+            # down projection (9 to 16 sequences: from tiles, the second residual inside; above: the library's GEMM and an
+            # addition) - instead of the library layer's ~26
             b, _, hidden = hidden_states.shape
             mlp, n1, n2, gate, _, down = mods
             h = torch.empty_like(hidden_states)
